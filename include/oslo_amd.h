@@ -1,0 +1,204 @@
+/*
+ * oslo_amd.h -- C ABI of the MI355X (gfx950) kernel-fusion library.
+ *
+ * One shared library, liboslo_amd.so, replaces the native module `oslo_kernels`
+ * of tunib-ai/oslo (oslo/fused_kernels/bindings/pybind_kernels.cpp:159-177) and
+ * the TorchScript-fused elementwise epilogues of
+ * oslo/fused_kernels_utils.py:259-308.
+ *
+ * Conventions shared by every entry point:
+ *   - plain device pointers and sizes; no torch or ATen type appears here;
+ *   - tensors are dense row-major ("contiguous"), last dimension fastest;
+ *   - `dtype` selects the storage type of every `void*` tensor argument of a
+ *     call (enum oslo_dtype); arithmetic is always done in fp32;
+ *   - work is enqueued on `stream` (a hipStream_t; NULL = the null stream) and
+ *     the call returns without synchronising;
+ *   - no entry point allocates or frees device memory;
+ *   - the return value is OSLO_OK (0) or a negative oslo_status; nothing throws.
+ *     oslo_last_error() gives the text of the calling thread's last failure.
+ */
+#ifndef OSLO_AMD_H_
+#define OSLO_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *oslo_stream_t; /* a hipStream_t */
+
+enum oslo_dtype { OSLO_F32 = 0, OSLO_F16 = 1, OSLO_BF16 = 2 };
+
+enum oslo_status {
+  OSLO_OK = 0,
+  OSLO_E_BAD_ARG = -1,     /* null pointer, negative size, unknown enum value   */
+  OSLO_E_UNSUPPORTED = -2, /* shape outside the supported range (see limits)   */
+  OSLO_E_LAUNCH = -3       /* the HIP runtime refused the launch               */
+};
+
+/* How a set mask byte changes a score (oslo_softmax_masked_fwd). */
+enum oslo_mask_mode {
+  /* e = scale*x + (-10000): what the unfused attention computes
+   * (oslo/models/gpt2/modeling_gpt2.py:214-216). */
+  OSLO_MASK_ADD = 0,
+  /* e = -10000: what the reference's fused kernel computes
+   * (oslo/fused_kernels/includes/fused_softmax.h:171-175). The two differ only
+   * on rows whose every key is masked. */
+  OSLO_MASK_REPLACE = 1
+};
+
+/* Library identity and limits ------------------------------------------- */
+
+/* ABI version of this header; bumped on any incompatible change. */
+int oslo_abi_version(void);
+/* Longest softmax row (key length) any softmax entry point accepts. The
+ * reference stops at 2048 (oslo/fused_kernels/fused_softmax.cu:48,
+ * oslo/fused_kernels/fused_triang_softmax.cu:39). */
+int oslo_softmax_max_cols(void);
+/* Text for a status code; never NULL. */
+const char *oslo_status_string(int status);
+/* Text of the calling thread's most recent failure ("" if none). */
+const char *oslo_last_error(void);
+
+/* Scale + causal mask + softmax ------------------------------------------ */
+
+/*
+ * y[b,h,r,k] = softmax over k<=r of ( scale*x[b,h,r,k] + pad_add[b,k] ),
+ * y[b,h,r,k] = 0 for k>r. x, y: [batch, heads, S, S]; y may alias x.
+ * pad_add: NULL or fp32 [batch, S], added after scaling (the order of the
+ * unfused path, oslo/models/gpt2/modeling_gpt2.py:197-216).
+ * Replaces scaled_upper_triang_masked_softmax::fwd
+ * (oslo/fused_kernels/bindings/pybind_kernels.cpp:98-105,
+ *  oslo/fused_kernels/fused_triang_softmax.cu:32-62,
+ *  kernel oslo/fused_kernels/includes/fused_triang_softmax.h:134-251), which
+ * has no pad argument: its caller adds the mask into a copy of x first
+ * (oslo/fused_kernels_utils.py:444-449).
+ */
+int oslo_softmax_causal_fwd(void *y, const void *x, const float *pad_add,
+                            float scale, int64_t batch, int64_t heads,
+                            int64_t S, int dtype, oslo_stream_t stream);
+
+/*
+ * dx[n,r,k] = scale * y[n,r,k] * ( g[n,r,k] - sum_{j<=r} g[n,r,j]*y[n,r,j] )
+ * for k<=r, 0 for k>r. g, y, dx: [bh, S, S]; dx may alias g (the reference
+ * always writes over g). Entries of g and y above the diagonal are not read.
+ * Replaces scaled_upper_triang_masked_softmax::bwd
+ * (oslo/fused_kernels/bindings/pybind_kernels.cpp:107-123,
+ *  oslo/fused_kernels/fused_triang_softmax.cu:64-96,
+ *  kernel oslo/fused_kernels/includes/fused_triang_softmax.h:253-351).
+ */
+int oslo_softmax_causal_bwd(void *dx, const void *g, const void *y, float scale,
+                            int64_t bh, int64_t S, int dtype,
+                            oslo_stream_t stream);
+
+/* Scale + key/padding mask + softmax -------------------------------------- */
+
+/*
+ * y[b,h,q,k] = softmax over k of e, e per `mask_mode` where
+ * mask[b*mask_stride_b + q*mask_stride_q + k] != 0, else scale*x[b,h,q,k].
+ * x, y: [B, H, Sq, Sk]; y may alias x. mask: NULL (nothing masked) or bytes;
+ * a stride of 0 broadcasts that dimension, so a [B,1,1,Sk] key mask is passed
+ * as (mask_stride_b=Sk, mask_stride_q=0) and the reference's materialised
+ * [B|1,1,Sq,Sk] mask as (Sq*Sk|0, Sk).
+ * Replaces scaled_masked_softmax::fwd
+ * (oslo/fused_kernels/bindings/pybind_kernels.cpp:46-57,
+ *  oslo/fused_kernels/fused_softmax.cu:37-80,
+ *  kernel oslo/fused_kernels/includes/fused_softmax.h:111-229).
+ */
+int oslo_softmax_masked_fwd(void *y, const void *x, const uint8_t *mask,
+                            int64_t mask_stride_b, int64_t mask_stride_q,
+                            int mask_mode, float scale, int64_t B, int64_t H,
+                            int64_t Sq, int64_t Sk, int dtype,
+                            oslo_stream_t stream);
+
+/*
+ * dx[n,k] = scale * y[n,k] * ( g[n,k] - sum_j g[n,j]*y[n,j] ).
+ * g, y, dx: [rows, Sk]; dx may alias g.
+ * Replaces scaled_masked_softmax::bwd
+ * (oslo/fused_kernels/bindings/pybind_kernels.cpp:59-75,
+ *  oslo/fused_kernels/fused_softmax.cu:82-115,
+ *  kernel oslo/fused_kernels/includes/fused_softmax.h:231-325).
+ */
+int oslo_softmax_masked_bwd(void *dx, const void *g, const void *y, float scale,
+                            int64_t rows, int64_t Sk, int dtype,
+                            oslo_stream_t stream);
+
+/*
+ * Rows of attention scores one 128-thread block of the reference's kernels
+ * handles: an implementation detail the reference exports so that its
+ * availability gate can test divisibility
+ * (oslo/fused_kernels/includes/fused_softmax.h:328-340,
+ *  oslo/fused_kernels/bindings/pybind_kernels.cpp:77-83,
+ *  used at oslo/fused_kernels_utils.py:465). Pure integer arithmetic with the
+ * reference's 32-lane constants, so callers see the reference's numbers. The
+ * kernels of this library have no divisibility requirement.
+ */
+int oslo_get_batch_per_block(int sq, int sk, int batches, int heads);
+
+/* Bias + GeLU (tanh form) -------------------------------------------------- */
+
+/*
+ * out[r,c] = gelu_tanh( y[r,c] + bias[c] ),
+ * gelu_tanh(x) = 0.5*x*(1 + tanh(0.79788456*x*(1 + 0.044715*x*x))).
+ * y, out: [rows, cols]; bias: [cols]; out may alias y.
+ * Replaces bias_gelu_fwb (oslo/fused_kernels_utils.py:295-298).
+ */
+int oslo_bias_gelu_fwd(void *out, const void *y, const void *bias, int64_t rows,
+                       int64_t cols, int dtype, oslo_stream_t stream);
+
+/*
+ * Bytes of fp32 workspace the two backward entry points below need to produce
+ * dbias for a [rows, cols] problem (0 if rows or cols is 0).
+ */
+size_t oslo_colsum_workspace_bytes(int64_t rows, int64_t cols);
+
+/*
+ * dy[r,c] = g[r,c] * gelu_tanh'( y[r,c] + bias[c] ) and, if dbias != NULL,
+ * dbias[c] = sum_r dy[r,c] (fp32 sum of the unrounded products, stored in
+ * `dtype`). workspace: oslo_colsum_workspace_bytes(rows, cols) bytes of device
+ * memory, required only when dbias != NULL. dy may alias g.
+ * Replaces bias_gelu_bwd (oslo/fused_kernels_utils.py:301-308) and the
+ * separate reduction autograd runs on the full-shape bias gradient that
+ * FusedBiasGeLU.backward returns (oslo/fused_kernels_utils.py:376-380).
+ */
+int oslo_bias_gelu_bwd(void *dy, void *dbias, float *workspace, const void *g,
+                       const void *y, const void *bias, int64_t rows,
+                       int64_t cols, int dtype, oslo_stream_t stream);
+
+/* Bias + dropout (+ residual) ----------------------------------------------- */
+
+/*
+ * out[r,c] = keep[r,c] * (x[r,c] + bias[c]) / (1-p) + residual[r,c].
+ * bias and residual may each be NULL (term dropped). p in [0,1); p == 0 keeps
+ * everything and draws no random numbers. keep[i] for the flat element index
+ * i = r*cols + c is word (i mod 4) of Philox4x32-10 with key = philox_seed and
+ * counter = (philox_offset/4 as 64 bits, i/4 as 64 bits), compared as
+ * keep = word >= floor(p * 2^32). One call consumes 4 units of generator
+ * offset. out may alias x.
+ * Replaces bias_dropout / bias_dropout_residual
+ * (oslo/fused_kernels_utils.py:259-292).
+ */
+int oslo_bias_dropout_add_fwd(void *out, const void *x, const void *bias,
+                              const void *residual, float p,
+                              uint64_t philox_seed, uint64_t philox_offset,
+                              int64_t rows, int64_t cols, int dtype,
+                              oslo_stream_t stream);
+
+/*
+ * dx[r,c] = keep[r,c] * g[r,c] / (1-p) with the mask regenerated from the same
+ * (seed, offset); if dbias != NULL, dbias[c] = sum_r dx[r,c] (workspace as for
+ * oslo_bias_gelu_bwd). The gradient of the residual is g itself. dx may alias
+ * g. The reference leaves this to TorchScript autodiff of
+ * oslo/fused_kernels_utils.py:259-292.
+ */
+int oslo_bias_dropout_add_bwd(void *dx, void *dbias, float *workspace,
+                              const void *g, float p, uint64_t philox_seed,
+                              uint64_t philox_offset, int64_t rows,
+                              int64_t cols, int dtype, oslo_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OSLO_AMD_H_ */

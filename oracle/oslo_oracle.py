@@ -1,0 +1,220 @@
+"""CPU restatement of the reference's arithmetic for the kernel-fusion path.
+
+THIS IS TEST INFRASTRUCTURE. Only tests, the smoke check and the cpu_baseline
+leg of the benchmark may import it; nothing the library ships routes through
+it. It is written with numpy only, one explicit step per line, and is pinned in
+tests/test_oracle.py against independent evidence: library routines
+(torch.softmax, torch.nn.functional.gelu(approximate="tanh"), autograd and
+gradcheck), pure-Python float64 loops on tiny inputs, closed-form special cases,
+and the published known-answer vectors of Philox4x32-10.
+
+What each function follows in the reference (paths relative to the reference
+root):
+
+* softmax_causal / softmax_masked(mode="add"): the unfused attention,
+  oslo/models/gpt2/modeling_gpt2.py:194-218 (scale, causal where(), additive
+  padding mask, softmax), which oslo/models/gptj/modeling_gptj.py:151-180 and
+  oslo/models/gpt_neo/modeling_gpt_neo.py:195-214 repeat;
+* softmax_masked(mode="replace"): the fused kernel,
+  oslo/fused_kernels/includes/fused_softmax.h:171-222;
+* softmax_bwd: oslo/fused_kernels/includes/fused_softmax.h:283-319 and
+  oslo/fused_kernels/includes/fused_triang_softmax.h:305-347;
+* bias_gelu_fwd / bias_gelu_bwd: oslo/fused_kernels_utils.py:295-308 and the
+  sum_to_size autograd applies to FusedBiasGeLU.backward's second output (:380);
+* bias_dropout_add_fwd / _bwd: oslo/fused_kernels_utils.py:259-292
+  (F.dropout(x + bias, p, training) + residual) given an explicit keep mask;
+* get_batch_per_block: oslo/fused_kernels/includes/fused_softmax.h:328-340;
+* reference_is_available: oslo/fused_kernels_utils.py:461-479;
+* philox4x32_10 / dropout_keep_mask: no counterpart in the reference (it uses
+  torch's generator through F.dropout); they restate the published Philox
+  algorithm and this library's documented element -> counter mapping.
+
+Parity unpinned: none of the functions above. The reference itself holds no
+golden vectors for this path.
+"""
+
+import numpy as np
+
+MASK_VALUE = -10000.0
+
+
+def _acc(dtype):
+    return np.dtype(dtype).type
+
+
+# ---------------------------------------------------------------------------
+# softmax
+# ---------------------------------------------------------------------------
+
+def _softmax_lastdim(e):
+    """softmax over the last axis of e, entries may be -inf (excluded)."""
+    m = np.max(e, axis=-1, keepdims=True)
+    p = np.exp(e - m)
+    return p / np.sum(p, axis=-1, keepdims=True, dtype=e.dtype)
+
+
+def softmax_causal(x, scale, pad_add=None, dtype=np.float32):
+    """x [B,H,S,S]; pad_add None or [B,S] additive. Row r attends keys 0..r."""
+    t = _acc(dtype)
+    x = np.asarray(x, dtype=dtype)
+    b, h, s, s2 = x.shape
+    assert s == s2
+    e = x * t(scale)                                      # scale first ...
+    if pad_add is not None:
+        e = e + np.asarray(pad_add, dtype=dtype)[:, None, None, :]  # ... then the mask
+    keep = np.tril(np.ones((s, s), dtype=bool))
+    e = np.where(keep, e, t(-np.inf))
+    return _softmax_lastdim(e)
+
+
+def softmax_masked(x, mask, scale, mode="add", dtype=np.float32):
+    """x [B,H,Sq,Sk]; mask None or boolean broadcastable to [B,1,Sq,Sk],
+    True = masked. mode "add": e = scale*x + (-10000); "replace": e = -10000."""
+    t = _acc(dtype)
+    x = np.asarray(x, dtype=dtype)
+    e = x * t(scale)
+    if mask is not None:
+        mask = np.broadcast_to(np.asarray(mask, dtype=bool), (x.shape[0], 1) + x.shape[2:])
+        if mode == "add":
+            e = np.where(mask, e + t(MASK_VALUE), e)
+        elif mode == "replace":
+            e = np.where(mask, t(MASK_VALUE), e)
+        else:
+            raise ValueError(mode)
+    return _softmax_lastdim(e)
+
+
+def softmax_bwd(g, y, scale, causal=False, dtype=np.float32):
+    """dx = scale * (g*y - y * sum_k(g*y)); with causal=True only k <= r takes
+    part and dx is 0 above the diagonal. g, y: [..., Sq, Sk]."""
+    t = _acc(dtype)
+    g = np.asarray(g, dtype=dtype)
+    y = np.asarray(y, dtype=dtype)
+    if causal:
+        s = y.shape[-1]
+        keep = np.tril(np.ones((s, s), dtype=bool))
+        g = np.where(keep, g, t(0))
+        y = np.where(keep, y, t(0))
+    gy = g * y
+    total = np.sum(gy, axis=-1, keepdims=True, dtype=dtype)
+    return t(scale) * (gy - y * total)
+
+
+def get_batch_per_block(sq, sk, batches, heads):
+    log2_elements = 0
+    while (1 << log2_elements) < sk:
+        log2_elements += 1
+    n2 = 1 << log2_elements
+    warp_size = n2 if n2 < 32 else 32
+    rows_per_warp = 2 if n2 <= 128 else 1
+    return rows_per_warp * (128 // warp_size)
+
+
+def reference_is_available(is_half, bsz, np_, sq, sk, use_triang_mask):
+    """The reference's gate, with `is_half` standing for dtype == torch.half."""
+    if not is_half or sk > 2048 or sk <= 0:
+        return False
+    bpb = get_batch_per_block(sq, sk, bsz, np_)
+    if use_triang_mask:
+        return sq == sk and (sk <= 64 or sk % 4 == 0) and (bsz * np_) % bpb == 0
+    return sq > 1 and sq % bpb == 0
+
+
+# ---------------------------------------------------------------------------
+# bias + GeLU
+# ---------------------------------------------------------------------------
+
+def bias_gelu_fwd(y, bias, dtype=np.float32):
+    t = _acc(dtype)
+    x = np.asarray(y, dtype=dtype) + np.asarray(bias, dtype=dtype)
+    return x * t(0.5) * (t(1.0) + np.tanh(t(0.79788456) * x * (t(1) + t(0.044715) * x * x)))
+
+
+def bias_gelu_bwd(g, y, bias, dtype=np.float32):
+    """Returns (dy, dbias); dbias sums dy over every axis but the last."""
+    t = _acc(dtype)
+    g = np.asarray(g, dtype=dtype)
+    x = np.asarray(y, dtype=dtype) + np.asarray(bias, dtype=dtype)
+    tanh_out = np.tanh(t(0.79788456) * x * (t(1) + t(0.044715) * x * x))
+    ff = t(0.5) * x * ((t(1) - tanh_out * tanh_out) * (t(0.79788456) + t(0.1070322243) * x * x)) \
+        + t(0.5) * (t(1) + tanh_out)
+    dy = ff * g
+    dbias = dy.reshape(-1, dy.shape[-1]).sum(axis=0, dtype=np.float64).astype(dtype)
+    return dy, dbias
+
+
+# ---------------------------------------------------------------------------
+# Philox4x32-10 and the dropout mask
+# ---------------------------------------------------------------------------
+
+_M0, _M1 = np.uint64(0xD2511F53), np.uint64(0xCD9E8D57)
+_W0, _W1 = np.uint32(0x9E3779B9), np.uint32(0xBB67AE85)
+_LO = np.uint64(0xFFFFFFFF)
+_S32 = np.uint64(32)
+
+
+def philox4x32_10(key, counter):
+    """key: 2 uint32 scalars; counter: 4 arrays of uint32 (same shape).
+    Returns 4 arrays of uint32: ten rounds of the Philox-4x32 bijection
+    (Salmon, Moraes, Dror, Shaw, SC'11), key bumped by the Weyl constants
+    between rounds."""
+    k0, k1 = np.uint32(key[0]), np.uint32(key[1])
+    c0, c1, c2, c3 = [np.asarray(c, dtype=np.uint32) for c in counter]
+    with np.errstate(over="ignore"):
+        for _ in range(10):
+            p0 = _M0 * c0.astype(np.uint64)
+            p1 = _M1 * c2.astype(np.uint64)
+            hi0, lo0 = (p0 >> _S32).astype(np.uint32), (p0 & _LO).astype(np.uint32)
+            hi1, lo1 = (p1 >> _S32).astype(np.uint32), (p1 & _LO).astype(np.uint32)
+            c0, c1, c2, c3 = hi1 ^ c1 ^ k0, lo1, hi0 ^ c3 ^ k1, lo0
+            k0 = np.uint32((int(k0) + int(_W0)) & 0xFFFFFFFF)
+            k1 = np.uint32((int(k1) + int(_W1)) & 0xFFFFFFFF)
+    return c0, c1, c2, c3
+
+
+def dropout_threshold(p):
+    t = float(np.float32(p)) * 4294967296.0
+    return 0xFFFFFFFF if t >= 4294967295.0 else int(t)
+
+
+def dropout_keep_mask(seed, offset, n, p):
+    """keep[i], i in [0, n): word (i mod 4) of Philox4x32-10 with key = seed
+    and counter = (offset // 4 as 64 bits, i // 4 as 64 bits), kept when
+    word >= floor(p * 2^32)."""
+    groups = (n + 3) // 4
+    g = np.arange(groups, dtype=np.uint64)
+    block = np.uint64(offset // 4)
+    c0 = np.full(groups, block & _LO, dtype=np.uint64).astype(np.uint32)
+    c1 = np.full(groups, block >> _S32, dtype=np.uint64).astype(np.uint32)
+    c2 = (g & _LO).astype(np.uint32)
+    c3 = (g >> _S32).astype(np.uint32)
+    key = (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)
+    words = np.stack(philox4x32_10(key, (c0, c1, c2, c3)), axis=1).reshape(-1)[:n]
+    return words >= np.uint32(dropout_threshold(p))
+
+
+def bias_dropout_add_fwd(x, bias, residual, p, keep, dtype=np.float32):
+    """F.dropout(x + bias, p) + residual with the keep mask given. keep: bool
+    array of x's shape (ignored when p == 0)."""
+    t = _acc(dtype)
+    out = np.asarray(x, dtype=dtype)
+    if bias is not None:
+        out = out + np.asarray(bias, dtype=dtype)
+    if p > 0:
+        scale = t(1.0 / (1.0 - float(np.float32(p))))
+        out = np.where(keep, out * scale, t(0))
+    if residual is not None:
+        out = out + np.asarray(residual, dtype=dtype)
+    return out
+
+
+def bias_dropout_add_bwd(g, p, keep, dtype=np.float32):
+    """Returns (dx, dbias, dresidual)."""
+    t = _acc(dtype)
+    g = np.asarray(g, dtype=dtype)
+    dx = g
+    if p > 0:
+        scale = t(1.0 / (1.0 - float(np.float32(p))))
+        dx = np.where(keep, g * scale, t(0))
+    dbias = dx.reshape(-1, dx.shape[-1]).sum(axis=0, dtype=np.float64).astype(dtype)
+    return dx, dbias, g

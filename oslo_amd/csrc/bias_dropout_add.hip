@@ -1,0 +1,257 @@
+// Bias + dropout (+ residual add), forward and backward, for gfx950:
+// out = dropout(x + bias, p) + residual, the arithmetic of bias_dropout /
+// bias_dropout_residual (oslo/fused_kernels_utils.py:259-292). The keep mask
+// is never stored: forward and backward both derive it from
+// (seed, offset, element index) with Philox4x32-10, so the backward reads only
+// the incoming gradient.
+
+#include "elementwise.hpp"
+#include "philox.h"
+
+namespace oslo {
+namespace {
+
+// keep flags of VEC consecutive elements starting at flat index i0 (a multiple
+// of VEC when VEC is 4 or 8; anything when VEC is 1).
+template <int VEC>
+__device__ __forceinline__ void keep_flags(bool (&keep)[VEC], uint64_t seed,
+                                           uint64_t offset, uint64_t i0,
+                                           uint32_t threshold) {
+  if constexpr (VEC == 1) {
+    const Philox4 d = dropout_draw(seed, offset, i0 >> 2);
+    keep[0] = d.w[i0 & 3] >= threshold;
+  } else {
+    static_assert(VEC % 4 == 0, "vector paths draw whole groups of four");
+#pragma unroll
+    for (int q = 0; q < VEC / 4; ++q) {
+      const Philox4 d = dropout_draw(seed, offset, (i0 >> 2) + q);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) keep[4 * q + j] = d.w[j] >= threshold;
+    }
+  }
+}
+
+template <typename T, int VEC, bool DROP, bool HAS_BIAS, bool HAS_RES>
+__global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_fwd_kernel(
+    T *out, const T *x, const T *__restrict__ bias, const T *residual,
+    float keep_scale, uint32_t threshold, uint64_t seed, uint64_t offset,
+    int64_t rows, int64_t cols, int rows_per_block) {
+  const int64_t c0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+  if (c0 >= cols) return; // no barrier in this kernel
+  float b[VEC];
+  if constexpr (HAS_BIAS) load_f32_cached<T, VEC>(b, bias + c0);
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+  const int64_t r1 = min(rows, r0 + rows_per_block);
+  const int TY = blockDim.y;
+  for (int64_t r = r0 + threadIdx.y; r < r1; r += (int64_t)TY * kRowUnroll) {
+    float tx[kRowUnroll][VEC], tr[kRowUnroll][VEC];
+#pragma unroll
+    for (int u = 0; u < kRowUnroll; ++u) {
+      const int64_t rr = r + (int64_t)u * TY;
+      if (rr < r1) {
+        load_f32<T, VEC>(tx[u], x + rr * cols + c0);
+        if constexpr (HAS_RES) load_f32<T, VEC>(tr[u], residual + rr * cols + c0);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kRowUnroll; ++u) {
+      const int64_t rr = r + (int64_t)u * TY;
+      if (rr < r1) {
+        bool keep[VEC];
+        if constexpr (DROP)
+          keep_flags<VEC>(keep, seed, offset, (uint64_t)(rr * cols + c0),
+                          threshold);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          float t = tx[u][j];
+          if constexpr (HAS_BIAS) t += b[j];
+          if constexpr (DROP) t = keep[j] ? t * keep_scale : 0.f;
+          if constexpr (HAS_RES) t += tr[u][j];
+          tx[u][j] = t;
+        }
+        store_f32<T, VEC>(out + rr * cols + c0, tx[u]);
+      }
+    }
+  }
+}
+
+template <typename T, int VEC, bool DROP, bool WANT_DBIAS>
+__global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_bwd_kernel(
+    T *dx, float *__restrict__ partial, const T *g, float keep_scale,
+    uint32_t threshold, uint64_t seed, uint64_t offset, int64_t rows,
+    int64_t cols, int rows_per_block) {
+  const int64_t c0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+  const bool col_ok = c0 < cols;
+  float acc[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+  if (col_ok) {
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = min(rows, r0 + rows_per_block);
+    const int TY = blockDim.y;
+    for (int64_t r = r0 + threadIdx.y; r < r1; r += (int64_t)TY * kRowUnroll) {
+      float tg[kRowUnroll][VEC];
+#pragma unroll
+      for (int u = 0; u < kRowUnroll; ++u) {
+        const int64_t rr = r + (int64_t)u * TY;
+        if (rr < r1) load_f32<T, VEC>(tg[u], g + rr * cols + c0);
+      }
+#pragma unroll
+      for (int u = 0; u < kRowUnroll; ++u) {
+        const int64_t rr = r + (int64_t)u * TY;
+        if (rr < r1) {
+          bool keep[VEC];
+          if constexpr (DROP)
+            keep_flags<VEC>(keep, seed, offset, (uint64_t)(rr * cols + c0),
+                            threshold);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            if constexpr (DROP)
+              tg[u][j] = keep[j] ? tg[u][j] * keep_scale : 0.f;
+            if constexpr (WANT_DBIAS) acc[j] += tg[u][j];
+          }
+          // with no dropout dx == g bit for bit; still written, dx may be a
+          // different buffer
+          store_f32<T, VEC>(dx + rr * cols + c0, tg[u]);
+        }
+      }
+    }
+  }
+  if constexpr (WANT_DBIAS)
+    write_colsum_partial<VEC>(acc, partial, cols, c0, col_ok);
+}
+
+struct DropArgs {
+  float keep_scale;
+  uint32_t threshold;
+  uint64_t seed, offset;
+  bool drop;
+};
+
+template <typename T, int VEC>
+int launch_fwd(T *out, const T *x, const T *bias, const T *res,
+               const DropArgs &a, int64_t rows, int64_t cols,
+               hipStream_t stream) {
+  const EwPlan p = plan_elementwise(rows, cols / VEC, kRowsPerBlockFwd);
+  auto go = [&]<bool DROP, bool HB, bool HR>() {
+    bias_dropout_add_fwd_kernel<T, VEC, DROP, HB, HR>
+        <<<p.grid, p.block, 0, stream>>>(out, x, bias, res, a.keep_scale,
+                                         a.threshold, a.seed, a.offset, rows,
+                                         cols, p.rows_per_block);
+  };
+  const int sel = (a.drop ? 4 : 0) | (bias ? 2 : 0) | (res ? 1 : 0);
+  switch (sel) {
+  case 0: go.template operator()<false, false, false>(); break;
+  case 1: go.template operator()<false, false, true>(); break;
+  case 2: go.template operator()<false, true, false>(); break;
+  case 3: go.template operator()<false, true, true>(); break;
+  case 4: go.template operator()<true, false, false>(); break;
+  case 5: go.template operator()<true, false, true>(); break;
+  case 6: go.template operator()<true, true, false>(); break;
+  default: go.template operator()<true, true, true>(); break;
+  }
+  return check_launch("bias_dropout_add_fwd");
+}
+
+template <typename T, int VEC>
+int launch_bwd(T *dx, T *dbias, float *ws, const T *g, const DropArgs &a,
+               int64_t rows, int64_t cols, hipStream_t stream) {
+  const EwPlan p = plan_elementwise(rows, cols / VEC, kRowsPerBlockBwd);
+  auto go = [&]<bool DROP, bool WANT>() {
+    bias_dropout_add_bwd_kernel<T, VEC, DROP, WANT>
+        <<<p.grid, p.block, 0, stream>>>(dx, ws, g, a.keep_scale, a.threshold,
+                                         a.seed, a.offset, rows, cols,
+                                         p.rows_per_block);
+  };
+  if (a.drop) {
+    if (dbias) go.template operator()<true, true>();
+    else go.template operator()<true, false>();
+  } else {
+    if (dbias) go.template operator()<false, true>();
+    else go.template operator()<false, false>();
+  }
+  int s = check_launch("bias_dropout_add_bwd");
+  if (s != OSLO_OK || !dbias) return s;
+  launch_colsum_finish<T>(dbias, ws, (int)p.grid.y, cols, stream);
+  return check_launch("bias_dropout_add_bwd(dbias)");
+}
+
+int make_args(const char *name, float p, uint64_t seed, uint64_t offset,
+              DropArgs *a) {
+  if (!(p >= 0.0f) || !(p < 1.0f))
+    return fail(OSLO_E_BAD_ARG, "%s: p = %g is outside [0, 1)", name, (double)p);
+  a->drop = p > 0.0f;
+  a->keep_scale = (float)(1.0 / (1.0 - (double)p));
+  a->threshold = dropout_threshold(p);
+  a->seed = seed;
+  a->offset = offset;
+  return OSLO_OK;
+}
+
+} // namespace
+} // namespace oslo
+
+extern "C" int oslo_bias_dropout_add_fwd(void *out, const void *x,
+                                         const void *bias, const void *residual,
+                                         float p, uint64_t philox_seed,
+                                         uint64_t philox_offset, int64_t rows,
+                                         int64_t cols, int dtype,
+                                         oslo_stream_t stream) {
+  using namespace oslo;
+  if (rows < 0 || cols < 0)
+    return fail(OSLO_E_BAD_ARG, "bias_dropout_add_fwd: negative size");
+  DropArgs a;
+  int s = make_args("bias_dropout_add_fwd", p, philox_seed, philox_offset, &a);
+  if (s != OSLO_OK) return s;
+  if (rows == 0 || cols == 0) return OSLO_OK;
+  if (!out || !x) return fail(OSLO_E_BAD_ARG, "bias_dropout_add_fwd: null tensor");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  OSLO_DISPATCH_DTYPE(dtype, {
+    constexpr int V = Io<T>::kVec;
+    const bool vec = cols % V == 0 && aligned16(out) && aligned16(x) &&
+                     aligned16(bias) && aligned16(residual);
+    T *o = static_cast<T *>(out);
+    const T *xx = static_cast<const T *>(x);
+    const T *bb = static_cast<const T *>(bias);
+    const T *rr = static_cast<const T *>(residual);
+    return vec ? launch_fwd<T, V>(o, xx, bb, rr, a, rows, cols, st)
+               : launch_fwd<T, 1>(o, xx, bb, rr, a, rows, cols, st);
+  });
+  return OSLO_OK;
+}
+
+extern "C" int oslo_bias_dropout_add_bwd(void *dx, void *dbias,
+                                         float *workspace, const void *g,
+                                         float p, uint64_t philox_seed,
+                                         uint64_t philox_offset, int64_t rows,
+                                         int64_t cols, int dtype,
+                                         oslo_stream_t stream) {
+  using namespace oslo;
+  if (rows < 0 || cols < 0)
+    return fail(OSLO_E_BAD_ARG, "bias_dropout_add_bwd: negative size");
+  DropArgs a;
+  int s = make_args("bias_dropout_add_bwd", p, philox_seed, philox_offset, &a);
+  if (s != OSLO_OK) return s;
+  if (cols == 0) return OSLO_OK;
+  if (dbias && !workspace && rows > 0)
+    return fail(OSLO_E_BAD_ARG, "bias_dropout_add_bwd: dbias needs a workspace");
+  if (rows > 0 && (!dx || !g))
+    return fail(OSLO_E_BAD_ARG, "bias_dropout_add_bwd: null tensor");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  OSLO_DISPATCH_DTYPE(dtype, {
+    if (rows == 0) {
+      if (dbias)
+        launch_colsum_finish<T>(static_cast<T *>(dbias), nullptr, 0, cols, st);
+      return check_launch("bias_dropout_add_bwd(dbias)");
+    }
+    constexpr int V = Io<T>::kVec;
+    const bool vec = cols % V == 0 && aligned16(dx) && aligned16(g) &&
+                     aligned16(workspace);
+    T *d = static_cast<T *>(dx);
+    T *db = static_cast<T *>(dbias);
+    const T *gg = static_cast<const T *>(g);
+    return vec ? launch_bwd<T, V>(d, db, workspace, gg, a, rows, cols, st)
+               : launch_bwd<T, 1>(d, db, workspace, gg, a, rows, cols, st);
+  });
+  return OSLO_OK;
+}

@@ -1,0 +1,199 @@
+// Bias + GeLU (tanh form), forward and backward, for gfx950. The arithmetic is
+// that of bias_gelu_fwb / bias_gelu_bwd (oslo/fused_kernels_utils.py:295-308)
+// rewritten around the identity 0.5*(1 + tanh(u)) = 1/(1 + exp(-2u)), which
+// needs one v_exp_f32 and one v_rcp_f32 per element. The backward also emits
+// the bias gradient (a column sum), which the reference leaves to a separate
+// full-tensor reduction by autograd (oslo/fused_kernels_utils.py:376-380).
+
+#include "elementwise.hpp"
+
+namespace oslo {
+namespace {
+
+// gelu_tanh(x) = x * s(x), s(x) = 1/(1 + exp(-2u)), u = K*x*(1 + A*x^2).
+constexpr float kGeluK = 0.79788456f;
+constexpr float kGeluA = 0.044715f;
+constexpr float kLog2eF = 1.4426950408889634f;
+// -2u*log2(e) = x * (kW0 + kW1*x^2)
+constexpr float kW0 = -2.0f * kLog2eF * kGeluK;
+constexpr float kW1 = kW0 * kGeluA;
+// 2*du/dx = kD0 + kD1*x^2   (kD1 = 2*3*A*K; 3*A*K is the reference's 0.1070322243)
+constexpr float kD0 = 2.0f * kGeluK;
+constexpr float kD1 = 2.0f * 0.1070322243f;
+
+__device__ __forceinline__ float sigmoid_2u(float x, float x2) {
+  const float w = x * __builtin_fmaf(x2, kW1, kW0);
+  const float e = __builtin_amdgcn_exp2f(w); // exp(-2u); inf for very negative x
+  return __builtin_amdgcn_rcpf(1.0f + e);    // rcp(inf) = 0
+}
+
+__device__ __forceinline__ float gelu_fwd(float x) {
+  return x * sigmoid_2u(x, x * x);
+}
+
+// d/dx [x*s] = s + x*s*(1-s)*2u'
+__device__ __forceinline__ float gelu_grad(float x) {
+  const float x2 = x * x;
+  const float s = sigmoid_2u(x, x2);
+  const float q = x * __builtin_fmaf(x2, kD1, kD0);
+  return __builtin_fmaf(q, s * (1.0f - s), s);
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlockThreads) void bias_gelu_fwd_kernel(
+    T *out, const T *y, const T *__restrict__ bias, int64_t rows, int64_t cols,
+    int rows_per_block) {
+  const int64_t c0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+  if (c0 >= cols) return; // no barrier in this kernel
+  float b[VEC];
+  load_f32_cached<T, VEC>(b, bias + c0);
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+  const int64_t r1 = min(rows, r0 + rows_per_block);
+  const int TY = blockDim.y;
+  for (int64_t r = r0 + threadIdx.y; r < r1; r += (int64_t)TY * kRowUnroll) {
+    float t[kRowUnroll][VEC];
+#pragma unroll
+    for (int u = 0; u < kRowUnroll; ++u) {
+      const int64_t rr = r + (int64_t)u * TY;
+      if (rr < r1) load_f32<T, VEC>(t[u], y + rr * cols + c0);
+    }
+#pragma unroll
+    for (int u = 0; u < kRowUnroll; ++u) {
+      const int64_t rr = r + (int64_t)u * TY;
+      if (rr < r1) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) t[u][j] = gelu_fwd(t[u][j] + b[j]);
+        store_f32<T, VEC>(out + rr * cols + c0, t[u]);
+      }
+    }
+  }
+}
+
+template <typename T, int VEC, bool WANT_DBIAS>
+__global__ __launch_bounds__(kBlockThreads) void bias_gelu_bwd_kernel(
+    T *dy, float *__restrict__ partial, const T *g, const T *y,
+    const T *__restrict__ bias, int64_t rows, int64_t cols,
+    int rows_per_block) {
+  const int64_t c0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+  const bool col_ok = c0 < cols;
+  float acc[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+  if (col_ok) {
+    float b[VEC];
+    load_f32_cached<T, VEC>(b, bias + c0);
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = min(rows, r0 + rows_per_block);
+    const int TY = blockDim.y;
+    for (int64_t r = r0 + threadIdx.y; r < r1; r += (int64_t)TY * kRowUnroll) {
+      float tg[kRowUnroll][VEC], ty_[kRowUnroll][VEC];
+#pragma unroll
+      for (int u = 0; u < kRowUnroll; ++u) {
+        const int64_t rr = r + (int64_t)u * TY;
+        if (rr < r1) {
+          load_f32<T, VEC>(tg[u], g + rr * cols + c0);
+          load_f32<T, VEC>(ty_[u], y + rr * cols + c0);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kRowUnroll; ++u) {
+        const int64_t rr = r + (int64_t)u * TY;
+        if (rr < r1) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            tg[u][j] = gelu_grad(ty_[u][j] + b[j]) * tg[u][j];
+            if constexpr (WANT_DBIAS) acc[j] += tg[u][j];
+          }
+          store_f32<T, VEC>(dy + rr * cols + c0, tg[u]);
+        }
+      }
+    }
+  }
+  if constexpr (WANT_DBIAS)
+    write_colsum_partial<VEC>(acc, partial, cols, c0, col_ok);
+}
+
+template <typename T, int VEC>
+int launch_fwd(T *out, const T *y, const T *bias, int64_t rows, int64_t cols,
+               hipStream_t stream) {
+  const EwPlan p = plan_elementwise(rows, cols / VEC, kRowsPerBlockFwd);
+  bias_gelu_fwd_kernel<T, VEC><<<p.grid, p.block, 0, stream>>>(
+      out, y, bias, rows, cols, p.rows_per_block);
+  return check_launch("bias_gelu_fwd");
+}
+
+template <typename T, int VEC>
+int launch_bwd(T *dy, T *dbias, float *ws, const T *g, const T *y,
+               const T *bias, int64_t rows, int64_t cols, hipStream_t stream) {
+  const EwPlan p = plan_elementwise(rows, cols / VEC, kRowsPerBlockBwd);
+  if (dbias) {
+    bias_gelu_bwd_kernel<T, VEC, true><<<p.grid, p.block, 0, stream>>>(
+        dy, ws, g, y, bias, rows, cols, p.rows_per_block);
+    int s = check_launch("bias_gelu_bwd");
+    if (s != OSLO_OK) return s;
+    launch_colsum_finish<T>(dbias, ws, (int)p.grid.y, cols, stream);
+    return check_launch("bias_gelu_bwd(dbias)");
+  }
+  bias_gelu_bwd_kernel<T, VEC, false><<<p.grid, p.block, 0, stream>>>(
+      dy, nullptr, g, y, bias, rows, cols, p.rows_per_block);
+  return check_launch("bias_gelu_bwd");
+}
+
+} // namespace
+} // namespace oslo
+
+extern "C" int oslo_bias_gelu_fwd(void *out, const void *y, const void *bias,
+                                  int64_t rows, int64_t cols, int dtype,
+                                  oslo_stream_t stream) {
+  using namespace oslo;
+  if (rows < 0 || cols < 0)
+    return fail(OSLO_E_BAD_ARG, "bias_gelu_fwd: negative size");
+  if (rows == 0 || cols == 0) return OSLO_OK;
+  if (!out || !y || !bias)
+    return fail(OSLO_E_BAD_ARG, "bias_gelu_fwd: null tensor");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  OSLO_DISPATCH_DTYPE(dtype, {
+    constexpr int V = Io<T>::kVec;
+    const bool vec = cols % V == 0 && aligned16(out) && aligned16(y) &&
+                     aligned16(bias);
+    T *o = static_cast<T *>(out);
+    const T *yy = static_cast<const T *>(y);
+    const T *bb = static_cast<const T *>(bias);
+    return vec ? launch_fwd<T, V>(o, yy, bb, rows, cols, st)
+               : launch_fwd<T, 1>(o, yy, bb, rows, cols, st);
+  });
+  return OSLO_OK;
+}
+
+extern "C" int oslo_bias_gelu_bwd(void *dy, void *dbias, float *workspace,
+                                  const void *g, const void *y,
+                                  const void *bias, int64_t rows, int64_t cols,
+                                  int dtype, oslo_stream_t stream) {
+  using namespace oslo;
+  if (rows < 0 || cols < 0)
+    return fail(OSLO_E_BAD_ARG, "bias_gelu_bwd: negative size");
+  if (cols == 0) return OSLO_OK;
+  if (dbias && !workspace && rows > 0)
+    return fail(OSLO_E_BAD_ARG, "bias_gelu_bwd: dbias needs a workspace");
+  if (rows > 0 && (!dy || !g || !y || !bias))
+    return fail(OSLO_E_BAD_ARG, "bias_gelu_bwd: null tensor");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  OSLO_DISPATCH_DTYPE(dtype, {
+    if (rows == 0) { // empty batch: the bias gradient is still defined (zero)
+      if (dbias)
+        launch_colsum_finish<T>(static_cast<T *>(dbias), nullptr, 0, cols, st);
+      return check_launch("bias_gelu_bwd(dbias)");
+    }
+    constexpr int V = Io<T>::kVec;
+    const bool vec = cols % V == 0 && aligned16(dy) && aligned16(g) &&
+                     aligned16(y) && aligned16(bias) && aligned16(workspace);
+    T *d = static_cast<T *>(dy);
+    T *db = static_cast<T *>(dbias);
+    const T *gg = static_cast<const T *>(g);
+    const T *yy = static_cast<const T *>(y);
+    const T *bb = static_cast<const T *>(bias);
+    return vec ? launch_bwd<T, V>(d, db, workspace, gg, yy, bb, rows, cols, st)
+               : launch_bwd<T, 1>(d, db, workspace, gg, yy, bb, rows, cols, st);
+  });
+  return OSLO_OK;
+}

@@ -1,0 +1,69 @@
+// Host-only part of the library: status text, per-thread error message, and the
+// integer helpers of the C ABI.
+
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "elementwise.hpp"
+#include "softmax.hpp"
+
+namespace oslo {
+namespace {
+thread_local char g_error[256] = "";
+}
+
+int fail(int status, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof g_error, fmt, ap);
+  va_end(ap);
+  return status;
+}
+
+int check_launch(const char *what) {
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return OSLO_OK;
+  return fail(OSLO_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+} // namespace oslo
+
+extern "C" int oslo_abi_version(void) { return 1; }
+
+extern "C" int oslo_softmax_max_cols(void) { return oslo::kSoftmaxMaxCols; }
+
+extern "C" const char *oslo_status_string(int status) {
+  switch (status) {
+  case OSLO_OK: return "ok";
+  case OSLO_E_BAD_ARG: return "bad argument";
+  case OSLO_E_UNSUPPORTED: return "unsupported shape";
+  case OSLO_E_LAUNCH: return "kernel launch failed";
+  default: return "unknown status";
+  }
+}
+
+extern "C" const char *oslo_last_error(void) { return oslo::g_error; }
+
+// The reference's arithmetic (oslo/fused_kernels/includes/fused_softmax.h
+// :328-340) with its constants: 32-lane warps, 128 threads per block, two rows
+// per warp up to 128 keys.
+extern "C" int oslo_get_batch_per_block(int sq, int sk, int batches, int heads) {
+  (void)sq;
+  (void)batches;
+  (void)heads;
+  int log2_elements = 0;
+  while ((1 << log2_elements) < sk) ++log2_elements;
+  const int next_pow2 = 1 << log2_elements;
+  const int warp_size = next_pow2 < 32 ? next_pow2 : 32;
+  const int rows_per_warp = next_pow2 <= 128 ? 2 : 1;
+  return rows_per_warp * (128 / warp_size);
+}
+
+extern "C" size_t oslo_colsum_workspace_bytes(int64_t rows, int64_t cols) {
+  if (rows <= 0 || cols <= 0) return 0;
+  // One fp32 partial row per block row range; a range is never shorter than
+  // kRowsPerBlockBwd rows whatever the column tiling.
+  int64_t parts = (rows + oslo::kRowsPerBlockBwd - 1) / oslo::kRowsPerBlockBwd;
+  if (parts > 32768) parts = 32768;
+  return (size_t)parts * (size_t)cols * sizeof(float);
+}

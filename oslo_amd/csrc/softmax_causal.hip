@@ -1,0 +1,314 @@
+// Scale + causal (upper-triangular) mask + softmax, forward and backward, for
+// gfx950. Behaviour follows oslo/fused_kernels/includes/fused_triang_softmax.h
+// :134-351 of the reference (row r sees keys 0..r, the rest of the output row
+// is zero) with the optional additive key mask of the unfused attention
+// (oslo/models/gpt2/modeling_gpt2.py:214-216) folded in.
+//
+// The mask is never materialised: the diagonal position follows from the row
+// index. Keys above the diagonal are not read (their lanes are switched off
+// for the load), and the zeros of the upper triangle are written by the same
+// 128-bit stores as the probabilities.
+
+#include "softmax.hpp"
+
+namespace oslo {
+namespace {
+
+// ---------------------------------------------------------------------------
+// Register-resident path: rows up to kSoftmaxMaxCols, S a multiple of VEC.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC, int NCHUNK, int WPR, bool HAS_PAD>
+__global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
+    T *y, const T *x, const float *__restrict__ pad, float scale, int S,
+    int heads, int64_t total_rows) {
+  using Tile = RowTile<VEC, NCHUNK, WPR>;
+  __shared__ float s_max[kWavesPerBlock];
+  __shared__ float s_sum[kWavesPerBlock];
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int sub = wave % WPR;
+  int64_t row = (int64_t)blockIdx.x * Tile::kRowsPerBlock + wave / WPR;
+  // A block past the end keeps its waves alive (they meet the same barriers)
+  // on the last row and only skips the stores.
+  const bool live = row < total_rows;
+  if (!live) row = total_rows - 1;
+  const int64_t slab = row / S;
+  const int r = (int)(row - slab * S);
+  const T *xr = x + row * S;
+  T *yr = y + row * S;
+  const float *padr = HAS_PAD ? pad + (slab / heads) * S : nullptr;
+
+  float v[NCHUNK][VEC];
+  float m = -INFINITY;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    const int k0 = Tile::col(c, sub, lane);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) v[c][j] = -INFINITY;
+    if (k0 <= r) { // implies k0 < S; lanes wholly above the diagonal load nothing
+      float t[VEC];
+      load_f32<T, VEC>(t, xr + k0);
+      float pv[VEC];
+      if constexpr (HAS_PAD) load_f32_cached<float, VEC>(pv, padr + k0);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        // scale then add, each rounded, as the unfused path does
+        float e = __fmul_rn(t[j], scale);
+        if constexpr (HAS_PAD) e = __fadd_rn(e, pv[j]);
+        if (k0 + j <= r) {
+          v[c][j] = e;
+          m = fmaxf(m, e);
+        }
+      }
+    }
+  }
+  m = row_allreduce<WPR>(m, OpMax(), s_max);
+
+  float sum = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    // wave-uniform: chunks wholly above the diagonal stay at exp(-inf) = 0
+    if (Tile::col(c, sub, 0) <= r) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        v[c][j] = exp_shifted(v[c][j], m);
+        sum += v[c][j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[c][j] = 0.f;
+    }
+  }
+  sum = row_allreduce<WPR>(sum, OpAdd(), s_sum);
+  const float inv = 1.0f / sum;
+
+  if (!live) return;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    const int k0 = Tile::col(c, sub, lane);
+    if (k0 < S) {
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o[j] = v[c][j] * inv;
+      store_f32<T, VEC>(yr + k0, o);
+    }
+  }
+}
+
+template <typename T, int VEC, int NCHUNK, int WPR>
+__global__ __launch_bounds__(kBlockThreads) void causal_bwd_kernel(
+    T *dx, const T *g, const T *y, float scale, int S, int64_t total_rows) {
+  using Tile = RowTile<VEC, NCHUNK, WPR>;
+  __shared__ float s_sum[kWavesPerBlock];
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int sub = wave % WPR;
+  int64_t row = (int64_t)blockIdx.x * Tile::kRowsPerBlock + wave / WPR;
+  const bool live = row < total_rows;
+  if (!live) row = total_rows - 1;
+  const int r = (int)(row % S);
+  const T *gr = g + row * S;
+  const T *yr = y + row * S;
+  T *dr = dx + row * S;
+
+  float gy[NCHUNK][VEC]; // g*y
+  float yy[NCHUNK][VEC]; // y
+  float sum = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    const int k0 = Tile::col(c, sub, lane);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) gy[c][j] = yy[c][j] = 0.f;
+    if (k0 <= r) {
+      float tg[VEC], ty[VEC];
+      load_f32<T, VEC>(tg, gr + k0);
+      load_f32<T, VEC>(ty, yr + k0);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        if (k0 + j <= r) {
+          yy[c][j] = ty[j];
+          gy[c][j] = tg[j] * ty[j];
+          sum += gy[c][j];
+        }
+      }
+    }
+  }
+  sum = row_allreduce<WPR>(sum, OpAdd(), s_sum);
+
+  if (!live) return;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    const int k0 = Tile::col(c, sub, lane);
+    if (k0 < S) {
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j)
+        o[j] = scale * (gy[c][j] - yy[c][j] * sum);
+      store_f32<T, VEC>(dr + k0, o);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Any-shape path: one wave per row, element-wise accesses, three passes over
+// the row (the second and third come from cache). Used when S is not a
+// multiple of the vector width or a pointer is not 16-byte aligned.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kBlockThreads) void causal_fwd_anyshape_kernel(
+    T *y, const T *x, const float *__restrict__ pad, float scale, int S,
+    int heads, int64_t total_rows) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  if (row >= total_rows) return; // whole wave leaves; no barriers below
+  const int64_t slab = row / S;
+  const int r = (int)(row - slab * S);
+  const T *xr = x + row * S;
+  T *yr = y + row * S;
+  const float *padr = pad ? pad + (slab / heads) * S : nullptr;
+
+  auto score = [&](int k) {
+    float e = __fmul_rn(static_cast<float>(xr[k]), scale);
+    if (padr) e = __fadd_rn(e, padr[k]);
+    return e;
+  };
+  float m = -INFINITY;
+  for (int k = lane; k <= r; k += kWave) m = fmaxf(m, score(k));
+  m = wave_allreduce(m, OpMax());
+  float sum = 0.f;
+  for (int k = lane; k <= r; k += kWave) sum += exp_shifted(score(k), m);
+  sum = wave_allreduce(sum, OpAdd());
+  const float inv = 1.0f / sum;
+  // x is read before y is written at the same index, so y may alias x
+  for (int k = lane; k < S; k += kWave) {
+    const float o = k <= r ? exp_shifted(score(k), m) * inv : 0.f;
+    yr[k] = static_cast<T>(o);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlockThreads) void causal_bwd_anyshape_kernel(
+    T *dx, const T *g, const T *y, float scale, int S, int64_t total_rows) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  if (row >= total_rows) return;
+  const int r = (int)(row % S);
+  const T *gr = g + row * S;
+  const T *yr = y + row * S;
+  T *dr = dx + row * S;
+  float sum = 0.f;
+  for (int k = lane; k <= r; k += kWave)
+    sum += static_cast<float>(gr[k]) * static_cast<float>(yr[k]);
+  sum = wave_allreduce(sum, OpAdd());
+  for (int k = lane; k < S; k += kWave) {
+    float o = 0.f;
+    if (k <= r) {
+      const float yk = static_cast<float>(yr[k]);
+      o = scale * (static_cast<float>(gr[k]) * yk - yk * sum);
+    }
+    dr[k] = static_cast<T>(o);
+  }
+}
+
+template <typename T>
+int launch_causal_fwd(T *y, const T *x, const float *pad, float scale,
+                      int64_t batch, int64_t heads, int64_t S,
+                      hipStream_t stream) {
+  constexpr int VEC = Io<T>::kVec;
+  const int64_t total_rows = batch * heads * S;
+  const bool vector_ok = S % VEC == 0 && aligned16(x) && aligned16(y) &&
+                         (pad == nullptr || aligned16(pad));
+  if (!vector_ok) {
+    const int64_t blocks = (total_rows + kWavesPerBlock - 1) / kWavesPerBlock;
+    causal_fwd_anyshape_kernel<T><<<dim3((unsigned)blocks), dim3(kBlockThreads),
+                                    0, stream>>>(y, x, pad, scale, (int)S,
+                                                 (int)heads, total_rows);
+    return check_launch("softmax_causal_fwd");
+  }
+  dispatch_row_tile<VEC>(S, [&]<int NCHUNK, int WPR>() {
+    constexpr int rpb = RowTile<VEC, NCHUNK, WPR>::kRowsPerBlock;
+    const int64_t blocks = (total_rows + rpb - 1) / rpb;
+    if (pad)
+      causal_fwd_kernel<T, VEC, NCHUNK, WPR, true>
+          <<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(
+              y, x, pad, scale, (int)S, (int)heads, total_rows);
+    else
+      causal_fwd_kernel<T, VEC, NCHUNK, WPR, false>
+          <<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(
+              y, x, nullptr, scale, (int)S, (int)heads, total_rows);
+  });
+  return check_launch("softmax_causal_fwd");
+}
+
+template <typename T>
+int launch_causal_bwd(T *dx, const T *g, const T *y, float scale, int64_t bh,
+                      int64_t S, hipStream_t stream) {
+  constexpr int VEC = Io<T>::kVec;
+  const int64_t total_rows = bh * S;
+  const bool vector_ok =
+      S % VEC == 0 && aligned16(dx) && aligned16(g) && aligned16(y);
+  if (!vector_ok) {
+    const int64_t blocks = (total_rows + kWavesPerBlock - 1) / kWavesPerBlock;
+    causal_bwd_anyshape_kernel<T><<<dim3((unsigned)blocks), dim3(kBlockThreads),
+                                    0, stream>>>(dx, g, y, scale, (int)S,
+                                                 total_rows);
+    return check_launch("softmax_causal_bwd");
+  }
+  dispatch_row_tile<VEC>(S, [&]<int NCHUNK, int WPR>() {
+    constexpr int rpb = RowTile<VEC, NCHUNK, WPR>::kRowsPerBlock;
+    const int64_t blocks = (total_rows + rpb - 1) / rpb;
+    causal_bwd_kernel<T, VEC, NCHUNK, WPR>
+        <<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(
+            dx, g, y, scale, (int)S, total_rows);
+  });
+  return check_launch("softmax_causal_bwd");
+}
+
+// Shared argument screening. Returns 1 when there is nothing to do.
+int screen(const char *name, int64_t rows, int64_t S) {
+  if (rows < 0 || S < 0)
+    return fail(OSLO_E_BAD_ARG, "%s: negative size", name);
+  if (S > kSoftmaxMaxCols)
+    return fail(OSLO_E_UNSUPPORTED, "%s: row length %lld exceeds %d", name,
+                (long long)S, kSoftmaxMaxCols);
+  if (S > 0 && rows > (int64_t)INT32_MAX / S)
+    return fail(OSLO_E_UNSUPPORTED, "%s: too many rows for one launch", name);
+  return (rows == 0 || S == 0) ? 1 : 0;
+}
+
+} // namespace
+} // namespace oslo
+
+extern "C" int oslo_softmax_causal_fwd(void *y, const void *x,
+                                       const float *pad_add, float scale,
+                                       int64_t batch, int64_t heads, int64_t S,
+                                       int dtype, oslo_stream_t stream) {
+  using namespace oslo;
+  if (batch < 0 || heads < 0)
+    return fail(OSLO_E_BAD_ARG, "softmax_causal_fwd: negative size");
+  const int s = screen("softmax_causal_fwd", batch * heads, S);
+  if (s != 0) return s < 0 ? s : OSLO_OK;
+  if (!x || !y) return fail(OSLO_E_BAD_ARG, "softmax_causal_fwd: null tensor");
+  OSLO_DISPATCH_DTYPE(dtype, return launch_causal_fwd<T>(
+                                 static_cast<T *>(y), static_cast<const T *>(x),
+                                 pad_add, scale, batch, heads, S,
+                                 static_cast<hipStream_t>(stream)));
+  return OSLO_OK;
+}
+
+extern "C" int oslo_softmax_causal_bwd(void *dx, const void *g, const void *y,
+                                       float scale, int64_t bh, int64_t S,
+                                       int dtype, oslo_stream_t stream) {
+  using namespace oslo;
+  const int s = screen("softmax_causal_bwd", bh, S);
+  if (s != 0) return s < 0 ? s : OSLO_OK;
+  if (!dx || !g || !y)
+    return fail(OSLO_E_BAD_ARG, "softmax_causal_bwd: null tensor");
+  OSLO_DISPATCH_DTYPE(dtype, return launch_causal_bwd<T>(
+                                 static_cast<T *>(dx), static_cast<const T *>(g),
+                                 static_cast<const T *>(y), scale, bh, S,
+                                 static_cast<hipStream_t>(stream)));
+  return OSLO_OK;
+}

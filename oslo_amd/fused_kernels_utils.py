@@ -1,0 +1,363 @@
+"""Fused operator API: the classes of oslo/fused_kernels_utils.py:259-479 and
+:524-566 of the reference, with the same names and ``apply`` / ``is_available``
+signatures, running on the gfx950 kernels of ``liboslo_amd.so``.
+
+Differences from the reference, all widening:
+
+* fp16, bf16 and fp32 scores up to 8192 keys are fused (the reference gates on
+  fp16 and 2048, oslo/fused_kernels_utils.py:462), with no divisibility rules;
+* the additive padding mask of the causal path is applied inside the kernel,
+  after scaling and in fp32 (the order of the unfused attention,
+  oslo/models/gpt2/modeling_gpt2.py:197-216), instead of being added into a
+  copy of the scores beforehand (oslo/fused_kernels_utils.py:444-449);
+* the key mask of the non-causal path is read through strides instead of being
+  repeated to [B,1,Sq,Sk] (oslo/fused_kernels_utils.py:456-458), and is
+  *added* as -10000 like the unfused attention does, where the reference's
+  kernel *replaces* the score (oslo/fused_kernels/includes/fused_softmax.h
+  :171-175); the two differ only on rows with every key masked;
+* bias-GeLU and bias-dropout(-residual) are single hand-written kernels rather
+  than TorchScript (oslo/fused_kernels_utils.py:259-308); their backward also
+  returns the reduced bias gradient.
+"""
+
+import inspect
+
+import torch
+
+from . import _lib, kernels
+
+_custom_kernels = None
+
+
+def get_custom_kernels():
+    """The native module (oslo/fused_kernels_utils.py:219-232). Nothing is
+    compiled here: the library is built ahead of time and only loaded.
+    Raises EnvironmentError if it is missing, like the reference does when its
+    build fails (:226-230)."""
+    global _custom_kernels
+    if _custom_kernels is None:
+        _lib.load()
+        _custom_kernels = kernels
+    return _custom_kernels
+
+
+# ---------------------------------------------------------------------------
+# softmax
+# ---------------------------------------------------------------------------
+
+class ScaledUpperTriangMaskedSoftmaxFunction(torch.autograd.Function):
+    """oslo/fused_kernels_utils.py:311-331. inputs: [attn_batches, S, S]."""
+
+    @staticmethod
+    def forward(ctx, inputs, scale):
+        scale_t = torch.tensor([scale])
+        softmax_results = get_custom_kernels().scaled_upper_triang_masked_softmax_forward(
+            inputs, scale_t[0]
+        )
+        ctx.save_for_backward(softmax_results, scale_t)
+        return softmax_results
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        softmax_results, scale_t = ctx.saved_tensors
+        input_grads = get_custom_kernels().scaled_upper_triang_masked_softmax_backward(
+            output_grads, softmax_results, scale_t[0]
+        )
+        return input_grads, None
+
+
+class ScaledMaskedSoftmaxFunction(torch.autograd.Function):
+    """oslo/fused_kernels_utils.py:334-352. inputs [B,H,Sq,Sk], mask bytes
+    [B or 1, 1, Sq, Sk]; a set byte replaces the score by -10000."""
+
+    @staticmethod
+    def forward(ctx, inputs, mask, scale):
+        scale_t = torch.tensor([scale])
+        softmax_results = get_custom_kernels().scaled_masked_softmax_forward(
+            inputs, mask, scale_t[0]
+        )
+        ctx.save_for_backward(softmax_results, scale_t)
+        return softmax_results
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        softmax_results, scale_t = ctx.saved_tensors
+        input_grads = get_custom_kernels().scaled_masked_softmax_backward(
+            output_grads, softmax_results, scale_t[0]
+        )
+        return input_grads, None, None
+
+
+class _CausalSoftmaxWithPad(torch.autograd.Function):
+    """Causal softmax of [B,H,S,S] scores with an fp32 additive key mask [B,S]
+    applied inside the kernel."""
+
+    @staticmethod
+    def forward(ctx, inputs, pad_add, scale):
+        y = get_custom_kernels().causal_softmax_forward(inputs, pad_add, scale)
+        ctx.save_for_backward(y)
+        ctx.scale = float(scale)
+        return y
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        (y,) = ctx.saved_tensors
+        b, h, s, _ = y.shape
+        dx = get_custom_kernels().scaled_upper_triang_masked_softmax_backward(
+            output_grads.reshape(b * h, s, s), y.view(b * h, s, s), ctx.scale
+        )
+        return dx.view(b, h, s, s), None, None
+
+
+class _KeyMaskedSoftmax(torch.autograd.Function):
+    """Softmax of [B,H,Sq,Sk] scores with a broadcastable byte mask that adds
+    -10000 to masked keys."""
+
+    @staticmethod
+    def forward(ctx, inputs, mask, scale):
+        y = get_custom_kernels().masked_softmax_forward(inputs, mask, scale, kernels.MASK_ADD)
+        ctx.save_for_backward(y)
+        ctx.scale = float(scale)
+        return y
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        (y,) = ctx.saved_tensors
+        dx = get_custom_kernels().scaled_masked_softmax_backward(output_grads, y, ctx.scale)
+        return dx, None, None
+
+
+def _key_mask_bytes(pad_mask):
+    """Any mask form -> bool, True = masked. Float masks follow the reference's
+    ``.bool()`` (oslo/fused_kernels_utils.py:453-457): non-zero means masked."""
+    return pad_mask if pad_mask.dtype == torch.bool else pad_mask != 0
+
+
+def _pad_additive_f32(pad_mask, bsz, sk):
+    """[B or 1, 1, 1, Sk] mask (bool/uint8: True = padded -> -10000; float:
+    additive as given) -> fp32 [B, Sk]."""
+    if pad_mask.dim() != 4 or pad_mask.shape[1] != 1 or pad_mask.shape[2] != 1 \
+            or pad_mask.shape[3] != sk or pad_mask.shape[0] not in (1, bsz):
+        raise RuntimeError(
+            "FusedScaleMaskSoftmax: with use_triang_mask the pad_mask must be "
+            f"[batch or 1, 1, 1, {sk}], got {tuple(pad_mask.shape)}"
+        )
+    m = pad_mask.reshape(pad_mask.shape[0], sk)
+    if m.dtype in (torch.bool, torch.uint8):
+        m = m.to(torch.float32) * -10000.0
+    else:
+        m = m.to(torch.float32)
+    return m.expand(bsz, sk).contiguous()
+
+
+class FusedScaleMaskSoftmax(object):
+    """
+    Kernel fusion function: Scale + Mask + Softmax
+    (oslo/fused_kernels_utils.py:431-479)
+
+    Before fusion: Matmul (Q * K^T) -> Scale -> Mask -> Softmax -> Matmul (Score * V) -> ...
+    After fusion: Matmul (Q * K^T) -> (Scale + Mask + Softmax) -> Matmul (Score * V) -> ...
+    """
+
+    @staticmethod
+    def apply(input, pad_mask, scale, use_triang_mask):
+        bsz, np, sq, sk = input.size()
+        scale = scale if scale is not None else 1.0
+
+        if use_triang_mask:
+            if pad_mask is None:
+                return ScaledUpperTriangMaskedSoftmaxFunction.apply(
+                    input.view(-1, sq, sk), scale
+                ).view(bsz, np, sq, sk)
+            return _CausalSoftmaxWithPad.apply(input, _pad_additive_f32(pad_mask, bsz, sk), scale)
+
+        if pad_mask is None:
+            return _KeyMaskedSoftmax.apply(input, None, scale)
+        return _KeyMaskedSoftmax.apply(input, _key_mask_bytes(pad_mask), scale)
+
+    @staticmethod
+    def is_available(dtype, bsz, np, sq, sk, use_triang_mask):
+        """Integer gate of oslo/fused_kernels_utils.py:461-479, widened: true
+        wherever the reference's is true."""
+        kernels_ = get_custom_kernels()
+        if dtype not in (torch.half, torch.bfloat16, torch.float32):
+            return False
+        if sk <= 0 or sk > _lib.load().oslo_softmax_max_cols():
+            return False
+        if bsz <= 0 or np <= 0 or sq <= 0:
+            return False
+        # kept for parity of side effects: the reference computes this number
+        # to test divisibility; no kernel here needs it
+        kernels_.get_batch_per_block(sq, sk, bsz, np)
+        if use_triang_mask:
+            return sq == sk
+        return True
+
+
+# ---------------------------------------------------------------------------
+# bias + GeLU
+# ---------------------------------------------------------------------------
+
+class FusedBiasGeLU(torch.autograd.Function):
+    """
+    Kernel fusion function: Bias + GeLU (oslo/fused_kernels_utils.py:366-380)
+    """
+
+    @staticmethod
+    def forward(ctx, input, bias):
+        ctx.save_for_backward(input, bias)
+        return get_custom_kernels().bias_gelu_forward(input, bias)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, bias = ctx.saved_tensors
+        want_dbias = ctx.needs_input_grad[1]
+        dy, dbias = get_custom_kernels().bias_gelu_backward(grad_output, input, bias, want_dbias)
+        return dy, dbias
+
+
+def _act2fn(act):
+    # Only reached for activations without "gelu" in the name, as in the
+    # reference (oslo/fused_kernels_utils.py:396).
+    from transformers.activations import ACT2FN
+
+    return ACT2FN[act]
+
+
+class FusedBiasActivation(object):
+    """
+    Kernel fusion function: Bias + Activation (oslo/fused_kernels_utils.py:383-396)
+
+    Before fusion: MLP FFN1 -> (Bias Addition -> Activation) -> MLP FFN2 -> ...
+    After fusion: MLP FFN1 -> Fused Bias Activation -> MLP FFN2 -> ...
+    """
+
+    @staticmethod
+    def apply(x, bias, act):
+        if "gelu" in act:
+            return FusedBiasGeLU.apply(x, bias)
+        else:
+            return _act2fn(act)(x + bias)
+
+
+# ---------------------------------------------------------------------------
+# bias + dropout (+ residual)
+# ---------------------------------------------------------------------------
+
+PHILOX_WORDS_PER_CALL = 4  # generator offset one dropout call consumes
+
+
+def _next_philox(device):
+    """Takes (seed, offset) from the device's default generator and advances it,
+    the way a torch random op does."""
+    gen = torch.cuda.default_generators[device.index if device.index is not None
+                                        else torch.cuda.current_device()]
+    seed = gen.initial_seed()
+    offset = gen.get_offset()
+    gen.set_offset(offset + PHILOX_WORDS_PER_CALL)
+    return seed, offset
+
+
+class _BiasDropoutAdd(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, bias, residual, p):
+        if p > 0.0:
+            seed, offset = _next_philox(x.device)
+        else:
+            seed, offset = 0, 0
+        ctx.p, ctx.seed, ctx.offset = p, seed, offset
+        return get_custom_kernels().bias_dropout_add_forward(x, bias, residual, p, seed, offset)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        want_dbias = ctx.needs_input_grad[1]
+        dx = dbias = None
+        if ctx.needs_input_grad[0] or want_dbias:
+            dx, dbias = get_custom_kernels().bias_dropout_add_backward(
+                grad_output, ctx.p, ctx.seed, ctx.offset, want_dbias
+            )
+        dres = grad_output if ctx.needs_input_grad[2] else None
+        return dx, dbias, dres, None
+
+
+def _bias_dropout_add(x, bias, residual, training, drop_prop):
+    p = float(drop_prop) if training else 0.0
+    if p < 0.0 or p > 1.0:
+        raise ValueError(f"dropout probability has to be between 0 and 1, but got {p}")
+    if p == 1.0:  # everything dropped: F.dropout returns zeros
+        out = torch.zeros_like(x)
+        return out if residual is None else out + residual
+    return _BiasDropoutAdd.apply(x, bias, residual, p)
+
+
+class FusedBiasDropout(object):
+    """
+    Kernel fusion function: Bias + Dropout (oslo/fused_kernels_utils.py:399-412)
+
+    Before fusion: MLP FFN2 -> (Bias Addition -> Dropout) -> Residual Addition ->. ..
+    After fusion: MLP FFN2 -> Fused Bias Dropout -> Residual Addition -> ...
+    """
+
+    @staticmethod
+    def apply(x, bias, training, drop_prop):
+        return _bias_dropout_add(x, bias, None, training, drop_prop)
+
+
+class FusedBiasDropoutResidual(object):
+    """
+    Kernel fusion function: Bias + Dropout + Residual
+    (oslo/fused_kernels_utils.py:415-428)
+
+    Before fusion: MLP FFN2 -> (Bias Addition -> Dropout -> Residual Addition) -> LayerNorm -> ...
+    After fusion: MLP FFN2 -> Fused Bias Dropout Residual -> LayerNorm -> ...
+    """
+
+    @staticmethod
+    def apply(x, bias, residual, training, drop_prop):
+        return _bias_dropout_add(x, bias, residual, training, drop_prop)
+
+
+# ---------------------------------------------------------------------------
+# model.fuse()
+# ---------------------------------------------------------------------------
+
+class FusedKernelMixin(object):
+    """oslo/fused_kernels_utils.py:524-566: swaps the class of every fusable
+    sub-module for its fused subclass; parameters and buffers are untouched."""
+
+    def fuse(self, modules=None):
+        user_modules = modules
+
+        assert user_modules is None or isinstance(
+            user_modules, list
+        ), "Param `modules` must be type of List[Class]."
+
+        if not getattr(self, "is_fusable", False):
+            raise RuntimeError(
+                "This model doesn't support kernel fusion. please check the document."
+            )
+
+        for policy in self.get_layer_policies():
+            fused_modules = policy.fused_modules()
+
+            if user_modules is not None:
+                for user_module in user_modules:
+                    assert user_module in fused_modules, (
+                        f"Module {user_module} can't be fused! "
+                        f"{self.__class__.__qualname__} only supports {list(fused_modules.keys())}"
+                    )
+                    assert inspect.isclass(user_module), (
+                        f"The element in the ``modules`` must be Class type. "
+                        f"but you input {type(user_module)}"
+                    )
+
+            for model_module in self.modules():
+                cls = model_module.__class__
+                if cls not in fused_modules:
+                    continue
+                if user_modules is not None and cls not in user_modules:
+                    continue  # not in the list the user asked for
+                model_module.__class__ = fused_modules[cls]
+                setattr(model_module, "config", self.config)
+
+        return self

@@ -1,0 +1,243 @@
+"""Tensor-level front of ``liboslo_amd.so``: the functions of the reference's
+native module ``oslo_kernels`` (oslo/fused_kernels/bindings/pybind_kernels.cpp
+:159-177) with the same names, argument order and error behaviour, plus the
+wider entry points the fused operators of this package use.
+
+Every function takes device tensors, allocates its output with torch, and
+enqueues one kernel on torch's current stream of that device. There is no CPU
+implementation: a CPU tensor is rejected with ``RuntimeError``.
+"""
+
+import ctypes
+
+import torch
+
+from . import _lib
+
+_DTYPE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+MASK_ADD = 0
+MASK_REPLACE = 1
+
+
+def _require(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _dtype_code(t, what):
+    _require(t.dtype in _DTYPE, f"{what}: only fp16, bf16 and fp32 are supported, got {t.dtype}")
+    return _DTYPE[t.dtype]
+
+
+def _device_tensor(t, what):
+    _require(isinstance(t, torch.Tensor), f"{what}: expected a tensor")
+    _require(t.is_cuda, f"{what}: expected a tensor on a ROCm device, got {t.device} "
+                        "(this library has no CPU path)")
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+# ---------------------------------------------------------------------------
+# the reference's five softmax symbols
+# ---------------------------------------------------------------------------
+
+def get_batch_per_block(query_seq_len, key_seq_len, batches, attn_heads):
+    """oslo/fused_kernels/bindings/pybind_kernels.cpp:77-83."""
+    return _lib.load().oslo_get_batch_per_block(
+        int(query_seq_len), int(key_seq_len), int(batches), int(attn_heads))
+
+
+def scaled_upper_triang_masked_softmax_forward(input, scale_factor):
+    """oslo/fused_kernels/bindings/pybind_kernels.cpp:98-105: input [attn_batches, S, S]."""
+    _require(input.dim() == 3, "expected 3D tensor")
+    return causal_softmax_forward(input.unsqueeze(0), None, scale_factor).squeeze(0)
+
+
+def scaled_upper_triang_masked_softmax_backward(output_grads, softmax_results, scale_factor):
+    """oslo/fused_kernels/bindings/pybind_kernels.cpp:107-123. Writes the input
+    gradient over ``output_grads`` (when it is contiguous) and returns it, as
+    the reference does (oslo/fused_kernels/fused_triang_softmax.cu:84-95)."""
+    _require(output_grads.dim() == 3, "expected 3D tensor")
+    _require(softmax_results.dim() == 3, "expected 3D tensor")
+    _device_tensor(output_grads, "output_grads")
+    _device_tensor(softmax_results, "softmax_results")
+    code = _dtype_code(output_grads, "output_grads")
+    _require(softmax_results.dtype == output_grads.dtype, "output_grads and softmax_results differ in dtype")
+    _require(softmax_results.shape == output_grads.shape, "output_grads and softmax_results differ in shape")
+    bh, sq, sk = output_grads.shape
+    _require(sq == sk, "causal softmax needs square score matrices")
+    g = output_grads.contiguous()
+    y = softmax_results.contiguous()
+    with torch.cuda.device(g.device):
+        _lib.check(_lib.load().oslo_softmax_causal_bwd(
+            _ptr(g), _ptr(g), _ptr(y), float(scale_factor), bh, sk, code, _stream(g)))
+    return g
+
+
+def scaled_masked_softmax_forward(input, mask, scale_factor):
+    """oslo/fused_kernels/bindings/pybind_kernels.cpp:46-57: input [B,H,Sq,Sk],
+    mask [B or 1, 1, Sq, Sk] bytes; a set byte replaces the score by -10000
+    (oslo/fused_kernels/includes/fused_softmax.h:171-175)."""
+    _require(input.dim() == 4, "expected 4D tensor")
+    _require(mask.dim() == 4, "expected 4D tensor")
+    return masked_softmax_forward(input, mask, scale_factor, MASK_REPLACE)
+
+
+def scaled_masked_softmax_backward(output_grads, softmax_results, scale_factor):
+    """oslo/fused_kernels/bindings/pybind_kernels.cpp:59-75; in place over
+    ``output_grads`` (oslo/fused_kernels/fused_softmax.cu:103-114)."""
+    _require(output_grads.dim() == 4, "expected 4D tensor")
+    _require(softmax_results.dim() == 4, "expected 4D tensor")
+    _device_tensor(output_grads, "output_grads")
+    _device_tensor(softmax_results, "softmax_results")
+    code = _dtype_code(output_grads, "output_grads")
+    _require(softmax_results.dtype == output_grads.dtype, "output_grads and softmax_results differ in dtype")
+    _require(softmax_results.shape == output_grads.shape, "output_grads and softmax_results differ in shape")
+    g = output_grads.contiguous()
+    y = softmax_results.contiguous()
+    sk = g.shape[-1]
+    rows = g.numel() // sk if sk else 0
+    with torch.cuda.device(g.device):
+        _lib.check(_lib.load().oslo_softmax_masked_bwd(
+            _ptr(g), _ptr(g), _ptr(y), float(scale_factor), rows, sk, code, _stream(g)))
+    return g
+
+
+# ---------------------------------------------------------------------------
+# wider entry points
+# ---------------------------------------------------------------------------
+
+def causal_softmax_forward(input, pad_add, scale_factor):
+    """input [B,H,S,S]; pad_add None or fp32 [B,S] added after scaling."""
+    _device_tensor(input, "input")
+    _require(input.dim() == 4, "expected 4D tensor")
+    code = _dtype_code(input, "input")
+    b, h, sq, sk = input.shape
+    _require(sq == sk, "causal softmax needs square score matrices")
+    x = input.contiguous()
+    if pad_add is not None:
+        _device_tensor(pad_add, "pad_add")
+        _require(pad_add.dtype == torch.float32 and tuple(pad_add.shape) == (b, sk),
+                 "pad_add must be fp32 [batch, S]")
+        pad_add = pad_add.contiguous()
+    y = torch.empty_like(x, requires_grad=False)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().oslo_softmax_causal_fwd(
+            _ptr(y), _ptr(x), _ptr(pad_add), float(scale_factor), b, h, sk, code, _stream(x)))
+    return y
+
+
+def masked_softmax_forward(input, mask, scale_factor, mask_mode=MASK_ADD):
+    """input [B,H,Sq,Sk]; mask None or bool/uint8 [B or 1, 1, Sq or 1, Sk]
+    (size-1 dimensions are broadcast by stride, not copied)."""
+    _device_tensor(input, "input")
+    _require(input.dim() == 4, "expected 4D tensor")
+    code = _dtype_code(input, "input")
+    b, h, sq, sk = input.shape
+    x = input.contiguous()
+    msb = msq = 0
+    if mask is not None:
+        _device_tensor(mask, "mask")
+        _require(mask.dim() == 4, "expected 4D tensor")
+        _require(mask.dtype in (torch.bool, torch.uint8), "mask must be bool or uint8")
+        mb, mh, mq, mk = mask.shape
+        _require(mb in (1, b), "mask batch must be 1 or the input's batch")
+        _require(mh == 1, "mask must have one head")
+        _require(mq in (1, sq), "mask rows must be 1 or the input's query length")
+        _require(mk == sk, "mask and input differ in key length")
+        mask = mask.contiguous()
+        if mask.dtype == torch.bool:
+            mask = mask.view(torch.uint8)
+        msb = mq * mk if mb == b and b > 1 else 0
+        msq = mk if mq == sq and sq > 1 else 0
+    y = torch.empty_like(x, requires_grad=False)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().oslo_softmax_masked_fwd(
+            _ptr(y), _ptr(x), _ptr(mask), msb, msq, int(mask_mode), float(scale_factor),
+            b, h, sq, sk, code, _stream(x)))
+    return y
+
+
+def _as_rows_cols(t, bias, what):
+    _device_tensor(t, what)
+    code = _dtype_code(t, what)
+    _require(t.dim() >= 1, f"{what}: expected at least 1 dimension")
+    cols = t.shape[-1]
+    if bias is not None:
+        _device_tensor(bias, "bias")
+        _require(bias.dim() == 1 and bias.shape[0] == cols, "bias must be [last dimension of the input]")
+        _require(bias.dtype == t.dtype, "bias and input differ in dtype")
+    rows = t.numel() // cols if cols else 0
+    return rows, cols, code
+
+
+def _workspace(rows, cols, device):
+    nbytes = _lib.load().oslo_colsum_workspace_bytes(rows, cols)
+    return torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=device)
+
+
+def bias_gelu_forward(y, bias):
+    rows, cols, code = _as_rows_cols(y, bias, "input")
+    y = y.contiguous()
+    bias = bias.contiguous()
+    out = torch.empty_like(y, requires_grad=False)
+    with torch.cuda.device(y.device):
+        _lib.check(_lib.load().oslo_bias_gelu_fwd(
+            _ptr(out), _ptr(y), _ptr(bias), rows, cols, code, _stream(y)))
+    return out
+
+
+def bias_gelu_backward(grad, y, bias, want_dbias=True):
+    """Returns (d_input, d_bias or None); d_input is a new tensor."""
+    rows, cols, code = _as_rows_cols(y, bias, "input")
+    _device_tensor(grad, "grad")
+    _require(grad.shape == y.shape and grad.dtype == y.dtype, "grad and input differ in shape or dtype")
+    grad = grad.contiguous()
+    y = y.contiguous()
+    bias = bias.contiguous()
+    dy = torch.empty_like(y, requires_grad=False)
+    dbias = torch.empty_like(bias, requires_grad=False) if want_dbias else None
+    ws = _workspace(rows, cols, y.device) if want_dbias else None
+    with torch.cuda.device(y.device):
+        _lib.check(_lib.load().oslo_bias_gelu_bwd(
+            _ptr(dy), _ptr(dbias), _ptr(ws), _ptr(grad), _ptr(y), _ptr(bias),
+            rows, cols, code, _stream(y)))
+    return dy, dbias
+
+
+def bias_dropout_add_forward(x, bias, residual, p, seed, offset):
+    rows, cols, code = _as_rows_cols(x, bias, "input")
+    x = x.contiguous()
+    if bias is not None:
+        bias = bias.contiguous()
+    if residual is not None:
+        _device_tensor(residual, "residual")
+        _require(residual.shape == x.shape and residual.dtype == x.dtype,
+                 "residual and input differ in shape or dtype")
+        residual = residual.contiguous()
+    out = torch.empty_like(x, requires_grad=False)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().oslo_bias_dropout_add_fwd(
+            _ptr(out), _ptr(x), _ptr(bias), _ptr(residual), float(p), int(seed), int(offset),
+            rows, cols, code, _stream(x)))
+    return out
+
+
+def bias_dropout_add_backward(grad, p, seed, offset, want_dbias=True):
+    """Returns (d_input, d_bias or None). The residual's gradient is ``grad``."""
+    rows, cols, code = _as_rows_cols(grad, None, "grad")
+    grad = grad.contiguous()
+    dx = torch.empty_like(grad, requires_grad=False)
+    dbias = torch.empty(cols, dtype=grad.dtype, device=grad.device) if want_dbias else None
+    ws = _workspace(rows, cols, grad.device) if want_dbias else None
+    with torch.cuda.device(grad.device):
+        _lib.check(_lib.load().oslo_bias_dropout_add_bwd(
+            _ptr(dx), _ptr(dbias), _ptr(ws), _ptr(grad), float(p), int(seed), int(offset),
+            rows, cols, code, _stream(grad)))
+    return dx, dbias

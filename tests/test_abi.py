@@ -1,0 +1,97 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header
+declares, and answers the calls that need no device (integer helpers and
+argument screening that fails before any launch)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from oracle import oslo_oracle as orc
+from oslo_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "oslo_amd.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(oslo_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree(lib):
+    names = declared_symbols()
+    assert len(names) >= 14
+    assert sorted(_lib.PROTOTYPES) == names
+    for name in names:
+        assert getattr(lib, name) is not None
+
+
+def test_header_compiles_as_plain_c(tmp_path):
+    src = tmp_path / "t.c"
+    src.write_text('#include "oslo_amd.h"\nint main(void){return OSLO_OK + OSLO_F32 + OSLO_MASK_ADD;}\n')
+    import subprocess
+
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic",
+                           f"-I{os.path.dirname(HEADER)}", "-c", str(src), "-o", str(tmp_path / "t.o")])
+
+
+def test_identity(lib):
+    assert lib.oslo_abi_version() == _lib.ABI_VERSION
+    assert lib.oslo_softmax_max_cols() == 8192
+    assert lib.oslo_status_string(0) == b"ok"
+    assert lib.oslo_status_string(-2) == b"unsupported shape"
+
+
+def test_get_batch_per_block_equals_reference_table(lib):
+    for sk in list(range(1, 300)) + [511, 512, 513, 1023, 1024, 1025, 2047, 2048]:
+        assert lib.oslo_get_batch_per_block(5, sk, 2, 3) == orc.get_batch_per_block(5, sk, 2, 3), sk
+
+
+def test_workspace_bytes(lib):
+    assert lib.oslo_colsum_workspace_bytes(0, 128) == 0
+    assert lib.oslo_colsum_workspace_bytes(128, 0) == 0
+    assert lib.oslo_colsum_workspace_bytes(1, 8) == 32
+    assert lib.oslo_colsum_workspace_bytes(16384, 16384) == 128 * 16384 * 4
+    assert lib.oslo_colsum_workspace_bytes(16385, 10) == 129 * 10 * 4
+
+
+def test_argument_screening_without_a_device(lib):
+    null = ctypes.c_void_p(0)
+    one = ctypes.c_void_p(16)  # never dereferenced: every call below fails or returns first
+    # negative sizes
+    assert lib.oslo_softmax_causal_fwd(one, one, null, 1.0, -1, 1, 8, 1, null) == -1
+    assert lib.oslo_softmax_masked_bwd(one, one, one, 1.0, -1, 8, 1, null) == -1
+    assert lib.oslo_bias_gelu_fwd(one, one, one, 4, -8, 1, null) == -1
+    # rows longer than the limit
+    assert lib.oslo_softmax_causal_fwd(one, one, null, 1.0, 1, 1, 8200, 1, null) == -2
+    assert b"8200" in lib.oslo_last_error()
+    assert lib.oslo_softmax_masked_fwd(one, one, null, 0, 0, 0, 1.0, 1, 1, 2, 8193, 1, null) == -2
+    # null tensors, unknown enums
+    assert lib.oslo_softmax_causal_bwd(null, one, one, 1.0, 1, 8, 1, null) == -1
+    assert lib.oslo_softmax_masked_fwd(one, one, null, 0, 0, 7, 1.0, 1, 1, 2, 8, 1, null) == -1
+    assert lib.oslo_softmax_causal_fwd(one, one, null, 1.0, 1, 1, 8, 9, null) == -1
+    assert lib.oslo_bias_gelu_bwd(one, one, null, one, one, one, 4, 8, 1, null) == -1  # dbias without workspace
+    # dropout probability outside [0, 1)
+    assert lib.oslo_bias_dropout_add_fwd(one, one, null, null, 1.0, 1, 0, 4, 8, 1, null) == -1
+    assert lib.oslo_bias_dropout_add_fwd(one, one, null, null, -0.1, 1, 0, 4, 8, 1, null) == -1
+    assert lib.oslo_bias_dropout_add_bwd(one, null, null, one, float("nan"), 1, 0, 4, 8, 1, null) == -1
+    # empty problems succeed without touching the device
+    assert lib.oslo_softmax_causal_fwd(null, null, null, 1.0, 0, 4, 8, 1, null) == 0
+    assert lib.oslo_softmax_masked_fwd(null, null, null, 0, 0, 0, 1.0, 2, 2, 0, 8, 1, null) == 0
+    assert lib.oslo_bias_gelu_fwd(null, null, null, 0, 8, 1, null) == 0
+    assert lib.oslo_bias_dropout_add_fwd(null, null, null, null, 0.5, 1, 0, 0, 8, 1, null) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/liboslo_amd.so")
+    with pytest.raises(EnvironmentError):
+        _lib.load()

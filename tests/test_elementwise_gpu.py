@@ -1,0 +1,161 @@
+"""Parity of the bias-GeLU and bias-dropout(-residual) kernels, called through
+the C ABI, with the CPU oracle. fp32 <= 1e-6, fp16/bf16 <= 2e-3 (relative above
+magnitude 1). The dropout keep mask must equal the oracle's bit for bit."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oslo_oracle as orc
+from oslo_amd import kernels
+from tests.util import DTYPES, IDS, assert_close, f32, randn
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+# (rows, cols): vector path, ragged tails, narrow and wide, column counts that
+# are not a multiple of the vector width, more rows than one block range
+SHAPES = [(1, 8), (3, 1), (5, 7), (33, 768), (129, 3072), (300, 4096), (257, 1000), (64, 16384), (2, 20000), (1025, 24)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("rows,cols", SHAPES)
+def test_bias_gelu_forward(rows, cols, dtype):
+    y = randn((rows, cols), dtype, seed=rows * 7 + cols, std=2.0)
+    b = randn((cols,), dtype, seed=cols, std=0.5)
+    want = orc.bias_gelu_fwd(f32(y), f32(b))
+    out = kernels.bias_gelu_forward(y.to(DEV), b.to(DEV))
+    assert out.dtype == dtype and out.shape == y.shape
+    assert_close(out, want, dtype, f"bias_gelu fwd {rows}x{cols}")
+
+
+def test_bias_gelu_forward_extremes_and_leading_dims():
+    y = torch.tensor([[0.0, 30.0, -30.0, 1e4, -1e4, 1e-8, -1e-8, 5.0]], dtype=torch.float32)
+    b = torch.zeros(8)
+    out = kernels.bias_gelu_forward(y.to(DEV), b.to(DEV))
+    assert_close(out, orc.bias_gelu_fwd(y.numpy(), b.numpy(), dtype=np.float64), torch.float32)
+    assert f32(out)[0, 4] == 0.0 and f32(out)[0, 3] == 1e4
+    y3 = randn((4, 6, 64), torch.bfloat16, seed=1)
+    b3 = randn((64,), torch.bfloat16, seed=2)
+    out3 = kernels.bias_gelu_forward(y3.to(DEV), b3.to(DEV))
+    assert out3.shape == y3.shape
+    assert_close(out3, orc.bias_gelu_fwd(f32(y3), f32(b3)), torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("rows,cols", SHAPES)
+def test_bias_gelu_backward(rows, cols, dtype):
+    y = randn((rows, cols), dtype, seed=rows * 7 + cols, std=2.0)
+    b = randn((cols,), dtype, seed=cols, std=0.5)
+    g = randn((rows, cols), dtype, seed=rows + cols)
+    want_dy, want_db = orc.bias_gelu_bwd(f32(g), f32(y), f32(b))
+    dy, db = kernels.bias_gelu_backward(g.to(DEV), y.to(DEV), b.to(DEV))
+    assert_close(dy, want_dy, dtype, f"bias_gelu bwd {rows}x{cols}")
+    # dbias sums `rows` terms: judged relative to sqrt(rows), the size such a sum reaches
+    assert_close(f32(db) / np.sqrt(rows), want_db / np.sqrt(rows), dtype, "dbias")
+    dy2, none = kernels.bias_gelu_backward(g.to(DEV), y.to(DEV), b.to(DEV), want_dbias=False)
+    assert none is None and torch.equal(dy2, dy)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("rows,cols", SHAPES)
+@pytest.mark.parametrize("p", [0.1, 0.5])
+def test_bias_dropout_add_forward_backward(rows, cols, dtype, p):
+    seed, offset = 1234, 8
+    x = randn((rows, cols), dtype, seed=rows * 3 + cols)
+    res = randn((rows, cols), dtype, seed=rows * 5 + cols)
+    b = randn((cols,), dtype, seed=cols, std=0.02)
+    keep = orc.dropout_keep_mask(seed, offset, rows * cols, p).reshape(rows, cols)
+    want = orc.bias_dropout_add_fwd(f32(x), f32(b), f32(res), p, keep)
+    out = kernels.bias_dropout_add_forward(x.to(DEV), b.to(DEV), res.to(DEV), p, seed, offset)
+    assert_close(out, want, dtype, f"bias_dropout_add fwd {rows}x{cols}")
+    # the mask itself, bit for bit: without bias/residual a dropped element is exactly 0
+    ones = torch.ones((rows, cols), dtype=dtype, device=DEV)
+    m = kernels.bias_dropout_add_forward(ones, None, None, p, seed, offset)
+    assert np.array_equal(f32(m) != 0, keep)
+    # no residual
+    out2 = kernels.bias_dropout_add_forward(x.to(DEV), b.to(DEV), None, p, seed, offset)
+    assert_close(out2, orc.bias_dropout_add_fwd(f32(x), f32(b), None, p, keep), dtype)
+    # backward regenerates the same mask
+    g = randn((rows, cols), dtype, seed=rows + cols + 1)
+    want_dx, want_db, _ = orc.bias_dropout_add_bwd(f32(g), p, keep)
+    dx, db = kernels.bias_dropout_add_backward(g.to(DEV), p, seed, offset)
+    assert_close(dx, want_dx, dtype, "bias_dropout_add bwd")
+    assert np.array_equal(f32(dx) != 0, keep & (f32(g) != 0))
+    assert_close(f32(db) / np.sqrt(rows), want_db / np.sqrt(rows), dtype, "dbias")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+def test_bias_dropout_add_p0_is_exact(dtype):
+    x = randn((37, 264), dtype, seed=1)
+    res = randn((37, 264), dtype, seed=2)
+    b = randn((264,), dtype, seed=3)
+    out = kernels.bias_dropout_add_forward(x.to(DEV), b.to(DEV), res.to(DEV), 0.0, 0, 0)
+    want = (x.float() + b.float() + res.float()).to(dtype)   # one rounding of the exact fp32 sum
+    assert torch.equal(out.cpu(), want)
+    g = randn((37, 264), dtype, seed=4)
+    dx, db = kernels.bias_dropout_add_backward(g.to(DEV), 0.0, 0, 0)
+    assert torch.equal(dx.cpu(), g)
+
+
+def test_dropout_keep_rate_and_seed_offset_semantics():
+    n_rows, n_cols, p = 4096, 1024, 0.1
+    ones = torch.ones((n_rows, n_cols), dtype=torch.bfloat16, device=DEV)
+    a = kernels.bias_dropout_add_forward(ones, None, None, p, 1234, 0)
+    rate = float((a != 0).float().mean())
+    sigma = (p * (1 - p) / (n_rows * n_cols)) ** 0.5
+    assert abs(rate - (1 - p)) < 4 * sigma
+    assert torch.equal(a, kernels.bias_dropout_add_forward(ones, None, None, p, 1234, 0))
+    assert not torch.equal(a, kernels.bias_dropout_add_forward(ones, None, None, p, 1234, 4))
+    assert not torch.equal(a, kernels.bias_dropout_add_forward(ones, None, None, p, 1235, 0))
+    kept = a[a != 0].float()
+    assert float((kept - 1 / (1 - p)).abs().max()) < 5e-3       # survivors scaled by 1/(1-p)
+    # 64-bit seed and offset are honoured
+    big = kernels.bias_dropout_add_forward(ones[:8], None, None, 0.5, 0xDEADBEEFCAFEF00D, (1 << 40) + 4)
+    keep = orc.dropout_keep_mask(0xDEADBEEFCAFEF00D, (1 << 40) + 4, 8 * n_cols, 0.5).reshape(8, n_cols)
+    assert np.array_equal(f32(big) != 0, keep)
+
+
+def test_elementwise_errors():
+    x = torch.zeros(4, 8, device=DEV)
+    with pytest.raises(RuntimeError):
+        kernels.bias_gelu_forward(x, torch.zeros(7, device=DEV))
+    with pytest.raises(RuntimeError):
+        kernels.bias_gelu_forward(x.cpu(), torch.zeros(8))
+    with pytest.raises(RuntimeError):
+        kernels.bias_dropout_add_forward(x, None, None, 1.0, 0, 0)
+    with pytest.raises(RuntimeError):
+        kernels.bias_dropout_add_forward(x, torch.zeros(8, device=DEV, dtype=torch.half), None, 0.1, 0, 0)
+
+
+def test_full_size_bias_gelu_and_dropout_properties():
+    """BASELINE shapes: [16384,16384] bias-GeLU and [16384,4096] dropout-add in
+    bf16; oracle on a band of rows, structural properties on the whole."""
+    dtype = torch.bfloat16
+    g = torch.Generator(device=DEV).manual_seed(0)
+    rows, cols = 16384, 16384
+    y = torch.randn((rows, cols), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+    b = (torch.randn((cols,), generator=g, device=DEV, dtype=torch.float32) * 0.02).to(dtype)
+    out = kernels.bias_gelu_forward(y, b)
+    for r0 in (0, 8000, 16380):
+        assert_close(out[r0:r0 + 4], orc.bias_gelu_fwd(f32(y[r0:r0 + 4]), f32(b)), dtype, f"rows {r0}")
+    go = torch.randn((rows, cols), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+    dy, db = kernels.bias_gelu_backward(go, y, b)
+    want_dy, _ = orc.bias_gelu_bwd(f32(go[5000:5004]), f32(y[5000:5004]), f32(b))
+    assert_close(dy[5000:5004], want_dy, dtype, "bwd band")
+    # dbias against a column sum of the kernel's own (rounded) dy, in fp32 on the device
+    colsum = dy.float().sum(0)
+    assert float(((db.float() - colsum).abs() / rows ** 0.5).max()) <= 2e-3
+    del y, out, go, dy
+    rows, cols, p = 16384, 4096, 0.1
+    x = torch.randn((rows, cols), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+    res = torch.randn((rows, cols), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+    b = b[:cols].contiguous()
+    o = kernels.bias_dropout_add_forward(x, b, res, p, 1234, 0)
+    keep = orc.dropout_keep_mask(1234, 0, rows * cols, p).reshape(rows, cols)
+    band = slice(9000, 9008)
+    assert_close(o[band], orc.bias_dropout_add_fwd(f32(x[band]), f32(b), f32(res[band]), p, keep[band]), dtype)
+    dropped = torch.from_numpy(~keep).to(DEV)
+    assert torch.equal(o[dropped], res[dropped])                # dropped elements are the residual, exactly
+    dx, db = kernels.bias_dropout_add_backward(x, p, 1234, 0)
+    assert torch.count_nonzero(dx[dropped]) == 0

@@ -1,0 +1,317 @@
+"""Pins the CPU oracle (oracle/oslo_oracle.py) against evidence that does not
+come from the oracle's own formulas: torch library routines, autograd, pure
+Python float64 loops, closed forms, published Philox known answers and the
+fixture written from torch's own Philox engine."""
+
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oslo_oracle as orc
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+# ---------------------------------------------------------------------------
+# softmax forward
+# ---------------------------------------------------------------------------
+
+def brute_softmax_row(scores):
+    """float64 loop; entries that are None are excluded."""
+    vals = [v for v in scores if v is not None]
+    m = max(vals)
+    exps = [math.exp(v - m) if v is not None else 0.0 for v in scores]
+    tot = sum(exps)
+    return [e / tot for e in exps]
+
+
+@pytest.mark.parametrize("s", [1, 2, 3, 5, 17])
+def test_causal_matches_python_loops(s):
+    x = rng(s).standard_normal((2, 2, s, s)) * 3
+    pad = rng(s + 1).choice([0.0, -10000.0], size=(2, s))
+    scale = 0.37
+    got = orc.softmax_causal(x, scale, pad, dtype=np.float64)
+    for b in range(2):
+        for h in range(2):
+            for r in range(s):
+                row = [x[b, h, r, k] * scale + pad[b, k] if k <= r else None for k in range(s)]
+                np.testing.assert_allclose(got[b, h, r], brute_softmax_row(row), rtol=1e-12, atol=1e-300)
+
+
+def test_causal_is_the_unfused_torch_expression():
+    # where(causal, scale*x, -1e9) + pad -> torch.softmax : the GPT-J form of
+    # the unfused attention. Right padding, so every row has a visible key.
+    g = torch.Generator().manual_seed(0)
+    b, h, s = 3, 2, 33
+    x = torch.randn(b, h, s, s, generator=g, dtype=torch.float64) * 4
+    lens = torch.tensor([33, 20, 1])
+    pad = torch.where(torch.arange(s)[None, :] < lens[:, None], 0.0, -10000.0).to(torch.float64)
+    causal = torch.tril(torch.ones(s, s, dtype=torch.bool))
+    e = torch.where(causal, x * 0.25, torch.tensor(-1e9, dtype=torch.float64)) + pad[:, None, None, :]
+    want = torch.softmax(e, dim=-1).numpy()
+    got = orc.softmax_causal(x.numpy(), 0.25, pad.numpy(), dtype=np.float64)
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-15)
+
+
+def test_causal_special_cases():
+    x = rng(3).standard_normal((1, 1, 6, 6))
+    y = orc.softmax_causal(x, 0.5, dtype=np.float64)
+    # row 0 is [1, 0, ...]; row 1 is [sigmoid(s*(x0-x1)), 1 - ...]
+    np.testing.assert_array_equal(y[0, 0, 0], [1, 0, 0, 0, 0, 0])
+    p = 1 / (1 + math.exp(-0.5 * (x[0, 0, 1, 0] - x[0, 0, 1, 1])))
+    np.testing.assert_allclose(y[0, 0, 1, :2], [p, 1 - p], rtol=1e-12)
+    assert np.all(np.triu(y[0, 0], 1) == 0)
+    np.testing.assert_allclose(y.sum(-1), 1, rtol=1e-12)
+    # adding a constant to a row changes nothing
+    y2 = orc.softmax_causal(x + 7.0, 0.5, dtype=np.float64)
+    np.testing.assert_allclose(y2, y, rtol=1e-10)
+    # scale 1, last row, no mask == library softmax of the full row
+    want = torch.softmax(torch.from_numpy(x[0, 0, 5]), -1).numpy()
+    np.testing.assert_allclose(orc.softmax_causal(x, 1.0, dtype=np.float64)[0, 0, 5], want, rtol=1e-12)
+
+
+@pytest.mark.parametrize("mode", ["add", "replace"])
+def test_masked_matches_python_loops(mode):
+    b, h, sq, sk = 2, 2, 3, 7
+    x = rng(5).standard_normal((b, h, sq, sk)) * 2
+    mask = rng(6).random((b, 1, sq, sk)) < 0.4
+    mask[0, 0, 1, :] = True  # a row with every key masked
+    scale = 1.7
+    got = orc.softmax_masked(x, mask, scale, mode, dtype=np.float64)
+    for bi in range(b):
+        for hi in range(h):
+            for q in range(sq):
+                row = []
+                for k in range(sk):
+                    e = x[bi, hi, q, k] * scale
+                    if mask[bi, 0, q, k]:
+                        e = e - 10000.0 if mode == "add" else -10000.0
+                    row.append(e)
+                np.testing.assert_allclose(got[bi, hi, q], brute_softmax_row(row), rtol=1e-9, atol=1e-300)
+    # fully masked row: "replace" is uniform, "add" is the softmax of the raw scores
+    if mode == "replace":
+        np.testing.assert_allclose(got[0, :, 1], 1.0 / sk, rtol=1e-12)
+    else:
+        want = torch.softmax(torch.from_numpy(x[0, :, 1] * scale), -1).numpy()
+        np.testing.assert_allclose(got[0, :, 1], want, rtol=1e-9)
+
+
+def test_masked_add_is_the_unfused_torch_expression_and_modes_agree():
+    g = torch.Generator().manual_seed(1)
+    b, h, sq, sk = 2, 3, 5, 19
+    x = torch.randn(b, h, sq, sk, generator=g, dtype=torch.float64) * 3
+    lens = torch.tensor([19, 6])
+    key_mask = (torch.arange(sk)[None, :] >= lens[:, None]).view(b, 1, 1, sk)
+    add = torch.where(key_mask, -10000.0, 0.0).to(torch.float64)
+    want = torch.softmax(x * 0.125 + add, dim=-1).numpy()
+    got = orc.softmax_masked(x.numpy(), key_mask.numpy(), 0.125, "add", dtype=np.float64)
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-300)
+    # with at least one visible key per row the two modes give the same fp32
+    # result: masked keys underflow to exactly 0 either way
+    a32 = orc.softmax_masked(x.numpy(), key_mask.numpy(), 0.125, "add", dtype=np.float32)
+    r32 = orc.softmax_masked(x.numpy(), key_mask.numpy(), 0.125, "replace", dtype=np.float32)
+    np.testing.assert_array_equal(a32, r32)
+    assert np.all(a32[1, :, :, 6:] == 0)
+    # no mask, scale 1 == library softmax
+    np.testing.assert_allclose(orc.softmax_masked(x.numpy(), None, 1.0, dtype=np.float64),
+                               torch.softmax(x, -1).numpy(), rtol=1e-12)
+
+
+# ---------------------------------------------------------------------------
+# softmax backward
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_softmax_bwd_matches_autograd(causal):
+    g = torch.Generator().manual_seed(2)
+    s = 9
+    x = torch.randn(2, 2, s, s, generator=g, dtype=torch.float64, requires_grad=True)
+    go = torch.randn(2, 2, s, s, generator=g, dtype=torch.float64)
+    scale = 0.3
+    e = x * scale
+    if causal:
+        e = e.masked_fill(~torch.tril(torch.ones(s, s, dtype=torch.bool)), float("-inf"))
+    y = torch.softmax(e, -1)
+    (dx,) = torch.autograd.grad(y, x, go)
+    got = orc.softmax_bwd(go.numpy(), y.detach().numpy(), scale, causal=causal, dtype=np.float64)
+    np.testing.assert_allclose(got, dx.numpy(), rtol=1e-10, atol=1e-14)
+    # gradient of a softmax row sums to zero; nothing flows above the diagonal
+    np.testing.assert_allclose(got.sum(-1), 0, atol=1e-13)
+    if causal:
+        assert np.all(np.triu(got, 1) == 0)
+        # upper-triangle garbage in g and y must not matter
+        junk_g = go.numpy() + np.triu(np.full((s, s), 123.0), 1)
+        junk_y = y.detach().numpy() + np.triu(np.full((s, s), 0.5), 1)
+        np.testing.assert_allclose(orc.softmax_bwd(junk_g, junk_y, scale, causal=True, dtype=np.float64),
+                                   got, rtol=1e-12, atol=1e-15)
+
+
+def test_softmax_gradcheck_of_the_forward():
+    # finite differences of the oracle's own forward agree with its backward
+    s, scale, eps = 5, 0.7, 1e-6
+    x = rng(8).standard_normal((1, 1, s, s))
+    go = rng(9).standard_normal((1, 1, s, s))
+    y = orc.softmax_causal(x, scale, dtype=np.float64)
+    dx = orc.softmax_bwd(go, y, scale, causal=True, dtype=np.float64)
+    for (r, k) in [(0, 0), (2, 1), (4, 4), (3, 0), (1, 3)]:
+        xp, xm = x.copy(), x.copy()
+        xp[0, 0, r, k] += eps
+        xm[0, 0, r, k] -= eps
+        fd = ((orc.softmax_causal(xp, scale, dtype=np.float64) -
+               orc.softmax_causal(xm, scale, dtype=np.float64)) * go).sum() / (2 * eps)
+        assert abs(fd - dx[0, 0, r, k]) < 1e-8
+
+
+# ---------------------------------------------------------------------------
+# integer helpers
+# ---------------------------------------------------------------------------
+
+def test_get_batch_per_block_known_answers():
+    # hand-derived from 128 threads / min(next_pow2(sk), 32) lanes, two rows per
+    # warp up to 128 keys
+    table = {1: 256, 2: 128, 3: 64, 4: 64, 8: 32, 16: 16, 17: 8, 32: 8, 33: 8, 64: 8, 128: 8,
+             129: 4, 256: 4, 1024: 4, 2047: 4, 2048: 4}
+    for sk, want in table.items():
+        assert orc.get_batch_per_block(7, sk, 3, 5) == want, sk
+
+
+def test_reference_gate_known_answers():
+    ok = orc.reference_is_available
+    assert ok(True, 8, 16, 2048, 2048, True)
+    assert not ok(False, 8, 16, 2048, 2048, True)       # not fp16
+    assert not ok(True, 8, 16, 4096, 4096, True)        # too long
+    assert not ok(True, 8, 16, 1, 2048, True)           # decode step: sq != sk
+    assert not ok(True, 1, 3, 1024, 1024, True)         # 3 rows-batches not divisible by 4
+    assert ok(True, 1, 1, 63, 63, True) is False        # bpb = 8 does not divide 1
+    assert ok(True, 2, 4, 63, 63, True)                 # sk <= 64 needs no sk % 4
+    assert not ok(True, 2, 4, 66, 66, True)             # sk > 64 and sk % 4 != 0
+    assert ok(True, 2, 4, 1024, 1024, False)
+    assert not ok(True, 2, 4, 1, 1024, False)           # sq == 1
+    assert not ok(True, 2, 4, 6, 1024, False)           # 6 % 4 != 0
+
+
+# ---------------------------------------------------------------------------
+# bias + GeLU
+# ---------------------------------------------------------------------------
+
+def test_bias_gelu_fwd_is_library_tanh_gelu():
+    g = torch.Generator().manual_seed(3)
+    y = torch.randn(7, 33, generator=g, dtype=torch.float64) * 3
+    b = torch.randn(33, generator=g, dtype=torch.float64)
+    want = torch.nn.functional.gelu(y + b, approximate="tanh").numpy()
+    got = orc.bias_gelu_fwd(y.numpy(), b.numpy(), dtype=np.float64)
+    # the reference's 8-digit constant 0.79788456 differs from sqrt(2/pi) by 8e-10 relative
+    np.testing.assert_allclose(got, want, rtol=2e-8, atol=2e-9)
+    # known values: gelu(0) = 0, gelu(large) = x, gelu(-large) = 0
+    pts = orc.bias_gelu_fwd(np.array([[0.0, 12.0, -12.0]]), np.zeros(3), dtype=np.float64)
+    np.testing.assert_allclose(pts, [[0.0, 12.0, 0.0]], atol=1e-12)
+    # and the installed transformers "gelu_new", the activation the models name
+    from transformers.activations import ACT2FN
+    want_new = ACT2FN["gelu_new"]((y + b).float()).numpy()
+    np.testing.assert_allclose(orc.bias_gelu_fwd(y.numpy(), b.numpy()), want_new, rtol=1e-5, atol=1e-6)
+
+
+def test_bias_gelu_bwd_matches_autograd_and_constant_identity():
+    assert abs(3 * 0.044715 * 0.79788456 - 0.1070322243) < 1e-10
+    g = torch.Generator().manual_seed(4)
+    y = torch.randn(5, 4, 11, generator=g, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(11, generator=g, dtype=torch.float64, requires_grad=True)
+    go = torch.randn(5, 4, 11, generator=g, dtype=torch.float64)
+    x = y + b
+    out = x * 0.5 * (1.0 + torch.tanh(0.79788456 * x * (1 + 0.044715 * x * x)))
+    dy, db = torch.autograd.grad(out, (y, b), go)
+    got_dy, got_db = orc.bias_gelu_bwd(go.numpy(), y.detach().numpy(), b.detach().numpy(), dtype=np.float64)
+    np.testing.assert_allclose(got_dy, dy.numpy(), rtol=1e-8, atol=1e-10)
+    np.testing.assert_allclose(got_db, db.numpy(), rtol=1e-8, atol=1e-10)
+
+
+# ---------------------------------------------------------------------------
+# Philox + dropout
+# ---------------------------------------------------------------------------
+
+def test_philox_published_known_answers():
+    # Random123 kat_vectors, philox4x32 with 10 rounds
+    kats = [
+        ((0, 0, 0, 0), (0, 0), (0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8)),
+        ((0xFFFFFFFF,) * 4, (0xFFFFFFFF,) * 2, (0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD)),
+        ((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0),
+         (0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1)),
+    ]
+    for ctr, key, want in kats:
+        got = orc.philox4x32_10(key, [np.array([c], dtype=np.uint32) for c in ctr])
+        assert tuple(int(w[0]) for w in got) == want
+
+
+def test_dropout_words_match_torch_engine_fixture():
+    fx = json.load(open(os.path.join(HERE, "golden", "philox_vectors.json")))
+    assert len(fx["vectors"]) >= 8
+    for v in fx["vectors"]:
+        grp, blk = v["group"], v["offset"] // 4
+        got = orc.philox4x32_10(
+            (v["seed"] & 0xFFFFFFFF, v["seed"] >> 32),
+            [np.array([c], dtype=np.uint32) for c in
+             (blk & 0xFFFFFFFF, blk >> 32, grp & 0xFFFFFFFF, grp >> 32)])
+        assert [int(w[0]) for w in got] == v["words"], v
+    # the mask generator lays groups out as documented: element i <- word i%4 of group i//4
+    v = fx["vectors"][1]  # seed 1234, group 0, offset 0
+    thr = orc.dropout_threshold(0.5)
+    keep = orc.dropout_keep_mask(1234, 0, 4, 0.5)
+    assert list(keep) == [w >= thr for w in v["words"]]
+    v = fx["vectors"][2]  # seed 1234, group 1, offset 0
+    keep = orc.dropout_keep_mask(1234, 0, 7, 0.5)
+    assert list(keep[4:7]) == [w >= thr for w in v["words"][:3]]
+    v = fx["vectors"][3]  # seed 1234, group 0, offset 4 (one counter block later)
+    keep = orc.dropout_keep_mask(1234, 4, 4, 0.5)
+    assert list(keep) == [w >= thr for w in v["words"]]
+
+
+def test_dropout_mask_statistics_and_thresholds():
+    assert orc.dropout_threshold(0.0) == 0
+    assert orc.dropout_threshold(0.5) == 2 ** 31
+    assert orc.dropout_threshold(0.25) == 2 ** 30
+    n, p = 1 << 20, 0.1
+    keep = orc.dropout_keep_mask(1234, 0, n, p)
+    rate = keep.mean()
+    sigma = math.sqrt(p * (1 - p) / n)
+    assert abs(rate - (1 - p)) < 4 * sigma
+    # a different offset or seed gives a different mask; the same pair repeats
+    assert (orc.dropout_keep_mask(1234, 4, n, p) != keep).mean() > 0.1
+    assert (orc.dropout_keep_mask(1235, 0, n, p) != keep).mean() > 0.1
+    assert np.array_equal(orc.dropout_keep_mask(1234, 0, n, p), keep)
+
+
+def test_bias_dropout_add_closed_forms():
+    r = rng(11)
+    x, res = r.standard_normal((6, 10)), r.standard_normal((6, 10))
+    b = r.standard_normal(10)
+    # p = 0: exactly x + b + res
+    np.testing.assert_array_equal(orc.bias_dropout_add_fwd(x, b, res, 0.0, None, dtype=np.float64), x + b + res)
+    keep = r.random((6, 10)) < 0.7
+    p = 0.3
+    out = orc.bias_dropout_add_fwd(x, b, res, p, keep, dtype=np.float64)
+    # same as torch: (x + b) * mask / (1 - p) + res
+    want = (torch.from_numpy(x + b) * torch.from_numpy(keep) / (1 - float(np.float32(p)))
+            + torch.from_numpy(res)).numpy()
+    np.testing.assert_allclose(out, want, rtol=1e-12)
+    go = r.standard_normal((6, 10))
+    dx, db, dres = orc.bias_dropout_add_bwd(go, p, keep, dtype=np.float64)
+    np.testing.assert_allclose(dx, go * keep / (1 - float(np.float32(p))), rtol=1e-12)
+    np.testing.assert_allclose(db, dx.sum(0), rtol=1e-12)
+    np.testing.assert_array_equal(dres, go)
+    # autograd through the same expression with the mask held fixed
+    xt = torch.from_numpy(x).requires_grad_()
+    bt = torch.from_numpy(b).requires_grad_()
+    rt = torch.from_numpy(res).requires_grad_()
+    o = (xt + bt) * torch.from_numpy(keep) / (1 - float(np.float32(p))) + rt
+    gx, gb, gr = torch.autograd.grad(o, (xt, bt, rt), torch.from_numpy(go))
+    np.testing.assert_allclose(dx, gx.numpy(), rtol=1e-12)
+    np.testing.assert_allclose(db, gb.numpy(), rtol=1e-12)
+    np.testing.assert_allclose(dres, gr.numpy(), rtol=1e-12)

