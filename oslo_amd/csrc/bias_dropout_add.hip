@@ -31,94 +31,89 @@ __device__ __forceinline__ void keep_flags(bool (&keep)[VEC], uint64_t seed,
   }
 }
 
-template <typename T, int VEC, bool DROP, bool HAS_BIAS, bool HAS_RES>
+template <typename T, int VEC, int U, bool DROP, bool HAS_BIAS, bool HAS_RES>
 __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_fwd_kernel(
     T *out, const T *x, const T *__restrict__ bias, const T *residual,
     float keep_scale, uint32_t threshold, uint64_t seed, uint64_t offset,
-    int64_t rows, int64_t cols, int rows_per_block) {
-  const int64_t c0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
-  if (c0 >= cols) return; // no barrier in this kernel
-  float b[VEC];
-  if constexpr (HAS_BIAS) load_f32_cached<T, VEC>(b, bias + c0);
-  const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
-  const int64_t r1 = min(rows, r0 + rows_per_block);
+    int64_t rows, int64_t cols, int col_tiles, int rows_per_block) {
+  const EwPos pos = ew_position<VEC>(col_tiles, rows_per_block);
+  if (pos.c0 >= cols) return; // no barrier in this kernel
   const int TY = blockDim.y;
-  for (int64_t r = r0 + threadIdx.y; r < r1; r += (int64_t)TY * kRowUnroll) {
-    float tx[kRowUnroll][VEC], tr[kRowUnroll][VEC];
+  const BufRsrc xrs = ew_rsrc<T>(x, pos, rows_per_block, rows, cols);
+  RawVec<T, VEC> xraw[U], rraw[HAS_RES ? U : 1];
 #pragma unroll
-    for (int u = 0; u < kRowUnroll; ++u) {
-      const int64_t rr = r + (int64_t)u * TY;
-      if (rr < r1) {
-        load_f32<T, VEC>(tx[u], x + rr * cols + c0);
-        if constexpr (HAS_RES) load_f32<T, VEC>(tr[u], residual + rr * cols + c0);
+  for (int u = 0; u < U; ++u)
+    xraw[u] = buffer_load_raw<T, VEC, true>(xrs, ew_offset<T>(pos, u, cols));
+  if constexpr (HAS_RES) {
+    const BufRsrc rrs = ew_rsrc<T>(residual, pos, rows_per_block, rows, cols);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      rraw[u] = buffer_load_raw<T, VEC, true>(rrs, ew_offset<T>(pos, u, cols));
+  }
+  float b[VEC];
+  if constexpr (HAS_BIAS) load_f32_cached<T, VEC>(b, bias + pos.c0);
+  float tx[U][VEC], tr[U][VEC];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t r = pos.r_base + (int64_t)u * TY;
+    raw_to_f32<T, VEC>(tx[u], xraw[u]);
+    if constexpr (HAS_RES) raw_to_f32<T, VEC>(tr[u], rraw[u]);
+    if (r < rows) {
+      bool keep[VEC];
+      if constexpr (DROP)
+        keep_flags<VEC>(keep, seed, offset, (uint64_t)(r * cols + pos.c0), threshold);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        float t = tx[u][j];
+        if constexpr (HAS_BIAS) t += b[j];
+        if constexpr (DROP) t = keep[j] ? t * keep_scale : 0.f;
+        if constexpr (HAS_RES) t += tr[u][j];
+        tx[u][j] = t;
       }
-    }
-#pragma unroll
-    for (int u = 0; u < kRowUnroll; ++u) {
-      const int64_t rr = r + (int64_t)u * TY;
-      if (rr < r1) {
-        bool keep[VEC];
-        if constexpr (DROP)
-          keep_flags<VEC>(keep, seed, offset, (uint64_t)(rr * cols + c0),
-                          threshold);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          float t = tx[u][j];
-          if constexpr (HAS_BIAS) t += b[j];
-          if constexpr (DROP) t = keep[j] ? t * keep_scale : 0.f;
-          if constexpr (HAS_RES) t += tr[u][j];
-          tx[u][j] = t;
-        }
-        store_f32<T, VEC>(out + rr * cols + c0, tx[u]);
-      }
+      store_f32<T, VEC>(out + r * cols + pos.c0, tx[u]);
     }
   }
 }
 
-template <typename T, int VEC, bool DROP, bool WANT_DBIAS>
+template <typename T, int VEC, int U, bool DROP, bool WANT_DBIAS>
 __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_bwd_kernel(
     T *dx, float *__restrict__ partial, const T *g, float keep_scale,
     uint32_t threshold, uint64_t seed, uint64_t offset, int64_t rows,
-    int64_t cols, int rows_per_block) {
-  const int64_t c0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
-  const bool col_ok = c0 < cols;
+    int64_t cols, int col_tiles, int rows_per_block) {
+  const EwPos pos = ew_position<VEC>(col_tiles, rows_per_block);
+  const bool col_ok = pos.c0 < cols;
+  const int TY = blockDim.y;
   float acc[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
   if (col_ok) {
-    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
-    const int64_t r1 = min(rows, r0 + rows_per_block);
-    const int TY = blockDim.y;
-    for (int64_t r = r0 + threadIdx.y; r < r1; r += (int64_t)TY * kRowUnroll) {
-      float tg[kRowUnroll][VEC];
+    const BufRsrc grs = ew_rsrc<T>(g, pos, rows_per_block, rows, cols);
+    RawVec<T, VEC> graw[U];
 #pragma unroll
-      for (int u = 0; u < kRowUnroll; ++u) {
-        const int64_t rr = r + (int64_t)u * TY;
-        if (rr < r1) load_f32<T, VEC>(tg[u], g + rr * cols + c0);
-      }
+    for (int u = 0; u < U; ++u)
+      graw[u] = buffer_load_raw<T, VEC, true>(grs, ew_offset<T>(pos, u, cols));
+    float tg[U][VEC];
 #pragma unroll
-      for (int u = 0; u < kRowUnroll; ++u) {
-        const int64_t rr = r + (int64_t)u * TY;
-        if (rr < r1) {
-          bool keep[VEC];
-          if constexpr (DROP)
-            keep_flags<VEC>(keep, seed, offset, (uint64_t)(rr * cols + c0),
-                            threshold);
+    for (int u = 0; u < U; ++u) {
+      const int64_t r = pos.r_base + (int64_t)u * TY;
+      raw_to_f32<T, VEC>(tg[u], graw[u]);
+      if (r < rows) {
+        bool keep[VEC];
+        if constexpr (DROP)
+          keep_flags<VEC>(keep, seed, offset, (uint64_t)(r * cols + pos.c0), threshold);
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            if constexpr (DROP)
-              tg[u][j] = keep[j] ? tg[u][j] * keep_scale : 0.f;
-            if constexpr (WANT_DBIAS) acc[j] += tg[u][j];
-          }
-          // with no dropout dx == g bit for bit; still written, dx may be a
-          // different buffer
-          store_f32<T, VEC>(dx + rr * cols + c0, tg[u]);
+        for (int j = 0; j < VEC; ++j) {
+          if constexpr (DROP) tg[u][j] = keep[j] ? tg[u][j] * keep_scale : 0.f;
+          if constexpr (WANT_DBIAS) acc[j] += tg[u][j];
         }
+        // with no dropout dx == g bit for bit; still written, dx may be a
+        // different buffer
+        store_f32<T, VEC>(dx + r * cols + pos.c0, tg[u]);
       }
     }
   }
   if constexpr (WANT_DBIAS)
-    write_colsum_partial<VEC>(acc, partial, cols, c0, col_ok);
+    write_colsum_partial<VEC>(acc, partial, cols, pos, col_ok);
 }
 
 struct DropArgs {
@@ -128,16 +123,20 @@ struct DropArgs {
   bool drop;
 };
 
+constexpr int kDropBwdUnroll = 4;
+static_assert(kDropBwdUnroll >= kBwdMinUnroll, "workspace bound");
+
 template <typename T, int VEC>
 int launch_fwd(T *out, const T *x, const T *bias, const T *res,
                const DropArgs &a, int64_t rows, int64_t cols,
                hipStream_t stream) {
-  const EwPlan p = plan_elementwise(rows, cols / VEC, kRowsPerBlockFwd);
+  const EwPlan p = plan_elementwise(rows, cols / VEC, kFwdMaxTx, kFwdUnroll);
+  if (!p.ok) return fail(OSLO_E_UNSUPPORTED, "bias_dropout_add_fwd: tensor too large for one launch");
   auto go = [&]<bool DROP, bool HB, bool HR>() {
-    bias_dropout_add_fwd_kernel<T, VEC, DROP, HB, HR>
+    bias_dropout_add_fwd_kernel<T, VEC, kFwdUnroll, DROP, HB, HR>
         <<<p.grid, p.block, 0, stream>>>(out, x, bias, res, a.keep_scale,
                                          a.threshold, a.seed, a.offset, rows,
-                                         cols, p.rows_per_block);
+                                         cols, p.col_tiles, p.rows_per_block);
   };
   const int sel = (a.drop ? 4 : 0) | (bias ? 2 : 0) | (res ? 1 : 0);
   switch (sel) {
@@ -156,12 +155,13 @@ int launch_fwd(T *out, const T *x, const T *bias, const T *res,
 template <typename T, int VEC>
 int launch_bwd(T *dx, T *dbias, float *ws, const T *g, const DropArgs &a,
                int64_t rows, int64_t cols, hipStream_t stream) {
-  const EwPlan p = plan_elementwise(rows, cols / VEC, kRowsPerBlockBwd);
+  const EwPlan p = plan_elementwise(rows, cols / VEC, kBwdMaxTx, kDropBwdUnroll);
+  if (!p.ok) return fail(OSLO_E_UNSUPPORTED, "bias_dropout_add_bwd: tensor too large for one launch");
   auto go = [&]<bool DROP, bool WANT>() {
-    bias_dropout_add_bwd_kernel<T, VEC, DROP, WANT>
+    bias_dropout_add_bwd_kernel<T, VEC, kDropBwdUnroll, DROP, WANT>
         <<<p.grid, p.block, 0, stream>>>(dx, ws, g, a.keep_scale, a.threshold,
                                          a.seed, a.offset, rows, cols,
-                                         p.rows_per_block);
+                                         p.col_tiles, p.rows_per_block);
   };
   if (a.drop) {
     if (dbias) go.template operator()<true, true>();
@@ -172,7 +172,7 @@ int launch_bwd(T *dx, T *dbias, float *ws, const T *g, const DropArgs &a,
   }
   int s = check_launch("bias_dropout_add_bwd");
   if (s != OSLO_OK || !dbias) return s;
-  launch_colsum_finish<T>(dbias, ws, (int)p.grid.y, cols, stream);
+  launch_colsum_finish<T>(dbias, ws, p.row_blocks, cols, stream);
   return check_launch("bias_dropout_add_bwd(dbias)");
 }
 
@@ -241,7 +241,7 @@ extern "C" int oslo_bias_dropout_add_bwd(void *dx, void *dbias,
   OSLO_DISPATCH_DTYPE(dtype, {
     if (rows == 0) {
       if (dbias)
-        launch_colsum_finish<T>(static_cast<T *>(dbias), nullptr, 0, cols, st);
+        launch_colsum_finish<T>(static_cast<T *>(dbias), nullptr, 0, cols, st); // writes zeros
       return check_launch("bias_dropout_add_bwd(dbias)");
     }
     constexpr int V = Io<T>::kVec;

@@ -21,121 +21,128 @@ constexpr float kW1 = kW0 * kGeluA;
 constexpr float kD0 = 2.0f * kGeluK;
 constexpr float kD1 = 2.0f * 0.1070322243f;
 
-__device__ __forceinline__ float sigmoid_2u(float x, float x2) {
-  const float w = x * __builtin_fmaf(x2, kW1, kW0);
-  const float e = __builtin_amdgcn_exp2f(w); // exp(-2u); inf for very negative x
-  return __builtin_amdgcn_rcpf(1.0f + e);    // rcp(inf) = 0
+// e = exp(-2u), clamped so that e stays finite (x below about -5.4 gives the
+// clamp; the results there are 0 to within 2^-126).
+__device__ __forceinline__ float exp_m2u(float x, float x2) {
+  const float w = fminf(x * __builtin_fmaf(x2, kW1, kW0), 126.0f);
+  return __builtin_amdgcn_exp2f(w);
 }
 
 __device__ __forceinline__ float gelu_fwd(float x) {
-  return x * sigmoid_2u(x, x * x);
+  const float e = exp_m2u(x, x * x);
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
-// d/dx [x*s] = s + x*s*(1-s)*2u'
+// d/dx [x*s] = s + x*s*(1-s)*2u' with s = r = 1/(1+e) and 1-s = e*r: written
+// as r + q*(e*r)*r so that no difference of nearly equal numbers is formed
+// (the reference's 1 - tanh^2 loses about two digits in fp32 for |x| > 2).
 __device__ __forceinline__ float gelu_grad(float x) {
   const float x2 = x * x;
-  const float s = sigmoid_2u(x, x2);
+  const float e = exp_m2u(x, x2);
+  const float r = __builtin_amdgcn_rcpf(1.0f + e);
   const float q = x * __builtin_fmaf(x2, kD1, kD0);
-  return __builtin_fmaf(q, s * (1.0f - s), s);
+  return __builtin_fmaf(q * (e * r), r, r);
 }
 
-template <typename T, int VEC>
+template <typename T, int VEC, int U>
 __global__ __launch_bounds__(kBlockThreads) void bias_gelu_fwd_kernel(
     T *out, const T *y, const T *__restrict__ bias, int64_t rows, int64_t cols,
-    int rows_per_block) {
-  const int64_t c0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
-  if (c0 >= cols) return; // no barrier in this kernel
-  float b[VEC];
-  load_f32_cached<T, VEC>(b, bias + c0);
-  const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
-  const int64_t r1 = min(rows, r0 + rows_per_block);
+    int col_tiles, int rows_per_block) {
+  const EwPos pos = ew_position<VEC>(col_tiles, rows_per_block);
+  if (pos.c0 >= cols) return; // no barrier in this kernel
   const int TY = blockDim.y;
-  for (int64_t r = r0 + threadIdx.y; r < r1; r += (int64_t)TY * kRowUnroll) {
-    float t[kRowUnroll][VEC];
+  const BufRsrc yrs = ew_rsrc<T>(y, pos, rows_per_block, rows, cols);
+  RawVec<T, VEC> raw[U];
 #pragma unroll
-    for (int u = 0; u < kRowUnroll; ++u) {
-      const int64_t rr = r + (int64_t)u * TY;
-      if (rr < r1) load_f32<T, VEC>(t[u], y + rr * cols + c0);
-    }
+  for (int u = 0; u < U; ++u)
+    raw[u] = buffer_load_raw<T, VEC, true>(yrs, ew_offset<T>(pos, u, cols));
+  float b[VEC];
+  load_f32_cached<T, VEC>(b, bias + pos.c0);
+  float t[U][VEC];
 #pragma unroll
-    for (int u = 0; u < kRowUnroll; ++u) {
-      const int64_t rr = r + (int64_t)u * TY;
-      if (rr < r1) {
+  for (int u = 0; u < U; ++u) {
+    const int64_t r = pos.r_base + (int64_t)u * TY;
+    raw_to_f32<T, VEC>(t[u], raw[u]);
+    if (r < rows) {
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) t[u][j] = gelu_fwd(t[u][j] + b[j]);
-        store_f32<T, VEC>(out + rr * cols + c0, t[u]);
-      }
+      for (int j = 0; j < VEC; ++j) t[u][j] = gelu_fwd(t[u][j] + b[j]);
+      store_f32<T, VEC>(out + r * cols + pos.c0, t[u]);
     }
   }
 }
 
-template <typename T, int VEC, bool WANT_DBIAS>
+template <typename T, int VEC, int U, bool WANT_DBIAS>
 __global__ __launch_bounds__(kBlockThreads) void bias_gelu_bwd_kernel(
     T *dy, float *__restrict__ partial, const T *g, const T *y,
-    const T *__restrict__ bias, int64_t rows, int64_t cols,
+    const T *__restrict__ bias, int64_t rows, int64_t cols, int col_tiles,
     int rows_per_block) {
-  const int64_t c0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
-  const bool col_ok = c0 < cols;
+  const EwPos pos = ew_position<VEC>(col_tiles, rows_per_block);
+  const bool col_ok = pos.c0 < cols;
+  const int TY = blockDim.y;
   float acc[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
   if (col_ok) {
+    const BufRsrc grs = ew_rsrc<T>(g, pos, rows_per_block, rows, cols);
+    const BufRsrc yrs = ew_rsrc<T>(y, pos, rows_per_block, rows, cols);
+    RawVec<T, VEC> graw[U], yraw[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      graw[u] = buffer_load_raw<T, VEC, true>(grs, ew_offset<T>(pos, u, cols));
+      yraw[u] = buffer_load_raw<T, VEC, true>(yrs, ew_offset<T>(pos, u, cols));
+    }
     float b[VEC];
-    load_f32_cached<T, VEC>(b, bias + c0);
-    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
-    const int64_t r1 = min(rows, r0 + rows_per_block);
-    const int TY = blockDim.y;
-    for (int64_t r = r0 + threadIdx.y; r < r1; r += (int64_t)TY * kRowUnroll) {
-      float tg[kRowUnroll][VEC], ty_[kRowUnroll][VEC];
+    load_f32_cached<T, VEC>(b, bias + pos.c0);
+    float tg[U][VEC], ty_[U][VEC];
 #pragma unroll
-      for (int u = 0; u < kRowUnroll; ++u) {
-        const int64_t rr = r + (int64_t)u * TY;
-        if (rr < r1) {
-          load_f32<T, VEC>(tg[u], g + rr * cols + c0);
-          load_f32<T, VEC>(ty_[u], y + rr * cols + c0);
+    for (int u = 0; u < U; ++u) {
+      const int64_t r = pos.r_base + (int64_t)u * TY;
+      raw_to_f32<T, VEC>(tg[u], graw[u]);
+      raw_to_f32<T, VEC>(ty_[u], yraw[u]);
+      if (r < rows) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          tg[u][j] = gelu_grad(ty_[u][j] + b[j]) * tg[u][j];
+          if constexpr (WANT_DBIAS) acc[j] += tg[u][j];
         }
-      }
-#pragma unroll
-      for (int u = 0; u < kRowUnroll; ++u) {
-        const int64_t rr = r + (int64_t)u * TY;
-        if (rr < r1) {
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            tg[u][j] = gelu_grad(ty_[u][j] + b[j]) * tg[u][j];
-            if constexpr (WANT_DBIAS) acc[j] += tg[u][j];
-          }
-          store_f32<T, VEC>(dy + rr * cols + c0, tg[u]);
-        }
+        store_f32<T, VEC>(dy + r * cols + pos.c0, tg[u]);
       }
     }
   }
   if constexpr (WANT_DBIAS)
-    write_colsum_partial<VEC>(acc, partial, cols, c0, col_ok);
+    write_colsum_partial<VEC>(acc, partial, cols, pos, col_ok);
 }
+
+constexpr int kGeluBwdUnroll = 2;
+static_assert(kGeluBwdUnroll >= kBwdMinUnroll, "workspace bound");
 
 template <typename T, int VEC>
 int launch_fwd(T *out, const T *y, const T *bias, int64_t rows, int64_t cols,
                hipStream_t stream) {
-  const EwPlan p = plan_elementwise(rows, cols / VEC, kRowsPerBlockFwd);
-  bias_gelu_fwd_kernel<T, VEC><<<p.grid, p.block, 0, stream>>>(
-      out, y, bias, rows, cols, p.rows_per_block);
+  const EwPlan p = plan_elementwise(rows, cols / VEC, kFwdMaxTx, kFwdUnroll);
+  if (!p.ok) return fail(OSLO_E_UNSUPPORTED, "bias_gelu_fwd: tensor too large for one launch");
+  bias_gelu_fwd_kernel<T, VEC, kFwdUnroll><<<p.grid, p.block, 0, stream>>>(
+      out, y, bias, rows, cols, p.col_tiles, p.rows_per_block);
   return check_launch("bias_gelu_fwd");
 }
 
 template <typename T, int VEC>
 int launch_bwd(T *dy, T *dbias, float *ws, const T *g, const T *y,
                const T *bias, int64_t rows, int64_t cols, hipStream_t stream) {
-  const EwPlan p = plan_elementwise(rows, cols / VEC, kRowsPerBlockBwd);
+  const EwPlan p = plan_elementwise(rows, cols / VEC, kBwdMaxTx, kGeluBwdUnroll);
+  if (!p.ok) return fail(OSLO_E_UNSUPPORTED, "bias_gelu_bwd: tensor too large for one launch");
   if (dbias) {
-    bias_gelu_bwd_kernel<T, VEC, true><<<p.grid, p.block, 0, stream>>>(
-        dy, ws, g, y, bias, rows, cols, p.rows_per_block);
+    bias_gelu_bwd_kernel<T, VEC, kGeluBwdUnroll, true>
+        <<<p.grid, p.block, 0, stream>>>(dy, ws, g, y, bias, rows, cols,
+                                         p.col_tiles, p.rows_per_block);
     int s = check_launch("bias_gelu_bwd");
     if (s != OSLO_OK) return s;
-    launch_colsum_finish<T>(dbias, ws, (int)p.grid.y, cols, stream);
+    launch_colsum_finish<T>(dbias, ws, p.row_blocks, cols, stream);
     return check_launch("bias_gelu_bwd(dbias)");
   }
-  bias_gelu_bwd_kernel<T, VEC, false><<<p.grid, p.block, 0, stream>>>(
-      dy, nullptr, g, y, bias, rows, cols, p.rows_per_block);
+  bias_gelu_bwd_kernel<T, VEC, kGeluBwdUnroll, false>
+      <<<p.grid, p.block, 0, stream>>>(dy, nullptr, g, y, bias, rows, cols,
+                                       p.col_tiles, p.rows_per_block);
   return check_launch("bias_gelu_bwd");
 }
 
@@ -181,7 +188,7 @@ extern "C" int oslo_bias_gelu_bwd(void *dy, void *dbias, float *workspace,
   OSLO_DISPATCH_DTYPE(dtype, {
     if (rows == 0) { // empty batch: the bias gradient is still defined (zero)
       if (dbias)
-        launch_colsum_finish<T>(static_cast<T *>(dbias), nullptr, 0, cols, st);
+        launch_colsum_finish<T>(static_cast<T *>(dbias), nullptr, 0, cols, st); // writes zeros
       return check_launch("bias_gelu_bwd(dbias)");
     }
     constexpr int V = Io<T>::kVec;

@@ -61,9 +61,9 @@ extern "C" int oslo_get_batch_per_block(int sq, int sk, int batches, int heads) 
 
 extern "C" size_t oslo_colsum_workspace_bytes(int64_t rows, int64_t cols) {
   if (rows <= 0 || cols <= 0) return 0;
-  // One fp32 partial row per block row range; a range is never shorter than
-  // kRowsPerBlockBwd rows whatever the column tiling.
-  int64_t parts = (rows + oslo::kRowsPerBlockBwd - 1) / oslo::kRowsPerBlockBwd;
-  if (parts > 32768) parts = 32768;
-  return (size_t)parts * (size_t)cols * sizeof(float);
+  // One fp32 partial row per block of rows; no backward kernel covers fewer
+  // than kBwdMinRowsPerBlock rows per block, whatever the dtype and alignment.
+  const int64_t parts =
+      (rows + oslo::kBwdMinRowsPerBlock - 1) / oslo::kBwdMinRowsPerBlock;
+  return (size_t)(parts + oslo::kColsumGroups) * (size_t)cols * sizeof(float);
 }

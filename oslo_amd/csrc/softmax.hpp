@@ -48,6 +48,15 @@ __device__ __forceinline__ float row_allreduce(float v, Op op, float *slots) {
   return v;
 }
 
+// Block order for the causal kernels. Row r of a slab reads r+1 keys and writes
+// S, so blocks taken in memory order alternate between write-only phases
+// (start of a slab) and read-heavy ones (end). Dealing blocks from both ends of
+// the launch alternately keeps the read:write mix of the work in flight
+// constant, which measured 5-6 % faster on MI355X than memory order.
+__device__ __forceinline__ int64_t paired_block(int64_t b, int64_t nblocks) {
+  return (b & 1) ? nblocks - 1 - (b >> 1) : (b >> 1);
+}
+
 // exp(v - m) for a score v and row max m, both in natural-log units.
 __device__ __forceinline__ float exp_shifted(float v, float m) {
   return __builtin_amdgcn_exp2f((v - m) * kLog2e);

@@ -26,9 +26,9 @@ __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
   __shared__ float s_sum[kWavesPerBlock];
 
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int sub = wave % WPR;
-  int64_t row = (int64_t)blockIdx.x * Tile::kRowsPerBlock + wave / WPR;
+  int64_t row = paired_block(blockIdx.x, gridDim.x) * Tile::kRowsPerBlock + wave / WPR;
   // A block past the end keeps its waves alive (they meet the same barriers)
   // on the last row and only skips the stores.
   const bool live = row < total_rows;
@@ -39,28 +39,40 @@ __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
   T *yr = y + row * S;
   const float *padr = HAS_PAD ? pad + (slab / heads) * S : nullptr;
 
+  // Every load of the row is issued first (raw), conversion comes afterwards.
+  // The row is bounded at the vector that holds key r: lanes wholly above the
+  // diagonal get zeros without touching memory.
+  const uint32_t keys = (uint32_t)(r / VEC + 1) * VEC;
+  const BufRsrc xrs = make_rsrc(xr, keys * (uint32_t)sizeof(T));
+  RawVec<T, VEC> raw[NCHUNK];
+  RawVec<float, VEC> praw[HAS_PAD ? NCHUNK : 1];
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c)
+    raw[c] = buffer_load_raw<T, VEC, false>(
+        xrs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T));
+  if constexpr (HAS_PAD) {
+    const BufRsrc prs = make_rsrc(padr, keys * (uint32_t)sizeof(float));
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c)
+      praw[c] = buffer_load_raw<float, VEC, false>(
+          prs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(float));
+  }
+
   float v[NCHUNK][VEC];
   float m = -INFINITY;
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
     const int k0 = Tile::col(c, sub, lane);
+    float t[VEC], pv[VEC];
+    raw_to_f32<T, VEC>(t, raw[c]);
+    if constexpr (HAS_PAD) raw_to_f32<float, VEC>(pv, praw[c]);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) v[c][j] = -INFINITY;
-    if (k0 <= r) { // implies k0 < S; lanes wholly above the diagonal load nothing
-      float t[VEC];
-      load_f32<T, VEC>(t, xr + k0);
-      float pv[VEC];
-      if constexpr (HAS_PAD) load_f32_cached<float, VEC>(pv, padr + k0);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        // scale then add, each rounded, as the unfused path does
-        float e = __fmul_rn(t[j], scale);
-        if constexpr (HAS_PAD) e = __fadd_rn(e, pv[j]);
-        if (k0 + j <= r) {
-          v[c][j] = e;
-          m = fmaxf(m, e);
-        }
-      }
+    for (int j = 0; j < VEC; ++j) {
+      // scale then add, each rounded, as the unfused path does
+      float e = __fmul_rn(t[j], scale);
+      if constexpr (HAS_PAD) e = __fadd_rn(e, pv[j]);
+      v[c][j] = (k0 + j <= r) ? e : -INFINITY;
+      m = fmaxf(m, v[c][j]);
     }
   }
   m = row_allreduce<WPR>(m, OpMax(), s_max);
@@ -103,9 +115,9 @@ __global__ __launch_bounds__(kBlockThreads) void causal_bwd_kernel(
   __shared__ float s_sum[kWavesPerBlock];
 
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int sub = wave % WPR;
-  int64_t row = (int64_t)blockIdx.x * Tile::kRowsPerBlock + wave / WPR;
+  int64_t row = paired_block(blockIdx.x, gridDim.x) * Tile::kRowsPerBlock + wave / WPR;
   const bool live = row < total_rows;
   if (!live) row = total_rows - 1;
   const int r = (int)(row % S);
@@ -113,26 +125,33 @@ __global__ __launch_bounds__(kBlockThreads) void causal_bwd_kernel(
   const T *yr = y + row * S;
   T *dr = dx + row * S;
 
+  // bounded at the vector that holds key r, all loads issued first
+  const uint32_t bytes = (uint32_t)(r / VEC + 1) * VEC * (uint32_t)sizeof(T);
+  const BufRsrc grs = make_rsrc(gr, bytes);
+  const BufRsrc yrs = make_rsrc(yr, bytes);
+  RawVec<T, VEC> graw[NCHUNK], yraw[NCHUNK];
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    const uint32_t off = (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T);
+    graw[c] = buffer_load_raw<T, VEC, false>(grs, off);
+    yraw[c] = buffer_load_raw<T, VEC, false>(yrs, off);
+  }
+
   float gy[NCHUNK][VEC]; // g*y
   float yy[NCHUNK][VEC]; // y
   float sum = 0.f;
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
     const int k0 = Tile::col(c, sub, lane);
+    float tg[VEC];
+    raw_to_f32<T, VEC>(tg, graw[c]);
+    raw_to_f32<T, VEC>(yy[c], yraw[c]);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) gy[c][j] = yy[c][j] = 0.f;
-    if (k0 <= r) {
-      float tg[VEC], ty[VEC];
-      load_f32<T, VEC>(tg, gr + k0);
-      load_f32<T, VEC>(ty, yr + k0);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        if (k0 + j <= r) {
-          yy[c][j] = ty[j];
-          gy[c][j] = tg[j] * ty[j];
-          sum += gy[c][j];
-        }
-      }
+    for (int j = 0; j < VEC; ++j) {
+      // entries above the diagonal are never used, whatever they hold
+      if (k0 + j > r) yy[c][j] = tg[j] = 0.f;
+      gy[c][j] = tg[j] * yy[c][j];
+      sum += gy[c][j];
     }
   }
   sum = row_allreduce<WPR>(sum, OpAdd(), s_sum);

@@ -30,7 +30,7 @@ __global__ __launch_bounds__(kBlockThreads) void masked_fwd_kernel(
   __shared__ float s_sum[kWavesPerBlock];
 
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int sub = wave % WPR;
   int64_t row = (int64_t)blockIdx.x * Tile::kRowsPerBlock + wave / WPR;
   const bool live = row < total_rows;
@@ -44,24 +44,39 @@ __global__ __launch_bounds__(kBlockThreads) void masked_fwd_kernel(
     mr = mask + (bh / heads) * mask_stride_b + q * mask_stride_q;
   }
 
+  // every load of the row is issued first (raw, bounded at Sk), conversion
+  // comes afterwards
+  const BufRsrc xrs = make_rsrc(xr, (uint32_t)Sk * (uint32_t)sizeof(T));
+  RawVec<T, VEC> raw[NCHUNK];
+  RawVec<uint8_t, VEC> mraw[HAS_MASK ? NCHUNK : 1];
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c)
+    raw[c] = buffer_load_raw<T, VEC, true>(
+        xrs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T));
+  if constexpr (HAS_MASK) {
+    const BufRsrc mrs = make_rsrc(mr, (uint32_t)Sk);
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c)
+      mraw[c] = buffer_load_raw<uint8_t, VEC, false>(
+          mrs, (uint32_t)Tile::col(c, sub, lane));
+  }
+
   float v[NCHUNK][VEC];
   float m = -INFINITY;
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
     const int k0 = Tile::col(c, sub, lane);
-    if (k0 < Sk) {
-      float t[VEC];
-      load_f32<T, VEC>(t, xr + k0);
-      uint8_t mk[VEC];
-      if constexpr (HAS_MASK) load_bytes<VEC>(mk, mr + k0);
+    float t[VEC];
+    raw_to_f32<T, VEC>(t, raw[c]);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        v[c][j] = masked_score<REPLACE>(t[j], scale, HAS_MASK ? mk[j] : 0);
-        m = fmaxf(m, v[c][j]);
+    for (int j = 0; j < VEC; ++j) {
+      uint8_t mk = 0;
+      if constexpr (HAS_MASK) {
+        if constexpr (VEC == 1) mk = mraw[c]; else mk = mraw[c][j];
       }
-    } else {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) v[c][j] = -INFINITY;
+      const float e = masked_score<REPLACE>(t[j], scale, mk);
+      v[c][j] = (k0 < Sk) ? e : -INFINITY;
+      m = fmaxf(m, v[c][j]);
     }
   }
   m = row_allreduce<WPR>(m, OpMax(), s_max);
@@ -100,7 +115,7 @@ __global__ __launch_bounds__(kBlockThreads) void masked_bwd_kernel(
   __shared__ float s_sum[kWavesPerBlock];
 
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int sub = wave % WPR;
   int64_t row = (int64_t)blockIdx.x * Tile::kRowsPerBlock + wave / WPR;
   const bool live = row < total_rows;
@@ -109,24 +124,29 @@ __global__ __launch_bounds__(kBlockThreads) void masked_bwd_kernel(
   const T *yr = y + row * Sk;
   T *dr = dx + row * Sk;
 
+  const uint32_t bytes = (uint32_t)Sk * (uint32_t)sizeof(T);
+  const BufRsrc grs = make_rsrc(gr, bytes);
+  const BufRsrc yrs = make_rsrc(yr, bytes);
+  RawVec<T, VEC> graw[NCHUNK], yraw[NCHUNK];
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    const uint32_t off = (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T);
+    graw[c] = buffer_load_raw<T, VEC, true>(grs, off);
+    yraw[c] = buffer_load_raw<T, VEC, true>(yrs, off);
+  }
+
   float gy[NCHUNK][VEC];
   float yy[NCHUNK][VEC];
   float sum = 0.f;
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
-    const int k0 = Tile::col(c, sub, lane);
-    if (k0 < Sk) {
-      float tg[VEC];
-      load_f32<T, VEC>(tg, gr + k0);
-      load_f32<T, VEC>(yy[c], yr + k0);
+    float tg[VEC];
+    raw_to_f32<T, VEC>(tg, graw[c]);
+    raw_to_f32<T, VEC>(yy[c], yraw[c]);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        gy[c][j] = tg[j] * yy[c][j];
-        sum += gy[c][j];
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) gy[c][j] = yy[c][j] = 0.f;
+    for (int j = 0; j < VEC; ++j) {
+      gy[c][j] = tg[j] * yy[c][j];
+      sum += gy[c][j];
     }
   }
   sum = row_allreduce<WPR>(sum, OpAdd(), s_sum);
