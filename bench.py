@@ -1,0 +1,293 @@
+#!/usr/bin/env python3
+"""Benchmark of the kernel-fusion hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one forward + backward pass of the fused causal scale-mask-softmax
+over one batch of synthetic attention scores: fp16 [8,16,2048,2048] ~ N(0,1)*8,
+scale 0.125, upstream gradient ~ N(0,1). Inputs are resident in HBM before the
+timed region. The JSON line printed at the end carries
+
+  value         algorithmic bytes of a step / time of a step, in GB/s
+  roofline      the causal forward kernel alone (its launches timed with events
+                on the launch stream), as a fraction of the 8 TB/s HBM peak
+  kernels       the same figure for every other kernel of the path at its
+                benchmark shape
+  cpu_baseline  the reference's unfused arithmetic on the host cores, timed on
+                a bounded sample of the same workload
+
+Algorithmic bytes count what the operation must move, not what the hardware
+moved: forward = lower triangle read + full matrix written; backward = two
+lower triangles read + full matrix written.
+"""
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+# HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` (KiB per dispatch, scaled by the reading of a 1 GiB copy
+# kernel: 2.0 for FETCH_SIZE, 1.0 for WRITE_SIZE), as recorded in
+# profiles/causal_softmax_fp16_8x16x2048x2048_hbm_traffic.md. Kernels that are
+# not listed were not measured (null in the output).
+MEASURED_TRAFFIC = {
+    "causal_fwd fp16 [8,16,2048,2048]": 1627451995,
+    "causal_bwd fp16 [8,16,2048,2048]": 2181095955,
+}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default="", help="run only the named kernel of the table (for profiling)")
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; every softmax row and every "
+                 "element is independent, so N GPUs would each run this same kernel on "
+                 "1/N of the batch*heads with no exchange. Run with --gpus 1.")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no ROCm device visible")
+    from oslo_amd import _lib
+
+    lib = _lib.load()  # raises if the HIP library is not built; there is no fallback
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream()
+    st = ctypes.c_void_p(stream.cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+    def check(rc):
+        if rc != 0:
+            raise RuntimeError(lib.oslo_last_error().decode())
+
+    def time_launches(fn, n, warm):
+        """Average seconds per call of fn over n calls, events on the launch stream."""
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(n):
+            fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / n
+
+    # ---------------- workload: causal softmax fwd+bwd, fp16 [8,16,2048,2048]
+    B, H, S = 8, 16, 2048
+    F16, BF16 = 1, 2
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0)
+    x = (torch.randn((B, H, S, S), generator=gen, device=dev, dtype=torch.float32) * 8).to(torch.float16)
+    gen.manual_seed(1)
+    g = torch.randn((B * H, S, S), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+    y = torch.empty_like(x)
+    dx = torch.empty_like(g)
+    tri = B * H * S * (S + 1) // 2
+    full = B * H * S * S
+    bytes_fwd = 2 * (tri + full)
+    bytes_bwd = 2 * (2 * tri + full)
+
+    def fwd():
+        check(lib.oslo_softmax_causal_fwd(P(y), P(x), None, 0.125, B, H, S, F16, st))
+
+    def bwd():
+        check(lib.oslo_softmax_causal_bwd(P(dx), P(g), P(y), 0.125, B * H, S, F16, st))
+
+    def step():
+        fwd()
+        bwd()
+
+    if args.only:
+        run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd)
+        return
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    value = (bytes_fwd + bytes_bwd) / (elapsed / args.steps) / 1e9
+
+    t_fwd = time_launches(fwd, args.steps, 5)
+    t_bwd = time_launches(bwd, args.steps, 5)
+
+    def roof(name, nbytes, seconds):
+        gbps = nbytes / seconds / 1e9
+        return {"kernel": name, "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
+                "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "us": round(seconds * 1e6, 1),
+                "algorithmic_bytes": nbytes, "traffic": MEASURED_TRAFFIC.get(name)}
+
+    roofline = roof("causal_fwd fp16 [8,16,2048,2048]", bytes_fwd, t_fwd)
+    kernels = [roof("causal_bwd fp16 [8,16,2048,2048]", bytes_bwd, t_bwd)]
+    del x, y, g, dx
+    kernels += other_kernels(lib, torch, dev, st, P, check, time_launches, roof, max(10, args.steps // 2))
+
+    out = {
+        "metric": "fused causal scale-mask-softmax fwd+bwd HBM GB/s",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "causal scaled softmax fwd+bwd, fp16 scores [8,16,2048,2048], scale 0.125, "
+                               "fp32 arithmetic",
+                   "algorithmic_bytes_per_step": bytes_fwd + bytes_bwd},
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch)
+    print(json.dumps(out))
+
+
+def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
+    """Every other kernel of the path at its benchmark shape."""
+    F16, BF16, F32 = 1, 2, 0
+    res = []
+    gen = torch.Generator(device=dev)
+
+    def randn(shape, seed, std, dtype):
+        gen.manual_seed(seed)
+        return (torch.randn(shape, generator=gen, device=dev, dtype=torch.float32) * std).to(dtype)
+
+    # causal, bf16 and fp32 variants of the workload
+    B, H, S = 8, 16, 2048
+    tri, full = B * H * S * (S + 1) // 2, B * H * S * S
+    for name, dt, code in (("bf16", torch.bfloat16, BF16), ("fp32", torch.float32, F32)):
+        x = randn((B, H, S, S), 0, 8.0, dt)
+        y = torch.empty_like(x)
+        es = x.element_size()
+        t = time_launches(lambda: check(lib.oslo_softmax_causal_fwd(P(y), P(x), None, 0.125, B, H, S, code, st)), n, 3)
+        res.append(roof(f"causal_fwd {name} [8,16,2048,2048]", es * (tri + full), t))
+        g = randn((B * H, S, S), 1, 1.0, dt)
+        t = time_launches(lambda: check(lib.oslo_softmax_causal_bwd(P(g), P(g), P(y), 0.125, B * H, S, code, st)), n, 3)
+        res.append(roof(f"causal_bwd {name} [8,16,2048,2048] (in place)", es * (2 * tri + full), t))
+        del x, y, g
+
+    # long rows: bf16 [1,16,8192,8192]
+    S8 = 8192
+    x = randn((1, 16, S8, S8), 0, 1.0, torch.bfloat16)
+    y = torch.empty_like(x)
+    t = time_launches(lambda: check(lib.oslo_softmax_causal_fwd(P(y), P(x), None, 1 / 16, 1, 16, S8, BF16, st)), n, 3)
+    res.append(roof("causal_fwd bf16 [1,16,8192,8192]", 2 * (16 * S8 * (S8 + 1) // 2 + x.numel()), t))
+    del x, y
+
+    # padded key mask: bf16 [16,16,1024,1024], lengths U{128..1024}
+    B, H, S = 16, 16, 1024
+    x = randn((B, H, S, S), 0, 8 ** 0.5, torch.bfloat16)
+    y = torch.empty_like(x)
+    gen.manual_seed(2)
+    lens = torch.randint(128, 1025, (B,), generator=gen, device=dev)
+    mask = (torch.arange(S, device=dev)[None, :] >= lens[:, None]).contiguous().view(torch.uint8)
+    t = time_launches(lambda: check(lib.oslo_softmax_masked_fwd(P(y), P(x), P(mask), S, 0, 0, 0.125, B, H, S, S, BF16, st)), n, 3)
+    res.append(roof("masked_fwd bf16 [16,16,1024,1024] key mask", 4 * x.numel() + mask.numel(), t))
+    g = randn((B, H, S, S), 1, 1.0, torch.bfloat16)
+    dxm = torch.empty_like(g)
+    t = time_launches(lambda: check(lib.oslo_softmax_masked_bwd(P(dxm), P(g), P(y), 0.125, B * H * S, S, BF16, st)), n, 3)
+    res.append(roof("masked_bwd bf16 [16,16,1024,1024]", 6 * x.numel(), t))
+    del x, y, g, dxm
+
+    # bias-GeLU and bias-dropout-residual, bf16
+    for rows, cols in ((16384, 16384), (16384, 4096)):
+        a = randn((rows, cols), 0, 1.0, torch.bfloat16)
+        r = randn((rows, cols), 1, 1.0, torch.bfloat16)
+        bias = randn((cols,), 3, 0.02, torch.bfloat16)
+        o = torch.empty_like(a)
+        db = torch.empty_like(bias)
+        ws = torch.empty(lib.oslo_colsum_workspace_bytes(rows, cols) // 4, dtype=torch.float32, device=dev)
+        n_el = rows * cols
+        shape = f"bf16 [{rows},{cols}]"
+        t = time_launches(lambda: check(lib.oslo_bias_gelu_fwd(P(o), P(a), P(bias), rows, cols, BF16, st)), n, 3)
+        res.append(roof(f"bias_gelu_fwd {shape}", 4 * n_el, t))
+        t = time_launches(lambda: check(lib.oslo_bias_gelu_bwd(P(o), P(db), P(ws), P(r), P(a), P(bias), rows, cols, BF16, st)), n, 3)
+        res.append(roof(f"bias_gelu_bwd+dbias {shape}", 6 * n_el, t))
+        t = time_launches(lambda: check(lib.oslo_bias_dropout_add_fwd(P(o), P(a), P(bias), P(r), 0.1, 1234, 0, rows, cols, BF16, st)), n, 3)
+        res.append(roof(f"bias_dropout_add_fwd p=0.1 {shape}", 6 * n_el, t))
+        t = time_launches(lambda: check(lib.oslo_bias_dropout_add_bwd(P(o), P(db), P(ws), P(r), 0.1, 1234, 0, rows, cols, BF16, st)), n, 3)
+        res.append(roof(f"bias_dropout_add_bwd+dbias p=0.1 {shape}", 4 * n_el, t))
+        del a, r, o, ws
+    return res
+
+
+def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
+    """--only causal_fwd | causal_bwd | copy: launch one kernel `steps` times
+    (profiling runs). `copy` is torch's device copy of 1 GiB, the kernel of
+    known traffic that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
+    if args.only == "copy":
+        a = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
+        b = torch.empty_like(a)
+        fn = lambda: b.copy_(a)
+    else:
+        fn = {"causal_fwd": fwd, "causal_bwd": bwd}.get(args.only)
+    if fn is None:
+        sys.exit("--only takes causal_fwd, causal_bwd or copy")
+    if args.only == "causal_bwd":
+        fwd()
+    t = time_launches(fn, args.steps, args.warmup)
+    print(json.dumps({"only": args.only, "us": round(t * 1e6, 2), "launches": args.steps}))
+
+
+def cpu_baseline(torch):
+    """The unfused arithmetic (scale, where(causal), softmax, autograd backward)
+    with torch's CPU operators on the host cores, fp32 (CPU half softmax is not
+    representative), on a bounded sample: [1,4,2048,2048] slabs of the same
+    workload, repeated for about 10 s."""
+    from oracle import unfused_torch as ref
+
+    cores = torch.get_num_threads()
+    b, h, s = 1, 4, 2048
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn((b, h, s, s), generator=gen) * 8
+    go = torch.randn((b, h, s, s), generator=gen)
+    tri, full = b * h * s * (s + 1) // 2, b * h * s * s
+    # same accounting as the GPU figure, at the fp16 element size of the workload
+    nbytes = 2 * (tri + full) + 2 * (2 * tri + full)
+
+    def one():
+        xx = x.clone().requires_grad_(True)
+        y = ref.attention_probs(xx, 0.125, causal=True)
+        y.backward(go)
+
+    one()
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < 10.0 or reps < 3:
+        one()
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"unfused fp32 fwd+bwd on [1,4,2048,2048] x {reps} reps, "
+                      f"{dt * 1e3:.1f} ms each, bytes counted at the workload's fp16 size"}
+
+
+if __name__ == "__main__":
+    main()
