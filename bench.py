@@ -50,6 +50,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gptj", action="store_true", help="skip the GPT-J-6B-shaped forward comparison")
     ap.add_argument("--only", default="", help="run only the named kernel of the table (for profiling)")
     return ap.parse_args()
 
@@ -165,6 +166,8 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    if not args.no_gptj:
+        out["gptj_fwd"] = gptj_forward(torch, dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(out))
@@ -255,6 +258,51 @@ def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
         fwd()
     t = time_launches(fn, args.steps, args.warmup)
     print(json.dumps({"only": args.only, "us": round(t * 1e6, 2), "launches": args.steps}))
+
+
+def gptj_forward(torch, dev, layers=28, batch=8, seq=2048, reps=5):
+    """GPT-J-6B-shaped forward (28 layers, d_model 4096, 16 heads of 256, rotary
+    64, d_ff 16384, vocab 50400; weights N(0, 0.02) in bf16; token ids uniform;
+    eval mode), unfused torch modules against the same model after fuse()."""
+    from oslo_amd import GPTJConfig, GPTJForCausalLM
+
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(dev):
+            torch.manual_seed(0)
+            model = GPTJForCausalLM(GPTJConfig(n_layer=layers)).eval()
+    finally:
+        torch.set_default_dtype(old)
+    ids = torch.randint(0, 50400, (batch, seq), device=dev)
+
+    def run():
+        with torch.no_grad():
+            return model(ids)["logits"]
+
+    def timed():
+        for _ in range(2):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            run()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps
+
+    t_unfused = timed()
+    ref_logits = run().float()
+    model.fuse()
+    t_fused = timed()
+    diff = (run().float() - ref_logits).abs().max().item()
+    del model, ref_logits
+    torch.cuda.empty_cache()
+    tokens = batch * seq
+    return {"config": f"{layers} layers, d_model 4096, 16x256 heads, rotary 64, d_ff 16384, vocab 50400, "
+                      f"bf16, batch {batch}, seq {seq}, eval",
+            "unfused_tokens_per_s": round(tokens / t_unfused, 1), "fused_tokens_per_s": round(tokens / t_fused, 1),
+            "unfused_ms": round(t_unfused * 1e3, 2), "fused_ms": round(t_fused * 1e3, 2),
+            "speedup": round(t_unfused / t_fused, 3), "max_abs_logit_diff": round(diff, 4)}
 
 
 def cpu_baseline(torch):

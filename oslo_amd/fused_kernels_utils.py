@@ -282,6 +282,8 @@ class _BiasDropoutAdd(torch.autograd.Function):
 
 def _bias_dropout_add(x, bias, residual, training, drop_prop):
     p = float(drop_prop) if training else 0.0
+    if not x.is_cuda:
+        raise RuntimeError(f"expected a tensor on a ROCm device, got {x.device} (this library has no CPU path)")
     if p < 0.0 or p > 1.0:
         raise ValueError(f"dropout probability has to be between 0 and 1, but got {p}")
     if p == 1.0:  # everything dropped: F.dropout returns zeros

@@ -1,0 +1,256 @@
+"""GPT-2 blocks with the reference's kernel-fusion hooks.
+
+``GPT2Attention`` / ``GPT2MLP`` compute what the reference's unfused modules
+compute (oslo/models/gpt2/modeling_gpt2.py:131-230, :385-399);
+``FusedGPT2Attention`` / ``FusedGPT2MLP`` are the classes ``fuse()`` swaps in
+(oslo/models/gpt2/modeling_gpt2.py:1434-1569). Sub-module and buffer names
+(c_attn, c_proj, c_fc, attn_dropout, resid_dropout, bias, masked_bias) are the
+reference's, so a state_dict moves between the two unchanged."""
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+from torch import nn
+
+from .fused_kernels_utils import FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax
+from .modeling_utils import (ACT2FN, Conv1D, LayerPolicy, PreTrainedModel, additive_attention_mask,
+                             causal_lm_loss)
+
+
+@dataclass
+class GPT2Config:
+    vocab_size: int = 50257
+    n_positions: int = 1024
+    n_embd: int = 768
+    n_layer: int = 12
+    n_head: int = 12
+    n_inner: Optional[int] = None
+    activation_function: str = "gelu_new"
+    resid_pdrop: float = 0.1
+    embd_pdrop: float = 0.1
+    attn_pdrop: float = 0.1
+    layer_norm_epsilon: float = 1e-5
+    scale_attn_weights: bool = True
+    scale_attn_by_inverse_layer_idx: bool = False
+    add_cross_attention: bool = False
+
+    @property
+    def hidden_size(self):
+        return self.n_embd
+
+    @property
+    def num_attention_heads(self):
+        return self.n_head
+
+    @property
+    def max_position_embeddings(self):
+        return self.n_positions
+
+
+class GPT2Attention(nn.Module):
+    def __init__(self, config, is_cross_attention=False, layer_idx=None):
+        super().__init__()
+        n_pos = config.max_position_embeddings
+        self.register_buffer(
+            "bias", torch.tril(torch.ones((n_pos, n_pos), dtype=torch.uint8)).view(1, 1, n_pos, n_pos))
+        self.register_buffer("masked_bias", torch.tensor(-1e4))
+        self.embed_dim = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.head_dim = self.embed_dim // self.num_heads
+        self.split_size = self.embed_dim
+        if self.head_dim * self.num_heads != self.embed_dim:
+            raise ValueError("`embed_dim` must be divisible by num_heads")
+        self.scale_attn_weights = config.scale_attn_weights
+        self.scale_attn_by_inverse_layer_idx = config.scale_attn_by_inverse_layer_idx
+        self.is_cross_attention = is_cross_attention
+        self.layer_idx = layer_idx
+        if is_cross_attention:
+            self.c_attn = Conv1D(2 * self.embed_dim, self.embed_dim)
+            self.q_attn = Conv1D(self.embed_dim, self.embed_dim)
+        else:
+            self.c_attn = Conv1D(3 * self.embed_dim, self.embed_dim)
+        self.c_proj = Conv1D(self.embed_dim, self.embed_dim)
+        self.attn_dropout = nn.Dropout(config.attn_pdrop)
+        self.resid_dropout = nn.Dropout(config.resid_pdrop)
+
+    def _split_heads(self, t, num_heads, head_dim):
+        return t.view(t.size()[:-1] + (num_heads, head_dim)).permute(0, 2, 1, 3)
+
+    def _merge_heads(self, t, num_heads, head_dim):
+        t = t.permute(0, 2, 1, 3).contiguous()
+        return t.view(t.size()[:-2] + (num_heads * head_dim,))
+
+    def _attention_scale(self, value):
+        scale = 1.0
+        if self.scale_attn_weights:
+            scale *= 1 / (float(value.size(-1)) ** 0.5)
+        if self.scale_attn_by_inverse_layer_idx:
+            scale *= 1 / float(self.layer_idx + 1)
+        return scale
+
+    def _attn(self, query, key, value, attention_mask=None, head_mask=None):
+        """The unfused path: scale, where(causal, w, -1e4), + mask, softmax, dropout."""
+        w = torch.matmul(query, key.transpose(-1, -2))
+        if self.scale_attn_weights:
+            w = w / (float(value.size(-1)) ** 0.5)
+        if self.scale_attn_by_inverse_layer_idx:
+            w = w / float(self.layer_idx + 1)
+        if not self.is_cross_attention:
+            sq, sk = query.size(-2), key.size(-2)
+            causal = self.bias[:, :, sk - sq:sk, :sk].bool()
+            w = torch.where(causal, w, self.masked_bias.to(w.dtype))
+        if attention_mask is not None:
+            w = w + attention_mask
+        w = nn.functional.softmax(w, dim=-1)
+        w = self.attn_dropout(w.type(value.dtype))
+        if head_mask is not None:
+            w = w * head_mask
+        return torch.matmul(w, value), w
+
+    def _project_qkv(self, hidden_states, layer_past, encoder_hidden_states, use_cache):
+        if encoder_hidden_states is not None:
+            if not hasattr(self, "q_attn"):
+                raise ValueError("cross attention needs GPT2Attention(..., is_cross_attention=True)")
+            query = self.q_attn(hidden_states)
+            key, value = self.c_attn(encoder_hidden_states).split(self.split_size, dim=2)
+        else:
+            query, key, value = self.c_attn(hidden_states).split(self.split_size, dim=2)
+        query = self._split_heads(query, self.num_heads, self.head_dim)
+        key = self._split_heads(key, self.num_heads, self.head_dim)
+        value = self._split_heads(value, self.num_heads, self.head_dim)
+        if layer_past is not None:
+            key = torch.cat((layer_past[0], key), dim=-2)
+            value = torch.cat((layer_past[1], value), dim=-2)
+        present = (key, value) if use_cache else None
+        return query, key, value, present
+
+    def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None,
+                encoder_hidden_states=None, encoder_attention_mask=None, use_cache=False,
+                output_attentions=False):
+        query, key, value, present = self._project_qkv(hidden_states, layer_past, encoder_hidden_states, use_cache)
+        if encoder_hidden_states is not None:
+            attention_mask = encoder_attention_mask
+        out, w = self._attn(query, key, value, attention_mask, head_mask)
+        out = self._merge_heads(out, self.num_heads, self.head_dim)
+        out = self.resid_dropout(self.c_proj(out))
+        return (out, present, w) if output_attentions else (out, present)
+
+
+class FusedGPT2Attention(GPT2Attention):
+    """oslo/models/gpt2/modeling_gpt2.py:1434-1542. Like the reference, the
+    fused path applies no attention-probability dropout."""
+
+    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
+        w = torch.matmul(query, key.transpose(-1, -2))
+        w = FusedScaleMaskSoftmax.apply(w, pad_mask=attention_mask, scale=self._attention_scale(value),
+                                        use_triang_mask=not self.is_cross_attention)
+        if head_mask is not None:
+            w = w * head_mask
+        return torch.matmul(w, value), w
+
+    def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None,
+                encoder_hidden_states=None, encoder_attention_mask=None, use_cache=False,
+                output_attentions=False):
+        query, key, value, present = self._project_qkv(hidden_states, layer_past, encoder_hidden_states, use_cache)
+        if encoder_hidden_states is not None:
+            attention_mask = encoder_attention_mask
+        (bsz, np_, sq, _), sk = query.size(), key.size(-2)
+        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk,
+                                              use_triang_mask=not self.is_cross_attention):
+            out, w = self._fused_attn(query, key, value, attention_mask, head_mask)
+        else:
+            out, w = self._attn(query, key, value, attention_mask, head_mask)
+        out = self._merge_heads(out, self.num_heads, self.head_dim)
+        out = out @ self.c_proj.weight  # projection without its bias ...
+        out = FusedBiasDropout.apply(out, self.c_proj.bias, self.training, self.resid_dropout.p)  # ... fused here
+        return (out, present, w) if output_attentions else (out, present)
+
+
+class GPT2MLP(nn.Module):
+    def __init__(self, intermediate_size, config):
+        super().__init__()
+        self.c_fc = Conv1D(intermediate_size, config.hidden_size)
+        self.c_proj = Conv1D(config.hidden_size, intermediate_size)
+        self.act = ACT2FN[config.activation_function]
+        self.dropout = nn.Dropout(config.resid_pdrop)
+
+    def forward(self, hidden_states):
+        return self.dropout(self.c_proj(self.act(self.c_fc(hidden_states))))
+
+
+class FusedGPT2MLP(GPT2MLP):
+    """oslo/models/gpt2/modeling_gpt2.py:1545-1569."""
+
+    def forward(self, x):
+        x = x @ self.c_fc.weight
+        x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
+        x = x @ self.c_proj.weight
+        return FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
+
+
+class GPT2Block(nn.Module):
+    def __init__(self, config, layer_idx=None):
+        super().__init__()
+        inner = config.n_inner if config.n_inner is not None else 4 * config.hidden_size
+        self.ln_1 = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_epsilon)
+        self.attn = GPT2Attention(config, layer_idx=layer_idx)
+        self.ln_2 = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_epsilon)
+        self.mlp = GPT2MLP(inner, config)
+
+    def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None, use_cache=False):
+        a = self.attn(self.ln_1(hidden_states), layer_past=layer_past, attention_mask=attention_mask,
+                      head_mask=head_mask, use_cache=use_cache)
+        hidden_states = a[0] + hidden_states
+        hidden_states = hidden_states + self.mlp(self.ln_2(hidden_states))
+        return hidden_states, a[1]
+
+
+class GPT2LayerPolicy(LayerPolicy):
+    """oslo/models/gpt2/configuration_gpt2.py:272-284."""
+
+    @staticmethod
+    def fused_modules():
+        return {GPT2Attention: FusedGPT2Attention, GPT2MLP: FusedGPT2MLP}
+
+
+class GPT2Model(nn.Module):
+    def __init__(self, config):
+        super().__init__()
+        self.wte = nn.Embedding(config.vocab_size, config.hidden_size)
+        self.wpe = nn.Embedding(config.max_position_embeddings, config.hidden_size)
+        self.drop = nn.Dropout(config.embd_pdrop)
+        self.h = nn.ModuleList([GPT2Block(config, layer_idx=i) for i in range(config.n_layer)])
+        self.ln_f = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_epsilon)
+
+    def forward(self, input_ids, attention_mask=None, past_key_values=None, use_cache=False):
+        past_len = 0 if past_key_values is None else past_key_values[0][0].size(-2)
+        pos = torch.arange(past_len, past_len + input_ids.size(-1), device=input_ids.device)
+        h = self.drop(self.wte(input_ids) + self.wpe(pos)[None])
+        mask = additive_attention_mask(attention_mask, h.dtype)
+        presents = []
+        for i, block in enumerate(self.h):
+            h, present = block(h, layer_past=None if past_key_values is None else past_key_values[i],
+                               attention_mask=mask, use_cache=use_cache)
+            presents.append(present)
+        return self.ln_f(h), (tuple(presents) if use_cache else None)
+
+
+class GPT2LMHeadModel(PreTrainedModel):
+    is_fusable = True
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.transformer = GPT2Model(config)
+        self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
+        self.init_weights()
+        self.lm_head.weight = self.transformer.wte.weight  # tied
+
+    def get_layer_policies(self):
+        return [GPT2LayerPolicy]
+
+    def forward(self, input_ids, attention_mask=None, past_key_values=None, use_cache=False, labels=None):
+        h, presents = self.transformer(input_ids, attention_mask, past_key_values, use_cache)
+        logits = self.lm_head(h)
+        loss = causal_lm_loss(logits, labels) if labels is not None else None
+        return {"loss": loss, "logits": logits, "past_key_values": presents}

@@ -1,0 +1,235 @@
+"""GPT-Neo blocks with the reference's kernel-fusion hooks.
+
+``GPTNeoSelfAttention`` / ``GPTNeoMLP`` compute what the reference's unfused
+modules compute (oslo/models/gpt_neo/modeling_gpt_neo.py:145-329): unscaled
+scores, fp32 softmax, global or sliding-window ("local") causal masks.
+``FusedGPTNeoSelfAttention`` / ``FusedGPTNeoMLP`` are what ``fuse()`` swaps in
+(oslo/models/gpt_neo/modeling_gpt_neo.py:993-1102). As in the reference, local
+attention layers are a separate class, so ``fuse()``'s exact-class match leaves
+them unfused (their mask is not a plain lower triangle;
+oslo/models/gpt_neo/modeling_gpt_neo.py:268-272)."""
+
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+import torch
+from torch import nn
+
+from .fused_kernels_utils import FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax
+from .modeling_utils import ACT2FN, LayerPolicy, PreTrainedModel, additive_attention_mask, causal_lm_loss
+
+
+@dataclass
+class GPTNeoConfig:
+    vocab_size: int = 50257
+    max_position_embeddings: int = 2048
+    hidden_size: int = 2048
+    num_layers: int = 24
+    num_heads: int = 16
+    attention_layers: List[str] = field(default_factory=list)  # "global" / "local" per layer
+    window_size: int = 256
+    intermediate_size: Optional[int] = None
+    activation_function: str = "gelu_new"
+    resid_dropout: float = 0.0
+    embed_dropout: float = 0.0
+    attention_dropout: float = 0.0
+    layer_norm_epsilon: float = 1e-5
+
+    def __post_init__(self):
+        if not self.attention_layers:
+            self.attention_layers = ["global", "local"] * (self.num_layers // 2) + \
+                                    ["global"] * (self.num_layers % 2)
+
+
+class GPTNeoSelfAttention(nn.Module):
+    def __init__(self, config, attention_type):
+        super().__init__()
+        n_pos = config.max_position_embeddings
+        bias = torch.tril(torch.ones((n_pos, n_pos), dtype=torch.uint8)).view(1, 1, n_pos, n_pos)
+        if attention_type == "local":  # keep only the last window_size keys of each row
+            bias = torch.bitwise_xor(bias, torch.tril(bias, -config.window_size))
+        self.register_buffer("bias", bias)
+        self.register_buffer("masked_bias", torch.tensor(-1e9))
+        self.attn_dropout = nn.Dropout(config.attention_dropout)
+        self.resid_dropout = nn.Dropout(config.resid_dropout)
+        self.embed_dim = config.hidden_size
+        self.num_heads = config.num_heads
+        self.head_dim = self.embed_dim // self.num_heads
+        if self.head_dim * self.num_heads != self.embed_dim:
+            raise ValueError("embed_dim must be divisible by num_heads")
+        self.k_proj = nn.Linear(self.embed_dim, self.embed_dim, bias=False)
+        self.v_proj = nn.Linear(self.embed_dim, self.embed_dim, bias=False)
+        self.q_proj = nn.Linear(self.embed_dim, self.embed_dim, bias=False)
+        self.out_proj = nn.Linear(self.embed_dim, self.embed_dim, bias=True)
+
+    def _split_heads(self, t):
+        return t.view(t.size()[:-1] + (self.num_heads, self.head_dim)).permute(0, 2, 1, 3)
+
+    def _merge_heads(self, t):
+        t = t.permute(0, 2, 1, 3).contiguous()
+        return t.view(t.size()[:-2] + (self.num_heads * self.head_dim,))
+
+    def _attn(self, query, key, value, attention_mask=None, head_mask=None):
+        """The unfused path: fp32 scores (no scaling), where(mask, w, -1e9), + mask, softmax."""
+        w = torch.matmul(query.to(torch.float32), key.to(torch.float32).transpose(-1, -2))
+        sq, sk = query.size(-2), key.size(-2)
+        causal = self.bias[:, :, sk - sq:sk, :sk].bool()
+        w = torch.where(causal, w, self.masked_bias.to(w.dtype))
+        if attention_mask is not None:
+            w = w + attention_mask
+        w = nn.functional.softmax(w, dim=-1).to(value.dtype)
+        w = self.attn_dropout(w)
+        if head_mask is not None:
+            w = w * head_mask
+        return torch.matmul(w, value), w
+
+    def _project_qkv(self, hidden_states, layer_past, use_cache):
+        query = self._split_heads(self.q_proj(hidden_states))
+        key = self._split_heads(self.k_proj(hidden_states))
+        value = self._split_heads(self.v_proj(hidden_states))
+        if layer_past is not None:
+            key = torch.cat((layer_past[0], key), dim=-2)
+            value = torch.cat((layer_past[1], value), dim=-2)
+        present = (key, value) if use_cache else None
+        return query, key, value, present
+
+    def forward(self, hidden_states, attention_mask=None, layer_past=None, head_mask=None,
+                use_cache=False, output_attentions=False):
+        query, key, value, present = self._project_qkv(hidden_states, layer_past, use_cache)
+        out, w = self._attn(query, key, value, attention_mask, head_mask)
+        out = self.resid_dropout(self.out_proj(self._merge_heads(out)))
+        return (out, present, w) if output_attentions else (out, present)
+
+
+class GPTNeoLocalSelfAttention(GPTNeoSelfAttention):
+    """Sliding-window layers; a class of their own so that fusion skips them."""
+
+
+class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
+    """oslo/models/gpt_neo/modeling_gpt_neo.py:993-1075."""
+
+    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
+        w = torch.matmul(query, key.transpose(-1, -2))
+        w = FusedScaleMaskSoftmax.apply(w, pad_mask=attention_mask, scale=None, use_triang_mask=True)
+        w = self.attn_dropout(w.to(value.dtype))
+        if head_mask is not None:
+            w = w * head_mask
+        return torch.matmul(w, value), w
+
+    def forward(self, hidden_states, attention_mask=None, layer_past=None, head_mask=None,
+                use_cache=False, output_attentions=False):
+        query, key, value, present = self._project_qkv(hidden_states, layer_past, use_cache)
+        (bsz, np_, sq, _), sk = query.size(), key.size(-2)
+        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=True):
+            out, w = self._fused_attn(query, key, value, attention_mask, head_mask)
+        else:
+            out, w = self._attn(query, key, value, attention_mask, head_mask)
+        out = self._merge_heads(out) @ self.out_proj.weight.t()
+        out = FusedBiasDropout.apply(out, self.out_proj.bias, self.training, self.resid_dropout.p)
+        return (out, present, w) if output_attentions else (out, present)
+
+
+class GPTNeoAttention(nn.Module):
+    def __init__(self, config, layer_id=0):
+        super().__init__()
+        self.attention_type = config.attention_layers[layer_id]
+        if self.attention_type == "local":
+            self.attention = GPTNeoLocalSelfAttention(config, "local")
+        elif self.attention_type == "global":
+            self.attention = GPTNeoSelfAttention(config, "global")
+        else:
+            raise NotImplementedError(f"unknown attention layer type {self.attention_type!r}")
+
+    def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None,
+                use_cache=False, output_attentions=False):
+        return self.attention(hidden_states, attention_mask=attention_mask, layer_past=layer_past,
+                              head_mask=head_mask, use_cache=use_cache, output_attentions=output_attentions)
+
+
+class GPTNeoMLP(nn.Module):
+    def __init__(self, intermediate_size, config):
+        super().__init__()
+        self.c_fc = nn.Linear(config.hidden_size, intermediate_size)
+        self.c_proj = nn.Linear(intermediate_size, config.hidden_size)
+        self.act = ACT2FN[config.activation_function]
+        self.dropout = nn.Dropout(config.resid_dropout)
+
+    def forward(self, hidden_states):
+        return self.dropout(self.c_proj(self.act(self.c_fc(hidden_states))))
+
+
+class FusedGPTNeoMLP(GPTNeoMLP):
+    """oslo/models/gpt_neo/modeling_gpt_neo.py:1078-1102."""
+
+    def forward(self, x):
+        x = x @ self.c_fc.weight.t()
+        x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
+        x = x @ self.c_proj.weight.t()
+        return FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
+
+
+class GPTNeoBlock(nn.Module):
+    def __init__(self, config, layer_id):
+        super().__init__()
+        inner = config.intermediate_size if config.intermediate_size is not None else 4 * config.hidden_size
+        self.ln_1 = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_epsilon)
+        self.attn = GPTNeoAttention(config, layer_id)
+        self.ln_2 = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_epsilon)
+        self.mlp = GPTNeoMLP(inner, config)
+
+    def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None, use_cache=False):
+        a = self.attn(self.ln_1(hidden_states), layer_past=layer_past, attention_mask=attention_mask,
+                      head_mask=head_mask, use_cache=use_cache)
+        hidden_states = a[0] + hidden_states
+        hidden_states = hidden_states + self.mlp(self.ln_2(hidden_states))
+        return hidden_states, a[1]
+
+
+class GPTNeoLayerPolicy(LayerPolicy):
+    """oslo/models/gpt_neo/configuration_gpt_neo.py:330-342."""
+
+    @staticmethod
+    def fused_modules():
+        return {GPTNeoSelfAttention: FusedGPTNeoSelfAttention, GPTNeoMLP: FusedGPTNeoMLP}
+
+
+class GPTNeoModel(nn.Module):
+    def __init__(self, config):
+        super().__init__()
+        self.wte = nn.Embedding(config.vocab_size, config.hidden_size)
+        self.wpe = nn.Embedding(config.max_position_embeddings, config.hidden_size)
+        self.drop = nn.Dropout(config.embed_dropout)
+        self.h = nn.ModuleList([GPTNeoBlock(config, layer_id=i) for i in range(config.num_layers)])
+        self.ln_f = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_epsilon)
+
+    def forward(self, input_ids, attention_mask=None, past_key_values=None, use_cache=False):
+        past_len = 0 if past_key_values is None else past_key_values[0][0].size(-2)
+        pos = torch.arange(past_len, past_len + input_ids.size(-1), device=input_ids.device)
+        h = self.drop(self.wte(input_ids) + self.wpe(pos)[None])
+        mask = additive_attention_mask(attention_mask, h.dtype)
+        presents = []
+        for i, block in enumerate(self.h):
+            h, present = block(h, layer_past=None if past_key_values is None else past_key_values[i],
+                               attention_mask=mask, use_cache=use_cache)
+            presents.append(present)
+        return self.ln_f(h), (tuple(presents) if use_cache else None)
+
+
+class GPTNeoForCausalLM(PreTrainedModel):
+    is_fusable = True
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.transformer = GPTNeoModel(config)
+        self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
+        self.init_weights()
+        self.lm_head.weight = self.transformer.wte.weight  # tied
+
+    def get_layer_policies(self):
+        return [GPTNeoLayerPolicy]
+
+    def forward(self, input_ids, attention_mask=None, past_key_values=None, use_cache=False, labels=None):
+        h, presents = self.transformer(input_ids, attention_mask, past_key_values, use_cache)
+        logits = self.lm_head(h)
+        loss = causal_lm_loss(logits, labels) if labels is not None else None
+        return {"loss": loss, "logits": logits, "past_key_values": presents}

@@ -1,0 +1,248 @@
+"""GPT-J blocks with the reference's kernel-fusion hooks.
+
+``GPTJAttention`` / ``GPTJMLP`` compute what the reference's unfused modules
+compute (oslo/models/gptj/modeling_gptj.py:49-257): rotary position embedding
+on the first ``rotary_dim`` features, scores and softmax in fp32, attention and
+MLP fed from the same LayerNorm. ``FusedGPTJAttention`` / ``FusedGPTJMLP`` are
+the classes ``fuse()`` swaps in (oslo/models/gptj/modeling_gptj.py:936-1065).
+
+One deliberate difference: the reference's fused attention passes
+``scale=self.scale_attn`` (= sqrt(head_dim)) to a kernel that multiplies by the
+scale (oslo/models/gptj/modeling_gptj.py:941-946), while its unfused attention
+divides by it (:175). The fused class here passes ``1/scale_attn``, so fused
+and unfused agree."""
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+from torch import nn
+
+from .fused_kernels_utils import FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax
+from .modeling_utils import ACT2FN, LayerPolicy, PreTrainedModel, additive_attention_mask, causal_lm_loss
+
+
+@dataclass
+class GPTJConfig:
+    vocab_size: int = 50400
+    n_positions: int = 2048
+    n_embd: int = 4096
+    n_layer: int = 28
+    n_head: int = 16
+    rotary_dim: Optional[int] = 64
+    n_inner: Optional[int] = None
+    activation_function: str = "gelu_new"
+    resid_pdrop: float = 0.0
+    embd_pdrop: float = 0.0
+    attn_pdrop: float = 0.0
+    layer_norm_epsilon: float = 1e-5
+
+    @property
+    def hidden_size(self):
+        return self.n_embd
+
+    @property
+    def num_attention_heads(self):
+        return self.n_head
+
+    @property
+    def max_position_embeddings(self):
+        return self.n_positions
+
+
+def rotary_tables(dim, seq_len, device):
+    """sin and cos of position * 10000^(-2i/dim), each [seq_len, dim/2], fp32."""
+    inv_freq = 1.0 / (10000 ** (torch.arange(0, dim, 2, device=device, dtype=torch.float32) / dim))
+    angles = torch.arange(seq_len, device=device, dtype=torch.float32)[:, None] * inv_freq[None, :]
+    return torch.sin(angles), torch.cos(angles)
+
+
+def apply_rotary(x, sin, cos, offset=0):
+    """x [B, S, H, D]: rotates consecutive feature pairs (2i, 2i+1) by the angle
+    of position offset+s."""
+    s = x.shape[1]
+    sin = sin[offset:offset + s].repeat_interleave(2, dim=-1)[None, :, None, :]
+    cos = cos[offset:offset + s].repeat_interleave(2, dim=-1)[None, :, None, :]
+    rotated = torch.stack((-x[..., 1::2], x[..., ::2]), dim=-1).flatten(-2)
+    return x * cos + rotated * sin
+
+
+class GPTJAttention(nn.Module):
+    def __init__(self, config):
+        super().__init__()
+        n_pos = config.max_position_embeddings
+        self.register_buffer(
+            "bias", torch.tril(torch.ones((n_pos, n_pos), dtype=torch.uint8)).view(1, 1, n_pos, n_pos))
+        self.register_buffer("masked_bias", torch.tensor(-1e9))
+        self.attn_dropout = nn.Dropout(config.attn_pdrop)
+        self.resid_dropout = nn.Dropout(config.resid_pdrop)
+        self.embed_dim = config.hidden_size
+        self.num_attention_heads = config.num_attention_heads
+        self.head_dim = self.embed_dim // self.num_attention_heads
+        if self.head_dim * self.num_attention_heads != self.embed_dim:
+            raise ValueError("embed_dim must be divisible by num_attention_heads")
+        self.scale_attn = float(self.head_dim) ** 0.5
+        self.k_proj = nn.Linear(self.embed_dim, self.embed_dim, bias=False)
+        self.v_proj = nn.Linear(self.embed_dim, self.embed_dim, bias=False)
+        self.q_proj = nn.Linear(self.embed_dim, self.embed_dim, bias=False)
+        self.out_proj = nn.Linear(self.embed_dim, self.embed_dim, bias=False)
+        self.rotary_dim = config.rotary_dim
+
+    def _merge_heads(self, t):
+        t = t.permute(0, 2, 1, 3).contiguous()
+        return t.view(t.size()[:-2] + (self.num_attention_heads * self.head_dim,))
+
+    def _attn(self, query, key, value, attention_mask=None, head_mask=None):
+        """The unfused path: fp32 scores, where(causal, w, -1e9), / sqrt(d), + mask, softmax."""
+        sq, sk = query.size(-2), key.size(-2)
+        causal = self.bias[:, :, sk - sq:sk, :sk].bool()
+        w = torch.matmul(query.to(torch.float32), key.to(torch.float32).transpose(-1, -2))
+        w = torch.where(causal, w, self.masked_bias.to(w.dtype))
+        w = w / self.scale_attn
+        if attention_mask is not None:
+            w = w + attention_mask
+        w = nn.functional.softmax(w, dim=-1).to(value.dtype)
+        w = self.attn_dropout(w)
+        if head_mask is not None:
+            w = w * head_mask
+        return torch.matmul(w, value), w
+
+    def _project_qkv(self, hidden_states, layer_past, use_cache):
+        b, s, _ = hidden_states.shape
+        shape = (b, s, self.num_attention_heads, self.head_dim)
+        query = self.q_proj(hidden_states).view(shape)
+        key = self.k_proj(hidden_states).view(shape)
+        value = self.v_proj(hidden_states).view(shape).permute(0, 2, 1, 3)
+        offset = 0 if layer_past is None else layer_past[0].shape[-2]
+        rot = self.rotary_dim if self.rotary_dim is not None else self.head_dim
+        sin, cos = rotary_tables(rot, s + offset, hidden_states.device)
+        if rot < self.head_dim:
+            key = torch.cat([apply_rotary(key[..., :rot], sin, cos, offset), key[..., rot:]], dim=-1)
+            query = torch.cat([apply_rotary(query[..., :rot], sin, cos, offset), query[..., rot:]], dim=-1)
+        else:
+            key = apply_rotary(key, sin, cos, offset)
+            query = apply_rotary(query, sin, cos, offset)
+        key = key.to(value.dtype).permute(0, 2, 1, 3)
+        query = query.to(value.dtype).permute(0, 2, 1, 3)
+        if layer_past is not None:
+            key = torch.cat((layer_past[0], key), dim=-2)
+            value = torch.cat((layer_past[1], value), dim=-2)
+        present = (key, value) if use_cache else None
+        return query, key, value, present
+
+    def forward(self, hidden_states, attention_mask=None, layer_past=None, head_mask=None,
+                use_cache=False, output_attentions=False):
+        query, key, value, present = self._project_qkv(hidden_states, layer_past, use_cache)
+        out, w = self._attn(query, key, value, attention_mask, head_mask)
+        out = self.resid_dropout(self.out_proj(self._merge_heads(out)))
+        return (out, present, w) if output_attentions else (out, present)
+
+
+class FusedGPTJAttention(GPTJAttention):
+    """oslo/models/gptj/modeling_gptj.py:936-1038."""
+
+    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
+        w = torch.matmul(query, key.transpose(-1, -2))
+        w = FusedScaleMaskSoftmax.apply(w, pad_mask=attention_mask, scale=1.0 / self.scale_attn,
+                                        use_triang_mask=True)
+        w = self.attn_dropout(w.to(value.dtype))
+        if head_mask is not None:
+            w = w * head_mask
+        return torch.matmul(w, value), w
+
+    def forward(self, hidden_states, attention_mask=None, layer_past=None, head_mask=None,
+                use_cache=False, output_attentions=False):
+        query, key, value, present = self._project_qkv(hidden_states, layer_past, use_cache)
+        (bsz, np_, sq, _), sk = query.size(), key.size(-2)
+        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=True):
+            out, w = self._fused_attn(query, key, value, attention_mask, head_mask)
+        else:
+            out, w = self._attn(query, key, value, attention_mask, head_mask)
+        # out_proj has no bias, so there is nothing to fuse after it
+        out = self.resid_dropout(self.out_proj(self._merge_heads(out)))
+        return (out, present, w) if output_attentions else (out, present)
+
+
+class GPTJMLP(nn.Module):
+    def __init__(self, intermediate_size, config):
+        super().__init__()
+        self.fc_in = nn.Linear(config.n_embd, intermediate_size)
+        self.fc_out = nn.Linear(intermediate_size, config.n_embd)
+        self.act = ACT2FN[config.activation_function]
+        self.dropout = nn.Dropout(config.resid_pdrop)
+
+    def forward(self, hidden_states):
+        return self.dropout(self.fc_out(self.act(self.fc_in(hidden_states))))
+
+
+class FusedGPTJMLP(GPTJMLP):
+    """oslo/models/gptj/modeling_gptj.py:1041-1065."""
+
+    def forward(self, x):
+        x = x @ self.fc_in.weight.t()
+        x = FusedBiasActivation.apply(x, self.fc_in.bias, self.config.activation_function)
+        x = x @ self.fc_out.weight.t()
+        return FusedBiasDropout.apply(x, self.fc_out.bias, self.training, self.dropout.p)
+
+
+class GPTJBlock(nn.Module):
+    def __init__(self, config):
+        super().__init__()
+        inner = config.n_inner if config.n_inner is not None else 4 * config.n_embd
+        self.ln_1 = nn.LayerNorm(config.n_embd, eps=config.layer_norm_epsilon)
+        self.attn = GPTJAttention(config)
+        self.mlp = GPTJMLP(inner, config)
+
+    def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None, use_cache=False):
+        residual = hidden_states
+        hidden_states = self.ln_1(hidden_states)
+        a = self.attn(hidden_states, layer_past=layer_past, attention_mask=attention_mask,
+                      head_mask=head_mask, use_cache=use_cache)
+        hidden_states = a[0] + self.mlp(hidden_states) + residual
+        return hidden_states, a[1]
+
+
+class GPTJLayerPolicy(LayerPolicy):
+    """oslo/models/gptj/configuration_gptj.py:155-167."""
+
+    @staticmethod
+    def fused_modules():
+        return {GPTJAttention: FusedGPTJAttention, GPTJMLP: FusedGPTJMLP}
+
+
+class GPTJModel(nn.Module):
+    def __init__(self, config):
+        super().__init__()
+        self.wte = nn.Embedding(config.vocab_size, config.n_embd)
+        self.drop = nn.Dropout(config.embd_pdrop)
+        self.h = nn.ModuleList([GPTJBlock(config) for _ in range(config.n_layer)])
+        self.ln_f = nn.LayerNorm(config.n_embd, eps=config.layer_norm_epsilon)
+
+    def forward(self, input_ids, attention_mask=None, past_key_values=None, use_cache=False):
+        h = self.drop(self.wte(input_ids))
+        mask = additive_attention_mask(attention_mask, h.dtype)
+        presents = []
+        for i, block in enumerate(self.h):
+            h, present = block(h, layer_past=None if past_key_values is None else past_key_values[i],
+                               attention_mask=mask, use_cache=use_cache)
+            presents.append(present)
+        return self.ln_f(h), (tuple(presents) if use_cache else None)
+
+
+class GPTJForCausalLM(PreTrainedModel):
+    is_fusable = True
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.transformer = GPTJModel(config)
+        self.lm_head = nn.Linear(config.n_embd, config.vocab_size)
+        self.init_weights()
+
+    def get_layer_policies(self):
+        return [GPTJLayerPolicy]
+
+    def forward(self, input_ids, attention_mask=None, past_key_values=None, use_cache=False, labels=None):
+        h, presents = self.transformer(input_ids, attention_mask, past_key_values, use_cache)
+        logits = self.lm_head(h)
+        loss = causal_lm_loss(logits, labels) if labels is not None else None
+        return {"loss": loss, "logits": logits, "past_key_values": presents}

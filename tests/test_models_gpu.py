@@ -1,0 +1,150 @@
+"""model.fuse() on the GPU: a fused model computes what the unfused model
+computes (dropout off), forward and backward, with and without padding, in the
+dtypes the families run in; and the operator API behaves like torch ops under
+autograd and the device generator."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oslo_oracle as orc
+from oslo_amd import (FusedBiasActivation, FusedBiasDropout, FusedBiasDropoutResidual, FusedScaleMaskSoftmax,
+                      GPT2Config, GPT2LMHeadModel, GPTJConfig, GPTJForCausalLM, GPTNeoConfig, GPTNeoForCausalLM)
+from oslo_amd import fused_kernels_utils as fku
+from tests.util import f32
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def models():
+    return {
+        "gpt2": lambda: GPT2LMHeadModel(GPT2Config(vocab_size=512, n_positions=128, n_embd=128, n_layer=2, n_head=4,
+                                                   resid_pdrop=0.0, embd_pdrop=0.0, attn_pdrop=0.0)),
+        "gptj": lambda: GPTJForCausalLM(GPTJConfig(vocab_size=512, n_positions=128, n_embd=128, n_layer=2, n_head=4,
+                                                   rotary_dim=16)),
+        "gpt_neo": lambda: GPTNeoForCausalLM(GPTNeoConfig(vocab_size=512, max_position_embeddings=128,
+                                                          hidden_size=128, num_layers=2, num_heads=4, window_size=32)),
+    }
+
+
+# logits are O(1); fused and unfused differ by the rounding of 16-bit
+# intermediates (the unfused path rounds after every operator)
+LOGIT_TOL = {torch.float32: 2e-4, torch.float16: 2e-2, torch.bfloat16: 1.5e-1}
+
+
+@pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("padded", [False, True], ids=["nopad", "pad"])
+def test_fused_model_matches_unfused(family, dtype, padded):
+    torch.manual_seed(0)
+    m = models()[family]().to(DEV, dtype).eval()
+    ids = torch.randint(0, 512, (3, 96), device=DEV)
+    mask = None
+    if padded:
+        mask = torch.ones(3, 96, device=DEV)
+        mask[1, 60:] = 0
+        mask[2, 17:] = 0
+    with torch.no_grad():
+        want = m(ids, attention_mask=mask)["logits"].float()
+        m.fuse()
+        got = m(ids, attention_mask=mask)["logits"].float()
+    assert torch.isfinite(got).all()
+    keep = torch.ones(3, 96, dtype=torch.bool, device=DEV) if mask is None else mask.bool()
+    err = (got - want).abs()[keep].max().item()     # rows of padded queries are not compared
+    assert err <= LOGIT_TOL[dtype], f"{family} {dtype}: logits differ by {err}"
+
+
+@pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
+def test_fused_model_backward_matches_unfused(family):
+    torch.manual_seed(1)
+    m = models()[family]().to(DEV).train()            # fp32, every dropout p = 0
+    ids = torch.randint(0, 512, (2, 64), device=DEV)
+    m(ids, labels=ids)["loss"].backward()
+    want = {k: p.grad.clone() for k, p in m.named_parameters() if p.grad is not None}
+    loss_want = m(ids, labels=ids)["loss"].item()
+    m.zero_grad()
+    m.fuse()
+    out = m(ids, labels=ids)
+    out["loss"].backward()
+    assert abs(out["loss"].item() - loss_want) <= 1e-5
+    for k, p in m.named_parameters():
+        if k in want:
+            scale = want[k].abs().max().item() + 1e-8
+            err = (p.grad - want[k]).abs().max().item()
+            assert err <= 2e-4 * max(1.0, scale) and err / scale <= 2e-3, f"{family} grad {k}: {err} (scale {scale})"
+
+
+def test_decode_step_routes_to_the_unfused_attention():
+    torch.manual_seed(2)
+    m = models()["gpt2"]().to(DEV, torch.float16).eval().fuse()
+    ids = torch.randint(0, 512, (2, 40), device=DEV)
+    with torch.no_grad():
+        full = m(ids)["logits"]
+        first = m(ids[:, :39], use_cache=True)
+        step = m(ids[:, 39:], past_key_values=first["past_key_values"], use_cache=True)
+    assert (step["logits"][:, 0].float() - full[:, 39].float()).abs().max().item() <= 2e-2
+
+
+def test_softmax_apply_autograd_matches_torch():
+    torch.manual_seed(3)
+    b, h, s = 2, 3, 72
+    x = torch.randn(b, h, s, s, device=DEV, requires_grad=True)
+    go = torch.randn(b, h, s, s, device=DEV)
+    pad = torch.zeros(b, 1, 1, s, device=DEV)
+    pad[1, :, :, 50:] = -10000.0
+    causal = torch.tril(torch.ones(s, s, dtype=torch.bool, device=DEV))
+    for tri in (True, False):
+        for mask in (None, pad, pad != 0):
+            e = x * 0.3
+            if tri:
+                e = e.masked_fill(~causal, float("-inf"))
+            if mask is not None:
+                e = e + (pad if mask.dtype != torch.bool else pad)
+            want = torch.softmax(e, -1)
+            (gx_want,) = torch.autograd.grad(want, x, go)
+            got = FusedScaleMaskSoftmax.apply(x, mask, 0.3, tri)
+            (gx,) = torch.autograd.grad(got, x, go.clone())
+            assert (got - want).abs().max().item() <= 1e-6
+            assert (gx - gx_want).abs().max().item() <= 1e-6
+    # scale=None means 1.0
+    got = FusedScaleMaskSoftmax.apply(x.detach(), None, None, True)
+    want = torch.softmax(x.detach().masked_fill(~causal, float("-inf")), -1)
+    assert (got - want).abs().max().item() <= 1e-6
+
+
+def test_bias_gelu_and_dropout_autograd():
+    torch.manual_seed(4)
+    x = torch.randn(5, 7, 96, device=DEV, requires_grad=True)
+    bias = torch.randn(96, device=DEV, requires_grad=True)
+    res = torch.randn(5, 7, 96, device=DEV, requires_grad=True)
+    go = torch.randn(5, 7, 96, device=DEV)
+    want = torch.nn.functional.gelu(x + bias, approximate="tanh")
+    gw = torch.autograd.grad(want, (x, bias), go)
+    got = FusedBiasActivation.apply(x, bias, "gelu_new")
+    gg = torch.autograd.grad(got, (x, bias), go)
+    assert (got - want).abs().max().item() <= 2e-6
+    assert (gg[0] - gw[0]).abs().max().item() <= 5e-6 and (gg[1] - gw[1]).abs().max().item() <= 5e-5
+    # inference: exactly x + bias (+ residual); gradients flow to all three
+    out = FusedBiasDropoutResidual.apply(x, bias, res, False, 0.1)
+    assert torch.equal(out, x + bias + res)
+    gx, gb, gr = torch.autograd.grad(out, (x, bias, res), go)
+    assert torch.equal(gx, go) and torch.equal(gr, go)
+    assert (gb - go.sum((0, 1))).abs().max().item() <= 1e-4
+    # training: mask from the device generator; same seed -> same mask, generator advances
+    torch.manual_seed(77)
+    gen = torch.cuda.default_generators[0]
+    seed, off0 = gen.initial_seed(), gen.get_offset()
+    a = FusedBiasDropout.apply(x, bias, True, 0.25)
+    assert gen.get_offset() == off0 + fku.PHILOX_WORDS_PER_CALL
+    b2 = FusedBiasDropout.apply(x, bias, True, 0.25)
+    assert not torch.equal(a, b2)
+    torch.manual_seed(77)
+    assert torch.equal(FusedBiasDropout.apply(x, bias, True, 0.25), a)
+    keep = orc.dropout_keep_mask(seed, off0, x.numel(), 0.25).reshape(5, 7, 96)
+    want = orc.bias_dropout_add_fwd(f32(x), f32(bias), None, 0.25, keep)
+    assert np.abs(f32(a) - want).max() <= 1e-6
+    (gx,) = torch.autograd.grad(a, x, go)                       # backward regenerates the mask
+    assert np.abs(f32(gx) - orc.bias_dropout_add_bwd(f32(go), 0.25, keep)[0]).max() <= 1e-6
+    # p = 1 drops everything, like F.dropout
+    assert torch.count_nonzero(FusedBiasDropout.apply(x, bias, True, 1.0)) == 0
