@@ -145,6 +145,24 @@ __device__ __forceinline__ RawVec<T, N> buffer_load_raw(BufRsrc rs,
   }
 }
 
+// Store N fp32 values as T through a buffer descriptor (offsets at or past the
+// bound are dropped). kStreamOut = sc1 + nt: write-through at device scope,
+// non-temporal; on the softmax rows it measured 2-3 % faster than nt alone and
+// 6 % faster than the default policy.
+constexpr int kStreamOut = 16 | 2;
+
+template <typename T, int N, int AUX>
+__device__ __forceinline__ void buffer_store_f32(BufRsrc rs, uint32_t byte_offset,
+                                                 const float (&src)[N]) {
+  static_assert(N * sizeof(T) == 16, "one 128-bit store");
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  RawVec<T, N> v;
+#pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = static_cast<T>(src[i]);
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rs,
+                                         byte_offset, 0, AUX);
+}
+
 template <typename T, int N>
 __device__ __forceinline__ void store_f32(T *p, const float (&src)[N]) {
   using V = typename VecOf<T, N>::type;

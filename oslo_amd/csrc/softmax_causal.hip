@@ -20,7 +20,7 @@ namespace {
 template <typename T, int VEC, int NCHUNK, int WPR, bool HAS_PAD>
 __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
     T *y, const T *x, const float *__restrict__ pad, float scale, int S,
-    int heads, int64_t total_rows) {
+    int heads, RowMap map) {
   using Tile = RowTile<VEC, NCHUNK, WPR>;
   __shared__ float s_max[kWavesPerBlock];
   __shared__ float s_sum[kWavesPerBlock];
@@ -28,11 +28,11 @@ __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int sub = wave % WPR;
-  int64_t row = paired_block(blockIdx.x, gridDim.x) * Tile::kRowsPerBlock + wave / WPR;
-  // A block past the end keeps its waves alive (they meet the same barriers)
-  // on the last row and only skips the stores.
-  const bool live = row < total_rows;
-  if (!live) row = total_rows - 1;
+  int64_t row = mapped_row(map, Tile::kRowsPerBlock, wave / WPR);
+  // A row slot past the end keeps its waves alive (they meet the same
+  // barriers) on the last row and only skips the stores.
+  const bool live = row < map.total_rows;
+  if (!live) row = map.total_rows - 1;
   const int64_t slab = row / S;
   const int r = (int)(row - slab * S);
   const T *xr = x + row * S;
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
   RawVec<float, VEC> praw[HAS_PAD ? NCHUNK : 1];
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c)
-    raw[c] = buffer_load_raw<T, VEC, false>(
+    raw[c] = buffer_load_raw<T, VEC, true>(
         xrs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T));
   if constexpr (HAS_PAD) {
     const BufRsrc prs = make_rsrc(padr, keys * (uint32_t)sizeof(float));
@@ -96,30 +96,29 @@ __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
   const float inv = 1.0f / sum;
 
   if (!live) return;
+  const BufRsrc yrs = make_rsrc(yr, (uint32_t)S * (uint32_t)sizeof(T));
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
-    const int k0 = Tile::col(c, sub, lane);
-    if (k0 < S) {
-      float o[VEC];
+    float o[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) o[j] = v[c][j] * inv;
-      store_f32<T, VEC>(yr + k0, o);
-    }
+    for (int j = 0; j < VEC; ++j) o[j] = v[c][j] * inv;
+    buffer_store_f32<T, VEC, kStreamOut>(
+        yrs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T), o);
   }
 }
 
 template <typename T, int VEC, int NCHUNK, int WPR>
 __global__ __launch_bounds__(kBlockThreads) void causal_bwd_kernel(
-    T *dx, const T *g, const T *y, float scale, int S, int64_t total_rows) {
+    T *dx, const T *g, const T *y, float scale, int S, RowMap map) {
   using Tile = RowTile<VEC, NCHUNK, WPR>;
   __shared__ float s_sum[kWavesPerBlock];
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int sub = wave % WPR;
-  int64_t row = paired_block(blockIdx.x, gridDim.x) * Tile::kRowsPerBlock + wave / WPR;
-  const bool live = row < total_rows;
-  if (!live) row = total_rows - 1;
+  int64_t row = mapped_row(map, Tile::kRowsPerBlock, wave / WPR);
+  const bool live = row < map.total_rows;
+  if (!live) row = map.total_rows - 1;
   const int r = (int)(row % S);
   const T *gr = g + row * S;
   const T *yr = y + row * S;
@@ -133,8 +132,8 @@ __global__ __launch_bounds__(kBlockThreads) void causal_bwd_kernel(
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
     const uint32_t off = (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T);
-    graw[c] = buffer_load_raw<T, VEC, false>(grs, off);
-    yraw[c] = buffer_load_raw<T, VEC, false>(yrs, off);
+    graw[c] = buffer_load_raw<T, VEC, true>(grs, off);
+    yraw[c] = buffer_load_raw<T, VEC, true>(yrs, off);
   }
 
   float gy[NCHUNK][VEC]; // g*y
@@ -157,16 +156,14 @@ __global__ __launch_bounds__(kBlockThreads) void causal_bwd_kernel(
   sum = row_allreduce<WPR>(sum, OpAdd(), s_sum);
 
   if (!live) return;
+  const BufRsrc drs = make_rsrc(dr, (uint32_t)S * (uint32_t)sizeof(T));
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
-    const int k0 = Tile::col(c, sub, lane);
-    if (k0 < S) {
-      float o[VEC];
+    float o[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j)
-        o[j] = scale * (gy[c][j] - yy[c][j] * sum);
-      store_f32<T, VEC>(dr + k0, o);
-    }
+    for (int j = 0; j < VEC; ++j) o[j] = scale * (gy[c][j] - yy[c][j] * sum);
+    buffer_store_f32<T, VEC, kStreamOut>(
+        drs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T), o);
   }
 }
 
@@ -248,15 +245,17 @@ int launch_causal_fwd(T *y, const T *x, const float *pad, float scale,
   }
   dispatch_row_tile<VEC>(S, [&]<int NCHUNK, int WPR>() {
     constexpr int rpb = RowTile<VEC, NCHUNK, WPR>::kRowsPerBlock;
-    const int64_t blocks = (total_rows + rpb - 1) / rpb;
+    const RowMap map = make_row_map(total_rows, rpb, S * (int64_t)sizeof(T), true);
+    const dim3 grid((unsigned)(map.blocks_per_xcd * kXcds));
+    const unsigned lds = occupancy_pad_bytes(false, S * (int64_t)sizeof(T));
     if (pad)
       causal_fwd_kernel<T, VEC, NCHUNK, WPR, true>
-          <<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(
-              y, x, pad, scale, (int)S, (int)heads, total_rows);
+          <<<grid, dim3(kBlockThreads), lds, stream>>>(
+              y, x, pad, scale, (int)S, (int)heads, map);
     else
       causal_fwd_kernel<T, VEC, NCHUNK, WPR, false>
-          <<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(
-              y, x, nullptr, scale, (int)S, (int)heads, total_rows);
+          <<<grid, dim3(kBlockThreads), lds, stream>>>(
+              y, x, nullptr, scale, (int)S, (int)heads, map);
   });
   return check_launch("softmax_causal_fwd");
 }
@@ -277,10 +276,11 @@ int launch_causal_bwd(T *dx, const T *g, const T *y, float scale, int64_t bh,
   }
   dispatch_row_tile<VEC>(S, [&]<int NCHUNK, int WPR>() {
     constexpr int rpb = RowTile<VEC, NCHUNK, WPR>::kRowsPerBlock;
-    const int64_t blocks = (total_rows + rpb - 1) / rpb;
+    const RowMap map = make_row_map(total_rows, rpb, S * (int64_t)sizeof(T), true);
     causal_bwd_kernel<T, VEC, NCHUNK, WPR>
-        <<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(
-            dx, g, y, scale, (int)S, total_rows);
+        <<<dim3((unsigned)(map.blocks_per_xcd * kXcds)), dim3(kBlockThreads),
+           occupancy_pad_bytes(true, S * (int64_t)sizeof(T)), stream>>>(
+            dx, g, y, scale, (int)S, map);
   });
   return check_launch("softmax_causal_bwd");
 }

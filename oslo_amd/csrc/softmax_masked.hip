@@ -24,7 +24,7 @@ template <typename T, int VEC, int NCHUNK, int WPR, bool HAS_MASK, bool REPLACE>
 __global__ __launch_bounds__(kBlockThreads) void masked_fwd_kernel(
     T *y, const T *x, const uint8_t *__restrict__ mask, int64_t mask_stride_b,
     int64_t mask_stride_q, float scale, int Sq, int Sk, int heads,
-    int64_t total_rows) {
+    RowMap map) {
   using Tile = RowTile<VEC, NCHUNK, WPR>;
   __shared__ float s_max[kWavesPerBlock];
   __shared__ float s_sum[kWavesPerBlock];
@@ -32,9 +32,9 @@ __global__ __launch_bounds__(kBlockThreads) void masked_fwd_kernel(
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int sub = wave % WPR;
-  int64_t row = (int64_t)blockIdx.x * Tile::kRowsPerBlock + wave / WPR;
-  const bool live = row < total_rows;
-  if (!live) row = total_rows - 1;
+  int64_t row = mapped_row(map, Tile::kRowsPerBlock, wave / WPR);
+  const bool live = row < map.total_rows;
+  if (!live) row = map.total_rows - 1;
   const T *xr = x + row * Sk;
   T *yr = y + row * Sk;
   const uint8_t *mr = nullptr;
@@ -96,30 +96,29 @@ __global__ __launch_bounds__(kBlockThreads) void masked_fwd_kernel(
   const float inv = 1.0f / sum;
 
   if (!live) return;
+  const BufRsrc yrs = make_rsrc(yr, (uint32_t)Sk * (uint32_t)sizeof(T));
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
-    const int k0 = Tile::col(c, sub, lane);
-    if (k0 < Sk) {
-      float o[VEC];
+    float o[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) o[j] = v[c][j] * inv;
-      store_f32<T, VEC>(yr + k0, o);
-    }
+    for (int j = 0; j < VEC; ++j) o[j] = v[c][j] * inv;
+    buffer_store_f32<T, VEC, kStreamOut>(
+        yrs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T), o);
   }
 }
 
 template <typename T, int VEC, int NCHUNK, int WPR>
 __global__ __launch_bounds__(kBlockThreads) void masked_bwd_kernel(
-    T *dx, const T *g, const T *y, float scale, int Sk, int64_t total_rows) {
+    T *dx, const T *g, const T *y, float scale, int Sk, RowMap map) {
   using Tile = RowTile<VEC, NCHUNK, WPR>;
   __shared__ float s_sum[kWavesPerBlock];
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int sub = wave % WPR;
-  int64_t row = (int64_t)blockIdx.x * Tile::kRowsPerBlock + wave / WPR;
-  const bool live = row < total_rows;
-  if (!live) row = total_rows - 1;
+  int64_t row = mapped_row(map, Tile::kRowsPerBlock, wave / WPR);
+  const bool live = row < map.total_rows;
+  if (!live) row = map.total_rows - 1;
   const T *gr = g + row * Sk;
   const T *yr = y + row * Sk;
   T *dr = dx + row * Sk;
@@ -152,16 +151,14 @@ __global__ __launch_bounds__(kBlockThreads) void masked_bwd_kernel(
   sum = row_allreduce<WPR>(sum, OpAdd(), s_sum);
 
   if (!live) return;
+  const BufRsrc drs = make_rsrc(dr, (uint32_t)Sk * (uint32_t)sizeof(T));
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
-    const int k0 = Tile::col(c, sub, lane);
-    if (k0 < Sk) {
-      float o[VEC];
+    float o[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j)
-        o[j] = scale * (gy[c][j] - yy[c][j] * sum);
-      store_f32<T, VEC>(dr + k0, o);
-    }
+    for (int j = 0; j < VEC; ++j) o[j] = scale * (gy[c][j] - yy[c][j] * sum);
+    buffer_store_f32<T, VEC, kStreamOut>(
+        drs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T), o);
   }
 }
 
@@ -240,20 +237,22 @@ int launch_masked_fwd(T *y, const T *x, const uint8_t *mask, int64_t msb,
   }
   dispatch_row_tile<VEC>(Sk, [&]<int NCHUNK, int WPR>() {
     constexpr int rpb = RowTile<VEC, NCHUNK, WPR>::kRowsPerBlock;
-    const dim3 grid((unsigned)((total_rows + rpb - 1) / rpb));
+    const RowMap map = make_row_map(total_rows, rpb, Sk * (int64_t)sizeof(T), false);
+    const dim3 grid((unsigned)(map.blocks_per_xcd * kXcds));
     const dim3 block(kBlockThreads);
+    const unsigned lds = occupancy_pad_bytes(false, Sk * (int64_t)sizeof(T));
     if (!mask)
       masked_fwd_kernel<T, VEC, NCHUNK, WPR, false, false>
-          <<<grid, block, 0, stream>>>(y, x, nullptr, 0, 0, scale, (int)Sq,
-                                       (int)Sk, (int)H, total_rows);
+          <<<grid, block, lds, stream>>>(y, x, nullptr, 0, 0, scale, (int)Sq,
+                                         (int)Sk, (int)H, map);
     else if (replace)
       masked_fwd_kernel<T, VEC, NCHUNK, WPR, true, true>
-          <<<grid, block, 0, stream>>>(y, x, mask, msb, msq, scale, (int)Sq,
-                                       (int)Sk, (int)H, total_rows);
+          <<<grid, block, lds, stream>>>(y, x, mask, msb, msq, scale, (int)Sq,
+                                         (int)Sk, (int)H, map);
     else
       masked_fwd_kernel<T, VEC, NCHUNK, WPR, true, false>
-          <<<grid, block, 0, stream>>>(y, x, mask, msb, msq, scale, (int)Sq,
-                                       (int)Sk, (int)H, total_rows);
+          <<<grid, block, lds, stream>>>(y, x, mask, msb, msq, scale, (int)Sq,
+                                         (int)Sk, (int)H, map);
   });
   return check_launch("softmax_masked_fwd");
 }
@@ -272,9 +271,11 @@ int launch_masked_bwd(T *dx, const T *g, const T *y, float scale, int64_t rows,
   }
   dispatch_row_tile<VEC>(Sk, [&]<int NCHUNK, int WPR>() {
     constexpr int rpb = RowTile<VEC, NCHUNK, WPR>::kRowsPerBlock;
+    const RowMap map = make_row_map(rows, rpb, Sk * (int64_t)sizeof(T), false);
     masked_bwd_kernel<T, VEC, NCHUNK, WPR>
-        <<<dim3((unsigned)((rows + rpb - 1) / rpb)), dim3(kBlockThreads), 0,
-           stream>>>(dx, g, y, scale, (int)Sk, rows);
+        <<<dim3((unsigned)(map.blocks_per_xcd * kXcds)), dim3(kBlockThreads),
+           occupancy_pad_bytes(true, Sk * (int64_t)sizeof(T)), stream>>>(
+            dx, g, y, scale, (int)Sk, map);
   });
   return check_launch("softmax_masked_bwd");
 }
