@@ -116,6 +116,9 @@ __device__ __forceinline__ BufRsrc make_rsrc(const void *base, uint32_t bytes) {
 }
 
 // NT sets the non-temporal bit of the cache policy (bit 1 on gfx94x/gfx950).
+// When the first use of a loaded value sits in a conditional block, follow the
+// loads with pin_loaded(): otherwise the optimiser sinks each load into that
+// block, next to a wait, and the loads of a wave are serialised again.
 template <typename T, int N, bool NT>
 __device__ __forceinline__ RawVec<T, N> buffer_load_raw(BufRsrc rs,
                                                         uint32_t byte_offset) {
@@ -143,6 +146,16 @@ __device__ __forceinline__ RawVec<T, N> buffer_load_raw(BufRsrc rs,
     return __builtin_bit_cast(
         V, __builtin_amdgcn_raw_buffer_load_b16(rs, byte_offset, 0, kAux));
   }
+}
+
+// An empty asm statement that "uses and redefines" the N raw vectors: every
+// load that produces them has to be issued before it and cannot be moved past
+// it. (The compiler also waits here for all of them; the waves of the other
+// rows cover that.)
+template <typename V, int N>
+__device__ __forceinline__ void pin_loaded(V (&raw)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(raw[i]));
 }
 
 // Store N fp32 values as T through a buffer descriptor (offsets at or past the

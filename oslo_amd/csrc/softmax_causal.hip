@@ -58,21 +58,44 @@ __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
           prs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(float));
   }
 
+  pin_loaded(raw);
+  if constexpr (HAS_PAD) pin_loaded(praw);
+
+  // With nothing added after scaling the row is kept in log2 units,
+  // exp(s*x - max) = exp2(x*(s*log2 e) - max'), which saves a multiply per key.
+  // With a padding mask the score is scale*x rounded, then + mask rounded, the
+  // two steps of the unfused path (they decide a fully masked row, where the
+  // sum is rounded at magnitude 1e4).
+  constexpr bool kLog2 = !HAS_PAD;
+  const float sc = kLog2 ? scale * kLog2e : scale;
   float v[NCHUNK][VEC];
   float m = -INFINITY;
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
+    // wave-uniform classification of the chunk against the diagonal
+    const int first = Tile::col(c, sub, 0);
+    if (first > r) continue; // wholly above: never converted, stored as zeros
     const int k0 = Tile::col(c, sub, lane);
     float t[VEC], pv[VEC];
     raw_to_f32<T, VEC>(t, raw[c]);
     if constexpr (HAS_PAD) raw_to_f32<float, VEC>(pv, praw[c]);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      // scale then add, each rounded, as the unfused path does
-      float e = __fmul_rn(t[j], scale);
-      if constexpr (HAS_PAD) e = __fadd_rn(e, pv[j]);
-      v[c][j] = (k0 + j <= r) ? e : -INFINITY;
-      m = fmaxf(m, v[c][j]);
+      t[j] = __fmul_rn(t[j], sc);
+      if constexpr (HAS_PAD) t[j] = __fadd_rn(t[j], pv[j]);
+    }
+    if (first + Tile::kSpan - 1 <= r) { // wholly at or below: no masking
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        v[c][j] = t[j];
+        m = fmaxf(m, t[j]);
+      }
+    } else { // the chunk the diagonal crosses
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        v[c][j] = (k0 + j <= r) ? t[j] : -INFINITY;
+        m = fmaxf(m, v[c][j]);
+      }
     }
   }
   m = row_allreduce<WPR>(m, OpMax(), s_max);
@@ -80,11 +103,10 @@ __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
   float sum = 0.f;
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
-    // wave-uniform: chunks wholly above the diagonal stay at exp(-inf) = 0
     if (Tile::col(c, sub, 0) <= r) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        v[c][j] = exp_shifted(v[c][j], m);
+        v[c][j] = kLog2 ? __builtin_amdgcn_exp2f(v[c][j] - m) : exp_shifted(v[c][j], m);
         sum += v[c][j];
       }
     } else {
@@ -136,19 +158,33 @@ __global__ __launch_bounds__(kBlockThreads) void causal_bwd_kernel(
     yraw[c] = buffer_load_raw<T, VEC, true>(yrs, off);
   }
 
+  pin_loaded(graw);
+  pin_loaded(yraw);
+
   float gy[NCHUNK][VEC]; // g*y
   float yy[NCHUNK][VEC]; // y
   float sum = 0.f;
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
+    // wave-uniform classification of the chunk against the diagonal
+    const int first = Tile::col(c, sub, 0);
+    if (first > r) { // wholly above: contributes nothing, stored as zeros
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) gy[c][j] = yy[c][j] = 0.f;
+      continue;
+    }
     const int k0 = Tile::col(c, sub, lane);
     float tg[VEC];
     raw_to_f32<T, VEC>(tg, graw[c]);
     raw_to_f32<T, VEC>(yy[c], yraw[c]);
+    if (first + Tile::kSpan - 1 > r) { // the chunk the diagonal crosses
+#pragma unroll
+      for (int j = 0; j < VEC; ++j)
+        // entries above the diagonal are never used, whatever they hold
+        if (k0 + j > r) yy[c][j] = tg[j] = 0.f;
+    }
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      // entries above the diagonal are never used, whatever they hold
-      if (k0 + j > r) yy[c][j] = tg[j] = 0.f;
       gy[c][j] = tg[j] * yy[c][j];
       sum += gy[c][j];
     }
