@@ -52,26 +52,27 @@ __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_fwd_kernel(
   }
   float b[VEC];
   if constexpr (HAS_BIAS) load_f32_cached<T, VEC>(b, bias + pos.c0);
+  // rows past the end were read as zeros and their stores are dropped by the
+  // same bound, so the body has no branch
+  const BufRsrc ors = ew_rsrc<T>(out, pos, rows_per_block, rows, cols);
   float tx[U][VEC], tr[U][VEC];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int64_t r = pos.r_base + (int64_t)u * TY;
     raw_to_f32<T, VEC>(tx[u], xraw[u]);
     if constexpr (HAS_RES) raw_to_f32<T, VEC>(tr[u], rraw[u]);
-    if (r < rows) {
-      bool keep[VEC];
-      if constexpr (DROP)
-        keep_flags<VEC>(keep, seed, offset, (uint64_t)(r * cols + pos.c0), threshold);
+    bool keep[VEC];
+    if constexpr (DROP)
+      keep_flags<VEC>(keep, seed, offset, (uint64_t)(r * cols + pos.c0), threshold);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        float t = tx[u][j];
-        if constexpr (HAS_BIAS) t += b[j];
-        if constexpr (DROP) t = keep[j] ? t * keep_scale : 0.f;
-        if constexpr (HAS_RES) t += tr[u][j];
-        tx[u][j] = t;
-      }
-      store_f32<T, VEC>(out + r * cols + pos.c0, tx[u]);
+    for (int j = 0; j < VEC; ++j) {
+      float t = tx[u][j];
+      if constexpr (HAS_BIAS) t += b[j];
+      if constexpr (DROP) t = keep[j] ? t * keep_scale : 0.f;
+      if constexpr (HAS_RES) t += tr[u][j];
+      tx[u][j] = t;
     }
+    buffer_store_f32<T, VEC, kStreamOut>(ors, ew_offset<T>(pos, u, cols), tx[u]);
   }
 }
 
@@ -92,24 +93,25 @@ __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_bwd_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u)
       graw[u] = buffer_load_raw<T, VEC, true>(grs, ew_offset<T>(pos, u, cols));
+    // rows past the end were read as zeros (they add nothing to dbias) and
+    // their stores are dropped by the same bound
+    const BufRsrc drs = ew_rsrc<T>(dx, pos, rows_per_block, rows, cols);
     float tg[U][VEC];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int64_t r = pos.r_base + (int64_t)u * TY;
       raw_to_f32<T, VEC>(tg[u], graw[u]);
-      if (r < rows) {
-        bool keep[VEC];
-        if constexpr (DROP)
-          keep_flags<VEC>(keep, seed, offset, (uint64_t)(r * cols + pos.c0), threshold);
+      bool keep[VEC];
+      if constexpr (DROP)
+        keep_flags<VEC>(keep, seed, offset, (uint64_t)(r * cols + pos.c0), threshold);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          if constexpr (DROP) tg[u][j] = keep[j] ? tg[u][j] * keep_scale : 0.f;
-          if constexpr (WANT_DBIAS) acc[j] += tg[u][j];
-        }
-        // with no dropout dx == g bit for bit; still written, dx may be a
-        // different buffer
-        store_f32<T, VEC>(dx + r * cols + pos.c0, tg[u]);
+      for (int j = 0; j < VEC; ++j) {
+        if constexpr (DROP) tg[u][j] = keep[j] ? tg[u][j] * keep_scale : 0.f;
+        if constexpr (WANT_DBIAS) acc[j] += tg[u][j];
       }
+      // with no dropout dx == g bit for bit; still written, dx may be a
+      // different buffer
+      buffer_store_f32<T, VEC, kStreamOut>(drs, ew_offset<T>(pos, u, cols), tg[u]);
     }
   }
   if constexpr (WANT_DBIAS)
@@ -123,7 +125,7 @@ struct DropArgs {
   bool drop;
 };
 
-constexpr int kDropBwdUnroll = 4;
+constexpr int kDropBwdUnroll = 8;
 static_assert(kDropBwdUnroll >= kBwdMinUnroll, "workspace bound");
 
 template <typename T, int VEC>

@@ -50,7 +50,6 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_fwd_kernel(
     int col_tiles, int rows_per_block) {
   const EwPos pos = ew_position<VEC>(col_tiles, rows_per_block);
   if (pos.c0 >= cols) return; // no barrier in this kernel
-  const int TY = blockDim.y;
   const BufRsrc yrs = ew_rsrc<T>(y, pos, rows_per_block, rows, cols);
   RawVec<T, VEC> raw[U];
 #pragma unroll
@@ -58,16 +57,16 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_fwd_kernel(
     raw[u] = buffer_load_raw<T, VEC, true>(yrs, ew_offset<T>(pos, u, cols));
   float b[VEC];
   load_f32_cached<T, VEC>(b, bias + pos.c0);
+  // rows past the end were read as zeros and their stores are dropped by the
+  // same bound, so the body has no branch
+  const BufRsrc ors = ew_rsrc<T>(out, pos, rows_per_block, rows, cols);
   float t[U][VEC];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    const int64_t r = pos.r_base + (int64_t)u * TY;
     raw_to_f32<T, VEC>(t[u], raw[u]);
-    if (r < rows) {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) t[u][j] = gelu_fwd(t[u][j] + b[j]);
-      store_f32<T, VEC>(out + r * cols + pos.c0, t[u]);
-    }
+    for (int j = 0; j < VEC; ++j) t[u][j] = gelu_fwd(t[u][j] + b[j]);
+    buffer_store_f32<T, VEC, kStreamOut>(ors, ew_offset<T>(pos, u, cols), t[u]);
   }
 }
 
@@ -78,7 +77,6 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_bwd_kernel(
     int rows_per_block) {
   const EwPos pos = ew_position<VEC>(col_tiles, rows_per_block);
   const bool col_ok = pos.c0 < cols;
-  const int TY = blockDim.y;
   float acc[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
@@ -93,27 +91,27 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_bwd_kernel(
     }
     float b[VEC];
     load_f32_cached<T, VEC>(b, bias + pos.c0);
+    // rows past the end were read as zeros (g = 0 makes their products 0, so
+    // they add nothing to dbias) and their stores are dropped by the bound
+    const BufRsrc drs = ew_rsrc<T>(dy, pos, rows_per_block, rows, cols);
     float tg[U][VEC], ty_[U][VEC];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t r = pos.r_base + (int64_t)u * TY;
       raw_to_f32<T, VEC>(tg[u], graw[u]);
       raw_to_f32<T, VEC>(ty_[u], yraw[u]);
-      if (r < rows) {
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          tg[u][j] = gelu_grad(ty_[u][j] + b[j]) * tg[u][j];
-          if constexpr (WANT_DBIAS) acc[j] += tg[u][j];
-        }
-        store_f32<T, VEC>(dy + r * cols + pos.c0, tg[u]);
+      for (int j = 0; j < VEC; ++j) {
+        tg[u][j] = gelu_grad(ty_[u][j] + b[j]) * tg[u][j];
+        if constexpr (WANT_DBIAS) acc[j] += tg[u][j];
       }
+      buffer_store_f32<T, VEC, kStreamOut>(drs, ew_offset<T>(pos, u, cols), tg[u]);
     }
   }
   if constexpr (WANT_DBIAS)
     write_colsum_partial<VEC>(acc, partial, cols, pos, col_ok);
 }
 
-constexpr int kGeluBwdUnroll = 2;
+constexpr int kGeluBwdUnroll = 4;
 static_assert(kGeluBwdUnroll >= kBwdMinUnroll, "workspace bound");
 
 template <typename T, int VEC>

@@ -167,13 +167,26 @@ constexpr int kStreamOut = 16 | 2;
 template <typename T, int N, int AUX>
 __device__ __forceinline__ void buffer_store_f32(BufRsrc rs, uint32_t byte_offset,
                                                  const float (&src)[N]) {
-  static_assert(N * sizeof(T) == 16, "one 128-bit store");
+  using V = RawVec<T, N>;
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-  RawVec<T, N> v;
+  V v;
+  if constexpr (N == 1) {
+    v = static_cast<T>(src[0]);
+  } else {
 #pragma unroll
-  for (int i = 0; i < N; ++i) v[i] = static_cast<T>(src[i]);
-  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rs,
-                                         byte_offset, 0, AUX);
+    for (int i = 0; i < N; ++i) v[i] = static_cast<T>(src[i]);
+  }
+  if constexpr (sizeof(V) == 16) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rs,
+                                           byte_offset, 0, AUX);
+  } else if constexpr (sizeof(V) == 4) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v),
+                                          rs, byte_offset, 0, AUX);
+  } else {
+    static_assert(sizeof(V) == 2, "unsupported vector size");
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v),
+                                          rs, byte_offset, 0, AUX);
+  }
 }
 
 template <typename T, int N>

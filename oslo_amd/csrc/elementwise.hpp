@@ -26,7 +26,7 @@ constexpr int kBwdMaxTx = 32;  // backward kernels: narrower and taller tiles,
                                // so that fewer dbias partial rows are written
 // Fewest rows a backward block covers (TY = 256/kBwdMaxTx threads x the
 // smallest unroll any backward kernel uses): bounds the number of partial rows.
-constexpr int kBwdMinUnroll = 2;
+constexpr int kBwdMinUnroll = 4;
 constexpr int kBwdMinRowsPerBlock = kBlockThreads / kBwdMaxTx * kBwdMinUnroll;
 
 struct EwPlan {
@@ -121,64 +121,49 @@ __device__ __forceinline__ void write_colsum_partial(
   }
 }
 
-// Column sum of fp32 partial rows, in one or two launches of the kernel below.
-// out[g, c] = sum of in[p, c] over the rows p of group g (per_group rows each).
-// A block owns 64 columns of one group; its four waves take every fourth row,
-// four rows in flight each, and meet in LDS. The order of the additions is
-// fixed, so the result is deterministic.
+// dbias[c] = sum of the fp32 partial rows in[p, c]. A block of 1024 threads owns
+// 64 columns; its 16 waves take every 16th row with eight rows in flight each
+// and meet in LDS, so even a few hundred partial rows are a handful of
+// dependent steps. The order of the additions is fixed: the result is
+// deterministic.
+constexpr int kFinishThreads = 1024;
+constexpr int kFinishWaves = kFinishThreads / kWave;
+
 template <typename OutT>
-__global__ __launch_bounds__(kBlockThreads) void colsum_reduce_kernel(
+__global__ __launch_bounds__(kFinishThreads) void colsum_finish_kernel(
     OutT *__restrict__ out, const float *__restrict__ in, int64_t nparts,
-    int64_t per_group, int64_t cols) {
-  __shared__ float red[kBlockThreads];
+    int64_t cols) {
+  __shared__ float red[kFinishThreads];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int64_t c = (int64_t)blockIdx.x * kWave + lane;
-  const int64_t p_begin = (int64_t)blockIdx.y * per_group;
-  const int64_t p_end = min(nparts, p_begin + per_group);
-  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  float s[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s[i] = 0.f;
   if (c < cols) {
-    int64_t p = p_begin + wave;
-    for (; p + 3 * kWavesPerBlock < p_end; p += 4 * kWavesPerBlock) {
-      s0 += in[p * cols + c];
-      s1 += in[(p + kWavesPerBlock) * cols + c];
-      s2 += in[(p + 2 * kWavesPerBlock) * cols + c];
-      s3 += in[(p + 3 * kWavesPerBlock) * cols + c];
+    int64_t p = wave;
+    for (; p + 7 * kFinishWaves < nparts; p += 8 * kFinishWaves) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s[i] += in[(p + i * kFinishWaves) * cols + c];
     }
-    for (; p < p_end; p += kWavesPerBlock) s0 += in[p * cols + c];
+    for (; p < nparts; p += kFinishWaves) s[0] += in[p * cols + c];
   }
-  red[threadIdx.x] = (s0 + s1) + (s2 + s3);
+  red[threadIdx.x] = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
   __syncthreads();
   if (wave == 0 && c < cols) {
-    float s = red[lane];
+    float t = red[lane];
 #pragma unroll
-    for (int w = 1; w < kWavesPerBlock; ++w) s += red[w * kWave + lane];
-    out[(int64_t)blockIdx.y * cols + c] = static_cast<OutT>(s);
+    for (int w = 1; w < kFinishWaves; ++w) t += red[w * kWave + lane];
+    out[c] = static_cast<OutT>(t);
   }
 }
 
-constexpr int kColsumGroups = 32;      // rows of the intermediate buffer
-constexpr int kColsumTwoStageMin = 64; // fewer partial rows: one launch
-
-// dbias = column sum of `nparts` partial rows at `partial`. The fp32 buffer
-// holds kColsumGroups more rows after the partials for the intermediate sums.
 template <typename T>
-inline void launch_colsum_finish(T *dbias, float *partial, int64_t nparts,
+inline void launch_colsum_finish(T *dbias, const float *partial, int64_t nparts,
                                  int64_t cols, hipStream_t stream) {
   const unsigned bx = (unsigned)((cols + kWave - 1) / kWave);
-  if (nparts <= kColsumTwoStageMin) {
-    colsum_reduce_kernel<T><<<dim3(bx, 1), dim3(kBlockThreads), 0, stream>>>(
-        dbias, partial, nparts, nparts, cols);
-    return;
-  }
-  float *mid = partial + nparts * cols;
-  const int64_t per_group = (nparts + kColsumGroups - 1) / kColsumGroups;
-  const unsigned groups = (unsigned)((nparts + per_group - 1) / per_group);
-  colsum_reduce_kernel<float>
-      <<<dim3(bx, groups), dim3(kBlockThreads), 0, stream>>>(
-          mid, partial, nparts, per_group, cols);
-  colsum_reduce_kernel<T><<<dim3(bx, 1), dim3(kBlockThreads), 0, stream>>>(
-      dbias, mid, groups, groups, cols);
+  colsum_finish_kernel<T><<<dim3(bx), dim3(kFinishThreads), 0, stream>>>(
+      dbias, partial, nparts, cols);
 }
 
 } // namespace oslo

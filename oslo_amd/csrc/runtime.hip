@@ -65,5 +65,5 @@ extern "C" size_t oslo_colsum_workspace_bytes(int64_t rows, int64_t cols) {
   // than kBwdMinRowsPerBlock rows per block, whatever the dtype and alignment.
   const int64_t parts =
       (rows + oslo::kBwdMinRowsPerBlock - 1) / oslo::kBwdMinRowsPerBlock;
-  return (size_t)(parts + oslo::kColsumGroups) * (size_t)cols * sizeof(float);
+  return (size_t)parts * (size_t)cols * sizeof(float);
 }

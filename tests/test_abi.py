@@ -58,10 +58,10 @@ def test_get_batch_per_block_equals_reference_table(lib):
 def test_workspace_bytes(lib):
     assert lib.oslo_colsum_workspace_bytes(0, 128) == 0
     assert lib.oslo_colsum_workspace_bytes(128, 0) == 0
-    # one partial row per 16 rows plus 32 rows for the second reduction stage
-    assert lib.oslo_colsum_workspace_bytes(1, 8) == (1 + 32) * 8 * 4
-    assert lib.oslo_colsum_workspace_bytes(16384, 16384) == (1024 + 32) * 16384 * 4
-    assert lib.oslo_colsum_workspace_bytes(16385, 10) == (1025 + 32) * 10 * 4
+    # one fp32 partial row per 32 rows
+    assert lib.oslo_colsum_workspace_bytes(1, 8) == 1 * 8 * 4
+    assert lib.oslo_colsum_workspace_bytes(16384, 16384) == 512 * 16384 * 4
+    assert lib.oslo_colsum_workspace_bytes(16385, 10) == 513 * 10 * 4
 
 
 def test_argument_screening_without_a_device(lib):
