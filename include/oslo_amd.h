@@ -198,6 +198,24 @@ int oslo_bias_dropout_add_bwd(void *dx, void *dbias, float *workspace,
                               uint64_t philox_offset, int64_t rows,
                               int64_t cols, int dtype, oslo_stream_t stream);
 
+/* Repeated n-gram blocking (beam search) ------------------------------------ */
+
+/*
+ * For every row and every i in [0, step-n+1]: if tokens[row, i .. i+n-2] equals
+ * the last n-1 tokens tokens[row, step-n+2 .. step], then
+ * lprobs[row, tokens[row, i+n-1]] = -inf. tokens: int64 [rows, max_len] holding
+ * step+1 generated tokens per row; lprobs: fp32 [rows, vocab], updated in
+ * place. Nothing happens while step+1 < n. Token ids outside [0, vocab) are
+ * ignored.
+ * Replaces ngram_repeat_block_forward
+ * (oslo/fused_kernels/bindings/pybind_kernels.cpp:129-157,
+ *  oslo/fused_kernels/fused_ngram_repeat_block.cu:18-75); `rows` is its
+ * bsz * beam_size.
+ */
+int oslo_ngram_repeat_block(float *lprobs, const int64_t *tokens, int64_t rows,
+                            int64_t max_len, int64_t step, int64_t vocab, int n,
+                            oslo_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

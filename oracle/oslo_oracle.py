@@ -24,6 +24,7 @@ root):
 * bias_dropout_add_fwd / _bwd: oslo/fused_kernels_utils.py:259-292
   (F.dropout(x + bias, p, training) + residual) given an explicit keep mask;
 * get_batch_per_block: oslo/fused_kernels/includes/fused_softmax.h:328-340;
+* ngram_banned_tokens: oslo/fused_kernels/fused_ngram_repeat_block.cu:18-49;
 * reference_is_available: oslo/fused_kernels_utils.py:461-479;
 * philox4x32_10 / dropout_keep_mask: no counterpart in the reference (it uses
   torch's generator through F.dropout); they restate the published Philox
@@ -118,6 +119,23 @@ def reference_is_available(is_half, bsz, np_, sq, sk, use_triang_mask):
     if use_triang_mask:
         return sq == sk and (sk <= 64 or sk % 4 == 0) and (bsz * np_) % bpb == 0
     return sq > 1 and sq % bpb == 0
+
+
+def ngram_banned_tokens(tokens, n):
+    """tokens: list of the generated ids of one hypothesis. Returns the set of
+    ids that would complete an n-gram already present: for every i with
+    tokens[i:i+n-1] == tokens[-(n-1):] (or every i, for n == 1), tokens[i+n-1].
+    Follows oslo/fused_kernels/fused_ngram_repeat_block.cu:18-49 (threads
+    0 .. step-n+1 compare their n-1 tokens with the last n-1)."""
+    cur_len = len(tokens)
+    banned = set()
+    if cur_len + 1 < n:
+        return banned
+    last = tokens[cur_len - (n - 1):] if n > 1 else []
+    for i in range(cur_len - n + 1):
+        if tokens[i:i + n - 1] == last:
+            banned.add(tokens[i + n - 1])
+    return banned
 
 
 # ---------------------------------------------------------------------------

@@ -320,6 +320,56 @@ class FusedBiasDropoutResidual(object):
 
 
 # ---------------------------------------------------------------------------
+# repeated n-gram blocking for generation
+# ---------------------------------------------------------------------------
+
+class NGramRepeatBlockFunction(torch.autograd.Function):
+    """oslo/fused_kernels_utils.py:355-363."""
+
+    @staticmethod
+    def forward(ctx, tokens, lprobs, bsz, step, beam_size, no_repeat_ngram_size):
+        return get_custom_kernels().ngram_repeat_block_forward(
+            tokens, lprobs, bsz, step, beam_size, no_repeat_ngram_size
+        )
+
+    def backward(*args):
+        raise NotImplementedError
+
+
+class FusedNoRepeatNGramLogitsProcessor(object):
+    """Logits processor that bans every token that would repeat an n-gram
+    (oslo/fused_kernels_utils.py:482-521). Callable as
+    ``processor(input_ids, scores)`` like a HuggingFace LogitsProcessor. The
+    reference computes the bans on the host for CPU tensors; here only device
+    tensors are accepted."""
+
+    def __init__(self, ngram_size: int, batch_size: int, beam_size: int):
+        if not isinstance(ngram_size, int) or ngram_size <= 0:
+            raise ValueError(
+                f"`ngram_size` has to be a strictly positive integer, but is {ngram_size}"
+            )
+        self.ngram_size = ngram_size
+        self.batch_size = batch_size
+        self.beam_size = beam_size
+
+    def __call__(self, input_ids, scores):
+        if not (input_ids.is_cuda and scores.is_cuda):
+            raise RuntimeError(
+                "FusedNoRepeatNGramLogitsProcessor: expected tensors on a ROCm device "
+                "(this library has no CPU path)"
+            )
+        cur_len = input_ids.shape[-1]
+        return NGramRepeatBlockFunction.apply(
+            input_ids.contiguous(),
+            scores.float().contiguous(),
+            self.batch_size,
+            cur_len - 1,
+            self.beam_size,
+            self.ngram_size,
+        )
+
+
+# ---------------------------------------------------------------------------
 # model.fuse()
 # ---------------------------------------------------------------------------
 

@@ -109,6 +109,28 @@ def scaled_masked_softmax_backward(output_grads, softmax_results, scale_factor):
     return g
 
 
+def ngram_repeat_block_forward(tokens, lprobs, bsz, step, beam_size, no_repeat_ngram_size):
+    """oslo/fused_kernels/bindings/pybind_kernels.cpp:143-157: tokens int64
+    [bsz*beam_size, len], lprobs fp32 [bsz*beam_size, vocab]; bans in place and
+    returns lprobs."""
+    _device_tensor(tokens, "tokens")
+    _device_tensor(lprobs, "lprobs")
+    _require(tokens.is_contiguous(), "tokens must be contiguous")
+    _require(lprobs.is_contiguous(), "lprobs must be contiguous")
+    _require(tokens.dtype == torch.int64, "tokens must be int64")
+    _require(lprobs.dtype == torch.float32, "lprobs must be float32")
+    _require(tokens.dim() == 2 and lprobs.dim() == 2, "expected 2D tensors")
+    assert bsz > 0 and step >= 0 and beam_size > 0 and no_repeat_ngram_size > 0
+    rows = bsz * beam_size
+    _require(tokens.shape[0] == rows and lprobs.shape[0] == rows,
+             "tokens and lprobs must have bsz * beam_size rows")
+    with torch.cuda.device(lprobs.device):
+        _lib.check(_lib.load().oslo_ngram_repeat_block(
+            _ptr(lprobs), _ptr(tokens), rows, tokens.shape[1], int(step), lprobs.shape[1],
+            int(no_repeat_ngram_size), _stream(lprobs)))
+    return lprobs
+
+
 # ---------------------------------------------------------------------------
 # wider entry points
 # ---------------------------------------------------------------------------
