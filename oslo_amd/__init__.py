@@ -9,7 +9,9 @@ from .fused_kernels_utils import (  # noqa: F401
     FusedBiasDropoutResidual,
     FusedBiasGeLU,
     FusedKernelMixin,
+    FusedNoRepeatNGramLogitsProcessor,
     FusedScaleMaskSoftmax,
+    FusedScaleMaskSoftmaxDropout,
     ScaledMaskedSoftmaxFunction,
     ScaledUpperTriangMaskedSoftmaxFunction,
     get_custom_kernels,

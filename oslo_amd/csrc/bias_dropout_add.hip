@@ -5,31 +5,11 @@
 // (seed, offset, element index) with Philox4x32-10, so the backward reads only
 // the incoming gradient.
 
+#include "dropout.hpp"
 #include "elementwise.hpp"
-#include "philox.h"
 
 namespace oslo {
 namespace {
-
-// keep flags of VEC consecutive elements starting at flat index i0 (a multiple
-// of VEC when VEC is 4 or 8; anything when VEC is 1).
-template <int VEC>
-__device__ __forceinline__ void keep_flags(bool (&keep)[VEC], uint64_t seed,
-                                           uint64_t offset, uint64_t i0,
-                                           uint32_t threshold) {
-  if constexpr (VEC == 1) {
-    const Philox4 d = dropout_draw(seed, offset, i0 >> 2);
-    keep[0] = d.w[i0 & 3] >= threshold;
-  } else {
-    static_assert(VEC % 4 == 0, "vector paths draw whole groups of four");
-#pragma unroll
-    for (int q = 0; q < VEC / 4; ++q) {
-      const Philox4 d = dropout_draw(seed, offset, (i0 >> 2) + q);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) keep[4 * q + j] = d.w[j] >= threshold;
-    }
-  }
-}
 
 template <typename T, int VEC, int U, bool DROP, bool HAS_BIAS, bool HAS_RES>
 __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_fwd_kernel(
@@ -118,13 +98,6 @@ __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_bwd_kernel(
     write_colsum_partial<VEC>(acc, partial, cols, pos, col_ok);
 }
 
-struct DropArgs {
-  float keep_scale;
-  uint32_t threshold;
-  uint64_t seed, offset;
-  bool drop;
-};
-
 constexpr int kDropBwdUnroll = 8;
 static_assert(kDropBwdUnroll >= kBwdMinUnroll, "workspace bound");
 
@@ -178,18 +151,6 @@ int launch_bwd(T *dx, T *dbias, float *ws, const T *g, const DropArgs &a,
   return check_launch("bias_dropout_add_bwd(dbias)");
 }
 
-int make_args(const char *name, float p, uint64_t seed, uint64_t offset,
-              DropArgs *a) {
-  if (!(p >= 0.0f) || !(p < 1.0f))
-    return fail(OSLO_E_BAD_ARG, "%s: p = %g is outside [0, 1)", name, (double)p);
-  a->drop = p > 0.0f;
-  a->keep_scale = (float)(1.0 / (1.0 - (double)p));
-  a->threshold = dropout_threshold(p);
-  a->seed = seed;
-  a->offset = offset;
-  return OSLO_OK;
-}
-
 } // namespace
 } // namespace oslo
 
@@ -203,7 +164,7 @@ extern "C" int oslo_bias_dropout_add_fwd(void *out, const void *x,
   if (rows < 0 || cols < 0)
     return fail(OSLO_E_BAD_ARG, "bias_dropout_add_fwd: negative size");
   DropArgs a;
-  int s = make_args("bias_dropout_add_fwd", p, philox_seed, philox_offset, &a);
+  int s = make_drop_args("bias_dropout_add_fwd", p, philox_seed, philox_offset, &a);
   if (s != OSLO_OK) return s;
   if (rows == 0 || cols == 0) return OSLO_OK;
   if (!out || !x) return fail(OSLO_E_BAD_ARG, "bias_dropout_add_fwd: null tensor");
@@ -232,7 +193,7 @@ extern "C" int oslo_bias_dropout_add_bwd(void *dx, void *dbias,
   if (rows < 0 || cols < 0)
     return fail(OSLO_E_BAD_ARG, "bias_dropout_add_bwd: negative size");
   DropArgs a;
-  int s = make_args("bias_dropout_add_bwd", p, philox_seed, philox_offset, &a);
+  int s = make_drop_args("bias_dropout_add_bwd", p, philox_seed, philox_offset, &a);
   if (s != OSLO_OK) return s;
   if (cols == 0) return OSLO_OK;
   if (dbias && !workspace && rows > 0)

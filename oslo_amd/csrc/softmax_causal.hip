@@ -9,6 +9,7 @@
 // for the load), and the zeros of the upper triangle are written by the same
 // 128-bit stores as the probabilities.
 
+#include "dropout.hpp"
 #include "softmax.hpp"
 
 namespace oslo {
@@ -17,10 +18,13 @@ namespace {
 // ---------------------------------------------------------------------------
 // Register-resident path: rows up to kSoftmaxMaxCols, S a multiple of VEC.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC, int NCHUNK, int WPR, bool HAS_PAD>
+// DROP: also writes yd = y * keep / (1-p), the probabilities after attention
+// dropout; the keep flag of element (row, k) is drawn for the flat index
+// row*S + k of the [batch*heads*S, S] tensor.
+template <typename T, int VEC, int NCHUNK, int WPR, bool HAS_PAD, bool DROP>
 __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
-    T *y, const T *x, const float *__restrict__ pad, float scale, int S,
-    int heads, RowMap map) {
+    T *y, T *yd, const T *x, const float *__restrict__ pad, float scale, int S,
+    int heads, RowMap map, DropArgs drop) {
   using Tile = RowTile<VEC, NCHUNK, WPR>;
   __shared__ float s_max[kWavesPerBlock];
   __shared__ float s_sum[kWavesPerBlock];
@@ -119,19 +123,32 @@ __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
 
   if (!live) return;
   const BufRsrc yrs = make_rsrc(yr, (uint32_t)S * (uint32_t)sizeof(T));
+  const BufRsrc ydrs = make_rsrc(DROP ? yd + row * S : yr, (uint32_t)S * (uint32_t)sizeof(T));
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
+    const uint32_t off = (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T);
     float o[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) o[j] = v[c][j] * inv;
-    buffer_store_f32<T, VEC, kStreamOut>(
-        yrs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T), o);
+    buffer_store_f32<T, VEC, kStreamOut>(yrs, off, o);
+    if constexpr (DROP) {
+      if (Tile::col(c, sub, 0) <= r) { // wave-uniform; above the diagonal o is 0 already
+        bool keep[VEC];
+        keep_flags<VEC>(keep, drop.seed, drop.offset,
+                        (uint64_t)row * S + Tile::col(c, sub, lane), drop.threshold);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] = keep[j] ? o[j] * drop.keep_scale : 0.f;
+      }
+      buffer_store_f32<T, VEC, kStreamOut>(ydrs, off, o);
+    }
   }
 }
 
-template <typename T, int VEC, int NCHUNK, int WPR>
+// DROP: g is the gradient of the probabilities after dropout; the keep mask is
+// regenerated and g' = g * keep / (1-p) takes g's place.
+template <typename T, int VEC, int NCHUNK, int WPR, bool DROP>
 __global__ __launch_bounds__(kBlockThreads) void causal_bwd_kernel(
-    T *dx, const T *g, const T *y, float scale, int S, RowMap map) {
+    T *dx, const T *g, const T *y, float scale, int S, RowMap map, DropArgs drop) {
   using Tile = RowTile<VEC, NCHUNK, WPR>;
   __shared__ float s_sum[kWavesPerBlock];
 
@@ -177,6 +194,12 @@ __global__ __launch_bounds__(kBlockThreads) void causal_bwd_kernel(
     float tg[VEC];
     raw_to_f32<T, VEC>(tg, graw[c]);
     raw_to_f32<T, VEC>(yy[c], yraw[c]);
+    if constexpr (DROP) {
+      bool keep[VEC];
+      keep_flags<VEC>(keep, drop.seed, drop.offset, (uint64_t)row * S + k0, drop.threshold);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) tg[j] = keep[j] ? tg[j] * drop.keep_scale : 0.f;
+    }
     if (first + Tile::kSpan - 1 > r) { // the chunk the diagonal crosses
 #pragma unroll
       for (int j = 0; j < VEC; ++j)
@@ -210,8 +233,8 @@ __global__ __launch_bounds__(kBlockThreads) void causal_bwd_kernel(
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(kBlockThreads) void causal_fwd_anyshape_kernel(
-    T *y, const T *x, const float *__restrict__ pad, float scale, int S,
-    int heads, int64_t total_rows) {
+    T *y, T *yd, const T *x, const float *__restrict__ pad, float scale, int S,
+    int heads, int64_t total_rows, DropArgs drop) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
   if (row >= total_rows) return; // whole wave leaves; no barriers below
@@ -237,12 +260,17 @@ __global__ __launch_bounds__(kBlockThreads) void causal_fwd_anyshape_kernel(
   for (int k = lane; k < S; k += kWave) {
     const float o = k <= r ? exp_shifted(score(k), m) * inv : 0.f;
     yr[k] = static_cast<T>(o);
+    if (drop.drop) {
+      const bool keep = keep_one(drop.seed, drop.offset, (uint64_t)row * S + k, drop.threshold);
+      yd[row * S + k] = static_cast<T>(keep ? o * drop.keep_scale : 0.f);
+    }
   }
 }
 
 template <typename T>
 __global__ __launch_bounds__(kBlockThreads) void causal_bwd_anyshape_kernel(
-    T *dx, const T *g, const T *y, float scale, int S, int64_t total_rows) {
+    T *dx, const T *g, const T *y, float scale, int S, int64_t total_rows,
+    DropArgs drop) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
   if (row >= total_rows) return;
@@ -250,33 +278,39 @@ __global__ __launch_bounds__(kBlockThreads) void causal_bwd_anyshape_kernel(
   const T *gr = g + row * S;
   const T *yr = y + row * S;
   T *dr = dx + row * S;
+  auto grad = [&](int k) { // gradient of the probabilities before dropout
+    float gk = static_cast<float>(gr[k]);
+    if (drop.drop)
+      gk = keep_one(drop.seed, drop.offset, (uint64_t)row * S + k, drop.threshold)
+               ? gk * drop.keep_scale : 0.f;
+    return gk;
+  };
   float sum = 0.f;
-  for (int k = lane; k <= r; k += kWave)
-    sum += static_cast<float>(gr[k]) * static_cast<float>(yr[k]);
+  for (int k = lane; k <= r; k += kWave) sum += grad(k) * static_cast<float>(yr[k]);
   sum = wave_allreduce(sum, OpAdd());
   for (int k = lane; k < S; k += kWave) {
     float o = 0.f;
     if (k <= r) {
       const float yk = static_cast<float>(yr[k]);
-      o = scale * (static_cast<float>(gr[k]) * yk - yk * sum);
+      o = scale * (grad(k) * yk - yk * sum);
     }
     dr[k] = static_cast<T>(o);
   }
 }
 
 template <typename T>
-int launch_causal_fwd(T *y, const T *x, const float *pad, float scale,
+int launch_causal_fwd(T *y, T *yd, const T *x, const float *pad, float scale,
                       int64_t batch, int64_t heads, int64_t S,
-                      hipStream_t stream) {
+                      const DropArgs &drop, hipStream_t stream) {
   constexpr int VEC = Io<T>::kVec;
   const int64_t total_rows = batch * heads * S;
   const bool vector_ok = S % VEC == 0 && aligned16(x) && aligned16(y) &&
-                         (pad == nullptr || aligned16(pad));
+                         aligned16(yd) && (pad == nullptr || aligned16(pad));
   if (!vector_ok) {
     const int64_t blocks = (total_rows + kWavesPerBlock - 1) / kWavesPerBlock;
     causal_fwd_anyshape_kernel<T><<<dim3((unsigned)blocks), dim3(kBlockThreads),
-                                    0, stream>>>(y, x, pad, scale, (int)S,
-                                                 (int)heads, total_rows);
+                                    0, stream>>>(y, yd, x, pad, scale, (int)S,
+                                                 (int)heads, total_rows, drop);
     return check_launch("softmax_causal_fwd");
   }
   dispatch_row_tile<VEC>(S, [&]<int NCHUNK, int WPR>() {
@@ -284,21 +318,25 @@ int launch_causal_fwd(T *y, const T *x, const float *pad, float scale,
     const RowMap map = make_row_map(total_rows, rpb, S * (int64_t)sizeof(T), true);
     const dim3 grid((unsigned)(map.blocks_per_xcd * kXcds));
     const unsigned lds = occupancy_pad_bytes(false, S * (int64_t)sizeof(T));
-    if (pad)
-      causal_fwd_kernel<T, VEC, NCHUNK, WPR, true>
+    auto go = [&]<bool HAS_PAD, bool DROP>() {
+      causal_fwd_kernel<T, VEC, NCHUNK, WPR, HAS_PAD, DROP>
           <<<grid, dim3(kBlockThreads), lds, stream>>>(
-              y, x, pad, scale, (int)S, (int)heads, map);
-    else
-      causal_fwd_kernel<T, VEC, NCHUNK, WPR, false>
-          <<<grid, dim3(kBlockThreads), lds, stream>>>(
-              y, x, nullptr, scale, (int)S, (int)heads, map);
+              y, yd, x, pad, scale, (int)S, (int)heads, map, drop);
+    };
+    if (drop.drop) {
+      if (pad) go.template operator()<true, true>();
+      else go.template operator()<false, true>();
+    } else {
+      if (pad) go.template operator()<true, false>();
+      else go.template operator()<false, false>();
+    }
   });
   return check_launch("softmax_causal_fwd");
 }
 
 template <typename T>
 int launch_causal_bwd(T *dx, const T *g, const T *y, float scale, int64_t bh,
-                      int64_t S, hipStream_t stream) {
+                      int64_t S, const DropArgs &drop, hipStream_t stream) {
   constexpr int VEC = Io<T>::kVec;
   const int64_t total_rows = bh * S;
   const bool vector_ok =
@@ -307,16 +345,20 @@ int launch_causal_bwd(T *dx, const T *g, const T *y, float scale, int64_t bh,
     const int64_t blocks = (total_rows + kWavesPerBlock - 1) / kWavesPerBlock;
     causal_bwd_anyshape_kernel<T><<<dim3((unsigned)blocks), dim3(kBlockThreads),
                                     0, stream>>>(dx, g, y, scale, (int)S,
-                                                 total_rows);
+                                                 total_rows, drop);
     return check_launch("softmax_causal_bwd");
   }
   dispatch_row_tile<VEC>(S, [&]<int NCHUNK, int WPR>() {
     constexpr int rpb = RowTile<VEC, NCHUNK, WPR>::kRowsPerBlock;
     const RowMap map = make_row_map(total_rows, rpb, S * (int64_t)sizeof(T), true);
-    causal_bwd_kernel<T, VEC, NCHUNK, WPR>
-        <<<dim3((unsigned)(map.blocks_per_xcd * kXcds)), dim3(kBlockThreads),
-           occupancy_pad_bytes(true, S * (int64_t)sizeof(T)), stream>>>(
-            dx, g, y, scale, (int)S, map);
+    const dim3 grid((unsigned)(map.blocks_per_xcd * kXcds));
+    const unsigned lds = occupancy_pad_bytes(true, S * (int64_t)sizeof(T));
+    if (drop.drop)
+      causal_bwd_kernel<T, VEC, NCHUNK, WPR, true>
+          <<<grid, dim3(kBlockThreads), lds, stream>>>(dx, g, y, scale, (int)S, map, drop);
+    else
+      causal_bwd_kernel<T, VEC, NCHUNK, WPR, false>
+          <<<grid, dim3(kBlockThreads), lds, stream>>>(dx, g, y, scale, (int)S, map, drop);
   });
   return check_launch("softmax_causal_bwd");
 }
@@ -336,34 +378,81 @@ int screen(const char *name, int64_t rows, int64_t S) {
 } // namespace
 } // namespace oslo
 
+namespace {
+int causal_fwd_entry(const char *name, void *y, void *yd, const void *x,
+                     const float *pad_add, float scale, const oslo::DropArgs &drop,
+                     int64_t batch, int64_t heads, int64_t S, int dtype,
+                     oslo_stream_t stream) {
+  using namespace oslo;
+  if (batch < 0 || heads < 0) return fail(OSLO_E_BAD_ARG, "%s: negative size", name);
+  const int s = screen(name, batch * heads, S);
+  if (s != 0) return s < 0 ? s : OSLO_OK;
+  if (!x || !y || (drop.drop && !yd)) return fail(OSLO_E_BAD_ARG, "%s: null tensor", name);
+  OSLO_DISPATCH_DTYPE(dtype, return launch_causal_fwd<T>(
+                                 static_cast<T *>(y), static_cast<T *>(yd),
+                                 static_cast<const T *>(x), pad_add, scale, batch,
+                                 heads, S, drop, static_cast<hipStream_t>(stream)));
+  return OSLO_OK;
+}
+
+int causal_bwd_entry(const char *name, void *dx, const void *g, const void *y,
+                     float scale, const oslo::DropArgs &drop, int64_t bh, int64_t S,
+                     int dtype, oslo_stream_t stream) {
+  using namespace oslo;
+  const int s = screen(name, bh, S);
+  if (s != 0) return s < 0 ? s : OSLO_OK;
+  if (!dx || !g || !y) return fail(OSLO_E_BAD_ARG, "%s: null tensor", name);
+  OSLO_DISPATCH_DTYPE(dtype, return launch_causal_bwd<T>(
+                                 static_cast<T *>(dx), static_cast<const T *>(g),
+                                 static_cast<const T *>(y), scale, bh, S, drop,
+                                 static_cast<hipStream_t>(stream)));
+  return OSLO_OK;
+}
+} // namespace
+
 extern "C" int oslo_softmax_causal_fwd(void *y, const void *x,
                                        const float *pad_add, float scale,
                                        int64_t batch, int64_t heads, int64_t S,
                                        int dtype, oslo_stream_t stream) {
-  using namespace oslo;
-  if (batch < 0 || heads < 0)
-    return fail(OSLO_E_BAD_ARG, "softmax_causal_fwd: negative size");
-  const int s = screen("softmax_causal_fwd", batch * heads, S);
-  if (s != 0) return s < 0 ? s : OSLO_OK;
-  if (!x || !y) return fail(OSLO_E_BAD_ARG, "softmax_causal_fwd: null tensor");
-  OSLO_DISPATCH_DTYPE(dtype, return launch_causal_fwd<T>(
-                                 static_cast<T *>(y), static_cast<const T *>(x),
-                                 pad_add, scale, batch, heads, S,
-                                 static_cast<hipStream_t>(stream)));
-  return OSLO_OK;
+  oslo::DropArgs none{};
+  return causal_fwd_entry("softmax_causal_fwd", y, nullptr, x, pad_add, scale, none,
+                          batch, heads, S, dtype, stream);
 }
 
 extern "C" int oslo_softmax_causal_bwd(void *dx, const void *g, const void *y,
                                        float scale, int64_t bh, int64_t S,
                                        int dtype, oslo_stream_t stream) {
-  using namespace oslo;
-  const int s = screen("softmax_causal_bwd", bh, S);
-  if (s != 0) return s < 0 ? s : OSLO_OK;
-  if (!dx || !g || !y)
-    return fail(OSLO_E_BAD_ARG, "softmax_causal_bwd: null tensor");
-  OSLO_DISPATCH_DTYPE(dtype, return launch_causal_bwd<T>(
-                                 static_cast<T *>(dx), static_cast<const T *>(g),
-                                 static_cast<const T *>(y), scale, bh, S,
-                                 static_cast<hipStream_t>(stream)));
-  return OSLO_OK;
+  oslo::DropArgs none{};
+  return causal_bwd_entry("softmax_causal_bwd", dx, g, y, scale, none, bh, S, dtype, stream);
+}
+
+extern "C" int oslo_softmax_causal_dropout_fwd(void *yd, void *y, const void *x,
+                                               const float *pad_add, float scale,
+                                               float p, uint64_t philox_seed,
+                                               uint64_t philox_offset, int64_t batch,
+                                               int64_t heads, int64_t S, int dtype,
+                                               oslo_stream_t stream) {
+  oslo::DropArgs drop;
+  const int s = oslo::make_drop_args("softmax_causal_dropout_fwd", p, philox_seed,
+                                     philox_offset, &drop);
+  if (s != OSLO_OK) return s;
+  if (!drop.drop && yd && yd != y)
+    return oslo::fail(OSLO_E_BAD_ARG,
+                      "softmax_causal_dropout_fwd: with p == 0 pass yd == y or NULL");
+  return causal_fwd_entry("softmax_causal_dropout_fwd", y, yd, x, pad_add, scale, drop,
+                          batch, heads, S, dtype, stream);
+}
+
+extern "C" int oslo_softmax_causal_dropout_bwd(void *dx, const void *g, const void *y,
+                                               float scale, float p,
+                                               uint64_t philox_seed,
+                                               uint64_t philox_offset, int64_t bh,
+                                               int64_t S, int dtype,
+                                               oslo_stream_t stream) {
+  oslo::DropArgs drop;
+  const int s = oslo::make_drop_args("softmax_causal_dropout_bwd", p, philox_seed,
+                                     philox_offset, &drop);
+  if (s != OSLO_OK) return s;
+  return causal_bwd_entry("softmax_causal_dropout_bwd", dx, g, y, scale, drop, bh, S,
+                          dtype, stream);
 }

@@ -127,6 +127,27 @@ class _KeyMaskedSoftmax(torch.autograd.Function):
         return dx, None, None
 
 
+class _CausalSoftmaxDropout(torch.autograd.Function):
+    """Causal softmax of [B,H,S,S] scores followed by dropout of the
+    probabilities, one kernel each way; the keep mask is regenerated in the
+    backward from the generator state taken in the forward."""
+
+    @staticmethod
+    def forward(ctx, inputs, pad_add, scale, p):
+        seed, offset = _next_philox(inputs.device)
+        yd, y = get_custom_kernels().causal_softmax_dropout_forward(inputs, pad_add, scale, p, seed, offset)
+        ctx.save_for_backward(y)
+        ctx.args = (float(scale), float(p), seed, offset)
+        return yd
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        (y,) = ctx.saved_tensors
+        scale, p, seed, offset = ctx.args
+        dx = get_custom_kernels().causal_softmax_dropout_backward(output_grads, y, scale, p, seed, offset)
+        return dx, None, None, None
+
+
 def _key_mask_bytes(pad_mask):
     """Any mask form -> bool, True = masked. Float masks follow the reference's
     ``.bool()`` (oslo/fused_kernels_utils.py:453-457): non-zero means masked."""
@@ -192,6 +213,33 @@ class FusedScaleMaskSoftmax(object):
         if use_triang_mask:
             return sq == sk
         return True
+
+
+class FusedScaleMaskSoftmaxDropout(object):
+    """
+    Kernel fusion function: Scale + Mask + Softmax + attention Dropout
+
+    Before fusion: ... -> (Scale + Mask + Softmax) -> Dropout -> Matmul (Score * V) -> ...
+    After fusion: ... -> (Scale + Mask + Softmax + Dropout) -> Matmul (Score * V) -> ...
+
+    Not in the reference, whose fused attention runs nn.Dropout as a separate
+    pass over the [B,H,S,S] probabilities (oslo/models/gptj/modeling_gptj.py
+    :947-948). ``apply`` has FusedScaleMaskSoftmax.apply's arguments plus the
+    dropout module's ``p`` and ``training``; causal scores in training with
+    0 < p < 1 take the fused kernel, everything else is the softmax operator
+    followed by torch's dropout.
+    """
+
+    @staticmethod
+    def apply(input, pad_mask, scale, use_triang_mask, drop_prop, training):
+        p = float(drop_prop) if training else 0.0
+        if not (use_triang_mask and 0.0 < p < 1.0):
+            y = FusedScaleMaskSoftmax.apply(input, pad_mask, scale, use_triang_mask)
+            return torch.nn.functional.dropout(y, p=p, training=training)
+        bsz, np, sq, sk = input.size()
+        scale = scale if scale is not None else 1.0
+        pad_add = None if pad_mask is None else _pad_additive_f32(pad_mask, bsz, sk)
+        return _CausalSoftmaxDropout.apply(input, pad_add, scale, p)
 
 
 # ---------------------------------------------------------------------------

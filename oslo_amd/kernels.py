@@ -155,6 +155,50 @@ def causal_softmax_forward(input, pad_add, scale_factor):
     return y
 
 
+def causal_softmax_dropout_forward(input, pad_add, scale_factor, p, seed, offset):
+    """Causal softmax + attention dropout in one pass. Returns (probs_after_
+    dropout, probs); the second is what the backward needs."""
+    _device_tensor(input, "input")
+    _require(input.dim() == 4, "expected 4D tensor")
+    code = _dtype_code(input, "input")
+    b, h, sq, sk = input.shape
+    _require(sq == sk, "causal softmax needs square score matrices")
+    x = input.contiguous()
+    if pad_add is not None:
+        _device_tensor(pad_add, "pad_add")
+        _require(pad_add.dtype == torch.float32 and tuple(pad_add.shape) == (b, sk),
+                 "pad_add must be fp32 [batch, S]")
+        pad_add = pad_add.contiguous()
+    y = torch.empty_like(x, requires_grad=False)
+    yd = torch.empty_like(x, requires_grad=False) if p > 0 else y
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().oslo_softmax_causal_dropout_fwd(
+            _ptr(yd), _ptr(y), _ptr(x), _ptr(pad_add), float(scale_factor), float(p),
+            int(seed), int(offset), b, h, sk, code, _stream(x)))
+    return yd, y
+
+
+def causal_softmax_dropout_backward(output_grads, softmax_results, scale_factor, p, seed, offset):
+    """output_grads: gradient of the probabilities after dropout, [B,H,S,S];
+    overwritten with the input gradient when contiguous, like the plain
+    backward."""
+    _device_tensor(output_grads, "output_grads")
+    _device_tensor(softmax_results, "softmax_results")
+    code = _dtype_code(output_grads, "output_grads")
+    _require(softmax_results.dtype == output_grads.dtype and softmax_results.shape == output_grads.shape,
+             "output_grads and softmax_results differ in dtype or shape")
+    _require(output_grads.dim() == 4 and output_grads.shape[-1] == output_grads.shape[-2],
+             "expected [B,H,S,S]")
+    b, h, s, _ = output_grads.shape
+    g = output_grads.contiguous()
+    y = softmax_results.contiguous()
+    with torch.cuda.device(g.device):
+        _lib.check(_lib.load().oslo_softmax_causal_dropout_bwd(
+            _ptr(g), _ptr(g), _ptr(y), float(scale_factor), float(p), int(seed), int(offset),
+            b * h, s, code, _stream(g)))
+    return g
+
+
 def masked_softmax_forward(input, mask, scale_factor, mask_mode=MASK_ADD):
     """input [B,H,Sq,Sk]; mask None or bool/uint8 [B or 1, 1, Sq or 1, Sk]
     (size-1 dimensions are broadcast by stride, not copied)."""

@@ -13,7 +13,8 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax,
+                                 FusedScaleMaskSoftmaxDropout)
 from .modeling_utils import (ACT2FN, Conv1D, LayerPolicy, PreTrainedModel, additive_attention_mask,
                              causal_lm_loss)
 
@@ -138,13 +139,16 @@ class GPT2Attention(nn.Module):
 
 
 class FusedGPT2Attention(GPT2Attention):
-    """oslo/models/gpt2/modeling_gpt2.py:1434-1542. Like the reference, the
-    fused path applies no attention-probability dropout."""
+    """oslo/models/gpt2/modeling_gpt2.py:1434-1542. The reference's fused
+    attention leaves out attn_dropout, which its unfused attention applies
+    (:222); here it is applied, inside the softmax kernel, so that fused and
+    unfused training agree."""
 
     def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
         w = torch.matmul(query, key.transpose(-1, -2))
-        w = FusedScaleMaskSoftmax.apply(w, pad_mask=attention_mask, scale=self._attention_scale(value),
-                                        use_triang_mask=not self.is_cross_attention)
+        w = FusedScaleMaskSoftmaxDropout.apply(w, attention_mask, self._attention_scale(value),
+                                               not self.is_cross_attention,
+                                               self.attn_dropout.p, self.training)
         if head_mask is not None:
             w = w * head_mask
         return torch.matmul(w, value), w

@@ -15,7 +15,8 @@ from typing import List, Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax,
+                                 FusedScaleMaskSoftmaxDropout)
 from .modeling_utils import ACT2FN, LayerPolicy, PreTrainedModel, additive_attention_mask, causal_lm_loss
 
 
@@ -110,8 +111,10 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
 
     def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
         w = torch.matmul(query, key.transpose(-1, -2))
-        w = FusedScaleMaskSoftmax.apply(w, pad_mask=attention_mask, scale=None, use_triang_mask=True)
-        w = self.attn_dropout(w.to(value.dtype))
+        # softmax and attn_dropout in one kernel (the reference runs nn.Dropout
+        # as a second pass over the probabilities)
+        w = FusedScaleMaskSoftmaxDropout.apply(w, attention_mask, None, True,
+                                               self.attn_dropout.p, self.training).to(value.dtype)
         if head_mask is not None:
             w = w * head_mask
         return torch.matmul(w, value), w

@@ -18,7 +18,8 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax,
+                                 FusedScaleMaskSoftmaxDropout)
 from .modeling_utils import ACT2FN, LayerPolicy, PreTrainedModel, additive_attention_mask, causal_lm_loss
 
 
@@ -143,9 +144,10 @@ class FusedGPTJAttention(GPTJAttention):
 
     def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
         w = torch.matmul(query, key.transpose(-1, -2))
-        w = FusedScaleMaskSoftmax.apply(w, pad_mask=attention_mask, scale=1.0 / self.scale_attn,
-                                        use_triang_mask=True)
-        w = self.attn_dropout(w.to(value.dtype))
+        # softmax and attn_dropout in one kernel (the reference runs nn.Dropout
+        # as a second pass over the probabilities)
+        w = FusedScaleMaskSoftmaxDropout.apply(w, attention_mask, 1.0 / self.scale_attn, True,
+                                               self.attn_dropout.p, self.training).to(value.dtype)
         if head_mask is not None:
             w = w * head_mask
         return torch.matmul(w, value), w

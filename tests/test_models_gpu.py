@@ -148,3 +148,40 @@ def test_bias_gelu_and_dropout_autograd():
     assert np.abs(f32(gx) - orc.bias_dropout_add_bwd(f32(go), 0.25, keep)[0]).max() <= 1e-6
     # p = 1 drops everything, like F.dropout
     assert torch.count_nonzero(FusedBiasDropout.apply(x, bias, True, 1.0)) == 0
+
+
+def test_fused_attention_dropout_operator_and_training_step():
+    from oslo_amd import FusedScaleMaskSoftmaxDropout
+
+    torch.manual_seed(5)
+    b, h, s, p = 2, 3, 136, 0.2
+    x = torch.randn(b, h, s, s, device=DEV, requires_grad=True)
+    go = torch.randn(b, h, s, s, device=DEV)
+    gen = torch.cuda.default_generators[0]
+    seed, off0 = gen.initial_seed(), gen.get_offset()
+    yd = FusedScaleMaskSoftmaxDropout.apply(x, None, 0.3, True, p, True)
+    assert gen.get_offset() == off0 + fku.PHILOX_WORDS_PER_CALL
+    keep = torch.from_numpy(orc.dropout_keep_mask(seed, off0, x.numel(), p).reshape(b, h, s, s)).to(DEV)
+    causal = torch.tril(torch.ones(s, s, dtype=torch.bool, device=DEV))
+    y = torch.softmax((x * 0.3).masked_fill(~causal, float("-inf")), -1)
+    want = y * keep / (1 - p)
+    (gx_want,) = torch.autograd.grad(want, x, go)
+    (gx,) = torch.autograd.grad(yd, x, go.clone())
+    assert (yd - want).abs().max().item() <= 1e-6 and (gx - gx_want).abs().max().item() <= 1e-6
+    # eval or p == 0: the plain softmax operator
+    assert torch.equal(FusedScaleMaskSoftmaxDropout.apply(x, None, 0.3, True, p, False),
+                       FusedScaleMaskSoftmax.apply(x, None, 0.3, True))
+    # a fused model with every dropout on trains: finite loss and gradients, reproducible from the seed
+    cfg = GPTJConfig(vocab_size=512, n_positions=128, n_embd=128, n_layer=2, n_head=4, rotary_dim=16,
+                     attn_pdrop=0.1, resid_pdrop=0.1, embd_pdrop=0.0)
+    m = GPTJForCausalLM(cfg).to(DEV).train().fuse()
+    ids = torch.randint(0, 512, (2, 64), device=DEV)
+    losses = []
+    for _ in range(2):
+        torch.manual_seed(9)
+        m.zero_grad()
+        loss = m(ids, labels=ids)["loss"]
+        loss.backward()
+        losses.append(loss.item())
+        assert all(torch.isfinite(q.grad).all() for q in m.parameters() if q.grad is not None)
+    assert losses[0] == losses[1]

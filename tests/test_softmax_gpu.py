@@ -193,3 +193,41 @@ def test_causal_full_size_properties(dtype):
     dx = kernels.scaled_upper_triang_masked_softmax_backward(go, y.view(-1, s, s), 0.125)
     assert_close(dx[77], want, dtype, "bwd slab 77")
     assert torch.count_nonzero(torch.triu(dx[::9], 1)) == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("s", [5, 64, 520, 1024, 2048, 2050, 4096])
+@pytest.mark.parametrize("with_pad", [False, True], ids=["nopad", "pad"])
+def test_causal_softmax_with_fused_dropout(s, dtype, with_pad):
+    """Softmax + attention dropout in one pass: the probabilities are the plain
+    kernel's, the dropped output is y*keep/(1-p) with the oracle's Philox mask
+    bit for bit, and the backward regenerates the same mask."""
+    b, h = (2, 2) if s <= 2048 else (1, 1)
+    p, seed, offset = 0.1, 4321, 12
+    x = randn((b, h, s, s), dtype, seed=s, std=8.0)
+    pad = None
+    if with_pad:
+        lens = torch.randint(1, s + 1, (b,), generator=torch.Generator().manual_seed(2))
+        pad = torch.where(torch.arange(s)[None, :] < lens[:, None], 0.0, -10000.0).float()
+    want_y = orc.softmax_causal(f32(x), 0.125, None if pad is None else pad.numpy())
+    keep = orc.dropout_keep_mask(seed, offset, b * h * s * s, p).reshape(b, h, s, s)
+    ks = np.float32(1.0 / (1.0 - float(np.float32(p))))
+    yd, y = kernels.causal_softmax_dropout_forward(x.to(DEV), None if pad is None else pad.to(DEV),
+                                                   0.125, p, seed, offset)
+    plain = kernels.causal_softmax_forward(x.to(DEV), None if pad is None else pad.to(DEV), 0.125)
+    assert torch.equal(y, plain)
+    assert_close(yd, np.where(keep, want_y * ks, np.float32(0)), dtype, f"softmax+dropout S={s}")
+    lower = np.tril(np.ones((s, s), dtype=bool))
+    nz = f32(yd) != 0
+    assert not nz[..., ~lower].any()
+    assert np.array_equal(nz & (f32(y) != 0), keep & (f32(y) != 0))   # the mask itself, where y is non-zero
+    # backward
+    g = randn((b, h, s, s), dtype, seed=s + 1)
+    gk = np.where(keep, f32(g) * ks, np.float32(0))
+    want_dx = orc.softmax_bwd(gk, f32(y), 0.125, causal=True)
+    dx = kernels.causal_softmax_dropout_backward(g.to(DEV), y, 0.125, p, seed, offset)
+    assert_close(dx, want_dx, dtype, f"softmax+dropout bwd S={s}")
+    # p == 0 is the plain kernel
+    yd0, y0 = kernels.causal_softmax_dropout_forward(x.to(DEV), None, 0.125, 0.0, 0, 0)
+    assert yd0.data_ptr() == y0.data_ptr()
+    assert torch.equal(y0, kernels.causal_softmax_forward(x.to(DEV), None, 0.125))
