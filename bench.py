@@ -195,6 +195,17 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         g = randn((B * H, S, S), 1, 1.0, dt)
         t = time_launches(lambda: check(lib.oslo_softmax_causal_bwd(P(g), P(g), P(y), 0.125, B * H, S, code, st)), n, 3)
         res.append(roof(f"causal_bwd {name} [8,16,2048,2048] (in place)", es * (2 * tri + full), t))
+        if name == "bf16":  # training: attention dropout inside the softmax kernels
+            stats = torch.empty((B * H * S, 2), dtype=torch.float32, device=dev)
+            t = time_launches(lambda: check(lib.oslo_softmax_causal_dropout_fwd(
+                P(y), P(stats), P(x), None, 0.125, 0.1, 1234, 0, B, H, S, code, st)), n, 3)
+            res.append(roof(f"causal_dropout_fwd p=0.1 {name} [8,16,2048,2048]",
+                            es * (tri + full) + 8 * B * H * S, t))
+            t = time_launches(lambda: check(lib.oslo_softmax_causal_dropout_bwd(
+                P(g), P(g), P(x), P(stats), None, 0.125, 0.1, 1234, 0, B, H, S, code, st)), n, 3)
+            res.append(roof(f"causal_dropout_bwd p=0.1 {name} [8,16,2048,2048] (in place)",
+                            es * (2 * tri + full) + 8 * B * H * S, t))
+            del stats
         del x, y, g
 
     # long rows: bf16 [1,16,8192,8192]

@@ -95,34 +95,42 @@ int oslo_softmax_causal_bwd(void *dx, const void *g, const void *y, float scale,
 
 /*
  * Causal softmax with attention-probability dropout in the same pass:
- * y as oslo_softmax_causal_fwd (kept for the backward), and
- * yd[b,h,r,k] = keep * y[b,h,r,k] / (1-p) (what is multiplied with V). keep for
- * the flat element index i of the [batch, heads, S, S] tensor is drawn like in
- * oslo_bias_dropout_add_fwd (Philox4x32-10, counter (offset/4, i/4), word
- * i mod 4, keep iff word >= floor(p*2^32)); one call consumes 4 units of
- * generator offset. p in [0,1); with p == 0 only y is written (pass yd == y or
- * NULL). yd must not alias y or x otherwise.
+ * yd[b,h,r,k] = keep * y[b,h,r,k] / (1-p) with y as oslo_softmax_causal_fwd
+ * (what is multiplied with V). keep for the flat element index i of the
+ * [batch, heads, S, S] tensor is drawn like in oslo_bias_dropout_add_fwd
+ * (Philox4x32-10, counter (offset/4, i/4), word i mod 4, keep iff
+ * word >= floor(p*2^32)); one call consumes 4 units of generator offset.
+ * p in [0,1). y itself is not stored. Instead row_stats (fp32,
+ * [batch*heads*S, 2], 8-byte aligned) receives per row the maximum of the
+ * exponent e and 1/sum_k exp(e_k - max), where e = scale*x*log2(e) in base-2
+ * units when pad_add is NULL and e = scale*x + pad_add in natural units
+ * otherwise; the backward recomputes y from x and these two numbers, so the
+ * caller keeps x (not y) for the backward. yd may alias x only if x is not
+ * needed afterwards.
  * Replaces the softmax kernel followed by the separate nn.Dropout of the
  * reference's fused GPT-Neo / GPT-J attention
  * (oslo/models/gptj/modeling_gptj.py:941-948,
  *  oslo/models/gpt_neo/modeling_gpt_neo.py:997-1005).
  */
-int oslo_softmax_causal_dropout_fwd(void *yd, void *y, const void *x,
+int oslo_softmax_causal_dropout_fwd(void *yd, float *row_stats, const void *x,
                                     const float *pad_add, float scale, float p,
                                     uint64_t philox_seed, uint64_t philox_offset,
                                     int64_t batch, int64_t heads, int64_t S,
                                     int dtype, oslo_stream_t stream);
 
 /*
- * Backward of the above: g is the gradient of yd; with g' = keep * g / (1-p)
- * (mask regenerated from the same seed and offset),
+ * Backward of the above: g is the gradient of yd; x, row_stats, pad_add,
+ * scale, p, seed and offset are the forward's. With g' = keep * g / (1-p)
+ * (mask regenerated) and y recomputed from x and row_stats,
  * dx = scale * y * ( g' - sum_{j<=r} g'_j * y_j ) for k<=r, 0 for k>r.
- * dx may alias g.
+ * dx may alias g or x.
  */
-int oslo_softmax_causal_dropout_bwd(void *dx, const void *g, const void *y,
+int oslo_softmax_causal_dropout_bwd(void *dx, const void *g, const void *x,
+                                    const float *row_stats, const float *pad_add,
                                     float scale, float p, uint64_t philox_seed,
-                                    uint64_t philox_offset, int64_t bh, int64_t S,
-                                    int dtype, oslo_stream_t stream);
+                                    uint64_t philox_offset, int64_t batch,
+                                    int64_t heads, int64_t S, int dtype,
+                                    oslo_stream_t stream);
 
 /* Scale + key/padding mask + softmax -------------------------------------- */
 

@@ -129,22 +129,27 @@ class _KeyMaskedSoftmax(torch.autograd.Function):
 
 class _CausalSoftmaxDropout(torch.autograd.Function):
     """Causal softmax of [B,H,S,S] scores followed by dropout of the
-    probabilities, one kernel each way; the keep mask is regenerated in the
-    backward from the generator state taken in the forward."""
+    probabilities, one kernel each way. Only the dropped probabilities are
+    written; the backward regenerates the keep mask from the generator state
+    taken in the forward and recomputes the probabilities from the scores and
+    two numbers per row, so the scores (not the probabilities) are what stays
+    alive between the two."""
 
     @staticmethod
     def forward(ctx, inputs, pad_add, scale, p):
         seed, offset = _next_philox(inputs.device)
-        yd, y = get_custom_kernels().causal_softmax_dropout_forward(inputs, pad_add, scale, p, seed, offset)
-        ctx.save_for_backward(y)
+        yd, stats = get_custom_kernels().causal_softmax_dropout_forward(inputs, pad_add, scale, p, seed, offset)
+        ctx.save_for_backward(inputs, stats)
+        ctx.pad_add = pad_add
         ctx.args = (float(scale), float(p), seed, offset)
         return yd
 
     @staticmethod
     def backward(ctx, output_grads):
-        (y,) = ctx.saved_tensors
+        inputs, stats = ctx.saved_tensors
         scale, p, seed, offset = ctx.args
-        dx = get_custom_kernels().causal_softmax_dropout_backward(output_grads, y, scale, p, seed, offset)
+        dx = get_custom_kernels().causal_softmax_dropout_backward(
+            output_grads, inputs, stats, ctx.pad_add, scale, p, seed, offset)
         return dx, None, None, None
 
 

@@ -155,47 +155,58 @@ def causal_softmax_forward(input, pad_add, scale_factor):
     return y
 
 
+def _pad_add_arg(pad_add, b, sk):
+    if pad_add is None:
+        return None
+    _device_tensor(pad_add, "pad_add")
+    _require(pad_add.dtype == torch.float32 and tuple(pad_add.shape) == (b, sk),
+             "pad_add must be fp32 [batch, S]")
+    return pad_add.contiguous()
+
+
 def causal_softmax_dropout_forward(input, pad_add, scale_factor, p, seed, offset):
     """Causal softmax + attention dropout in one pass. Returns (probs_after_
-    dropout, probs); the second is what the backward needs."""
+    dropout, row_stats): the probabilities themselves are not stored; the
+    backward recomputes them from ``input`` and the fp32 [B,H,S,2] row_stats
+    (row maximum and reciprocal row sum)."""
     _device_tensor(input, "input")
     _require(input.dim() == 4, "expected 4D tensor")
     code = _dtype_code(input, "input")
     b, h, sq, sk = input.shape
     _require(sq == sk, "causal softmax needs square score matrices")
     x = input.contiguous()
-    if pad_add is not None:
-        _device_tensor(pad_add, "pad_add")
-        _require(pad_add.dtype == torch.float32 and tuple(pad_add.shape) == (b, sk),
-                 "pad_add must be fp32 [batch, S]")
-        pad_add = pad_add.contiguous()
-    y = torch.empty_like(x, requires_grad=False)
-    yd = torch.empty_like(x, requires_grad=False) if p > 0 else y
+    pad_add = _pad_add_arg(pad_add, b, sk)
+    yd = torch.empty_like(x, requires_grad=False)
+    stats = torch.empty((b, h, sq, 2), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
         _lib.check(_lib.load().oslo_softmax_causal_dropout_fwd(
-            _ptr(yd), _ptr(y), _ptr(x), _ptr(pad_add), float(scale_factor), float(p),
+            _ptr(yd), _ptr(stats), _ptr(x), _ptr(pad_add), float(scale_factor), float(p),
             int(seed), int(offset), b, h, sk, code, _stream(x)))
-    return yd, y
+    return yd, stats
 
 
-def causal_softmax_dropout_backward(output_grads, softmax_results, scale_factor, p, seed, offset):
+def causal_softmax_dropout_backward(output_grads, input, row_stats, pad_add, scale_factor, p, seed, offset):
     """output_grads: gradient of the probabilities after dropout, [B,H,S,S];
     overwritten with the input gradient when contiguous, like the plain
-    backward."""
+    backward. input, row_stats, pad_add: the forward's."""
     _device_tensor(output_grads, "output_grads")
-    _device_tensor(softmax_results, "softmax_results")
+    _device_tensor(input, "input")
+    _device_tensor(row_stats, "row_stats")
     code = _dtype_code(output_grads, "output_grads")
-    _require(softmax_results.dtype == output_grads.dtype and softmax_results.shape == output_grads.shape,
-             "output_grads and softmax_results differ in dtype or shape")
+    _require(input.dtype == output_grads.dtype and input.shape == output_grads.shape,
+             "output_grads and input differ in dtype or shape")
     _require(output_grads.dim() == 4 and output_grads.shape[-1] == output_grads.shape[-2],
              "expected [B,H,S,S]")
     b, h, s, _ = output_grads.shape
+    _require(row_stats.dtype == torch.float32 and tuple(row_stats.shape) == (b, h, s, 2)
+             and row_stats.is_contiguous(), "row_stats must be contiguous fp32 [B,H,S,2]")
     g = output_grads.contiguous()
-    y = softmax_results.contiguous()
+    x = input.contiguous()
+    pad_add = _pad_add_arg(pad_add, b, s)
     with torch.cuda.device(g.device):
         _lib.check(_lib.load().oslo_softmax_causal_dropout_bwd(
-            _ptr(g), _ptr(g), _ptr(y), float(scale_factor), float(p), int(seed), int(offset),
-            b * h, s, code, _stream(g)))
+            _ptr(g), _ptr(g), _ptr(x), _ptr(row_stats), _ptr(pad_add), float(scale_factor), float(p),
+            int(seed), int(offset), b, h, s, code, _stream(g)))
     return g
 
 

@@ -199,9 +199,10 @@ def test_causal_full_size_properties(dtype):
 @pytest.mark.parametrize("s", [5, 64, 520, 1024, 2048, 2050, 4096])
 @pytest.mark.parametrize("with_pad", [False, True], ids=["nopad", "pad"])
 def test_causal_softmax_with_fused_dropout(s, dtype, with_pad):
-    """Softmax + attention dropout in one pass: the probabilities are the plain
-    kernel's, the dropped output is y*keep/(1-p) with the oracle's Philox mask
-    bit for bit, and the backward regenerates the same mask."""
+    """Softmax + attention dropout in one pass: the output is y*keep/(1-p) with
+    the oracle's Philox mask bit for bit, the row statistics are the row's
+    maximum and reciprocal sum, and the backward (which regenerates the mask and
+    recomputes y from the scores and the statistics) matches the oracle."""
     b, h = (2, 2) if s <= 2048 else (1, 1)
     p, seed, offset = 0.1, 4321, 12
     x = randn((b, h, s, s), dtype, seed=s, std=8.0)
@@ -212,22 +213,42 @@ def test_causal_softmax_with_fused_dropout(s, dtype, with_pad):
     want_y = orc.softmax_causal(f32(x), 0.125, None if pad is None else pad.numpy())
     keep = orc.dropout_keep_mask(seed, offset, b * h * s * s, p).reshape(b, h, s, s)
     ks = np.float32(1.0 / (1.0 - float(np.float32(p))))
-    yd, y = kernels.causal_softmax_dropout_forward(x.to(DEV), None if pad is None else pad.to(DEV),
-                                                   0.125, p, seed, offset)
-    plain = kernels.causal_softmax_forward(x.to(DEV), None if pad is None else pad.to(DEV), 0.125)
-    assert torch.equal(y, plain)
+    pad_dev = None if pad is None else pad.to(DEV)
+    x_dev = x.to(DEV)
+    yd, stats = kernels.causal_softmax_dropout_forward(x_dev, pad_dev, 0.125, p, seed, offset)
     assert_close(yd, np.where(keep, want_y * ks, np.float32(0)), dtype, f"softmax+dropout S={s}")
     lower = np.tril(np.ones((s, s), dtype=bool))
     nz = f32(yd) != 0
     assert not nz[..., ~lower].any()
-    assert np.array_equal(nz & (f32(y) != 0), keep & (f32(y) != 0))   # the mask itself, where y is non-zero
-    # backward
+    y = f32(kernels.causal_softmax_forward(x_dev, pad_dev, 0.125))
+    assert np.array_equal(nz & (y != 0), keep & (y != 0))   # the mask itself, where y is non-zero
+    # row statistics: the reciprocal of sum_k exp(e_k - max)
+    e = f32(x).astype(np.float64) * 0.125
+    if pad is not None:
+        e = e + pad.numpy().astype(np.float64)[:, None, None, :]
+    e = np.where(lower, e, -np.inf)
+    inv = 1.0 / np.exp(e - e.max(-1, keepdims=True)).sum(-1)
+    got = stats.cpu().numpy()
+    assert got.shape == (b, h, s, 2)
+    np.testing.assert_allclose(got[..., 1], inv, rtol=2e-6)
+    unit = np.log2(np.e) if pad is None else 1.0
+    np.testing.assert_allclose(got[..., 0], e.max(-1) * unit, rtol=1e-6, atol=1e-6)
+    # backward: probabilities recomputed from x and the statistics
     g = randn((b, h, s, s), dtype, seed=s + 1)
     gk = np.where(keep, f32(g) * ks, np.float32(0))
-    want_dx = orc.softmax_bwd(gk, f32(y), 0.125, causal=True)
-    dx = kernels.causal_softmax_dropout_backward(g.to(DEV), y, 0.125, p, seed, offset)
+    want_dx = orc.softmax_bwd(gk, want_y, 0.125, causal=True)
+    dx = kernels.causal_softmax_dropout_backward(g.to(DEV), x_dev, stats, pad_dev, 0.125, p, seed, offset)
     assert_close(dx, want_dx, dtype, f"softmax+dropout bwd S={s}")
-    # p == 0 is the plain kernel
-    yd0, y0 = kernels.causal_softmax_dropout_forward(x.to(DEV), None, 0.125, 0.0, 0, 0)
-    assert yd0.data_ptr() == y0.data_ptr()
-    assert torch.equal(y0, kernels.causal_softmax_forward(x.to(DEV), None, 0.125))
+    # in place over the scores
+    x2 = x_dev.clone()
+    dx2 = torch.empty_like(x2)
+    from oslo_amd import _lib
+    with torch.cuda.device(DEV):
+        _lib.check(_lib.load().oslo_softmax_causal_dropout_bwd(
+            x2.data_ptr(), g.to(DEV).data_ptr(), x2.data_ptr(), stats.data_ptr(),
+            None if pad_dev is None else pad_dev.data_ptr(), 0.125, p, seed, offset, b, h, s,
+            kernels._dtype_code(x2, "x"), torch.cuda.current_stream().cuda_stream))
+    assert torch.equal(x2, dx)
+    # p == 0: the plain probabilities
+    yd0, _ = kernels.causal_softmax_dropout_forward(x_dev, pad_dev, 0.125, 0.0, 0, 0)
+    assert torch.equal(yd0, kernels.causal_softmax_forward(x_dev, pad_dev, 0.125))
