@@ -80,10 +80,20 @@ def main():
             raise RuntimeError(lib.oslo_last_error().decode())
 
     def time_launches(fn, n, warm):
-        """Average seconds per call of fn over n calls, events on the launch stream."""
+        """Average seconds per call of fn over n calls, events on the launch stream.
+        Warm-up: `warm` calls and then until 30 ms have passed. After a change of
+        workload the device's clocks take some milliseconds to settle (the same
+        kernel on the same buffers was seen 15-25 % slower for its first few dozen
+        launches after a set-up phase), and a kernel table is about the settled
+        rate."""
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
+        t_end = time.perf_counter() + 0.03
+        while time.perf_counter() < t_end:
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         e0.record(stream)

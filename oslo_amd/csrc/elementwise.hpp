@@ -65,12 +65,20 @@ struct EwPos {
   int64_t row_block;
 };
 
+// Column tile and row block of workgroup `block`: column tile fastest.
+struct EwTile {
+  int64_t col_tile, row_block;
+};
+__host__ __device__ inline EwTile ew_tile(int col_tiles, int64_t block) {
+  return EwTile{block % col_tiles, block / col_tiles};
+}
+
 template <int VEC>
 __device__ __forceinline__ EwPos ew_position(int col_tiles, int rows_per_block) {
-  const int64_t ct = blockIdx.x % col_tiles;
+  const EwTile t = ew_tile(col_tiles, blockIdx.x);
   EwPos p;
-  p.row_block = blockIdx.x / col_tiles;
-  p.c0 = (ct * blockDim.x + threadIdx.x) * VEC;
+  p.row_block = t.row_block;
+  p.c0 = (t.col_tile * blockDim.x + threadIdx.x) * VEC;
   p.c0_in_row = (uint32_t)p.c0;
   p.r_base = p.row_block * rows_per_block + threadIdx.y;
   return p;

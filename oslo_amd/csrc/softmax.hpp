@@ -89,16 +89,20 @@ inline RowMap make_row_map(int64_t total_rows, int rows_per_block,
   return m;
 }
 
-// Row of the `w`-th row slot (0 .. rows_per_block-1) of this block; may be
-// >= total_rows (a slot past the end).
-__device__ __forceinline__ int64_t mapped_row(const RowMap &m, int rows_per_block,
-                                              int w) {
-  const int64_t xcd = blockIdx.x % kXcds;
-  int64_t q = blockIdx.x / kXcds;
+// Row of the `w`-th row slot (0 .. rows_per_block-1) of workgroup `block`; may
+// be >= total_rows (a slot past the end).
+__host__ __device__ inline int64_t mapped_row_of(const RowMap &m, int rows_per_block,
+                                                 int64_t block, int w) {
+  const int64_t xcd = block % kXcds;
+  int64_t q = block / kXcds;
   if (m.paired) q = (q & 1) ? m.blocks_per_xcd - 1 - (q >> 1) : (q >> 1);
   const int units_per_block = rows_per_block / m.unit_rows;
   const int64_t unit = xcd + kXcds * (q * units_per_block + w / m.unit_rows);
   return unit * m.unit_rows + w % m.unit_rows;
+}
+__device__ __forceinline__ int64_t mapped_row(const RowMap &m, int rows_per_block,
+                                              int w) {
+  return mapped_row_of(m, rows_per_block, blockIdx.x, w);
 }
 
 // Dynamic LDS a softmax launch asks for without using it, to cap the blocks
@@ -121,21 +125,25 @@ __device__ __forceinline__ float exp_shifted(float v, float m) {
 }
 
 // Picks <NCHUNK, WPR> for a row length and calls fn.template operator()<...>().
-// Rows are kept at <= 32 fp32 values per lane (NCHUNK*VEC <= 32).
+// A lane holds at most four vectors wherever the row length allows it: four
+// 128-bit loads in flight per lane, 4 KiB per wave, measured best (fp32 rows of
+// 2048 as one wave x 8 vectors: 76 % of HBM peak forward, as two waves x 4: 84
+// %). Only fp32 rows beyond 4096 take eight (32 fp32 values per lane).
 template <int VEC, typename Fn>
 inline bool dispatch_row_tile(int64_t cols, Fn &&fn) {
   constexpr int kSpan = kWave * VEC;
-  constexpr int kMaxChunk = 32 / VEC;
   if (cols <= kSpan * 1) {
     fn.template operator()<1, 1>();
   } else if (cols <= kSpan * 2) {
     fn.template operator()<2, 1>();
-  } else if (cols <= kSpan * kMaxChunk) {
-    fn.template operator()<kMaxChunk, 1>();
-  } else if (cols <= kSpan * kMaxChunk * 2) {
-    fn.template operator()<kMaxChunk, 2>();
-  } else if (cols <= kSpan * kMaxChunk * 4) {
-    fn.template operator()<kMaxChunk, 4>();
+  } else if (cols <= kSpan * 4) {
+    fn.template operator()<4, 1>();
+  } else if (cols <= kSpan * 8) {
+    fn.template operator()<4, 2>();
+  } else if (cols <= kSpan * 16) {
+    fn.template operator()<4, 4>();
+  } else if (VEC * 8 <= 32 && cols <= kSpan * 32) {
+    if constexpr (VEC * 8 <= 32) fn.template operator()<8, 4>();
   } else {
     return false;
   }
