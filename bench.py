@@ -260,6 +260,16 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         t = time_launches(lambda: check(lib.oslo_bias_dropout_add_bwd(P(o), P(db), P(ws), P(r), 0.1, 1234, 0, rows, cols, BF16, st)), n, 3)
         res.append(roof(f"bias_dropout_add_bwd+dbias p=0.1 {shape}", 4 * n_el, t))
         del a, r, o, ws
+
+    # rotary embedding + split heads of q, k, v at the GPT-J-6B shape
+    B, S, H, D, rot = 8, 2048, 16, 256, 64
+    q, k, v = (randn((B, S, H, D), 10 + i, 1.0, torch.bfloat16) for i in range(3))
+    qo, ko, vo = (torch.empty((B, H, S, D), dtype=torch.bfloat16, device=dev) for _ in range(3))
+    from oslo_amd.modeling_gptj import rotary_tables
+    sin, cos = rotary_tables(rot, S, dev)
+    t = time_launches(lambda: check(lib.oslo_rotary_qkv(P(qo), P(ko), P(vo), P(q), P(k), P(v), P(sin), P(cos),
+                                                        S, B, S, H, D, rot, 0, 0, BF16, st)), n, 3)
+    res.append(roof("rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64", 3 * 4 * q.numel(), t))
     return res
 
 

@@ -237,6 +237,32 @@ int oslo_bias_dropout_add_bwd(void *dx, void *dbias, float *workspace,
                               uint64_t philox_offset, int64_t rows,
                               int64_t cols, int dtype, oslo_stream_t stream);
 
+/* Rotary position embedding + split-heads transposition ----------------------- */
+
+/*
+ * q_in, k_in, v_in: [batch, seq, heads, head_dim] (the projections viewed by
+ * head); q_out, k_out, v_out: [batch, heads, seq, head_dim]. For q and k the
+ * first rotary_dim features are rotated pairwise by the angle of position
+ * offset + s, in fp32 and in the reference's order of operations:
+ *   out[2i]   = x[2i]  *cos[pos,i] + (-x[2i+1])*sin[pos,i]
+ *   out[2i+1] = x[2i+1]*cos[pos,i] +   x[2i]   *sin[pos,i]
+ * the remaining features and all of v are only moved. sin_table, cos_table:
+ * fp32 [table_positions, rotary_dim/2]. Any of the three tensor pairs may be
+ * NULL (both pointers). inverse != 0 runs the transposed map, the backward:
+ * *_in are then [batch, heads, seq, head_dim] gradients, *_out
+ * [batch, seq, heads, head_dim], rotation by the opposite angle. head_dim must
+ * be a multiple of 16 bytes, rotary_dim even; no output may alias an input.
+ * Replaces fixed_pos_embedding / rotate_every_two / apply_rotary_pos_emb, the
+ * torch.cat of rotated and passed-through features and the permute of
+ * GPTJAttention.forward (oslo/models/gptj/modeling_gptj.py:49-80, :205-233).
+ */
+int oslo_rotary_qkv(void *q_out, void *k_out, void *v_out, const void *q_in,
+                    const void *k_in, const void *v_in, const float *sin_table,
+                    const float *cos_table, int64_t table_positions,
+                    int64_t batch, int64_t seq, int64_t heads, int64_t head_dim,
+                    int64_t rotary_dim, int64_t offset, int inverse, int dtype,
+                    oslo_stream_t stream);
+
 /* Repeated n-gram blocking (beam search) ------------------------------------ */
 
 /*

@@ -236,3 +236,42 @@ def bias_dropout_add_bwd(g, p, keep, dtype=np.float32):
         dx = np.where(keep, g * scale, t(0))
     dbias = dx.reshape(-1, dx.shape[-1]).sum(axis=0, dtype=np.float64).astype(dtype)
     return dx, dbias, g
+
+
+# ---------------------------------------------------------------------------
+# rotary position embedding (GPT-J)
+# ---------------------------------------------------------------------------
+
+def rotary_tables(rotary_dim, positions):
+    """fixed_pos_embedding (oslo/models/gptj/modeling_gptj.py:49-60): fp32 sin
+    and cos of position * 10000^(-2i/rotary_dim), each [positions, rotary_dim/2];
+    exponent, power, reciprocal and product each rounded to fp32."""
+    expo = (np.arange(0, rotary_dim, 2, dtype=np.float32) / np.float32(rotary_dim)).astype(np.float32)
+    inv_freq = (np.float32(1.0) / np.power(np.float32(10000.0), expo, dtype=np.float32)).astype(np.float32)
+    angle = (np.arange(positions, dtype=np.float32)[:, None] * inv_freq[None, :]).astype(np.float32)
+    return np.sin(angle, dtype=np.float32), np.cos(angle, dtype=np.float32)
+
+
+def rotary_split_heads(x, sin, cos, rotary_dim, offset=0, rotate=True, inverse=False):
+    """apply_rotary_pos_emb + cat + permute (modeling_gptj.py:63-80, :205-233)
+    for one projection. Forward: x [B,S,H,D] -> [B,H,S,D] with
+    out[2i] = x[2i]*cos_i + (-x[2i+1])*sin_i, out[2i+1] = x[2i+1]*cos_i + x[2i]*sin_i
+    on the first rotary_dim features, every product and sum rounded to fp32.
+    inverse: the transposed map, x [B,H,S,D] -> [B,S,H,D] with sin negated."""
+    x = np.asarray(x, dtype=np.float32)
+    if inverse:
+        x = x.transpose(0, 2, 1, 3)          # work in [B,S,H,D]
+    out = x.copy()
+    if rotate and rotary_dim > 0:
+        s_len = x.shape[1]
+        sn = sin[offset:offset + s_len][None, :, None, :].astype(np.float32)
+        cs = cos[offset:offset + s_len][None, :, None, :].astype(np.float32)
+        if inverse:
+            sn = -sn
+        x0 = x[..., 0:rotary_dim:2]
+        x1 = x[..., 1:rotary_dim:2]
+        out[..., 0:rotary_dim:2] = (x0 * cs).astype(np.float32) + ((-x1) * sn).astype(np.float32)
+        out[..., 1:rotary_dim:2] = (x1 * cs).astype(np.float32) + (x0 * sn).astype(np.float32)
+    if inverse:
+        return np.ascontiguousarray(out)
+    return np.ascontiguousarray(out.transpose(0, 2, 1, 3))

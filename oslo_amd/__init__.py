@@ -10,6 +10,7 @@ from .fused_kernels_utils import (  # noqa: F401
     FusedBiasGeLU,
     FusedKernelMixin,
     FusedNoRepeatNGramLogitsProcessor,
+    FusedRotaryPositionEmbedding,
     FusedScaleMaskSoftmax,
     FusedScaleMaskSoftmaxDropout,
     ScaledMaskedSoftmaxFunction,

@@ -24,7 +24,7 @@ SOURCES = [
     "softmax_masked.hip",
     "bias_gelu.hip",
     "bias_dropout_add.hip",
-    "ngram_repeat_block.hip",
+    "ngram_repeat_block.hip", "rotary.hip",
 ]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

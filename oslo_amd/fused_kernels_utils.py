@@ -248,6 +248,55 @@ class FusedScaleMaskSoftmaxDropout(object):
 
 
 # ---------------------------------------------------------------------------
+# rotary position embedding + split heads
+# ---------------------------------------------------------------------------
+
+class _RotaryQKV(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, query, key, value, sin, cos, rotary_dim, offset):
+        ctx.save_for_backward(sin, cos)
+        ctx.args = (int(rotary_dim), int(offset))
+        return get_custom_kernels().rotary_qkv_forward(query, key, value, sin, cos, rotary_dim, offset)
+
+    @staticmethod
+    def backward(ctx, grad_query, grad_key, grad_value):
+        sin, cos = ctx.saved_tensors
+        rotary_dim, offset = ctx.args
+        gq, gk, gv = get_custom_kernels().rotary_qkv_backward(
+            grad_query, grad_key, grad_value, sin, cos, rotary_dim, offset)
+        return gq, gk, gv, None, None, None, None
+
+
+class FusedRotaryPositionEmbedding(object):
+    """
+    Kernel fusion function: rotary position embedding + split heads
+
+    Before fusion: view -> slice -> (x * cos) + (rotate_every_two(x) * sin) -> cat -> permute -> copy
+    After fusion: view -> (Rotary + Permute)
+
+    Not in the reference, whose fused GPT-J attention keeps the torch
+    operators of oslo/models/gptj/modeling_gptj.py:49-80, :205-233. ``apply``
+    takes the query / key / value projections viewed as [B, S, H, D] and the
+    fp32 (sin, cos) tables of ``fixed_pos_embedding``, and returns the three
+    tensors as contiguous [B, H, S, D], query and key rotated in their first
+    ``rotary_dim`` features by the angle of position ``offset + s``, in fp32
+    and rounded once to the input dtype.
+    """
+
+    @staticmethod
+    def apply(query, key, value, sincos, rotary_dim, offset=0):
+        sin, cos = sincos
+        return _RotaryQKV.apply(query, key, value, sin, cos, rotary_dim, offset)
+
+    @staticmethod
+    def is_available(dtype, head_dim, rotary_dim):
+        if dtype not in (torch.half, torch.bfloat16, torch.float32):
+            return False
+        vec = 4 if dtype == torch.float32 else 8
+        return head_dim % vec == 0 and rotary_dim % 2 == 0 and 0 <= rotary_dim <= head_dim
+
+
+# ---------------------------------------------------------------------------
 # bias + GeLU
 # ---------------------------------------------------------------------------
 

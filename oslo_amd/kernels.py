@@ -318,3 +318,61 @@ def bias_dropout_add_backward(grad, p, seed, offset, want_dbias=True):
             _ptr(dx), _ptr(dbias), _ptr(ws), _ptr(grad), float(p), int(seed), int(offset),
             rows, cols, code, _stream(grad)))
     return dx, dbias
+
+
+# ---------------------------------------------------------------------------
+# rotary position embedding + split-heads transposition
+# ---------------------------------------------------------------------------
+
+def _rotary_call(tensors, sin, cos, rotary_dim, offset, inverse):
+    first = next(t for t in tensors if t is not None)
+    _device_tensor(first, "rotary input")
+    code = _dtype_code(first, "rotary input")
+    _require(first.dim() == 4, "expected 4D tensors")
+    if inverse:
+        b, h, s, d = first.shape
+        out_shape = (b, s, h, d)
+    else:
+        b, s, h, d = first.shape
+        out_shape = (b, h, s, d)
+    ins, outs = [], []
+    for t in tensors:
+        if t is None:
+            ins.append(None)
+            outs.append(None)
+            continue
+        _device_tensor(t, "rotary input")
+        _require(t.shape == first.shape and t.dtype == first.dtype, "q, k and v differ in shape or dtype")
+        ins.append(t.contiguous())
+        outs.append(torch.empty(out_shape, dtype=t.dtype, device=t.device))
+    positions = 0
+    if rotary_dim > 0:
+        _device_tensor(sin, "sin")
+        _device_tensor(cos, "cos")
+        _require(sin.dtype == torch.float32 and cos.dtype == torch.float32 and sin.dim() == 2
+                 and sin.shape == cos.shape and sin.shape[1] == rotary_dim // 2,
+                 "sin and cos must be fp32 [positions, rotary_dim/2]")
+        sin, cos = sin.contiguous(), cos.contiguous()
+        positions = sin.shape[0]
+    else:
+        sin = cos = None
+    with torch.cuda.device(first.device):
+        _lib.check(_lib.load().oslo_rotary_qkv(
+            _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _ptr(ins[0]), _ptr(ins[1]), _ptr(ins[2]),
+            _ptr(sin), _ptr(cos), positions, b, s, h, d, int(rotary_dim), int(offset),
+            1 if inverse else 0, code, _stream(first)))
+    return tuple(outs)
+
+
+def rotary_qkv_forward(query, key, value, sin, cos, rotary_dim, offset=0):
+    """query, key, value: [B, S, H, D] (any may be None); sin, cos: fp32
+    [positions, rotary_dim/2]. Returns the three tensors as [B, H, S, D], query
+    and key with their first rotary_dim features rotated by the angle of
+    position offset + s (oslo/models/gptj/modeling_gptj.py:49-80, :205-233)."""
+    return _rotary_call((query, key, value), sin, cos, rotary_dim, offset, inverse=False)
+
+
+def rotary_qkv_backward(grad_query, grad_key, grad_value, sin, cos, rotary_dim, offset=0):
+    """Gradients [B, H, S, D] of rotary_qkv_forward's outputs -> gradients
+    [B, S, H, D] of its inputs."""
+    return _rotary_call((grad_query, grad_key, grad_value), sin, cos, rotary_dim, offset, inverse=True)

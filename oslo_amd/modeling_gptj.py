@@ -18,8 +18,8 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax,
-                                 FusedScaleMaskSoftmaxDropout)
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedRotaryPositionEmbedding,
+                                 FusedScaleMaskSoftmax, FusedScaleMaskSoftmaxDropout)
 from .modeling_utils import ACT2FN, LayerPolicy, PreTrainedModel, additive_attention_mask, causal_lm_loss
 
 
@@ -140,7 +140,27 @@ class GPTJAttention(nn.Module):
 
 
 class FusedGPTJAttention(GPTJAttention):
-    """oslo/models/gptj/modeling_gptj.py:936-1038."""
+    """oslo/models/gptj/modeling_gptj.py:936-1038. Beyond the reference's fused
+    class, the rotary embedding of q and k and the split-heads permute of
+    q, k and v run as one kernel (the reference keeps the torch operators)."""
+
+    def _project_qkv(self, hidden_states, layer_past, use_cache):
+        rot = self.rotary_dim if self.rotary_dim is not None else self.head_dim
+        if not (hidden_states.is_cuda and
+                FusedRotaryPositionEmbedding.is_available(hidden_states.dtype, self.head_dim, rot)):
+            return super()._project_qkv(hidden_states, layer_past, use_cache)
+        b, s, _ = hidden_states.shape
+        shape = (b, s, self.num_attention_heads, self.head_dim)
+        offset = 0 if layer_past is None else layer_past[0].shape[-2]
+        sincos = rotary_tables(rot, s + offset, hidden_states.device)
+        query, key, value = FusedRotaryPositionEmbedding.apply(
+            self.q_proj(hidden_states).view(shape), self.k_proj(hidden_states).view(shape),
+            self.v_proj(hidden_states).view(shape), sincos, rot, offset)
+        if layer_past is not None:
+            key = torch.cat((layer_past[0], key), dim=-2)
+            value = torch.cat((layer_past[1], value), dim=-2)
+        present = (key, value) if use_cache else None
+        return query, key, value, present
 
     def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
         w = torch.matmul(query, key.transpose(-1, -2))

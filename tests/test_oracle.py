@@ -315,3 +315,64 @@ def test_bias_dropout_add_closed_forms():
     np.testing.assert_allclose(dx, gx.numpy(), rtol=1e-12)
     np.testing.assert_allclose(db, gb.numpy(), rtol=1e-12)
     np.testing.assert_allclose(dres, gr.numpy(), rtol=1e-12)
+
+
+# ---------------------------------------------------------------------------
+# rotary position embedding
+# ---------------------------------------------------------------------------
+
+def test_rotary_is_complex_multiplication_by_the_position_angle():
+    rng = np.random.default_rng(5)
+    b, s, h, d, rot, off = 2, 9, 3, 16, 12, 4
+    x = rng.standard_normal((b, s, h, d)).astype(np.float32)
+    sin, cos = orc.rotary_tables(rot, s + off)
+    got = orc.rotary_split_heads(x, sin, cos, rot, offset=off)
+    assert got.shape == (b, h, s, d)
+    # (x0 + i x1) * e^{i theta}, theta = pos * 10000^(-2j/rot), in float64
+    j = np.arange(rot // 2)
+    theta = (np.arange(s) + off)[:, None] * 10000.0 ** (-2.0 * j / rot)[None, :]
+    z = (x[..., 0:rot:2].astype(np.float64) + 1j * x[..., 1:rot:2]) * np.exp(1j * theta)[None, :, None, :]
+    want = x.astype(np.float64).copy()
+    want[..., 0:rot:2], want[..., 1:rot:2] = z.real, z.imag
+    # the angle is rounded to fp32 (positions up to 12: error ~1e-6), the rest is exact to fp32
+    np.testing.assert_allclose(got, want.transpose(0, 2, 1, 3), atol=2e-5)
+    assert np.array_equal(got[..., rot:], x.transpose(0, 2, 1, 3)[..., rot:])      # pass-through features
+    # position 0 is the identity
+    first = orc.rotary_split_heads(x[:, :1], sin, cos, rot, offset=0)
+    assert np.array_equal(first, x[:, :1].transpose(0, 2, 1, 3))
+    # rotations preserve the norm of every pair
+    n_in = np.hypot(x[..., 0:rot:2], x[..., 1:rot:2]).transpose(0, 2, 1, 3)
+    np.testing.assert_allclose(np.hypot(got[..., 0:rot:2], got[..., 1:rot:2]), n_in, rtol=1e-5, atol=1e-6)
+
+
+def test_rotary_inverse_is_the_adjoint_and_undoes_the_rotation():
+    rng = np.random.default_rng(6)
+    b, s, h, d, rot = 1, 7, 2, 8, 8
+    x = rng.standard_normal((b, s, h, d)).astype(np.float32)
+    g = rng.standard_normal((b, h, s, d)).astype(np.float32)
+    sin, cos = orc.rotary_tables(rot, s)
+    y = orc.rotary_split_heads(x, sin, cos, rot)
+    back = orc.rotary_split_heads(g, sin, cos, rot, inverse=True)
+    assert back.shape == x.shape
+    # <R x, g> == <x, R^T g>
+    np.testing.assert_allclose((y.astype(np.float64) * g).sum(), (x.astype(np.float64) * back).sum(), rtol=1e-6)
+    np.testing.assert_allclose(orc.rotary_split_heads(y, sin, cos, rot, inverse=True), x, atol=1e-6)
+    # v is only transposed
+    assert np.array_equal(orc.rotary_split_heads(x, sin, cos, rot, rotate=False), x.transpose(0, 2, 1, 3))
+
+
+def test_rotary_matches_the_torch_restatement_of_the_unfused_attention():
+    """The torch operators of the unfused GPT-J attention, in its order (tables,
+    x*cos + rotate_every_two(x)*sin, cat, permute), against the numpy oracle."""
+    from oslo_amd.modeling_gptj import apply_rotary, rotary_tables
+
+    torch.manual_seed(3)
+    b, s, h, d, rot, off = 2, 11, 3, 16, 8, 5
+    x = torch.randn(b, s, h, d)
+    sin_t, cos_t = rotary_tables(rot, s + off, "cpu")
+    sin, cos = orc.rotary_tables(rot, s + off)
+    np.testing.assert_allclose(sin_t.numpy(), sin, atol=1e-6)
+    np.testing.assert_allclose(cos_t.numpy(), cos, atol=1e-6)
+    want = torch.cat([apply_rotary(x[..., :rot], sin_t, cos_t, off), x[..., rot:]], dim=-1).permute(0, 2, 1, 3)
+    got = orc.rotary_split_heads(x.numpy(), sin_t.numpy(), cos_t.numpy(), rot, offset=off)
+    assert np.array_equal(got, want.numpy())   # same tables -> the same fp32 operations, bit for bit
