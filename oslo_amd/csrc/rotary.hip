@@ -39,7 +39,7 @@ struct RotaryArgs {
 // fastest, then position within a tile of `ts` positions, then head: a wave
 // writes (forward) or reads (inverse) contiguous pieces of the [B,H,S,D] side
 // and pieces of one D-row of the [B,S,H,D] side.
-template <typename T, int VEC, bool INVERSE>
+template <typename T, int VEC, bool INVERSE, bool TABLE_VEC>
 __global__ __launch_bounds__(kBlockThreads) void rotary_transpose_kernel(
     RotaryArgs a, const float *__restrict__ sin_t, const float *__restrict__ cos_t,
     int S, int H, int D, int rotary_dim, int offset, int ts, int items_per_tile,
@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kBlockThreads) void rotary_transpose_kernel(
     const int s = s0 + sl;
     const bool ok = item < items_per_tile && s < S;
     col[u] = d8 * VEC;
-    pos[u] = s + offset;
+    pos[u] = (ok ? s : 0) + offset; // a table row that exists
     const uint32_t bshd = (uint32_t)(((int64_t)s * H + h) * D + col[u]) * (uint32_t)sizeof(T);
     const uint32_t bhsd = (uint32_t)(((int64_t)h * S + s) * D + col[u]) * (uint32_t)sizeof(T);
     const uint32_t off_in = ok ? (INVERSE ? bhsd : bshd) : kOutside;
@@ -82,21 +82,46 @@ __global__ __launch_bounds__(kBlockThreads) void rotary_transpose_kernel(
     raw[u] = buffer_load_raw<T, VEC, true>(irs, off_in);
   }
 
+  // sin/cos of the thread's pairs, issued before the data is waited for. A
+  // vector past the rotary features reads the row's first entries (cached,
+  // unused) so that the loads sit outside any branch.
+  constexpr int HALF = VEC / 2;
+  float sn[kRotaryUnroll][HALF], cs[kRotaryUnroll][HALF];
+  const int half_rot = rotary_dim / 2;
+  if (rotate) {
+#pragma unroll
+    for (int u = 0; u < kRotaryUnroll; ++u) {
+      const int64_t row = (int64_t)pos[u] * half_rot;
+      if constexpr (TABLE_VEC) {
+        // rotary_dim/2 is a multiple of HALF and the tables are aligned: the
+        // thread's entries are one aligned vector, wholly inside the row or not
+        const int i = col[u] / 2;
+        load_f32_cached<float, HALF>(sn[u], sin_t + row + (i < half_rot ? i : 0));
+        load_f32_cached<float, HALF>(cs[u], cos_t + row + (i < half_rot ? i : 0));
+      } else {
+#pragma unroll
+        for (int j = 0; j < HALF; ++j) {
+          const int i = col[u] / 2 + j;
+          const int64_t at = row + (i < half_rot ? i : 0);
+          sn[u][j] = sin_t[at];
+          cs[u][j] = cos_t[at];
+        }
+      }
+    }
+  }
+
 #pragma unroll
   for (int u = 0; u < kRotaryUnroll; ++u) {
     float x[VEC];
     raw_to_f32<T, VEC>(x, raw[u]);
-    if (rotate && col[u] < rotary_dim) {
-      const float *sr = sin_t + (int64_t)pos[u] * (rotary_dim / 2) + col[u] / 2;
-      const float *cr = cos_t + (int64_t)pos[u] * (rotary_dim / 2) + col[u] / 2;
+    if (rotate) {
 #pragma unroll
-      for (int j = 0; j < VEC; j += 2) {
-        if (col[u] + j < rotary_dim) { // rotary_dim is even, so the pair is whole
-          const float sn = INVERSE ? -sr[j / 2] : sr[j / 2];
-          const float cs = cr[j / 2];
-          const float x0 = x[j], x1 = x[j + 1];
-          x[j] = __fadd_rn(__fmul_rn(x0, cs), __fmul_rn(-x1, sn));
-          x[j + 1] = __fadd_rn(__fmul_rn(x1, cs), __fmul_rn(x0, sn));
+      for (int j = 0; j < HALF; ++j) {
+        if (col[u] + 2 * j < rotary_dim) { // rotary_dim is even, so the pair is whole
+          const float s1 = INVERSE ? -sn[u][j] : sn[u][j];
+          const float x0 = x[2 * j], x1 = x[2 * j + 1];
+          x[2 * j] = __fadd_rn(__fmul_rn(x0, cs[u][j]), __fmul_rn(-x1, s1));
+          x[2 * j + 1] = __fadd_rn(__fmul_rn(x1, cs[u][j]), __fmul_rn(x0, s1));
         }
       }
     }
@@ -121,14 +146,21 @@ int launch_rotary(const RotaryArgs &a, const float *sin_t, const float *cos_t,
   if (blocks > INT32_MAX || items_per_tile > INT32_MAX)
     return fail(OSLO_E_UNSUPPORTED, "rotary_qkv: tensor too large for one launch");
   const dim3 grid((unsigned)blocks, (unsigned)a.count);
-  if (inverse)
-    rotary_transpose_kernel<T, VEC, true><<<grid, dim3(kBlockThreads), 0, stream>>>(
-        a, sin_t, cos_t, (int)S, (int)H, (int)D, (int)rotary_dim, (int)offset, ts,
-        (int)items_per_tile, blocks_per_tile, s_tiles);
-  else
-    rotary_transpose_kernel<T, VEC, false><<<grid, dim3(kBlockThreads), 0, stream>>>(
-        a, sin_t, cos_t, (int)S, (int)H, (int)D, (int)rotary_dim, (int)offset, ts,
-        (int)items_per_tile, blocks_per_tile, s_tiles);
+  const bool table_vec = rotary_dim > 0 && (rotary_dim / 2) % (VEC / 2) == 0 &&
+                         aligned16(sin_t) && aligned16(cos_t);
+  auto go = [&]<bool INVERSE, bool TABLE_VEC>() {
+    rotary_transpose_kernel<T, VEC, INVERSE, TABLE_VEC>
+        <<<grid, dim3(kBlockThreads), 0, stream>>>(
+            a, sin_t, cos_t, (int)S, (int)H, (int)D, (int)rotary_dim, (int)offset, ts,
+            (int)items_per_tile, blocks_per_tile, s_tiles);
+  };
+  if (inverse) {
+    if (table_vec) go.template operator()<true, true>();
+    else go.template operator()<true, false>();
+  } else {
+    if (table_vec) go.template operator()<false, true>();
+    else go.template operator()<false, false>();
+  }
   return check_launch("rotary_qkv");
 }
 
