@@ -98,8 +98,8 @@ int oslo_softmax_causal_bwd(void *dx, const void *g, const void *y, float scale,
  * yd[b,h,r,k] = keep * y[b,h,r,k] / (1-p) with y as oslo_softmax_causal_fwd
  * (what is multiplied with V). keep for the flat element index i of the
  * [batch, heads, S, S] tensor is drawn like in oslo_bias_dropout_add_fwd
- * (Philox4x32-10, counter (offset/4, i/4), word i mod 4, keep iff
- * word >= floor(p*2^32)); one call consumes 4 units of generator offset.
+ * (Philox4x32-10, counter (offset/4, i/8), 16 bits per element); one call
+ * consumes 4 units of generator offset.
  * p in [0,1). y itself is not stored. Instead row_stats (fp32,
  * [batch*heads*S, 2], 8-byte aligned) receives per row the maximum of the
  * exponent e and 1/sum_k exp(e_k - max), where e = scale*x*log2(e) in base-2
@@ -212,10 +212,11 @@ int oslo_bias_gelu_bwd(void *dy, void *dbias, float *workspace, const void *g,
  * out[r,c] = keep[r,c] * (x[r,c] + bias[c]) / (1-p) + residual[r,c].
  * bias and residual may each be NULL (term dropped). p in [0,1); p == 0 keeps
  * everything and draws no random numbers. keep[i] for the flat element index
- * i = r*cols + c is word (i mod 4) of Philox4x32-10 with key = philox_seed and
- * counter = (philox_offset/4 as 64 bits, i/4 as 64 bits), compared as
- * keep = word >= floor(p * 2^32). One call consumes 4 units of generator
- * offset. out may alias x.
+ * i = r*cols + c comes from Philox4x32-10 with key = philox_seed and
+ * counter = (philox_offset/4 as 64 bits, i/8 as 64 bits): element i owns 16 of
+ * the 128 bits, the low half of word (i mod 8)/2 when i is even, the high half
+ * when odd, and keep = bits >= floor(p * 2^16) (p is quantised to a multiple
+ * of 2^-16). One call consumes 4 units of generator offset. out may alias x.
  * Replaces bias_dropout / bias_dropout_residual
  * (oslo/fused_kernels_utils.py:259-292).
  */

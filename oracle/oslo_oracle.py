@@ -191,15 +191,17 @@ def philox4x32_10(key, counter):
 
 
 def dropout_threshold(p):
-    t = float(np.float32(p)) * 4294967296.0
-    return 0xFFFFFFFF if t >= 4294967295.0 else int(t)
+    """floor(p * 2^16), at most 0xFFFF: an element is dropped with probability
+    threshold / 2^16."""
+    t = float(np.float32(p)) * 65536.0
+    return 0xFFFF if t >= 65535.0 else int(t)
 
 
-def dropout_keep_mask(seed, offset, n, p):
-    """keep[i], i in [0, n): word (i mod 4) of Philox4x32-10 with key = seed
-    and counter = (offset // 4 as 64 bits, i // 4 as 64 bits), kept when
-    word >= floor(p * 2^32)."""
-    groups = (n + 3) // 4
+def dropout_bits(seed, offset, n):
+    """The 16 random bits of elements 0..n-1: element i owns the low (i even)
+    or high (i odd) half of word (i mod 8) // 2 of Philox4x32-10 with
+    key = seed and counter = (offset // 4 as 64 bits, i // 8 as 64 bits)."""
+    groups = (n + 7) // 8
     g = np.arange(groups, dtype=np.uint64)
     block = np.uint64(offset // 4)
     c0 = np.full(groups, block & _LO, dtype=np.uint64).astype(np.uint32)
@@ -207,8 +209,14 @@ def dropout_keep_mask(seed, offset, n, p):
     c2 = (g & _LO).astype(np.uint32)
     c3 = (g >> _S32).astype(np.uint32)
     key = (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)
-    words = np.stack(philox4x32_10(key, (c0, c1, c2, c3)), axis=1).reshape(-1)[:n]
-    return words >= np.uint32(dropout_threshold(p))
+    words = np.stack(philox4x32_10(key, (c0, c1, c2, c3)), axis=1)          # [groups, 4]
+    halves = np.stack((words & np.uint32(0xFFFF), words >> np.uint32(16)), axis=2)  # [groups, 4, 2]
+    return halves.reshape(-1)[:n]
+
+
+def dropout_keep_mask(seed, offset, n, p):
+    """keep[i], i in [0, n): the element's 16 bits >= floor(p * 2^16)."""
+    return dropout_bits(seed, offset, n) >= np.uint32(dropout_threshold(p))
 
 
 def bias_dropout_add_fwd(x, bias, residual, p, keep, dtype=np.float32):

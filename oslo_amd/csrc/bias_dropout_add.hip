@@ -98,7 +98,7 @@ __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_bwd_kernel(
     write_colsum_partial<VEC>(acc, partial, cols, pos, col_ok);
 }
 
-constexpr int kDropBwdUnroll = 8;
+constexpr int kDropBwdUnroll = 4;
 static_assert(kDropBwdUnroll >= kBwdMinUnroll, "workspace bound");
 
 template <typename T, int VEC>

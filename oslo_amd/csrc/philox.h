@@ -38,12 +38,15 @@ OSLO_HD Philox4 philox4x32_10(uint32_t k0, uint32_t k1, uint32_t c0,
   return Philox4{{c0, c1, c2, c3}};
 }
 
-// Dropout draw for a group of four consecutive elements: key = seed,
+// Dropout draw for a group of eight consecutive elements: key = seed,
 // counter = (offset/4 as 64 bits, group index as 64 bits). The generator
 // offset counts 32-bit words, a counter step yields four of them. The four
 // words equal the first four outputs of
 // at::Philox4_32(seed, /*subsequence=*/group, /*offset=*/offset/4) from
-// ATen/core/PhiloxRNGEngine.h.
+// ATen/core/PhiloxRNGEngine.h. Element e (0..7) of the group owns 16 of the
+// 128 bits: the low half of word e/2 when e is even, the high half when odd.
+// Ten Philox rounds cost about as much issue time as the memory traffic of
+// eight 16-bit elements, so a draw is shared by eight elements, not four.
 OSLO_HD Philox4 dropout_draw(uint64_t seed, uint64_t offset, uint64_t group) {
   const uint64_t block = offset >> 2;
   return philox4x32_10((uint32_t)seed, (uint32_t)(seed >> 32), (uint32_t)block,
@@ -51,10 +54,15 @@ OSLO_HD Philox4 dropout_draw(uint64_t seed, uint64_t offset, uint64_t group) {
                        (uint32_t)(group >> 32));
 }
 
-// keep = word >= threshold, threshold = floor(p * 2^32): P(drop) = threshold/2^32.
+OSLO_HD uint32_t dropout_bits(const Philox4 &d, int e) {
+  return (d.w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu;
+}
+
+// keep = bits >= threshold, threshold = floor(p * 2^16): P(drop) = threshold/2^16
+// (p is quantised to a multiple of 2^-16).
 OSLO_HD uint32_t dropout_threshold(float p) {
-  const double t = (double)p * 4294967296.0;
-  return t >= 4294967295.0 ? 0xFFFFFFFFu : (uint32_t)t;
+  const double t = (double)p * 65536.0;
+  return t >= 65535.0 ? 0xFFFFu : (uint32_t)t;
 }
 
 } // namespace oslo

@@ -260,23 +260,27 @@ def test_dropout_words_match_torch_engine_fixture():
             [np.array([c], dtype=np.uint32) for c in
              (blk & 0xFFFFFFFF, blk >> 32, grp & 0xFFFFFFFF, grp >> 32)])
         assert [int(w[0]) for w in got] == v["words"], v
-    # the mask generator lays groups out as documented: element i <- word i%4 of group i//4
-    v = fx["vectors"][1]  # seed 1234, group 0, offset 0
+    # the mask generator lays groups out as documented: element i <- 16 bits of group i//8,
+    # low half of word (i%8)//2 when i is even, high half when odd
+    def halves(words):
+        return [h for w in words for h in (w & 0xFFFF, w >> 16)]
+
     thr = orc.dropout_threshold(0.5)
-    keep = orc.dropout_keep_mask(1234, 0, 4, 0.5)
-    assert list(keep) == [w >= thr for w in v["words"]]
+    v = fx["vectors"][1]  # seed 1234, group 0, offset 0
+    assert list(orc.dropout_bits(1234, 0, 8)) == halves(v["words"])
+    assert list(orc.dropout_keep_mask(1234, 0, 8, 0.5)) == [h >= thr for h in halves(v["words"])]
     v = fx["vectors"][2]  # seed 1234, group 1, offset 0
-    keep = orc.dropout_keep_mask(1234, 0, 7, 0.5)
-    assert list(keep[4:7]) == [w >= thr for w in v["words"][:3]]
+    keep = orc.dropout_keep_mask(1234, 0, 13, 0.5)
+    assert list(keep[8:13]) == [h >= thr for h in halves(v["words"])[:5]]
     v = fx["vectors"][3]  # seed 1234, group 0, offset 4 (one counter block later)
-    keep = orc.dropout_keep_mask(1234, 4, 4, 0.5)
-    assert list(keep) == [w >= thr for w in v["words"]]
+    assert list(orc.dropout_keep_mask(1234, 4, 8, 0.5)) == [h >= thr for h in halves(v["words"])]
 
 
 def test_dropout_mask_statistics_and_thresholds():
     assert orc.dropout_threshold(0.0) == 0
-    assert orc.dropout_threshold(0.5) == 2 ** 31
-    assert orc.dropout_threshold(0.25) == 2 ** 30
+    assert orc.dropout_threshold(0.5) == 2 ** 15
+    assert orc.dropout_threshold(0.25) == 2 ** 14
+    assert orc.dropout_threshold(0.999999) == 0xFFFF
     n, p = 1 << 20, 0.1
     keep = orc.dropout_keep_mask(1234, 0, n, p)
     rate = keep.mean()
