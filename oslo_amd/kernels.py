@@ -29,10 +29,12 @@ def _dtype_code(t, what):
     return _DTYPE[t.dtype]
 
 
-def _device_tensor(t, what):
+def _device_tensor(t, what, like=None):
     _require(isinstance(t, torch.Tensor), f"{what}: expected a tensor")
     _require(t.is_cuda, f"{what}: expected a tensor on a ROCm device, got {t.device} "
                         "(this library has no CPU path)")
+    if like is not None:
+        _require(t.device == like.device, f"{what} is on {t.device}, the input on {like.device}")
 
 
 def _stream(t):
@@ -66,7 +68,7 @@ def scaled_upper_triang_masked_softmax_backward(output_grads, softmax_results, s
     _require(output_grads.dim() == 3, "expected 3D tensor")
     _require(softmax_results.dim() == 3, "expected 3D tensor")
     _device_tensor(output_grads, "output_grads")
-    _device_tensor(softmax_results, "softmax_results")
+    _device_tensor(softmax_results, "softmax_results", output_grads)
     code = _dtype_code(output_grads, "output_grads")
     _require(softmax_results.dtype == output_grads.dtype, "output_grads and softmax_results differ in dtype")
     _require(softmax_results.shape == output_grads.shape, "output_grads and softmax_results differ in shape")
@@ -95,7 +97,7 @@ def scaled_masked_softmax_backward(output_grads, softmax_results, scale_factor):
     _require(output_grads.dim() == 4, "expected 4D tensor")
     _require(softmax_results.dim() == 4, "expected 4D tensor")
     _device_tensor(output_grads, "output_grads")
-    _device_tensor(softmax_results, "softmax_results")
+    _device_tensor(softmax_results, "softmax_results", output_grads)
     code = _dtype_code(output_grads, "output_grads")
     _require(softmax_results.dtype == output_grads.dtype, "output_grads and softmax_results differ in dtype")
     _require(softmax_results.shape == output_grads.shape, "output_grads and softmax_results differ in shape")
@@ -114,7 +116,7 @@ def ngram_repeat_block_forward(tokens, lprobs, bsz, step, beam_size, no_repeat_n
     [bsz*beam_size, len], lprobs fp32 [bsz*beam_size, vocab]; bans in place and
     returns lprobs."""
     _device_tensor(tokens, "tokens")
-    _device_tensor(lprobs, "lprobs")
+    _device_tensor(lprobs, "lprobs", tokens)
     _require(tokens.is_contiguous(), "tokens must be contiguous")
     _require(lprobs.is_contiguous(), "lprobs must be contiguous")
     _require(tokens.dtype == torch.int64, "tokens must be int64")
@@ -144,7 +146,7 @@ def causal_softmax_forward(input, pad_add, scale_factor):
     _require(sq == sk, "causal softmax needs square score matrices")
     x = input.contiguous()
     if pad_add is not None:
-        _device_tensor(pad_add, "pad_add")
+        _device_tensor(pad_add, "pad_add", input)
         _require(pad_add.dtype == torch.float32 and tuple(pad_add.shape) == (b, sk),
                  "pad_add must be fp32 [batch, S]")
         pad_add = pad_add.contiguous()
@@ -155,10 +157,10 @@ def causal_softmax_forward(input, pad_add, scale_factor):
     return y
 
 
-def _pad_add_arg(pad_add, b, sk):
+def _pad_add_arg(pad_add, b, sk, like):
     if pad_add is None:
         return None
-    _device_tensor(pad_add, "pad_add")
+    _device_tensor(pad_add, "pad_add", like)
     _require(pad_add.dtype == torch.float32 and tuple(pad_add.shape) == (b, sk),
              "pad_add must be fp32 [batch, S]")
     return pad_add.contiguous()
@@ -175,7 +177,7 @@ def causal_softmax_dropout_forward(input, pad_add, scale_factor, p, seed, offset
     b, h, sq, sk = input.shape
     _require(sq == sk, "causal softmax needs square score matrices")
     x = input.contiguous()
-    pad_add = _pad_add_arg(pad_add, b, sk)
+    pad_add = _pad_add_arg(pad_add, b, sk, input)
     yd = torch.empty_like(x, requires_grad=False)
     stats = torch.empty((b, h, sq, 2), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
@@ -190,8 +192,8 @@ def causal_softmax_dropout_backward(output_grads, input, row_stats, pad_add, sca
     overwritten with the input gradient when contiguous, like the plain
     backward. input, row_stats, pad_add: the forward's."""
     _device_tensor(output_grads, "output_grads")
-    _device_tensor(input, "input")
-    _device_tensor(row_stats, "row_stats")
+    _device_tensor(input, "input", output_grads)
+    _device_tensor(row_stats, "row_stats", output_grads)
     code = _dtype_code(output_grads, "output_grads")
     _require(input.dtype == output_grads.dtype and input.shape == output_grads.shape,
              "output_grads and input differ in dtype or shape")
@@ -202,7 +204,7 @@ def causal_softmax_dropout_backward(output_grads, input, row_stats, pad_add, sca
              and row_stats.is_contiguous(), "row_stats must be contiguous fp32 [B,H,S,2]")
     g = output_grads.contiguous()
     x = input.contiguous()
-    pad_add = _pad_add_arg(pad_add, b, s)
+    pad_add = _pad_add_arg(pad_add, b, s, output_grads)
     with torch.cuda.device(g.device):
         _lib.check(_lib.load().oslo_softmax_causal_dropout_bwd(
             _ptr(g), _ptr(g), _ptr(x), _ptr(row_stats), _ptr(pad_add), float(scale_factor), float(p),
@@ -220,7 +222,7 @@ def masked_softmax_forward(input, mask, scale_factor, mask_mode=MASK_ADD):
     x = input.contiguous()
     msb = msq = 0
     if mask is not None:
-        _device_tensor(mask, "mask")
+        _device_tensor(mask, "mask", input)
         _require(mask.dim() == 4, "expected 4D tensor")
         _require(mask.dtype in (torch.bool, torch.uint8), "mask must be bool or uint8")
         mb, mh, mq, mk = mask.shape
@@ -247,7 +249,7 @@ def _as_rows_cols(t, bias, what):
     _require(t.dim() >= 1, f"{what}: expected at least 1 dimension")
     cols = t.shape[-1]
     if bias is not None:
-        _device_tensor(bias, "bias")
+        _device_tensor(bias, "bias", t)
         _require(bias.dim() == 1 and bias.shape[0] == cols, "bias must be [last dimension of the input]")
         _require(bias.dtype == t.dtype, "bias and input differ in dtype")
     rows = t.numel() // cols if cols else 0
@@ -273,7 +275,7 @@ def bias_gelu_forward(y, bias):
 def bias_gelu_backward(grad, y, bias, want_dbias=True):
     """Returns (d_input, d_bias or None); d_input is a new tensor."""
     rows, cols, code = _as_rows_cols(y, bias, "input")
-    _device_tensor(grad, "grad")
+    _device_tensor(grad, "grad", y)
     _require(grad.shape == y.shape and grad.dtype == y.dtype, "grad and input differ in shape or dtype")
     grad = grad.contiguous()
     y = y.contiguous()
@@ -294,7 +296,7 @@ def bias_dropout_add_forward(x, bias, residual, p, seed, offset):
     if bias is not None:
         bias = bias.contiguous()
     if residual is not None:
-        _device_tensor(residual, "residual")
+        _device_tensor(residual, "residual", x)
         _require(residual.shape == x.shape and residual.dtype == x.dtype,
                  "residual and input differ in shape or dtype")
         residual = residual.contiguous()
@@ -325,7 +327,8 @@ def bias_dropout_add_backward(grad, p, seed, offset, want_dbias=True):
 # ---------------------------------------------------------------------------
 
 def _rotary_call(tensors, sin, cos, rotary_dim, offset, inverse):
-    first = next(t for t in tensors if t is not None)
+    first = next((t for t in tensors if t is not None), None)
+    _require(first is not None, "rotary: at least one of query, key and value is needed")
     _device_tensor(first, "rotary input")
     code = _dtype_code(first, "rotary input")
     _require(first.dim() == 4, "expected 4D tensors")
@@ -341,14 +344,14 @@ def _rotary_call(tensors, sin, cos, rotary_dim, offset, inverse):
             ins.append(None)
             outs.append(None)
             continue
-        _device_tensor(t, "rotary input")
+        _device_tensor(t, "rotary input", first)
         _require(t.shape == first.shape and t.dtype == first.dtype, "q, k and v differ in shape or dtype")
         ins.append(t.contiguous())
         outs.append(torch.empty(out_shape, dtype=t.dtype, device=t.device))
     positions = 0
     if rotary_dim > 0:
-        _device_tensor(sin, "sin")
-        _device_tensor(cos, "cos")
+        _device_tensor(sin, "sin", first)
+        _device_tensor(cos, "cos", first)
         _require(sin.dtype == torch.float32 and cos.dtype == torch.float32 and sin.dim() == 2
                  and sin.shape == cos.shape and sin.shape[1] == rotary_dim // 2,
                  "sin and cos must be fp32 [positions, rotary_dim/2]")
