@@ -282,6 +282,46 @@ int oslo_ngram_repeat_block(float *lprobs, const int64_t *tokens, int64_t rows,
                             int64_t max_len, int64_t step, int64_t vocab, int n,
                             oslo_stream_t stream);
 
+/* Dataset index builders (host memory, no device work) ------------------------ */
+
+/*
+ * Rows of the array oslo_build_sample_idx fills:
+ * (num_epochs * tokens_per_epoch - 1) / seq_length + 1, or -1 for arguments the
+ * builder rejects (seq_length <= 1, num_epochs <= 0, tokens_per_epoch <= 1).
+ */
+int64_t oslo_sample_idx_rows(int32_t seq_length, int32_t num_epochs,
+                             int64_t tokens_per_epoch);
+
+/*
+ * sample_idx: int32 [rows, 2], host memory. The documents, taken in doc_idx
+ * order, form one token stream (document d has sizes[d] tokens); sample k is
+ * seq_length + 1 tokens of it and starts on the last token of sample k-1.
+ * Row k = (position in doc_idx, offset inside that document) of the first
+ * token of sample k; the last row is the end of the last sample. Fails with
+ * OSLO_E_BAD_ARG, leaving sample_idx partly written, if doc_idx names a
+ * document outside [0, num_docs) or runs out of tokens.
+ * Replaces build_sample_idx
+ * (oslo/fused_kernels/bindings/pybind_datasets.cpp:85-160), which allocates
+ * the array itself and checks nothing.
+ */
+int oslo_build_sample_idx(int32_t *sample_idx, int64_t rows, const int32_t *sizes,
+                          int64_t num_docs, const int32_t *doc_idx,
+                          int64_t doc_idx_len, int32_t seq_length,
+                          int32_t num_epochs, int64_t tokens_per_epoch);
+
+/*
+ * dataset_index: int32 [size]; dataset_sample_index: int64 [size]; weights:
+ * double [num_datasets]; host memory. Sample i is given to the dataset d that
+ * maximises weights[d] * max(i, 1) - (samples given to d so far), lowest d on
+ * ties; dataset_sample_index[i] is that dataset's count before the sample.
+ * Replaces build_blending_indices
+ * (oslo/fused_kernels/bindings/pybind_datasets.cpp:35-82).
+ */
+int oslo_build_blending_indices(int32_t *dataset_index,
+                                int64_t *dataset_sample_index,
+                                const double *weights, int32_t num_datasets,
+                                int64_t size);
+
 #ifdef __cplusplus
 }
 #endif

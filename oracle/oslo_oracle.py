@@ -283,3 +283,48 @@ def rotary_split_heads(x, sin, cos, rotary_dim, offset=0, rotate=True, inverse=F
     if inverse:
         return np.ascontiguousarray(out)
     return np.ascontiguousarray(out.transpose(0, 2, 1, 3))
+
+
+# ---------------------------------------------------------------------------
+# dataset index builders
+# ---------------------------------------------------------------------------
+
+def build_sample_idx(sizes, doc_idx, seq_length, num_epochs, tokens_per_epoch):
+    """oslo/fused_kernels/bindings/pybind_datasets.cpp:85-160 (and its Python
+    twin, oslo/data/datasets/dataset_causal_lm.py:323-358), one step per line.
+    Returns int32 [num_samples + 1, 2]."""
+    num_samples = (num_epochs * tokens_per_epoch - 1) // seq_length
+    out = np.zeros((num_samples + 1, 2), dtype=np.int32)
+    at, offset = 0, 0
+    for k in range(1, num_samples + 1):
+        remaining = seq_length + 1
+        while remaining != 0:
+            left_in_doc = int(sizes[doc_idx[at]]) - offset
+            remaining -= left_in_doc
+            if remaining <= 0:
+                offset += remaining + left_in_doc - 1
+                remaining = 0
+            else:
+                at += 1
+                offset = 0
+        out[k] = (at, offset)
+    return out
+
+
+def build_blending_indices(weights, num_datasets, size):
+    """oslo/fused_kernels/bindings/pybind_datasets.cpp:35-82. Returns
+    (dataset_index int32 [size], dataset_sample_index int64 [size])."""
+    dataset_index = np.zeros(size, dtype=np.int32)
+    dataset_sample_index = np.zeros(size, dtype=np.int64)
+    drawn = [0] * num_datasets
+    for i in range(size):
+        at = max(float(i), 1.0)
+        best, best_error = 0, float(weights[0]) * at - drawn[0]
+        for d in range(1, num_datasets):
+            error = float(weights[d]) * at - drawn[d]
+            if error > best_error:
+                best, best_error = d, error
+        dataset_index[i] = best
+        dataset_sample_index[i] = drawn[best]
+        drawn[best] += 1
+    return dataset_index, dataset_sample_index

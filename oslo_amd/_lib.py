@@ -47,6 +47,10 @@ PROTOTYPES = {
                    _c.c_int, _c.c_int, _P]),
     "oslo_ngram_repeat_block": (
         _c.c_int, [_P, _P, _I64, _I64, _I64, _I64, _c.c_int, _P]),
+    "oslo_sample_idx_rows": (_I64, [_c.c_int32, _c.c_int32, _I64]),
+    "oslo_build_sample_idx": (
+        _c.c_int, [_P, _I64, _P, _I64, _P, _I64, _c.c_int32, _c.c_int32, _I64]),
+    "oslo_build_blending_indices": (_c.c_int, [_P, _P, _P, _c.c_int32, _I64]),
 }
 
 ABI_VERSION = 1

@@ -24,7 +24,9 @@ SOURCES = [
     "softmax_masked.hip",
     "bias_gelu.hip",
     "bias_dropout_add.hip",
-    "ngram_repeat_block.hip", "rotary.hip",
+    "ngram_repeat_block.hip",
+    "rotary.hip",
+    "dataset_index.hip",
 ]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -41,6 +41,17 @@ def get_custom_kernels():
     return _custom_kernels
 
 
+def get_datasets_builder():
+    """The native index builders of the data pipeline
+    (oslo/fused_kernels_utils.py:235-256). The reference returns None when its
+    C++ module does not compile and falls back to Python loops; here the
+    library either loads or EnvironmentError is raised."""
+    from . import datasets_builder
+
+    _lib.load()
+    return datasets_builder
+
+
 # ---------------------------------------------------------------------------
 # softmax
 # ---------------------------------------------------------------------------
