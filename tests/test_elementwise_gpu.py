@@ -129,7 +129,7 @@ def test_elementwise_errors():
 
 
 def test_full_size_bias_gelu_and_dropout_properties():
-    """BASELINE shapes: [16384,16384] bias-GeLU and [16384,4096] dropout-add in
+    """The benchmark shapes: [16384,16384] bias-GeLU and [16384,4096] dropout-add in
     bf16; oracle on a band of rows, structural properties on the whole."""
     dtype = torch.bfloat16
     g = torch.Generator(device=DEV).manual_seed(0)

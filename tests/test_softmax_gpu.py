@@ -170,7 +170,7 @@ def test_reference_symbol_names_and_errors():
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=IDS.get)
 def test_causal_full_size_properties(dtype):
-    """BASELINE configuration [8,16,2048,2048]: size-independent properties on
+    """The benchmark configuration [8,16,2048,2048]: size-independent properties on
     the whole tensor, the oracle on three slabs."""
     b, h, s = 8, 16, 2048
     g = torch.Generator(device=DEV).manual_seed(0)
