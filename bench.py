@@ -196,6 +196,7 @@ def main():
     }
     if not args.no_gptj:
         out["gptj_fwd"] = gptj_forward(torch, dev)
+        out["gptj_train_step"] = gptj_train_step(torch, dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(out))
@@ -352,6 +353,61 @@ def gptj_forward(torch, dev, layers=28, batch=8, seq=2048, reps=5):
             "unfused_tokens_per_s": round(tokens / t_unfused, 1), "fused_tokens_per_s": round(tokens / t_fused, 1),
             "unfused_ms": round(t_unfused * 1e3, 2), "fused_ms": round(t_fused * 1e3, 2),
             "speedup": round(t_unfused / t_fused, 3), "max_abs_logit_diff": round(diff, 4)}
+
+
+def gptj_train_step(torch, dev, layers=4, batch=8, seq=2048, reps=3):
+    """Forward + backward (loss on the input ids, no optimizer) of a GPT-J-6B-
+    shaped stack cut to `layers` layers, with attention and residual dropout at
+    0.1, unfused torch modules against the same model after fuse(): the
+    backward kernels and the dropout kernels in place."""
+    from oslo_amd import GPTJConfig, GPTJForCausalLM
+
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(dev):
+            torch.manual_seed(0)
+            model = GPTJForCausalLM(GPTJConfig(n_layer=layers, attn_pdrop=0.1, resid_pdrop=0.1)).train()
+    finally:
+        torch.set_default_dtype(old)
+    ids = torch.randint(0, 50400, (batch, seq), device=dev)
+
+    def run():
+        model.zero_grad(set_to_none=True)
+        loss = model(ids, labels=ids)["loss"]
+        loss.backward()
+        return loss
+
+    def timed():
+        for _ in range(2):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            run()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps
+
+    t_unfused = timed()
+    torch.cuda.reset_peak_memory_stats(dev)
+    run()
+    mem_unfused = torch.cuda.max_memory_allocated(dev)
+    model.fuse()
+    t_fused = timed()
+    torch.cuda.reset_peak_memory_stats(dev)
+    loss = run()
+    mem_fused = torch.cuda.max_memory_allocated(dev)
+    finite = bool(torch.isfinite(loss).item())
+    del model
+    torch.cuda.empty_cache()
+    tokens = batch * seq
+    return {"config": f"{layers} layers of the 6B shape, bf16, batch {batch}, seq {seq}, attn/resid dropout 0.1, "
+                      "forward + backward",
+            "unfused_tokens_per_s": round(tokens / t_unfused, 1), "fused_tokens_per_s": round(tokens / t_fused, 1),
+            "unfused_ms": round(t_unfused * 1e3, 2), "fused_ms": round(t_fused * 1e3, 2),
+            "speedup": round(t_unfused / t_fused, 3),
+            "unfused_peak_GiB": round(mem_unfused / 2 ** 30, 2), "fused_peak_GiB": round(mem_fused / 2 ** 30, 2),
+            "loss_finite": finite}
 
 
 def cpu_baseline(torch):
