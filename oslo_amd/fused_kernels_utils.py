@@ -402,6 +402,8 @@ def _bias_dropout_add(x, bias, residual, training, drop_prop):
     if p == 1.0:  # everything dropped: F.dropout returns zeros
         out = torch.zeros_like(x)
         return out if residual is None else out + residual
+    if p == 0.0 and bias is None and residual is None:
+        return x  # nothing to add and nothing to drop
     return _BiasDropoutAdd.apply(x, bias, residual, p)
 
 

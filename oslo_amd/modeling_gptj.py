@@ -180,8 +180,10 @@ class FusedGPTJAttention(GPTJAttention):
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask)
         else:
             out, w = self._attn(query, key, value, attention_mask, head_mask)
-        # out_proj has no bias, so there is nothing to fuse after it
-        out = self.resid_dropout(self.out_proj(self._merge_heads(out)))
+        # out_proj has no bias: the epilogue kernel runs with the bias term
+        # dropped (in training; it is skipped when there is nothing to drop)
+        out = FusedBiasDropout.apply(self.out_proj(self._merge_heads(out)), None,
+                                     self.training, self.resid_dropout.p)
         return (out, present, w) if output_attentions else (out, present)
 
 

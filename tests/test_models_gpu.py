@@ -185,3 +185,19 @@ def test_fused_attention_dropout_operator_and_training_step():
         losses.append(loss.item())
         assert all(torch.isfinite(q.grad).all() for q in m.parameters() if q.grad is not None)
     assert losses[0] == losses[1]
+
+
+def test_bias_dropout_without_bias():
+    """The epilogue with no bias term (GPT-J's out_proj): eval returns the input
+    itself, training drops with the documented mask and back-propagates it."""
+    torch.manual_seed(2)
+    x = torch.randn(48, 256, device=DEV, requires_grad=True)
+    assert FusedBiasDropout.apply(x, None, False, 0.3) is x
+    gen = torch.cuda.default_generators[0]
+    seed, off0 = gen.initial_seed(), gen.get_offset()
+    out = FusedBiasDropout.apply(x, None, True, 0.25)
+    keep = torch.from_numpy(orc.dropout_keep_mask(seed, off0, x.numel(), 0.25).reshape(x.shape)).to(DEV)
+    assert torch.equal(out, torch.where(keep, x.detach() * (1 / 0.75), torch.zeros_like(x)))
+    go = torch.randn_like(x)
+    (gx,) = torch.autograd.grad(out, x, go)
+    assert torch.equal(gx, torch.where(keep, go * (1 / 0.75), torch.zeros_like(go)))
