@@ -307,6 +307,28 @@ class FusedRotaryPositionEmbedding(object):
         return head_dim % vec == 0 and rotary_dim % 2 == 0 and 0 <= rotary_dim <= head_dim
 
 
+class _MergeHeads(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        return get_custom_kernels().rotary_qkv_backward(None, None, x, None, None, 0)[2]
+
+    @staticmethod
+    def backward(ctx, grad):
+        return get_custom_kernels().rotary_qkv_forward(None, None, grad, None, None, 0)[2]
+
+
+class FusedMergeHeads(object):
+    """[B, H, S, D] -> contiguous [B, S, H*D]: the ``permute(0, 2, 1, 3)
+    .contiguous().view(...)`` of ``_merge_heads``
+    (oslo/models/gptj/modeling_gptj.py:129-140) as one pass of the
+    transposition kernel, forward and backward."""
+
+    @staticmethod
+    def apply(x):
+        b, h, s, d = x.shape
+        return _MergeHeads.apply(x).view(b, s, h * d)
+
+
 # ---------------------------------------------------------------------------
 # bias + GeLU
 # ---------------------------------------------------------------------------

@@ -18,7 +18,8 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedRotaryPositionEmbedding,
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedMergeHeads,
+                                 FusedRotaryPositionEmbedding,
                                  FusedScaleMaskSoftmax, FusedScaleMaskSoftmaxDropout)
 from .modeling_utils import ACT2FN, LayerPolicy, PreTrainedModel, additive_attention_mask, causal_lm_loss
 
@@ -182,8 +183,9 @@ class FusedGPTJAttention(GPTJAttention):
             out, w = self._attn(query, key, value, attention_mask, head_mask)
         # out_proj has no bias: the epilogue kernel runs with the bias term
         # dropped (in training; it is skipped when there is nothing to drop)
-        out = FusedBiasDropout.apply(self.out_proj(self._merge_heads(out)), None,
-                                     self.training, self.resid_dropout.p)
+        vec_ok = FusedRotaryPositionEmbedding.is_available(out.dtype, self.head_dim, 0)
+        out = FusedMergeHeads.apply(out) if out.is_cuda and vec_ok else self._merge_heads(out)
+        out = FusedBiasDropout.apply(self.out_proj(out), None, self.training, self.resid_dropout.p)
         return (out, present, w) if output_attentions else (out, present)
 
 

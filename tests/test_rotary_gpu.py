@@ -118,3 +118,17 @@ def test_argument_errors():
         kernels.rotary_qkv_forward(torch.randn(1, 4, 2, 6, device=DEV), None, None, sin[:, :1], sin[:, :1], 2)
     with pytest.raises(RuntimeError, match="no CPU path"):
         kernels.rotary_qkv_forward(x.cpu(), None, None, sin, sin, 8)
+
+
+def test_merge_heads_operator():
+    from oslo_amd import FusedMergeHeads
+
+    torch.manual_seed(4)
+    x = torch.randn(2, 3, 17, 32, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    got = FusedMergeHeads.apply(x)
+    want = x.permute(0, 2, 1, 3).contiguous().view(2, 17, 96)
+    assert got.is_contiguous() and torch.equal(got, want)
+    go = torch.randn_like(want)
+    (gx,) = torch.autograd.grad(got, x, go)
+    (gw,) = torch.autograd.grad(want, x, go)
+    assert torch.equal(gx, gw)
