@@ -197,6 +197,7 @@ def main():
     if not args.no_gptj:
         out["gptj_fwd"] = gptj_forward(torch, dev)
         out["gptj_train_step"] = gptj_train_step(torch, dev)
+        out["other_families_fwd"] = other_families_forward(torch, dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(out))
@@ -408,6 +409,67 @@ def gptj_train_step(torch, dev, layers=4, batch=8, seq=2048, reps=3):
             "speedup": round(t_unfused / t_fused, 3),
             "unfused_peak_GiB": round(mem_unfused / 2 ** 30, 2), "fused_peak_GiB": round(mem_fused / 2 ** 30, 2),
             "loss_finite": finite}
+
+
+def other_families_forward(torch, dev, reps=5):
+    """fuse() on the two other model families of the path, forward in eval mode,
+    at published shapes cut to a few layers: GPT-2 XL blocks (d_model 1600, 25
+    heads of 64, 1024 positions) in fp16 and GPT-Neo 2.7B blocks (d_model 2560,
+    20 heads of 128, 2048 positions; every second layer is a sliding-window
+    layer, which fusion leaves alone) in fp16, the one dtype the reference's
+    gate admits. GPT-Neo does not scale its scores; with random N(0, 0.02)
+    weights at this width they have a standard deviation of about 11, and the
+    fused attention (the reference's too) takes them from a GEMM in the model
+    dtype where the unfused attention computes them in fp32: the logit
+    difference reported for this family is that quantisation, not the kernels
+    (in fp32 the two paths agree to 2e-4)."""
+    from oslo_amd import GPT2Config, GPT2LMHeadModel, GPTNeoConfig, GPTNeoForCausalLM
+
+    cases = [
+        ("gpt2_xl_blocks", torch.float16, 16, 1024,
+         lambda: GPT2LMHeadModel(GPT2Config(n_embd=1600, n_head=25, n_layer=6, n_positions=1024))),
+        ("gpt_neo_2.7b_blocks", torch.float16, 8, 2048,
+         lambda: GPTNeoForCausalLM(GPTNeoConfig(hidden_size=2560, num_heads=20, num_layers=6,
+                                                max_position_embeddings=2048))),
+    ]
+    res = {}
+    for name, dtype, batch, seq, ctor in cases:
+        old = torch.get_default_dtype()
+        torch.set_default_dtype(dtype)
+        try:
+            with torch.device(dev):
+                torch.manual_seed(0)
+                model = ctor().eval()
+        finally:
+            torch.set_default_dtype(old)
+        ids = torch.randint(0, 50257, (batch, seq), device=dev)
+
+        def run():
+            with torch.no_grad():
+                return model(ids)["logits"]
+
+        def timed():
+            for _ in range(2):
+                run()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                run()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / reps
+
+        t_unfused = timed()
+        ref_logits = run().float()
+        model.fuse()
+        t_fused = timed()
+        diff = (run().float() - ref_logits).abs().max().item()
+        del model, ref_logits
+        torch.cuda.empty_cache()
+        res[name] = {"dtype": str(dtype).replace("torch.", ""), "batch": batch, "seq": seq, "layers": 6,
+                     "unfused_tokens_per_s": round(batch * seq / t_unfused, 1),
+                     "fused_tokens_per_s": round(batch * seq / t_fused, 1),
+                     "speedup": round(t_unfused / t_fused, 3), "max_abs_logit_diff": round(diff, 4)}
+    return res
 
 
 def cpu_baseline(torch):
