@@ -501,7 +501,40 @@ def cpu_baseline(torch):
     dt = (time.perf_counter() - t0) / reps
     return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": f"unfused fp32 fwd+bwd on [1,4,2048,2048] x {reps} reps, "
-                      f"{dt * 1e3:.1f} ms each, bytes counted at the workload's fp16 size"}
+                      f"{dt * 1e3:.1f} ms each, bytes counted at the workload's fp16 size",
+            "gpt2_small_fwd": gpt2_small_forward(torch)}
+
+
+def gpt2_small_forward(torch):
+    """The CPU-runnable configuration: GPT-2 small (12 layers, d_model 768, 12
+    heads, vocab 50257), random fp32 weights, batch 4 x 512 tokens, eval. The
+    unfused model on the host cores against the same weights after fuse() on
+    the GPU."""
+    from oslo_amd import GPT2Config, GPT2LMHeadModel
+
+    torch.manual_seed(0)
+    model = GPT2LMHeadModel(GPT2Config()).eval()
+    ids = torch.randint(0, 50257, (4, 512))
+    with torch.no_grad():
+        model(ids)
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 5.0 or reps < 2:
+            cpu_logits = model(ids)["logits"]
+            reps += 1
+        t_cpu = (time.perf_counter() - t0) / reps
+        model = model.to("cuda:0").fuse()
+        dev_ids = ids.to("cuda:0")
+        for _ in range(3):
+            gpu_logits = model(dev_ids)["logits"]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            model(dev_ids)
+        torch.cuda.synchronize()
+        t_gpu = (time.perf_counter() - t0) / 20
+    diff = (gpu_logits.cpu() - cpu_logits).abs().max().item()
+    return {"cpu_unfused_tokens_per_s": round(2048 / t_cpu, 1), "cpu_cores": torch.get_num_threads(),
+            "gpu_fused_tokens_per_s": round(2048 / t_gpu, 1), "max_abs_logit_diff": round(diff, 6)}
 
 
 if __name__ == "__main__":

@@ -35,23 +35,8 @@ struct Io {
   static constexpr int kVec = 16 / sizeof(T);
 };
 
-// Load N consecutive elements (address aligned to N*sizeof(T)) as fp32, marked
-// non-temporal (read once).
-template <typename T, int N>
-__device__ __forceinline__ void load_f32(float (&dst)[N], const T *p) {
-  using V = typename VecOf<T, N>::type;
-  if constexpr (N == 1) {
-    dst[0] = static_cast<float>(__builtin_nontemporal_load(p));
-  } else {
-    V v = __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
-#pragma unroll
-    for (int i = 0; i < N; ++i) dst[i] = static_cast<float>(v[i]);
-  }
-}
-
-// Same without the non-temporal hint: for small operands reused by many rows
-// (bias vectors, masks), and for the causal kernels' score reads, where it
-// measured 1-2 % faster than the hinted form.
+// Loads N consecutive elements (address aligned to N*sizeof(T)) as fp32 through
+// the caches: for small operands reused by many rows (bias vectors, tables).
 template <typename T, int N>
 __device__ __forceinline__ void load_f32_cached(float (&dst)[N], const T *p) {
   using V = typename VecOf<T, N>::type;
@@ -71,25 +56,6 @@ __device__ __forceinline__ void load_f32_cached(float (&dst)[N], const T *p) {
 template <typename T, int N>
 using RawVec = typename VecOf<T, N>::type;
 
-template <typename T, int N>
-__device__ __forceinline__ RawVec<T, N> load_raw(const T *p) {
-  return __builtin_nontemporal_load(reinterpret_cast<const RawVec<T, N> *>(p));
-}
-template <typename T, int N>
-__device__ __forceinline__ RawVec<T, N> load_raw_cached(const T *p) {
-  return *reinterpret_cast<const RawVec<T, N> *>(p);
-}
-template <typename T, int N>
-__device__ __forceinline__ RawVec<T, N> zero_raw() {
-  if constexpr (N == 1) {
-    return static_cast<T>(0.0f);
-  } else {
-    RawVec<T, N> v;
-#pragma unroll
-    for (int i = 0; i < N; ++i) v[i] = static_cast<T>(0.0f);
-    return v;
-  }
-}
 template <typename T, int N>
 __device__ __forceinline__ void raw_to_f32(float (&dst)[N],
                                            const RawVec<T, N> &v) {
@@ -186,31 +152,6 @@ __device__ __forceinline__ void buffer_store_f32(BufRsrc rs, uint32_t byte_offse
     static_assert(sizeof(V) == 2, "unsupported vector size");
     __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v),
                                           rs, byte_offset, 0, AUX);
-  }
-}
-
-template <typename T, int N>
-__device__ __forceinline__ void store_f32(T *p, const float (&src)[N]) {
-  using V = typename VecOf<T, N>::type;
-  if constexpr (N == 1) {
-    __builtin_nontemporal_store(static_cast<T>(src[0]), p);
-  } else {
-    V v;
-#pragma unroll
-    for (int i = 0; i < N; ++i) v[i] = static_cast<T>(src[i]);
-    __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
-  }
-}
-
-template <int N>
-__device__ __forceinline__ void load_bytes(uint8_t (&dst)[N], const uint8_t *p) {
-  using V = typename VecOf<uint8_t, N>::type;
-  if constexpr (N == 1) {
-    dst[0] = *p;
-  } else {
-    V v = *reinterpret_cast<const V *>(p);
-#pragma unroll
-    for (int i = 0; i < N; ++i) dst[i] = v[i];
   }
 }
 
