@@ -108,7 +108,7 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_bwd_kernel(
     }
   }
   if constexpr (WANT_DBIAS)
-    write_colsum_partial<VEC>(acc, partial, cols, pos, col_ok);
+    write_colsum_partial<VEC>(acc, partial, cols, pos);
 }
 
 constexpr int kGeluBwdUnroll = 4;

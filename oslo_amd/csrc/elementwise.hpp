@@ -104,28 +104,29 @@ __device__ __forceinline__ uint32_t ew_offset(const EwPos &pos, int u,
 }
 
 // Block-level finish of a per-thread column accumulator: sums acc over the TY
-// threads that share a column vector and writes one fp32 partial row.
+// threads that share a column vector and writes the tile's part of one fp32
+// partial row. The accumulators go to LDS as TY rows of the tile's width; then
+// every thread adds up one column (consecutive threads, consecutive columns:
+// no bank conflicts, one coalesced store per wave), in a fixed order.
 // Every thread of the block must call this (it contains a barrier).
 template <int VEC>
 __device__ __forceinline__ void write_colsum_partial(
     const float (&acc)[VEC], float *__restrict__ partial, int64_t cols,
-    const EwPos &pos, bool col_ok) {
+    const EwPos &pos) {
   __shared__ float red[kBlockThreads * VEC];
-  const int tx = threadIdx.x, ty = threadIdx.y;
   const int TX = blockDim.x, TY = blockDim.y;
-  if (TY > 1) {
+  const int width = TX * VEC; // columns of the tile
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) red[(ty * TX + tx) * VEC + j] = acc[j];
-    __syncthreads();
-  }
-  if (ty == 0 && col_ok) {
-    float *dst = partial + pos.row_block * cols + pos.c0;
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      float s = acc[j];
-      for (int t = 1; t < TY; ++t) s += red[(t * TX + tx) * VEC + j];
-      dst[j] = s;
-    }
+  for (int j = 0; j < VEC; ++j)
+    red[threadIdx.y * width + threadIdx.x * VEC + j] = acc[j];
+  __syncthreads();
+  const int tid = threadIdx.y * TX + threadIdx.x;
+  const int64_t tile_c0 = pos.c0 - (int64_t)threadIdx.x * VEC;
+  float *dst = partial + pos.row_block * cols + tile_c0;
+  for (int c = tid; c < width && tile_c0 + c < cols; c += kBlockThreads) {
+    float s = red[c];
+    for (int t = 1; t < TY; ++t) s += red[t * width + c];
+    dst[c] = s;
   }
 }
 
