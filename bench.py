@@ -50,15 +50,15 @@ MEASURED_TRAFFIC = {
     "causal_fwd bf16 [1,16,8192,8192]": 3229695590,
     "masked_fwd bf16 [16,16,1024,1024] key mask": 1073948672,
     "masked_bwd bf16 [16,16,1024,1024]": 1610650624,
-    "bias_gelu_fwd bf16 [16384,16384]": 1073873305,
-    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1679904563,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610759168,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1145228595,
-    "bias_gelu_fwd bf16 [16384,4096]": 268489523,
-    "bias_gelu_bwd+dbias bf16 [16384,4096]": 420024115,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402726502,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 286330982,
-    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807774617,
+    "bias_gelu_fwd bf16 [16384,16384]": 1073873510,
+    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677932748,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610758758,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141058969,
+    "bias_gelu_fwd bf16 [16384,4096]": 268489318,
+    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419568025,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402726297,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285348249,
+    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807780147,
 }
 
 
