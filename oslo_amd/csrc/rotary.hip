@@ -96,8 +96,13 @@ __global__ __launch_bounds__(kBlockThreads) void rotary_transpose_kernel(
         // rotary_dim/2 is a multiple of HALF and the tables are aligned: the
         // thread's entries are one aligned vector, wholly inside the row or not
         const int i = col[u] / 2;
-        load_f32_cached<float, HALF>(sn[u], sin_t + row + (i < half_rot ? i : 0));
-        load_f32_cached<float, HALF>(cs[u], cos_t + row + (i < half_rot ? i : 0));
+        if (i < half_rot) {
+          load_f32_cached<float, HALF>(sn[u], sin_t + row + i);
+          load_f32_cached<float, HALF>(cs[u], cos_t + row + i);
+        } else {
+#pragma unroll
+          for (int j = 0; j < HALF; ++j) sn[u][j] = cs[u][j] = 0.f;
+        }
       } else {
 #pragma unroll
         for (int j = 0; j < HALF; ++j) {
