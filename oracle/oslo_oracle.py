@@ -26,9 +26,19 @@ root):
 * get_batch_per_block: oslo/fused_kernels/includes/fused_softmax.h:328-340;
 * ngram_banned_tokens: oslo/fused_kernels/fused_ngram_repeat_block.cu:18-49;
 * reference_is_available: oslo/fused_kernels_utils.py:461-479;
-* philox4x32_10 / dropout_keep_mask: no counterpart in the reference (it uses
-  torch's generator through F.dropout); they restate the published Philox
-  algorithm and this library's documented element -> counter mapping.
+* philox4x32_10 / dropout_bits / dropout_keep_mask: no counterpart in the
+  reference (it uses torch's generator through F.dropout); they restate the
+  published Philox algorithm and this library's documented element -> counter
+  mapping (pinned by the Random123 known answers and a fixture written from
+  torch's own Philox engine, tests/golden/philox_vectors.json);
+* rotary_tables / rotary_split_heads: oslo/models/gptj/modeling_gptj.py:49-80
+  and :205-233 (pinned by complex multiplication in float64, the adjoint
+  identity and the torch operators of the unfused attention);
+* build_sample_idx / build_blending_indices:
+  oslo/fused_kernels/bindings/pybind_datasets.cpp:35-160 (pinned by the closed
+  form "sample k starts at token k*seq_length", the share bound of the
+  blending, and, where oracle/_ref holds a build of it, the reference's own
+  module).
 
 Parity unpinned: none of the functions above. The reference itself holds no
 golden vectors for this path.
