@@ -84,6 +84,26 @@ def test_argument_screening_without_a_device(lib):
     assert lib.oslo_bias_dropout_add_fwd(one, one, null, null, 1.0, 1, 0, 4, 8, 1, null) == -1
     assert lib.oslo_bias_dropout_add_fwd(one, one, null, null, -0.1, 1, 0, 4, 8, 1, null) == -1
     assert lib.oslo_bias_dropout_add_bwd(one, null, null, one, float("nan"), 1, 0, 4, 8, 1, null) == -1
+    # softmax with fused dropout: p, the statistics buffer, sizes
+    assert lib.oslo_softmax_causal_dropout_fwd(one, one, one, null, 1.0, 1.0, 1, 0, 1, 1, 8, 1, null) == -1
+    assert lib.oslo_softmax_causal_dropout_fwd(one, null, one, null, 1.0, 0.1, 1, 0, 1, 1, 8, 1, null) == -1
+    assert lib.oslo_softmax_causal_dropout_bwd(one, one, one, null, null, 1.0, 0.1, 1, 0, 1, 1, 8, 1, null) == -1
+    assert lib.oslo_softmax_causal_dropout_bwd(one, one, one, one, null, 1.0, 0.1, 1, 0, 1, 1, 9000, 1, null) == -2
+    assert lib.oslo_softmax_causal_dropout_fwd(null, null, null, null, 1.0, 0.1, 1, 0, 0, 1, 8, 1, null) == 0
+    # rotary: odd or oversized rotary_dim, head_dim not a multiple of the vector, table too short,
+    # one pointer of a pair, in place
+    two = ctypes.c_void_p(32)
+    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 3, 0, 0, 1, null) == -1
+    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 32, 0, 0, 1, null) == -1
+    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 12, 4, 0, 0, 1, null) == -2
+    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 4, 1, 0, 1, null) == -1
+    assert b"table" in lib.oslo_last_error()
+    assert lib.oslo_rotary_qkv(one, null, null, null, null, null, one, one, 8, 1, 8, 2, 16, 4, 0, 0, 1, null) == -1
+    assert lib.oslo_rotary_qkv(two, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 4, 0, 0, 1, null) == -1
+    assert lib.oslo_rotary_qkv(null, null, null, null, null, null, null, null, 0, 1, 8, 2, 16, 4, 0, 0, 1, null) == 0
+    # n-gram blocking
+    assert lib.oslo_ngram_repeat_block(one, one, 2, 4, 3, 8, 0, null) == -1
+    assert lib.oslo_ngram_repeat_block(null, one, 2, 4, 3, 8, 2, null) == -1
     # empty problems succeed without touching the device
     assert lib.oslo_softmax_causal_fwd(null, null, null, 1.0, 0, 4, 8, 1, null) == 0
     assert lib.oslo_softmax_masked_fwd(null, null, null, 0, 0, 0, 1.0, 2, 2, 0, 8, 1, null) == 0
