@@ -464,10 +464,12 @@ int launch_causal_fwd(T *y, float *stats, const T *x, const float *pad,
     constexpr int rpb = RowTile<VEC, NCHUNK, WPR>::kRowsPerBlock;
     const RowMap map = make_row_map(total_rows, rpb, S * (int64_t)sizeof(T), true);
     const dim3 grid((unsigned)(map.blocks_per_xcd * kXcds));
-    // the dropout variant is bound by the Philox arithmetic, not by the write
-    // stream, and wants every wave the registers allow
-    const unsigned lds =
-        with_dropout ? 0u : occupancy_pad_bytes(false, S * (int64_t)sizeof(T));
+    // the variants with dropout (Philox) or a padding mask (its loads, and one
+    // more multiply and add per key) carry more arithmetic per byte and want
+    // every wave the registers allow: measured 277 -> 267 us with the mask
+    const unsigned lds = (with_dropout || pad)
+                             ? 0u
+                             : occupancy_pad_bytes(false, S * (int64_t)sizeof(T));
     auto go = [&]<bool HAS_PAD, bool DROP>() {
       causal_fwd_kernel<T, VEC, NCHUNK, WPR, HAS_PAD, DROP>
           <<<grid, dim3(kBlockThreads), lds, stream>>>(
