@@ -225,6 +225,12 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         g = randn((B * H, S, S), 1, 1.0, dt)
         t = time_launches(lambda: check(lib.oslo_softmax_causal_bwd(P(g), P(g), P(y), 0.125, B * H, S, code, st)), n, 3)
         res.append(roof(f"causal_bwd {name} [8,16,2048,2048] (in place)", es * (2 * tri + full), t))
+        if name == "bf16":  # padded batches: additive key mask, lengths U{1024..2048}
+            gen.manual_seed(2)
+            lens = torch.randint(1024, S + 1, (B,), generator=gen, device=dev)
+            pad = torch.where(torch.arange(S, device=dev)[None, :] < lens[:, None], 0.0, -10000.0).float().contiguous()
+            t = time_launches(lambda: check(lib.oslo_softmax_causal_fwd(P(y), P(x), P(pad), 0.125, B, H, S, code, st)), n, 3)
+            res.append(roof(f"causal_fwd {name} [8,16,2048,2048] with padding mask", es * (tri + full) + 4 * B * S, t))
         if name == "bf16":  # training: attention dropout inside the softmax kernels
             stats = torch.empty((B * H * S, 2), dtype=torch.float32, device=dev)
             t = time_launches(lambda: check(lib.oslo_softmax_causal_dropout_fwd(
