@@ -164,14 +164,15 @@ def main():
     t_fwd = time_launches(fwd, args.steps, 5)
     t_bwd = time_launches(bwd, args.steps, 5)
 
-    def roof(name, nbytes, seconds):
+    def roof(name, nbytes, seconds, elements):
+        """elements: scores or activations the launch produces."""
         gbps = nbytes / seconds / 1e9
-        return {"kernel": name, "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
+        return {"kernel": name, "elements_per_s": round(elements / seconds, 1), "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "us": round(seconds * 1e6, 1),
                 "algorithmic_bytes": nbytes, "traffic": MEASURED_TRAFFIC.get(name)}
 
-    roofline = roof("causal_fwd fp16 [8,16,2048,2048]", bytes_fwd, t_fwd)
-    kernels = [roof("causal_bwd fp16 [8,16,2048,2048]", bytes_bwd, t_bwd)]
+    roofline = roof("causal_fwd fp16 [8,16,2048,2048]", bytes_fwd, t_fwd, full)
+    kernels = [roof("causal_bwd fp16 [8,16,2048,2048]", bytes_bwd, t_bwd, full)]
     del x, y, g, dx
     kernels += other_kernels(lib, torch, dev, st, P, check, time_launches, roof, max(10, args.steps // 2))
 
@@ -221,26 +222,26 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         y = torch.empty_like(x)
         es = x.element_size()
         t = time_launches(lambda: check(lib.oslo_softmax_causal_fwd(P(y), P(x), None, 0.125, B, H, S, code, st)), n, 3)
-        res.append(roof(f"causal_fwd {name} [8,16,2048,2048]", es * (tri + full), t))
+        res.append(roof(f"causal_fwd {name} [8,16,2048,2048]", es * (tri + full), t, full))
         g = randn((B * H, S, S), 1, 1.0, dt)
         t = time_launches(lambda: check(lib.oslo_softmax_causal_bwd(P(g), P(g), P(y), 0.125, B * H, S, code, st)), n, 3)
-        res.append(roof(f"causal_bwd {name} [8,16,2048,2048] (in place)", es * (2 * tri + full), t))
+        res.append(roof(f"causal_bwd {name} [8,16,2048,2048] (in place)", es * (2 * tri + full), t, full))
         if name == "bf16":  # padded batches: additive key mask, lengths U{1024..2048}
             gen.manual_seed(2)
             lens = torch.randint(1024, S + 1, (B,), generator=gen, device=dev)
             pad = torch.where(torch.arange(S, device=dev)[None, :] < lens[:, None], 0.0, -10000.0).float().contiguous()
             t = time_launches(lambda: check(lib.oslo_softmax_causal_fwd(P(y), P(x), P(pad), 0.125, B, H, S, code, st)), n, 3)
-            res.append(roof(f"causal_fwd {name} [8,16,2048,2048] with padding mask", es * (tri + full) + 4 * B * S, t))
+            res.append(roof(f"causal_fwd {name} [8,16,2048,2048] with padding mask", es * (tri + full) + 4 * B * S, t, full))
         if name == "bf16":  # training: attention dropout inside the softmax kernels
             stats = torch.empty((B * H * S, 2), dtype=torch.float32, device=dev)
             t = time_launches(lambda: check(lib.oslo_softmax_causal_dropout_fwd(
                 P(y), P(stats), P(x), None, 0.125, 0.1, 1234, 0, B, H, S, code, st)), n, 3)
             res.append(roof(f"causal_dropout_fwd p=0.1 {name} [8,16,2048,2048]",
-                            es * (tri + full) + 8 * B * H * S, t))
+                            es * (tri + full) + 8 * B * H * S, t, full))
             t = time_launches(lambda: check(lib.oslo_softmax_causal_dropout_bwd(
                 P(g), P(g), P(x), P(stats), None, 0.125, 0.1, 1234, 0, B, H, S, code, st)), n, 3)
             res.append(roof(f"causal_dropout_bwd p=0.1 {name} [8,16,2048,2048] (in place)",
-                            es * (2 * tri + full) + 8 * B * H * S, t))
+                            es * (2 * tri + full) + 8 * B * H * S, t, full))
             del stats
         del x, y, g
 
@@ -249,7 +250,7 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
     x = randn((1, 16, S8, S8), 0, 1.0, torch.bfloat16)
     y = torch.empty_like(x)
     t = time_launches(lambda: check(lib.oslo_softmax_causal_fwd(P(y), P(x), None, 1 / 16, 1, 16, S8, BF16, st)), n, 3)
-    res.append(roof("causal_fwd bf16 [1,16,8192,8192]", 2 * (16 * S8 * (S8 + 1) // 2 + x.numel()), t))
+    res.append(roof("causal_fwd bf16 [1,16,8192,8192]", 2 * (16 * S8 * (S8 + 1) // 2 + x.numel()), t, x.numel()))
     del x, y
 
     # padded key mask: bf16 [16,16,1024,1024], lengths U{128..1024}
@@ -260,11 +261,11 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
     lens = torch.randint(128, 1025, (B,), generator=gen, device=dev)
     mask = (torch.arange(S, device=dev)[None, :] >= lens[:, None]).contiguous().view(torch.uint8)
     t = time_launches(lambda: check(lib.oslo_softmax_masked_fwd(P(y), P(x), P(mask), S, 0, 0, 0.125, B, H, S, S, BF16, st)), n, 3)
-    res.append(roof("masked_fwd bf16 [16,16,1024,1024] key mask", 4 * x.numel() + mask.numel(), t))
+    res.append(roof("masked_fwd bf16 [16,16,1024,1024] key mask", 4 * x.numel() + mask.numel(), t, x.numel()))
     g = randn((B, H, S, S), 1, 1.0, torch.bfloat16)
     dxm = torch.empty_like(g)
     t = time_launches(lambda: check(lib.oslo_softmax_masked_bwd(P(dxm), P(g), P(y), 0.125, B * H * S, S, BF16, st)), n, 3)
-    res.append(roof("masked_bwd bf16 [16,16,1024,1024]", 6 * x.numel(), t))
+    res.append(roof("masked_bwd bf16 [16,16,1024,1024]", 6 * x.numel(), t, x.numel()))
     del x, y, g, dxm
 
     # bias-GeLU and bias-dropout-residual, bf16
@@ -278,13 +279,13 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         n_el = rows * cols
         shape = f"bf16 [{rows},{cols}]"
         t = time_launches(lambda: check(lib.oslo_bias_gelu_fwd(P(o), P(a), P(bias), rows, cols, BF16, st)), n, 3)
-        res.append(roof(f"bias_gelu_fwd {shape}", 4 * n_el, t))
+        res.append(roof(f"bias_gelu_fwd {shape}", 4 * n_el, t, n_el))
         t = time_launches(lambda: check(lib.oslo_bias_gelu_bwd(P(o), P(db), P(ws), P(r), P(a), P(bias), rows, cols, BF16, st)), n, 3)
-        res.append(roof(f"bias_gelu_bwd+dbias {shape}", 6 * n_el, t))
+        res.append(roof(f"bias_gelu_bwd+dbias {shape}", 6 * n_el, t, n_el))
         t = time_launches(lambda: check(lib.oslo_bias_dropout_add_fwd(P(o), P(a), P(bias), P(r), 0.1, 1234, 0, rows, cols, BF16, st)), n, 3)
-        res.append(roof(f"bias_dropout_add_fwd p=0.1 {shape}", 6 * n_el, t))
+        res.append(roof(f"bias_dropout_add_fwd p=0.1 {shape}", 6 * n_el, t, n_el))
         t = time_launches(lambda: check(lib.oslo_bias_dropout_add_bwd(P(o), P(db), P(ws), P(r), 0.1, 1234, 0, rows, cols, BF16, st)), n, 3)
-        res.append(roof(f"bias_dropout_add_bwd+dbias p=0.1 {shape}", 4 * n_el, t))
+        res.append(roof(f"bias_dropout_add_bwd+dbias p=0.1 {shape}", 4 * n_el, t, n_el))
         del a, r, o, ws
 
     # rotary embedding + split heads of q, k, v at the GPT-J-6B shape
@@ -295,7 +296,7 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
     sin, cos = rotary_tables(rot, S, dev)
     t = time_launches(lambda: check(lib.oslo_rotary_qkv(P(qo), P(ko), P(vo), P(q), P(k), P(v), P(sin), P(cos),
                                                         S, B, S, H, D, rot, 0, 0, BF16, st)), n, 3)
-    res.append(roof("rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64", 3 * 4 * q.numel(), t))
+    res.append(roof("rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64", 3 * 4 * q.numel(), t, 3 * q.numel()))
     return res
 
 
