@@ -21,6 +21,7 @@ Differences from the reference, all widening:
 """
 
 import inspect
+import weakref
 
 import torch
 
@@ -170,9 +171,19 @@ def _key_mask_bytes(pad_mask):
     return pad_mask if pad_mask.dtype == torch.bool else pad_mask != 0
 
 
+_pad_cache = None  # (weakref to the mask, its version, the fp32 [B, Sk] form)
+
+
 def _pad_additive_f32(pad_mask, bsz, sk):
     """[B or 1, 1, 1, Sk] mask (bool/uint8: True = padded -> -10000; float:
-    additive as given) -> fp32 [B, Sk]."""
+    additive as given) -> fp32 [B, Sk]. Every layer of a model passes the same
+    mask tensor, so the last conversion is kept and reused while that tensor is
+    alive and unmodified."""
+    global _pad_cache
+    if _pad_cache is not None:
+        ref, version, converted = _pad_cache
+        if ref() is pad_mask and pad_mask._version == version and tuple(converted.shape) == (bsz, sk):
+            return converted
     if pad_mask.dim() != 4 or pad_mask.shape[1] != 1 or pad_mask.shape[2] != 1 \
             or pad_mask.shape[3] != sk or pad_mask.shape[0] not in (1, bsz):
         raise RuntimeError(
@@ -184,7 +195,9 @@ def _pad_additive_f32(pad_mask, bsz, sk):
         m = m.to(torch.float32) * -10000.0
     else:
         m = m.to(torch.float32)
-    return m.expand(bsz, sk).contiguous()
+    m = m.expand(bsz, sk).contiguous()
+    _pad_cache = (weakref.ref(pad_mask), pad_mask._version, m)
+    return m
 
 
 class FusedScaleMaskSoftmax(object):

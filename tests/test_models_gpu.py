@@ -201,3 +201,20 @@ def test_bias_dropout_without_bias():
     go = torch.randn_like(x)
     (gx,) = torch.autograd.grad(out, x, go)
     assert torch.equal(gx, torch.where(keep, go * (1 / 0.75), torch.zeros_like(go)))
+
+
+def test_padding_mask_conversion_is_reused_and_invalidated():
+    b, h, s = 2, 2, 64
+    x = torch.randn(b, h, s, s, device=DEV)
+    mask = torch.zeros(b, 1, 1, s, device=DEV)
+    mask[1, :, :, 40:] = -10000.0
+    y1 = FusedScaleMaskSoftmax.apply(x, mask, 0.5, True)
+    first = fku._pad_cache[2]
+    y2 = FusedScaleMaskSoftmax.apply(x, mask, 0.5, True)
+    assert fku._pad_cache[2] is first and torch.equal(y1, y2)      # same tensor, unmodified: reused
+    mask[0, :, :, 10:] = -10000.0                                    # in-place change bumps the version
+    y3 = FusedScaleMaskSoftmax.apply(x, mask, 0.5, True)
+    assert fku._pad_cache[2] is not first
+    want = torch.softmax((x * 0.5 + mask).masked_fill(
+        ~torch.tril(torch.ones(s, s, dtype=torch.bool, device=DEV)), float("-inf")), -1)
+    assert (y3 - want).abs().max().item() <= 1e-6
