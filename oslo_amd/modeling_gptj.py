@@ -52,11 +52,23 @@ class GPTJConfig:
         return self.n_positions
 
 
+_rotary_table_cache = {}
+
+
 def rotary_tables(dim, seq_len, device):
-    """sin and cos of position * 10000^(-2i/dim), each [seq_len, dim/2], fp32."""
+    """sin and cos of position * 10000^(-2i/dim), each [seq_len, dim/2], fp32.
+    Every layer asks for the same tables, so the last few are kept."""
+    key = (int(dim), int(seq_len), str(device))
+    hit = _rotary_table_cache.get(key)
+    if hit is not None:
+        return hit
     inv_freq = 1.0 / (10000 ** (torch.arange(0, dim, 2, device=device, dtype=torch.float32) / dim))
     angles = torch.arange(seq_len, device=device, dtype=torch.float32)[:, None] * inv_freq[None, :]
-    return torch.sin(angles), torch.cos(angles)
+    tables = (torch.sin(angles), torch.cos(angles))
+    if len(_rotary_table_cache) >= 8:
+        _rotary_table_cache.pop(next(iter(_rotary_table_cache)))
+    _rotary_table_cache[key] = tables
+    return tables
 
 
 def apply_rotary(x, sin, cos, offset=0):
