@@ -232,6 +232,17 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
             pad = torch.where(torch.arange(S, device=dev)[None, :] < lens[:, None], 0.0, -10000.0).float().contiguous()
             t = time_launches(lambda: check(lib.oslo_softmax_causal_fwd(P(y), P(x), P(pad), 0.125, B, H, S, code, st)), n, 3)
             res.append(roof(f"causal_fwd {name} [8,16,2048,2048] with padding mask", es * (tri + full) + 4 * B * S, t, full))
+        if name == "bf16":  # sliding-window rows (GPT-Neo local attention), window 256
+            W = 256
+            band = B * H * (W * (W + 1) // 2 + (S - W) * W)
+            t = time_launches(lambda: check(lib.oslo_softmax_causal_window_fwd(
+                P(y), P(x), None, 0.125, W, B, H, S, code, st)), n, 3)
+            res.append(roof(f"causal_window_fwd window 256 {name} [8,16,2048,2048]", es * (band + full), t, full))
+            t = time_launches(lambda: check(lib.oslo_softmax_causal_window_bwd(
+                P(g), P(g), P(y), 0.125, W, B * H, S, code, st)), n, 3)
+            res.append(roof(f"causal_window_bwd window 256 {name} [8,16,2048,2048] (in place)",
+                            es * (2 * band + full), t, full))
+            check(lib.oslo_softmax_causal_fwd(P(y), P(x), None, 0.125, B, H, S, code, st))
         if name == "bf16":  # training: attention dropout inside the softmax kernels
             stats = torch.empty((B * H * S, 2), dtype=torch.float32, device=dev)
             t = time_launches(lambda: check(lib.oslo_softmax_causal_dropout_fwd(

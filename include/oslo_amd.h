@@ -132,6 +132,27 @@ int oslo_softmax_causal_dropout_bwd(void *dx, const void *g, const void *x,
                                     int64_t heads, int64_t S, int dtype,
                                     oslo_stream_t stream);
 
+/*
+ * Sliding-window causal softmax: as oslo_softmax_causal_fwd, but row r sees only
+ * the keys max(0, r-window+1) .. r (window >= 1; window >= S is the plain causal
+ * softmax). y is zero outside the window.
+ * This is the mask of GPT-Neo's local attention layers, bias = tril(ones) xor
+ * tril(ones, -window) (oslo/models/gpt_neo/modeling_gpt_neo.py:153-163), which
+ * the reference computes on its unfused path only (:268-272).
+ */
+int oslo_softmax_causal_window_fwd(void *y, const void *x, const float *pad_add,
+                                   float scale, int64_t window, int64_t batch,
+                                   int64_t heads, int64_t S, int dtype,
+                                   oslo_stream_t stream);
+
+/*
+ * Backward of the above: dx = scale * y * (g - sum_j g_j*y_j) over the keys of
+ * the window, 0 outside it. dx may alias g.
+ */
+int oslo_softmax_causal_window_bwd(void *dx, const void *g, const void *y,
+                                   float scale, int64_t window, int64_t bh,
+                                   int64_t S, int dtype, oslo_stream_t stream);
+
 /* Scale + key/padding mask + softmax -------------------------------------- */
 
 /*

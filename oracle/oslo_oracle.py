@@ -64,8 +64,10 @@ def _softmax_lastdim(e):
     return p / np.sum(p, axis=-1, keepdims=True, dtype=e.dtype)
 
 
-def softmax_causal(x, scale, pad_add=None, dtype=np.float32):
-    """x [B,H,S,S]; pad_add None or [B,S] additive. Row r attends keys 0..r."""
+def softmax_causal(x, scale, pad_add=None, dtype=np.float32, window=None):
+    """x [B,H,S,S]; pad_add None or [B,S] additive. Row r attends keys 0..r, or,
+    with a window, the keys max(0, r-window+1)..r of GPT-Neo's local attention
+    (oslo/models/gpt_neo/modeling_gpt_neo.py:153-163)."""
     t = _acc(dtype)
     x = np.asarray(x, dtype=dtype)
     b, h, s, s2 = x.shape
@@ -74,6 +76,8 @@ def softmax_causal(x, scale, pad_add=None, dtype=np.float32):
     if pad_add is not None:
         e = e + np.asarray(pad_add, dtype=dtype)[:, None, None, :]  # ... then the mask
     keep = np.tril(np.ones((s, s), dtype=bool))
+    if window is not None:
+        keep &= ~np.tril(np.ones((s, s), dtype=bool), -int(window))
     e = np.where(keep, e, t(-np.inf))
     return _softmax_lastdim(e)
 
@@ -95,15 +99,18 @@ def softmax_masked(x, mask, scale, mode="add", dtype=np.float32):
     return _softmax_lastdim(e)
 
 
-def softmax_bwd(g, y, scale, causal=False, dtype=np.float32):
-    """dx = scale * (g*y - y * sum_k(g*y)); with causal=True only k <= r takes
-    part and dx is 0 above the diagonal. g, y: [..., Sq, Sk]."""
+def softmax_bwd(g, y, scale, causal=False, dtype=np.float32, window=None):
+    """dx = scale * (g*y - y * sum_k(g*y)); with causal=True only k <= r (and,
+    with a window, k > r - window) takes part and dx is 0 elsewhere.
+    g, y: [..., Sq, Sk]."""
     t = _acc(dtype)
     g = np.asarray(g, dtype=dtype)
     y = np.asarray(y, dtype=dtype)
     if causal:
         s = y.shape[-1]
         keep = np.tril(np.ones((s, s), dtype=bool))
+        if window is not None:
+            keep &= ~np.tril(np.ones((s, s), dtype=bool), -int(window))
         g = np.where(keep, g, t(0))
         y = np.where(keep, y, t(0))
     gy = g * y

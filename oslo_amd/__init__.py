@@ -14,6 +14,7 @@ from .fused_kernels_utils import (  # noqa: F401
     FusedRotaryPositionEmbedding,
     FusedScaleMaskSoftmax,
     FusedScaleMaskSoftmaxDropout,
+    FusedScaleMaskWindowSoftmax,
     ScaledMaskedSoftmaxFunction,
     ScaledUpperTriangMaskedSoftmaxFunction,
     get_custom_kernels,

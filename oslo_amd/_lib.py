@@ -28,6 +28,10 @@ PROTOTYPES = {
         _c.c_int, [_P, _P, _P, _P, _c.c_float, _c.c_float, _U64, _U64, _I64, _I64, _I64, _c.c_int, _P]),
     "oslo_softmax_causal_dropout_bwd": (
         _c.c_int, [_P, _P, _P, _P, _P, _c.c_float, _c.c_float, _U64, _U64, _I64, _I64, _I64, _c.c_int, _P]),
+    "oslo_softmax_causal_window_fwd": (
+        _c.c_int, [_P, _P, _P, _c.c_float, _I64, _I64, _I64, _I64, _c.c_int, _P]),
+    "oslo_softmax_causal_window_bwd": (
+        _c.c_int, [_P, _P, _P, _c.c_float, _I64, _I64, _I64, _c.c_int, _P]),
     "oslo_softmax_masked_fwd": (
         _c.c_int, [_P, _P, _P, _I64, _I64, _c.c_int, _c.c_float,
                    _I64, _I64, _I64, _I64, _c.c_int, _P]),

@@ -22,6 +22,7 @@ SOURCES = [
     "runtime.hip",
     "softmax_causal.hip",
     "softmax_masked.hip",
+    "softmax_window.hip",
     "bias_gelu.hip",
     "bias_dropout_add.hip",
     "ngram_repeat_block.hip",

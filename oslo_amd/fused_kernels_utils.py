@@ -139,6 +139,25 @@ class _KeyMaskedSoftmax(torch.autograd.Function):
         return dx, None, None
 
 
+class _CausalWindowSoftmax(torch.autograd.Function):
+    """Sliding-window causal softmax of [B,H,S,S] scores, optional fp32 additive
+    key mask [B,S] applied inside the kernel."""
+
+    @staticmethod
+    def forward(ctx, inputs, pad_add, scale, window):
+        y = get_custom_kernels().causal_window_softmax_forward(inputs, pad_add, scale, window)
+        ctx.save_for_backward(y)
+        ctx.args = (float(scale), int(window))
+        return y
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        (y,) = ctx.saved_tensors
+        scale, window = ctx.args
+        dx = get_custom_kernels().causal_window_softmax_backward(output_grads, y, scale, window)
+        return dx, None, None, None
+
+
 class _CausalSoftmaxDropout(torch.autograd.Function):
     """Causal softmax of [B,H,S,S] scores followed by dropout of the
     probabilities, one kernel each way. Only the dropped probabilities are
@@ -242,6 +261,29 @@ class FusedScaleMaskSoftmax(object):
         if use_triang_mask:
             return sq == sk
         return True
+
+
+class FusedScaleMaskWindowSoftmax(object):
+    """
+    Kernel fusion function: Scale + sliding-window causal Mask + Softmax
+
+    Not in the reference, which leaves GPT-Neo's local attention layers on the
+    unfused path (oslo/models/gpt_neo/modeling_gpt_neo.py:268-272). ``apply``
+    is FusedScaleMaskSoftmax.apply with use_triang_mask=True and one more
+    argument: row r attends the keys max(0, r-window+1) .. r, the band
+    ``tril(ones) xor tril(ones, -window)`` of :153-163.
+    """
+
+    @staticmethod
+    def apply(input, pad_mask, scale, window):
+        bsz, np, sq, sk = input.size()
+        scale = scale if scale is not None else 1.0
+        pad_add = None if pad_mask is None else _pad_additive_f32(pad_mask, bsz, sk)
+        return _CausalWindowSoftmax.apply(input, pad_add, scale, window)
+
+    @staticmethod
+    def is_available(dtype, bsz, np, sq, sk, window):
+        return window >= 1 and FusedScaleMaskSoftmax.is_available(dtype, bsz, np, sq, sk, True)
 
 
 class FusedScaleMaskSoftmaxDropout(object):

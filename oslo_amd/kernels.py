@@ -157,6 +157,39 @@ def causal_softmax_forward(input, pad_add, scale_factor):
     return y
 
 
+def causal_window_softmax_forward(input, pad_add, scale_factor, window):
+    """input [B,H,S,S]; row r attends the keys max(0, r-window+1) .. r."""
+    _device_tensor(input, "input")
+    _require(input.dim() == 4, "expected 4D tensor")
+    code = _dtype_code(input, "input")
+    b, h, sq, sk = input.shape
+    _require(sq == sk, "causal softmax needs square score matrices")
+    x = input.contiguous()
+    pad_add = _pad_add_arg(pad_add, b, sk, input)
+    y = torch.empty_like(x, requires_grad=False)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().oslo_softmax_causal_window_fwd(
+            _ptr(y), _ptr(x), _ptr(pad_add), float(scale_factor), int(window), b, h, sk, code, _stream(x)))
+    return y
+
+
+def causal_window_softmax_backward(output_grads, softmax_results, scale_factor, window):
+    """[B,H,S,S] gradients; written over ``output_grads`` when it is contiguous."""
+    _device_tensor(output_grads, "output_grads")
+    _device_tensor(softmax_results, "softmax_results", output_grads)
+    code = _dtype_code(output_grads, "output_grads")
+    _require(softmax_results.dtype == output_grads.dtype and softmax_results.shape == output_grads.shape,
+             "output_grads and softmax_results differ in dtype or shape")
+    _require(output_grads.dim() == 4 and output_grads.shape[-1] == output_grads.shape[-2], "expected [B,H,S,S]")
+    b, h, s, _ = output_grads.shape
+    g = output_grads.contiguous()
+    y = softmax_results.contiguous()
+    with torch.cuda.device(g.device):
+        _lib.check(_lib.load().oslo_softmax_causal_window_bwd(
+            _ptr(g), _ptr(g), _ptr(y), float(scale_factor), int(window), b * h, s, code, _stream(g)))
+    return g
+
+
 def _pad_add_arg(pad_add, b, sk, like):
     if pad_add is None:
         return None

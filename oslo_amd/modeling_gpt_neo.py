@@ -5,9 +5,10 @@ modules compute (oslo/models/gpt_neo/modeling_gpt_neo.py:145-329): unscaled
 scores, fp32 softmax, global or sliding-window ("local") causal masks.
 ``FusedGPTNeoSelfAttention`` / ``FusedGPTNeoMLP`` are what ``fuse()`` swaps in
 (oslo/models/gpt_neo/modeling_gpt_neo.py:993-1102). As in the reference, local
-attention layers are a separate class, so ``fuse()``'s exact-class match leaves
-them unfused (their mask is not a plain lower triangle;
-oslo/models/gpt_neo/modeling_gpt_neo.py:268-272)."""
+attention layers are a separate class
+(oslo/models/gpt_neo/modeling_gpt_neo.py:268-272); the reference leaves them
+unfused because their mask is not a plain lower triangle, here they get a fused
+class of their own on the sliding-window softmax kernel."""
 
 from dataclasses import dataclass, field
 from typing import List, Optional
@@ -16,7 +17,7 @@ import torch
 from torch import nn
 
 from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax,
-                                 FusedScaleMaskSoftmaxDropout)
+                                 FusedScaleMaskSoftmaxDropout, FusedScaleMaskWindowSoftmax)
 from .modeling_utils import ACT2FN, LayerPolicy, PreTrainedModel, additive_attention_mask, causal_lm_loss
 
 
@@ -132,6 +133,19 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
         return (out, present, w) if output_attentions else (out, present)
 
 
+class FusedGPTNeoLocalSelfAttention(FusedGPTNeoSelfAttention, GPTNeoLocalSelfAttention):
+    """The fused attention on the sliding-window kernel: row r attends the last
+    ``window_size`` keys up to r. No counterpart in the reference."""
+
+    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
+        w = torch.matmul(query, key.transpose(-1, -2))
+        w = FusedScaleMaskWindowSoftmax.apply(w, attention_mask, None, self.config.window_size)
+        w = self.attn_dropout(w.to(value.dtype))
+        if head_mask is not None:
+            w = w * head_mask
+        return torch.matmul(w, value), w
+
+
 class GPTNeoAttention(nn.Module):
     def __init__(self, config, layer_id=0):
         super().__init__()
@@ -193,7 +207,8 @@ class GPTNeoLayerPolicy(LayerPolicy):
 
     @staticmethod
     def fused_modules():
-        return {GPTNeoSelfAttention: FusedGPTNeoSelfAttention, GPTNeoMLP: FusedGPTNeoMLP}
+        return {GPTNeoSelfAttention: FusedGPTNeoSelfAttention, GPTNeoMLP: FusedGPTNeoMLP,
+                GPTNeoLocalSelfAttention: FusedGPTNeoLocalSelfAttention}
 
 
 class GPTNeoModel(nn.Module):

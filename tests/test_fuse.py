@@ -124,8 +124,13 @@ def test_fuse_modules_filter_and_errors():
         Plain(None).fuse()
 
 
-def test_gpt_neo_local_attention_is_not_fused():
+def test_gpt_neo_local_attention_has_a_fused_class_of_its_own():
     m = tiny_neo().fuse()
+    kinds = [type(b.attn.attention) for b in m.transformer.h]
+    assert kinds == [modeling_gpt_neo.FusedGPTNeoSelfAttention, modeling_gpt_neo.FusedGPTNeoLocalSelfAttention]
+    assert isinstance(m.transformer.h[1].attn.attention, modeling_gpt_neo.GPTNeoLocalSelfAttention)
+    # the reference's behaviour (local layers left alone) is one filter away
+    m = tiny_neo().fuse(modules=[modeling_gpt_neo.GPTNeoSelfAttention, modeling_gpt_neo.GPTNeoMLP])
     kinds = [type(b.attn.attention) for b in m.transformer.h]
     assert kinds == [modeling_gpt_neo.FusedGPTNeoSelfAttention, modeling_gpt_neo.GPTNeoLocalSelfAttention]
 

@@ -380,3 +380,28 @@ def test_rotary_matches_the_torch_restatement_of_the_unfused_attention():
     want = torch.cat([apply_rotary(x[..., :rot], sin_t, cos_t, off), x[..., rot:]], dim=-1).permute(0, 2, 1, 3)
     got = orc.rotary_split_heads(x.numpy(), sin_t.numpy(), cos_t.numpy(), rot, offset=off)
     assert np.array_equal(got, want.numpy())   # same tables -> the same fp32 operations, bit for bit
+
+
+def test_window_softmax_is_torch_softmax_over_the_local_attention_band():
+    """GPT-Neo's local mask, built the way the unfused attention builds it:
+    tril(ones) xor tril(ones, -window), where(mask, w, -1e9), softmax."""
+    torch.manual_seed(8)
+    b, h, s, window = 2, 2, 23, 5
+    x = torch.randn(b, h, s, s) * 3
+    ones = torch.tril(torch.ones(s, s, dtype=torch.uint8))
+    band = torch.bitwise_xor(ones, torch.tril(ones, -window)).bool()
+    assert band[10].nonzero().flatten().tolist() == [6, 7, 8, 9, 10]          # keys r-window+1 .. r
+    want = torch.softmax(torch.where(band, x * 0.7, torch.tensor(-1e9)), -1)
+    got = orc.softmax_causal(x.numpy(), 0.7, window=window)
+    np.testing.assert_allclose(got, want.numpy(), atol=1e-6)
+    assert (got[..., ~band.numpy()] == 0).all()
+    # window >= S is the plain causal softmax; window = 1 is the identity on the diagonal
+    assert np.array_equal(orc.softmax_causal(x.numpy(), 0.7, window=s), orc.softmax_causal(x.numpy(), 0.7))
+    assert np.array_equal(orc.softmax_causal(x.numpy(), 0.7, window=1)[0, 0], np.eye(s, dtype=np.float32))
+    # backward against autograd through the same expression
+    xt = x.clone().double().requires_grad_(True)
+    y = torch.softmax(torch.where(band, xt * 0.7, torch.tensor(-1e9, dtype=torch.float64)), -1)
+    go = torch.randn(b, h, s, s, dtype=torch.float64)
+    (gx,) = torch.autograd.grad(y, xt, go)
+    got_dx = orc.softmax_bwd(go.numpy(), y.detach().numpy(), 0.7, causal=True, dtype=np.float64, window=window)
+    np.testing.assert_allclose(got_dx, gx.numpy(), atol=1e-12)

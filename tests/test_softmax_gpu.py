@@ -252,3 +252,36 @@ def test_causal_softmax_with_fused_dropout(s, dtype, with_pad):
     # p == 0: the plain probabilities
     yd0, _ = kernels.causal_softmax_dropout_forward(x_dev, pad_dev, 0.125, 0.0, 0, 0)
     assert torch.equal(yd0, kernels.causal_softmax_forward(x_dev, pad_dev, 0.125))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("s,window", [(5, 2), (64, 1), (64, 64), (130, 7), (512, 256), (1000, 256), (1001, 33),
+                                      (2048, 256), (2048, 2047), (4096, 256), (8192, 256)])
+@pytest.mark.parametrize("with_pad", [False, True], ids=["nopad", "pad"])
+def test_window_softmax_forward_backward(s, window, dtype, with_pad):
+    """Sliding-window causal softmax (GPT-Neo's local attention) against the
+    oracle, forward and backward; zero outside the band; NaNs outside the band
+    are never read."""
+    b, h = (2, 2) if s <= 2048 else (1, 1)
+    x = randn((b, h, s, s), dtype, seed=s + window, std=8.0)
+    band = np.tril(np.ones((s, s), dtype=bool)) & ~np.tril(np.ones((s, s), dtype=bool), -window)
+    pad = None
+    if with_pad:
+        lens = torch.randint(1, s + 1, (b,), generator=torch.Generator().manual_seed(3))
+        pad = torch.where(torch.arange(s)[None, :] < lens[:, None], 0.0, -10000.0).float()
+    want = orc.softmax_causal(f32(x), 0.125, None if pad is None else pad.numpy(), window=window)
+    poisoned = x.clone()
+    poisoned[..., torch.from_numpy(~band)] = float("nan")
+    y = kernels.causal_window_softmax_forward(poisoned.to(DEV), None if pad is None else pad.to(DEV), 0.125, window)
+    assert_close(y, want, dtype, f"window softmax S={s} W={window}")
+    assert (f32(y)[..., ~band] == 0).all()
+    check_rowsums(y, dtype, want)
+    g = randn((b, h, s, s), dtype, seed=s + window + 1)
+    want_dx = orc.softmax_bwd(f32(g), f32(y), 0.125, causal=True, window=window)
+    gp = g.clone()
+    gp[..., torch.from_numpy(~band)] = float("nan")
+    dx = kernels.causal_window_softmax_backward(gp.to(DEV), y, 0.125, window)
+    assert_close(dx, want_dx, dtype, f"window softmax bwd S={s} W={window}")
+    assert (f32(dx)[..., ~band] == 0).all()
+    if window >= s:   # the plain causal kernel
+        assert torch.equal(y, kernels.causal_softmax_forward(x.to(DEV), None if pad is None else pad.to(DEV), 0.125))
