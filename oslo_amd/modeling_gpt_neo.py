@@ -16,7 +16,8 @@ from typing import List, Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax,
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedMergeHeads,
+                                 FusedRotaryPositionEmbedding, FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedScaleMaskWindowSoftmax)
 from .modeling_utils import ACT2FN, LayerPolicy, PreTrainedModel, additive_attention_mask, causal_lm_loss
 
@@ -108,7 +109,27 @@ class GPTNeoLocalSelfAttention(GPTNeoSelfAttention):
 
 
 class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
-    """oslo/models/gpt_neo/modeling_gpt_neo.py:993-1075."""
+    """oslo/models/gpt_neo/modeling_gpt_neo.py:993-1075. Beyond the reference's
+    fused class, the split-heads permutes of q, k, v and the merge-heads
+    permute run through the transposition kernel (one launch for q, k and v)
+    instead of torch's strided copies."""
+
+    def _transposes_fused(self, t):
+        return t.is_cuda and FusedRotaryPositionEmbedding.is_available(t.dtype, self.head_dim, 0)
+
+    def _project_qkv(self, hidden_states, layer_past, use_cache):
+        if not self._transposes_fused(hidden_states):
+            return super()._project_qkv(hidden_states, layer_past, use_cache)
+        b, s, _ = hidden_states.shape
+        shape = (b, s, self.num_heads, self.head_dim)
+        query, key, value = FusedRotaryPositionEmbedding.apply(
+            self.q_proj(hidden_states).view(shape), self.k_proj(hidden_states).view(shape),
+            self.v_proj(hidden_states).view(shape), (None, None), 0)
+        if layer_past is not None:
+            key = torch.cat((layer_past[0], key), dim=-2)
+            value = torch.cat((layer_past[1], value), dim=-2)
+        present = (key, value) if use_cache else None
+        return query, key, value, present
 
     def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
         w = torch.matmul(query, key.transpose(-1, -2))
@@ -128,7 +149,8 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask)
         else:
             out, w = self._attn(query, key, value, attention_mask, head_mask)
-        out = self._merge_heads(out) @ self.out_proj.weight.t()
+        out = FusedMergeHeads.apply(out) if self._transposes_fused(out) else self._merge_heads(out)
+        out = out @ self.out_proj.weight.t()
         out = FusedBiasDropout.apply(out, self.out_proj.bias, self.training, self.resid_dropout.p)
         return (out, present, w) if output_attentions else (out, present)
 
