@@ -306,7 +306,7 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
     from oslo_amd.modeling_gptj import rotary_tables
     sin, cos = rotary_tables(rot, S, dev)
     t = time_launches(lambda: check(lib.oslo_rotary_qkv(P(qo), P(ko), P(vo), P(q), P(k), P(v), P(sin), P(cos),
-                                                        S, B, S, H, D, rot, 0, 0, BF16, st)), n, 3)
+                                                        S, B, S, H, D, 0, rot, 0, 0, BF16, st)), n, 3)
     res.append(roof("rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64", 3 * 4 * q.numel(), t, 3 * q.numel()))
     return res
 

@@ -274,6 +274,12 @@ int oslo_bias_dropout_add_bwd(void *dx, void *dbias, float *workspace,
  * *_in are then [batch, heads, seq, head_dim] gradients, *_out
  * [batch, seq, heads, head_dim], rotation by the opposite angle. head_dim must
  * be a multiple of 16 bytes, rotary_dim even; no output may alias an input.
+ * row_stride is the distance, in elements, between consecutive positions of
+ * the [batch, seq, heads, head_dim] side (its batch stride is seq*row_stride):
+ * 0 or heads*head_dim for a dense tensor, 3*heads*head_dim when q, k and v are
+ * the three slices of one packed [batch, seq, 3*hidden] projection, as in
+ * GPT-2's c_attn (oslo/models/gpt2/modeling_gpt2.py:176-183, :300-306). The
+ * [batch, heads, seq, head_dim] side is always dense.
  * Replaces fixed_pos_embedding / rotate_every_two / apply_rotary_pos_emb, the
  * torch.cat of rotated and passed-through features and the permute of
  * GPTJAttention.forward (oslo/models/gptj/modeling_gptj.py:49-80, :205-233).
@@ -282,8 +288,8 @@ int oslo_rotary_qkv(void *q_out, void *k_out, void *v_out, const void *q_in,
                     const void *k_in, const void *v_in, const float *sin_table,
                     const float *cos_table, int64_t table_positions,
                     int64_t batch, int64_t seq, int64_t heads, int64_t head_dim,
-                    int64_t rotary_dim, int64_t offset, int inverse, int dtype,
-                    oslo_stream_t stream);
+                    int64_t row_stride, int64_t rotary_dim, int64_t offset,
+                    int inverse, int dtype, oslo_stream_t stream);
 
 /* Repeated n-gram blocking (beam search) ------------------------------------ */
 

@@ -13,6 +13,7 @@ from .fused_kernels_utils import (  # noqa: F401
     FusedNoRepeatNGramLogitsProcessor,
     FusedRotaryPositionEmbedding,
     FusedScaleMaskSoftmax,
+    FusedSplitHeads,
     FusedScaleMaskSoftmaxDropout,
     FusedScaleMaskWindowSoftmax,
     ScaledMaskedSoftmaxFunction,

@@ -47,7 +47,7 @@ PROTOTYPES = {
     "oslo_bias_dropout_add_bwd": (
         _c.c_int, [_P, _P, _P, _P, _c.c_float, _U64, _U64, _I64, _I64, _c.c_int, _P]),
     "oslo_rotary_qkv": (
-        _c.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
+        _c.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                    _c.c_int, _c.c_int, _P]),
     "oslo_ngram_repeat_block": (
         _c.c_int, [_P, _P, _I64, _I64, _I64, _I64, _c.c_int, _P]),

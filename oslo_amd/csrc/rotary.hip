@@ -42,8 +42,8 @@ struct RotaryArgs {
 template <typename T, int VEC, bool INVERSE, bool TABLE_VEC>
 __global__ __launch_bounds__(kBlockThreads) void rotary_transpose_kernel(
     RotaryArgs a, const float *__restrict__ sin_t, const float *__restrict__ cos_t,
-    int S, int H, int D, int rotary_dim, int offset, int ts, int items_per_tile,
-    int blocks_per_tile, int s_tiles) {
+    int S, int H, int D, int64_t row_stride, int rotary_dim, int offset, int ts,
+    int items_per_tile, int blocks_per_tile, int s_tiles) {
   const int which = blockIdx.y;
   const T *in = static_cast<const T *>(a.in[which]);
   T *out = static_cast<T *>(a.out[which]);
@@ -55,11 +55,18 @@ __global__ __launch_bounds__(kBlockThreads) void rotary_transpose_kernel(
   const int s0 = (tile - b * s_tiles) * ts;
   const int lpr = D / VEC; // lanes per D-row
 
-  // [B,S,H,D] side and [B,H,S,D] side of batch b
-  const int64_t slab = (int64_t)S * H * D;
-  const uint32_t slab_bytes = (uint32_t)slab * (uint32_t)sizeof(T);
-  const BufRsrc irs = make_rsrc(in + b * slab, slab_bytes);
-  const BufRsrc ors = make_rsrc(out + b * slab, slab_bytes);
+  // [B,S,H,D] side (a position every row_stride elements: H*D when dense, more
+  // when q, k, v are slices of one packed projection) and dense [B,H,S,D] side
+  // of batch b
+  const int64_t dense_slab = (int64_t)S * H * D;
+  const int64_t strided_slab = (int64_t)S * row_stride;
+  const uint32_t dense_bytes = (uint32_t)dense_slab * (uint32_t)sizeof(T);
+  const uint32_t strided_bytes =
+      (uint32_t)((int64_t)(S - 1) * row_stride + (int64_t)H * D) * (uint32_t)sizeof(T);
+  const BufRsrc irs = make_rsrc(in + b * (INVERSE ? dense_slab : strided_slab),
+                                INVERSE ? dense_bytes : strided_bytes);
+  const BufRsrc ors = make_rsrc(out + b * (INVERSE ? strided_slab : dense_slab),
+                                INVERSE ? strided_bytes : dense_bytes);
 
   RawVec<T, VEC> raw[kRotaryUnroll];
   uint32_t off_out[kRotaryUnroll];
@@ -75,7 +82,7 @@ __global__ __launch_bounds__(kBlockThreads) void rotary_transpose_kernel(
     const bool ok = item < items_per_tile && s < S;
     col[u] = d8 * VEC;
     pos[u] = (ok ? s : 0) + offset; // a table row that exists
-    const uint32_t bshd = (uint32_t)(((int64_t)s * H + h) * D + col[u]) * (uint32_t)sizeof(T);
+    const uint32_t bshd = (uint32_t)((int64_t)s * row_stride + h * D + col[u]) * (uint32_t)sizeof(T);
     const uint32_t bhsd = (uint32_t)(((int64_t)h * S + s) * D + col[u]) * (uint32_t)sizeof(T);
     const uint32_t off_in = ok ? (INVERSE ? bhsd : bshd) : kOutside;
     off_out[u] = ok ? (INVERSE ? bshd : bhsd) : kOutside;
@@ -136,8 +143,8 @@ __global__ __launch_bounds__(kBlockThreads) void rotary_transpose_kernel(
 
 template <typename T>
 int launch_rotary(const RotaryArgs &a, const float *sin_t, const float *cos_t,
-                  int64_t B, int64_t S, int64_t H, int64_t D, int64_t rotary_dim,
-                  int64_t offset, bool inverse, hipStream_t stream) {
+                  int64_t B, int64_t S, int64_t H, int64_t D, int64_t row_stride,
+                  int64_t rotary_dim, int64_t offset, bool inverse, hipStream_t stream) {
   constexpr int VEC = Io<T>::kVec;
   const int lpr = (int)(D / VEC);
   // positions per tile: enough for a wave to cover whole D-rows, at least 8
@@ -156,8 +163,8 @@ int launch_rotary(const RotaryArgs &a, const float *sin_t, const float *cos_t,
   auto go = [&]<bool INVERSE, bool TABLE_VEC>() {
     rotary_transpose_kernel<T, VEC, INVERSE, TABLE_VEC>
         <<<grid, dim3(kBlockThreads), 0, stream>>>(
-            a, sin_t, cos_t, (int)S, (int)H, (int)D, (int)rotary_dim, (int)offset, ts,
-            (int)items_per_tile, blocks_per_tile, s_tiles);
+            a, sin_t, cos_t, (int)S, (int)H, (int)D, row_stride, (int)rotary_dim, (int)offset,
+            ts, (int)items_per_tile, blocks_per_tile, s_tiles);
   };
   if (inverse) {
     if (table_vec) go.template operator()<true, true>();
@@ -176,12 +183,13 @@ extern "C" int oslo_rotary_qkv(void *q_out, void *k_out, void *v_out,
                                const void *q_in, const void *k_in, const void *v_in,
                                const float *sin_table, const float *cos_table,
                                int64_t table_positions, int64_t batch, int64_t seq,
-                               int64_t heads, int64_t head_dim, int64_t rotary_dim,
-                               int64_t offset, int inverse, int dtype,
+                               int64_t heads, int64_t head_dim, int64_t row_stride,
+                               int64_t rotary_dim, int64_t offset, int inverse, int dtype,
                                oslo_stream_t stream) {
   using namespace oslo;
   const char *name = "rotary_qkv";
-  if (batch < 0 || seq < 0 || heads < 0 || head_dim < 0 || rotary_dim < 0 || offset < 0)
+  if (batch < 0 || seq < 0 || heads < 0 || head_dim < 0 || row_stride < 0 || rotary_dim < 0 ||
+      offset < 0)
     return fail(OSLO_E_BAD_ARG, "%s: negative size", name);
   if (rotary_dim > head_dim || rotary_dim % 2 != 0)
     return fail(OSLO_E_BAD_ARG, "%s: rotary_dim %lld must be even and <= head_dim %lld", name,
@@ -194,7 +202,11 @@ extern "C" int oslo_rotary_qkv(void *q_out, void *k_out, void *v_out,
   if (head_dim % vec != 0)
     return fail(OSLO_E_UNSUPPORTED, "%s: head_dim %lld is not a multiple of %lld", name,
                 (long long)head_dim, (long long)vec);
-  if (seq > INT32_MAX / (heads * head_dim) || seq * heads * head_dim * es >= (int64_t)kOutside)
+  if (row_stride == 0) row_stride = heads * head_dim; // dense
+  if (row_stride < heads * head_dim || row_stride % vec != 0)
+    return fail(OSLO_E_BAD_ARG, "%s: row_stride %lld must be a multiple of %lld and at least heads*head_dim",
+                name, (long long)row_stride, (long long)vec);
+  if (seq > INT32_MAX / row_stride || seq * row_stride * es >= (int64_t)kOutside)
     return fail(OSLO_E_UNSUPPORTED, "%s: one batch entry must stay under 2 GiB", name);
   RotaryArgs a{};
   const void *ins[3] = {q_in, k_in, v_in};
@@ -220,7 +232,8 @@ extern "C" int oslo_rotary_qkv(void *q_out, void *k_out, void *v_out,
                   (long long)offset, (long long)(offset + seq - 1), (long long)table_positions);
   }
   OSLO_DISPATCH_DTYPE(dtype, return launch_rotary<T>(a, sin_table, cos_table, batch, seq, heads,
-                                                     head_dim, rotary_dim, offset, inverse != 0,
+                                                     head_dim, row_stride, rotary_dim, offset,
+                                                     inverse != 0,
                                                      static_cast<hipStream_t>(stream)));
   return OSLO_OK;
 }

@@ -384,6 +384,31 @@ class FusedMergeHeads(object):
         return _MergeHeads.apply(x).view(b, s, h * d)
 
 
+class _SplitHeadsPacked(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, qkv, heads):
+        return get_custom_kernels().split_heads_packed_forward(qkv, heads)
+
+    @staticmethod
+    def backward(ctx, grad_query, grad_key, grad_value):
+        return get_custom_kernels().split_heads_packed_backward(grad_query, grad_key, grad_value), None
+
+
+class FusedSplitHeads(object):
+    """[B, S, 3*H*D] packed q|k|v projection -> query, key, value as contiguous
+    [B, H, S, D]: GPT-2's ``split(split_size, dim=2)`` and three
+    ``_split_heads`` permutes (oslo/models/gpt2/modeling_gpt2.py:300-306,
+    :176-183) in one pass of the transposition kernel, forward and backward."""
+
+    @staticmethod
+    def apply(qkv, heads):
+        return _SplitHeadsPacked.apply(qkv, heads)
+
+    @staticmethod
+    def is_available(dtype, head_dim):
+        return FusedRotaryPositionEmbedding.is_available(dtype, head_dim, 0)
+
+
 # ---------------------------------------------------------------------------
 # bias + GeLU
 # ---------------------------------------------------------------------------

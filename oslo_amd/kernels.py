@@ -395,7 +395,7 @@ def _rotary_call(tensors, sin, cos, rotary_dim, offset, inverse):
     with torch.cuda.device(first.device):
         _lib.check(_lib.load().oslo_rotary_qkv(
             _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _ptr(ins[0]), _ptr(ins[1]), _ptr(ins[2]),
-            _ptr(sin), _ptr(cos), positions, b, s, h, d, int(rotary_dim), int(offset),
+            _ptr(sin), _ptr(cos), positions, b, s, h, d, 0, int(rotary_dim), int(offset),
             1 if inverse else 0, code, _stream(first)))
     return tuple(outs)
 
@@ -412,3 +412,47 @@ def rotary_qkv_backward(grad_query, grad_key, grad_value, sin, cos, rotary_dim, 
     """Gradients [B, H, S, D] of rotary_qkv_forward's outputs -> gradients
     [B, S, H, D] of its inputs."""
     return _rotary_call((grad_query, grad_key, grad_value), sin, cos, rotary_dim, offset, inverse=True)
+
+
+def split_heads_packed_forward(qkv, heads):
+    """qkv: [B, S, 3*H*D], the packed projection of GPT-2's c_attn
+    (oslo/models/gpt2/modeling_gpt2.py:300-306). Returns query, key and value as
+    contiguous [B, H, S, D]: the split and the three split-heads permutes in one
+    launch, reading the slices in place."""
+    _device_tensor(qkv, "qkv")
+    code = _dtype_code(qkv, "qkv")
+    _require(qkv.dim() == 3 and qkv.shape[2] % (3 * heads) == 0, "expected [B, S, 3*heads*head_dim]")
+    qkv = qkv.contiguous()
+    b, s, e3 = qkv.shape
+    e = e3 // 3
+    d = e // heads
+    outs = [torch.empty((b, heads, s, d), dtype=qkv.dtype, device=qkv.device) for _ in range(3)]
+    step = e * qkv.element_size()
+    ins = [ctypes.c_void_p(qkv.data_ptr() + i * step) for i in range(3)]
+    with torch.cuda.device(qkv.device):
+        _lib.check(_lib.load().oslo_rotary_qkv(
+            _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), ins[0], ins[1], ins[2], None, None, 0,
+            b, s, heads, d, e3, 0, 0, 0, code, _stream(qkv)))
+    return tuple(outs)
+
+
+def split_heads_packed_backward(grad_query, grad_key, grad_value):
+    """Gradients [B, H, S, D] of split_heads_packed_forward's outputs -> the
+    gradient [B, S, 3*H*D] of the packed projection."""
+    grads = []
+    for t in (grad_query, grad_key, grad_value):
+        _device_tensor(t, "gradient", grad_query)
+        _require(t.shape == grad_query.shape and t.dtype == grad_query.dtype and t.dim() == 4,
+                 "gradients differ in shape or dtype")
+        grads.append(t.contiguous())
+    code = _dtype_code(grad_query, "gradient")
+    b, h, s, d = grad_query.shape
+    e = h * d
+    out = torch.empty((b, s, 3 * e), dtype=grad_query.dtype, device=grad_query.device)
+    step = e * out.element_size()
+    outs = [ctypes.c_void_p(out.data_ptr() + i * step) for i in range(3)]
+    with torch.cuda.device(out.device):
+        _lib.check(_lib.load().oslo_rotary_qkv(
+            outs[0], outs[1], outs[2], _ptr(grads[0]), _ptr(grads[1]), _ptr(grads[2]), None, None, 0,
+            b, s, h, d, 3 * e, 0, 0, 1, code, _stream(out)))
+    return out

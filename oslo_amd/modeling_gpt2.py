@@ -13,8 +13,8 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedScaleMaskSoftmax,
-                                 FusedScaleMaskSoftmaxDropout)
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedMergeHeads, FusedScaleMaskSoftmax,
+                                 FusedScaleMaskSoftmaxDropout, FusedSplitHeads)
 from .modeling_utils import (ACT2FN, Conv1D, LayerPolicy, PreTrainedModel, additive_attention_mask,
                              causal_lm_loss)
 
@@ -142,7 +142,21 @@ class FusedGPT2Attention(GPT2Attention):
     """oslo/models/gpt2/modeling_gpt2.py:1434-1542. The reference's fused
     attention leaves out attn_dropout, which its unfused attention applies
     (:222); here it is applied, inside the softmax kernel, so that fused and
-    unfused training agree."""
+    unfused training agree. Beyond the reference's fused class, the split of the
+    packed c_attn projection with its three split-heads permutes, and the
+    merge-heads permute, run through the transposition kernel instead of torch's
+    strided copies."""
+
+    def _project_qkv(self, hidden_states, layer_past, encoder_hidden_states, use_cache):
+        if encoder_hidden_states is not None or not (
+                hidden_states.is_cuda and FusedSplitHeads.is_available(hidden_states.dtype, self.head_dim)):
+            return super()._project_qkv(hidden_states, layer_past, encoder_hidden_states, use_cache)
+        query, key, value = FusedSplitHeads.apply(self.c_attn(hidden_states), self.num_heads)
+        if layer_past is not None:
+            key = torch.cat((layer_past[0], key), dim=-2)
+            value = torch.cat((layer_past[1], value), dim=-2)
+        present = (key, value) if use_cache else None
+        return query, key, value, present
 
     def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
         w = torch.matmul(query, key.transpose(-1, -2))
@@ -165,7 +179,10 @@ class FusedGPT2Attention(GPT2Attention):
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask)
         else:
             out, w = self._attn(query, key, value, attention_mask, head_mask)
-        out = self._merge_heads(out, self.num_heads, self.head_dim)
+        if out.is_cuda and FusedSplitHeads.is_available(out.dtype, self.head_dim):
+            out = FusedMergeHeads.apply(out)
+        else:
+            out = self._merge_heads(out, self.num_heads, self.head_dim)
         out = out @ self.c_proj.weight  # projection without its bias ...
         out = FusedBiasDropout.apply(out, self.c_proj.bias, self.training, self.resid_dropout.p)  # ... fused here
         return (out, present, w) if output_attentions else (out, present)

@@ -93,14 +93,16 @@ def test_argument_screening_without_a_device(lib):
     # rotary: odd or oversized rotary_dim, head_dim not a multiple of the vector, table too short,
     # one pointer of a pair, in place
     two = ctypes.c_void_p(32)
-    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 3, 0, 0, 1, null) == -1
-    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 32, 0, 0, 1, null) == -1
-    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 12, 4, 0, 0, 1, null) == -2
-    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 4, 1, 0, 1, null) == -1
+    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 0, 3, 0, 0, 1, null) == -1
+    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 0, 32, 0, 0, 1, null) == -1
+    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 12, 0, 4, 0, 0, 1, null) == -2
+    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 0, 4, 1, 0, 1, null) == -1
     assert b"table" in lib.oslo_last_error()
-    assert lib.oslo_rotary_qkv(one, null, null, null, null, null, one, one, 8, 1, 8, 2, 16, 4, 0, 0, 1, null) == -1
-    assert lib.oslo_rotary_qkv(two, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 4, 0, 0, 1, null) == -1
-    assert lib.oslo_rotary_qkv(null, null, null, null, null, null, null, null, 0, 1, 8, 2, 16, 4, 0, 0, 1, null) == 0
+    assert lib.oslo_rotary_qkv(one, null, null, null, null, null, one, one, 8, 1, 8, 2, 16, 0, 4, 0, 0, 1, null) == -1
+    assert lib.oslo_rotary_qkv(two, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 0, 4, 0, 0, 1, null) == -1
+    assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 24, 4, 0, 0, 1, null) == -1
+    assert b"row_stride" in lib.oslo_last_error()      # smaller than heads*head_dim
+    assert lib.oslo_rotary_qkv(null, null, null, null, null, null, null, null, 0, 1, 8, 2, 16, 0, 4, 0, 0, 1, null) == 0
     # n-gram blocking
     assert lib.oslo_ngram_repeat_block(one, one, 2, 4, 3, 8, 0, null) == -1
     assert lib.oslo_ngram_repeat_block(null, one, 2, 4, 3, 8, 2, null) == -1

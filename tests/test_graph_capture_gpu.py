@@ -63,7 +63,7 @@ def test_captured_sequence_replays_like_eager():
             lib.oslo_bias_dropout_add_bwd(P(o["ddrop"]), P(o["dbias2"]), P(o["ws"]), P(ga), 0.1, 77, 12,
                                           rows, cols, BF16, st),
             lib.oslo_rotary_qkv(P(o["qo"]), None, None, P(q), None, None, P(sin), P(cos), s,
-                                bs, s, hs, d, rot, 0, 0, BF16, st),
+                                bs, s, hs, d, 0, rot, 0, 0, BF16, st),
         ]
         assert all(r == 0 for r in rc), lib.oslo_last_error().decode()
 

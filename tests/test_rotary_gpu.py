@@ -132,3 +132,24 @@ def test_merge_heads_operator():
     (gx,) = torch.autograd.grad(got, x, go)
     (gw,) = torch.autograd.grad(want, x, go)
     assert torch.equal(gx, gw)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+def test_split_heads_of_a_packed_projection(dtype):
+    """GPT-2's c_attn output [B, S, 3E]: the three slices are read in place
+    (row stride 3E) and come out as [B, H, S, D]; the backward writes the three
+    gradients back into one [B, S, 3E] tensor."""
+    from oslo_amd import FusedSplitHeads
+
+    torch.manual_seed(6)
+    b, s, h, d = 2, 19, 3, 16
+    e = h * d
+    qkv = torch.randn(b, s, 3 * e, device=DEV).to(dtype).requires_grad_(True)
+    outs = FusedSplitHeads.apply(qkv, h)
+    wants = [t.view(b, s, h, d).permute(0, 2, 1, 3) for t in qkv.split(e, dim=2)]
+    for got, want in zip(outs, wants):
+        assert got.is_contiguous() and torch.equal(got, want)
+    gos = [torch.randn(b, h, s, d, device=DEV).to(dtype) for _ in range(3)]
+    (g_got,) = torch.autograd.grad(outs, qkv, gos)
+    (g_want,) = torch.autograd.grad(wants, qkv, gos)
+    assert torch.equal(g_got, g_want)
