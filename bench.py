@@ -39,26 +39,26 @@ HBM_PEAK_GBPS = 8000.0
 # profiles/bench_kernels_hbm_traffic.md and, for the two kernels of the step,
 # profiles/causal_softmax_fp16_8x16x2048x2048_hbm_traffic.md.
 MEASURED_TRAFFIC = {
-    "causal_fwd fp16 [8,16,2048,2048]": 1627472076,
-    "causal_bwd fp16 [8,16,2048,2048]": 2181120204,
+    "causal_fwd fp16 [8,16,2048,2048]": 1627471872,
+    "causal_bwd fp16 [8,16,2048,2048]": 2181120000,
     "causal_fwd bf16 [8,16,2048,2048]": 1627472076,
     "causal_bwd bf16 [8,16,2048,2048] (in place)": 2181120204,
-    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635891200,
+    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635890995,
     "causal_dropout_bwd p=0.1 bf16 [8,16,2048,2048] (in place)": 2214719488,
     "causal_fwd fp32 [8,16,2048,2048]": 3238062284,
     "causal_bwd fp32 [8,16,2048,2048] (in place)": 4328582963,
     "causal_fwd bf16 [1,16,8192,8192]": 3229695590,
     "masked_fwd bf16 [16,16,1024,1024] key mask": 1073948672,
     "masked_bwd bf16 [16,16,1024,1024]": 1610650624,
-    "bias_gelu_fwd bf16 [16384,16384]": 1073873510,
-    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677932748,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610758758,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141058969,
+    "bias_gelu_fwd bf16 [16384,16384]": 1073871872,
+    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677933363,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610759168,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141059584,
     "bias_gelu_fwd bf16 [16384,4096]": 268489318,
-    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419568025,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402726297,
+    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419567820,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402726502,
     "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285348249,
-    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807780147,
+    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807997644,
 }
 
 
