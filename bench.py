@@ -550,9 +550,23 @@ def gpt2_small_forward(torch):
             model(dev_ids)
         torch.cuda.synchronize()
         t_gpu = (time.perf_counter() - t0) / 20
+        # the same forward captured once as a HIP graph and replayed
+        from oslo_amd import GraphedForward
+        graphed = GraphedForward(model, dev_ids)
+        for _ in range(3):
+            graph_logits = graphed(dev_ids)["logits"]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            graphed(dev_ids)
+        torch.cuda.synchronize()
+        t_graph = (time.perf_counter() - t0) / 20
     diff = (gpu_logits.cpu() - cpu_logits).abs().max().item()
     return {"cpu_unfused_tokens_per_s": round(2048 / t_cpu, 1), "cpu_cores": torch.get_num_threads(),
-            "gpu_fused_tokens_per_s": round(2048 / t_gpu, 1), "max_abs_logit_diff": round(diff, 6)}
+            "gpu_fused_tokens_per_s": round(2048 / t_gpu, 1),
+            "gpu_fused_graph_replay_tokens_per_s": round(2048 / t_graph, 1),
+            "graph_equals_eager": bool(torch.equal(graph_logits, gpu_logits)),
+            "max_abs_logit_diff": round(diff, 6)}
 
 
 if __name__ == "__main__":

@@ -20,6 +20,7 @@ from .fused_kernels_utils import (  # noqa: F401
     ScaledUpperTriangMaskedSoftmaxFunction,
     get_custom_kernels,
 )
+from .graphs import GraphedForward  # noqa: F401
 from .modeling_gpt2 import GPT2Config, GPT2LMHeadModel  # noqa: F401
 from .modeling_gpt_neo import GPTNeoConfig, GPTNeoForCausalLM  # noqa: F401
 from .modeling_gptj import GPTJConfig, GPTJForCausalLM  # noqa: F401

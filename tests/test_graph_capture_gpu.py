@@ -89,3 +89,44 @@ def test_captured_sequence_replays_like_eager():
                 continue
             assert torch.equal(captured[name], eager[name]), f"replay {replay}: {name} differs from eager"
             assert not torch.isnan(captured[name].float()).any(), f"replay {replay}: {name} not written"
+
+
+@pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
+def test_graphed_forward_of_a_fused_model(family):
+    """The whole fused forward captured once and replayed with new token ids and
+    padding masks; every replay equals the eager forward bit for bit, with eager
+    work between the replays."""
+    from oslo_amd import (GPT2Config, GPT2LMHeadModel, GPTJConfig, GPTJForCausalLM, GPTNeoConfig,
+                          GPTNeoForCausalLM, GraphedForward)
+
+    torch.manual_seed(0)
+    make = {
+        "gpt2": lambda: GPT2LMHeadModel(GPT2Config(vocab_size=512, n_positions=128, n_embd=128, n_layer=2, n_head=4)),
+        "gptj": lambda: GPTJForCausalLM(GPTJConfig(vocab_size=512, n_positions=128, n_embd=128, n_layer=2, n_head=4,
+                                                   rotary_dim=16)),
+        "gpt_neo": lambda: GPTNeoForCausalLM(GPTNeoConfig(vocab_size=512, max_position_embeddings=128,
+                                                          hidden_size=128, num_layers=2, num_heads=4,
+                                                          window_size=32)),
+    }[family]
+    model = make().half().to(DEV).eval().fuse()
+    b, s = 3, 96
+
+    def batch(seed):
+        g = torch.Generator(device=DEV).manual_seed(seed)
+        ids = torch.randint(0, 512, (b, s), device=DEV, generator=g)
+        lens = torch.randint(s // 2, s + 1, (b,), device=DEV, generator=g)
+        mask = (torch.arange(s, device=DEV)[None, :] < lens[:, None]).to(torch.int64)
+        return ids, mask
+
+    ids, mask = batch(1)
+    graphed = GraphedForward(model, ids, attention_mask=mask)
+    for replay in range(4):
+        ids, mask = batch(10 + replay)
+        got = graphed(ids, attention_mask=mask)["logits"].clone()
+        with torch.no_grad():
+            want = model(ids, attention_mask=mask)["logits"]      # eager work between replays
+        assert torch.equal(got, want), f"{family} replay {replay}"
+    with pytest.raises(RuntimeError, match="captured for"):
+        graphed(ids[:, :50], attention_mask=mask[:, :50])
+    with pytest.raises(RuntimeError, match="eval"):
+        GraphedForward(model.train(), ids, attention_mask=mask)
