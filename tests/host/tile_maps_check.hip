@@ -98,6 +98,23 @@ int main() {
     check_rows(9, 4, 10, paired);
     check_rows(1, 4, 2, paired);
   }
+  // a few hundred pseudo-random shapes on top of the hand-picked ones
+  uint64_t state = 0x9E3779B97F4A7C15ull;
+  auto next = [&](uint64_t n) {
+    state = state * 6364136223846793005ull + 1442695040888963407ull;
+    return (state >> 33) % n;
+  };
+  for (int i = 0; i < 300; ++i) {
+    const int64_t rows = 1 + (int64_t)next(5000);
+    const int vec = next(2) ? 8 : 4;
+    const int64_t cols = vec * (1 + (int64_t)next(700));
+    const int k = (int)next(3);
+    check_elementwise(rows, cols, vec, k == 0 ? kFwdMaxTx : kBwdMaxTx,
+                      k == 0 ? kFwdUnroll : (k == 1 ? 4 : 8));
+    const int rpb = 1 << next(3);                        // 1, 2 or 4 rows per block
+    const int64_t row_bytes = 16 * (1 + (int64_t)next(1024)); // up to 16 KiB
+    check_rows(1 + (int64_t)next(20000), rpb, row_bytes, next(2) != 0);
+  }
   if (failures == 0) std::printf("tile maps ok\n");
   return failures == 0 ? 0 : 1;
 }
