@@ -6,7 +6,6 @@ oracle/_ref holds a build of it."""
 
 import importlib.util
 import os
-import sys
 
 import numpy as np
 import pytest

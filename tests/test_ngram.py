@@ -2,7 +2,6 @@
 NoRepeatNGramLogitsProcessor (an independent implementation of the same rule)
 and a hand-worked case; the HIP kernel against the oracle."""
 
-import numpy as np
 import pytest
 import torch
 
