@@ -359,11 +359,28 @@ def gptj_forward(torch, dev, layers=28, batch=8, seq=2048, reps=5):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / reps
 
+    def decode_ms(context=1024, steps=20):
+        """One new token for one sequence over a key/value cache of `context`
+        tokens: milliseconds per step (bound by launches, not by the kernels)."""
+        with torch.no_grad():
+            past = model(ids[:1, :context], use_cache=True)["past_key_values"]
+            nxt = ids[:1, context - 1:context]
+            for _ in range(3):
+                model(nxt, past_key_values=past, use_cache=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                model(nxt, past_key_values=past, use_cache=True)
+            torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
     t_unfused = timed()
     ref_logits = run().float()
+    d_unfused = decode_ms()
     model.fuse()
     t_fused = timed()
     diff = (run().float() - ref_logits).abs().max().item()
+    d_fused = decode_ms()
     del model, ref_logits
     torch.cuda.empty_cache()
     tokens = batch * seq
@@ -371,7 +388,9 @@ def gptj_forward(torch, dev, layers=28, batch=8, seq=2048, reps=5):
                       f"bf16, batch {batch}, seq {seq}, eval",
             "unfused_tokens_per_s": round(tokens / t_unfused, 1), "fused_tokens_per_s": round(tokens / t_fused, 1),
             "unfused_ms": round(t_unfused * 1e3, 2), "fused_ms": round(t_fused * 1e3, 2),
-            "speedup": round(t_unfused / t_fused, 3), "max_abs_logit_diff": round(diff, 4)}
+            "speedup": round(t_unfused / t_fused, 3), "max_abs_logit_diff": round(diff, 4),
+            "decode_step_batch1_context1024": {"unfused_ms": round(d_unfused, 2), "fused_ms": round(d_fused, 2),
+                                               "speedup": round(d_unfused / d_fused, 3)}}
 
 
 def gptj_train_step(torch, dev, layers=4, batch=8, seq=2048, reps=3):

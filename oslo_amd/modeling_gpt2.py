@@ -158,10 +158,9 @@ class FusedGPT2Attention(GPT2Attention):
         present = (key, value) if use_cache else None
         return query, key, value, present
 
-    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
+    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
         w = torch.matmul(query, key.transpose(-1, -2))
-        w = FusedScaleMaskSoftmaxDropout.apply(w, attention_mask, self._attention_scale(value),
-                                               not self.is_cross_attention,
+        w = FusedScaleMaskSoftmaxDropout.apply(w, attention_mask, self._attention_scale(value), causal,
                                                self.attn_dropout.p, self.training)
         if head_mask is not None:
             w = w * head_mask
@@ -174,9 +173,11 @@ class FusedGPT2Attention(GPT2Attention):
         if encoder_hidden_states is not None:
             attention_mask = encoder_attention_mask
         (bsz, np_, sq, _), sk = query.size(), key.size(-2)
-        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk,
-                                              use_triang_mask=not self.is_cross_attention):
-            out, w = self._fused_attn(query, key, value, attention_mask, head_mask)
+        # a single query over a key/value cache (a decoding step) sees every key:
+        # the causal mask is empty and the key-mask kernel applies
+        causal = not self.is_cross_attention and sq > 1
+        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal):
+            out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)
         else:
             out, w = self._attn(query, key, value, attention_mask, head_mask)
         if out.is_cuda and FusedSplitHeads.is_available(out.dtype, self.head_dim):

@@ -131,11 +131,11 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
         present = (key, value) if use_cache else None
         return query, key, value, present
 
-    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
+    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
         w = torch.matmul(query, key.transpose(-1, -2))
         # softmax and attn_dropout in one kernel (the reference runs nn.Dropout
         # as a second pass over the probabilities)
-        w = FusedScaleMaskSoftmaxDropout.apply(w, attention_mask, None, True,
+        w = FusedScaleMaskSoftmaxDropout.apply(w, attention_mask, None, causal,
                                                self.attn_dropout.p, self.training).to(value.dtype)
         if head_mask is not None:
             w = w * head_mask
@@ -145,8 +145,12 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
                 use_cache=False, output_attentions=False):
         query, key, value, present = self._project_qkv(hidden_states, layer_past, use_cache)
         (bsz, np_, sq, _), sk = query.size(), key.size(-2)
-        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=True):
-            out, w = self._fused_attn(query, key, value, attention_mask, head_mask)
+        # a single query over a key/value cache (a decoding step) sees every key
+        # of a global layer: the causal mask is empty and the key-mask kernel
+        # applies. A local layer still has its window and stays unfused then.
+        causal = sq > 1 or isinstance(self, GPTNeoLocalSelfAttention)
+        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal):
+            out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)
         else:
             out, w = self._attn(query, key, value, attention_mask, head_mask)
         out = FusedMergeHeads.apply(out) if self._transposes_fused(out) else self._merge_heads(out)
@@ -159,7 +163,7 @@ class FusedGPTNeoLocalSelfAttention(FusedGPTNeoSelfAttention, GPTNeoLocalSelfAtt
     """The fused attention on the sliding-window kernel: row r attends the last
     ``window_size`` keys up to r. No counterpart in the reference."""
 
-    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
+    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
         w = torch.matmul(query, key.transpose(-1, -2))
         w = FusedScaleMaskWindowSoftmax.apply(w, attention_mask, None, self.config.window_size)
         w = self.attn_dropout(w.to(value.dtype))

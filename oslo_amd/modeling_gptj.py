@@ -175,11 +175,11 @@ class FusedGPTJAttention(GPTJAttention):
         present = (key, value) if use_cache else None
         return query, key, value, present
 
-    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None):
+    def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
         w = torch.matmul(query, key.transpose(-1, -2))
         # softmax and attn_dropout in one kernel (the reference runs nn.Dropout
         # as a second pass over the probabilities)
-        w = FusedScaleMaskSoftmaxDropout.apply(w, attention_mask, 1.0 / self.scale_attn, True,
+        w = FusedScaleMaskSoftmaxDropout.apply(w, attention_mask, 1.0 / self.scale_attn, causal,
                                                self.attn_dropout.p, self.training).to(value.dtype)
         if head_mask is not None:
             w = w * head_mask
@@ -189,8 +189,11 @@ class FusedGPTJAttention(GPTJAttention):
                 use_cache=False, output_attentions=False):
         query, key, value, present = self._project_qkv(hidden_states, layer_past, use_cache)
         (bsz, np_, sq, _), sk = query.size(), key.size(-2)
-        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=True):
-            out, w = self._fused_attn(query, key, value, attention_mask, head_mask)
+        # a single query over a key/value cache (a decoding step) sees every key:
+        # the causal mask is empty and the key-mask kernel applies
+        causal = sq > 1
+        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal):
+            out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)
         else:
             out, w = self._attn(query, key, value, attention_mask, head_mask)
         # out_proj has no bias: the epilogue kernel runs with the bias term

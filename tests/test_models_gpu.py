@@ -75,15 +75,28 @@ def test_fused_model_backward_matches_unfused(family):
             assert err <= 2e-4 * max(1.0, scale) and err / scale <= 2e-3, f"{family} grad {k}: {err} (scale {scale})"
 
 
-def test_decode_step_routes_to_the_unfused_attention():
+@pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
+def test_decode_step_with_a_key_value_cache(family, monkeypatch):
+    """A single new token over cached keys and values: the step's logits equal
+    the full forward's last position, the fused classes take the key-mask kernel
+    (one query sees every key) and, for GPT-Neo, the local layer stays unfused."""
     torch.manual_seed(2)
-    m = models()["gpt2"]().to(DEV, torch.float16).eval().fuse()
+    m = models()[family]().to(DEV, torch.float16).eval().fuse()
     ids = torch.randint(0, 512, (2, 40), device=DEV)
+    mask = torch.ones(2, 40, dtype=torch.int64, device=DEV)
+    mask[1, :5] = 0                                       # left padding survives into the cache
+    calls = []
+    real = fku.FusedScaleMaskSoftmax.apply
+    monkeypatch.setattr(fku.FusedScaleMaskSoftmax, "apply",
+                        staticmethod(lambda x, pm, sc, tri: (calls.append((tuple(x.shape), tri)), real(x, pm, sc, tri))[1]))
     with torch.no_grad():
-        full = m(ids)["logits"]
-        first = m(ids[:, :39], use_cache=True)
-        step = m(ids[:, 39:], past_key_values=first["past_key_values"], use_cache=True)
+        full = m(ids, attention_mask=mask)["logits"]
+        first = m(ids[:, :39], attention_mask=mask[:, :39], use_cache=True)
+        calls.clear()
+        step = m(ids[:, 39:], attention_mask=mask, past_key_values=first["past_key_values"], use_cache=True)
     assert (step["logits"][:, 0].float() - full[:, 39].float()).abs().max().item() <= 2e-2
+    fused_layers = 1 if family == "gpt_neo" else 2
+    assert calls == [((2, 4, 1, 40), False)] * fused_layers
 
 
 def test_softmax_apply_autograd_matches_torch():
