@@ -30,6 +30,13 @@ from . import _lib, kernels
 _custom_kernels = None
 
 
+def _needs_grad(*tensors):
+    """False when autograd would record nothing: the operators then call the
+    kernels directly and skip the autograd.Function machinery (a decoding step
+    is bound by such per-call overheads, not by its kernels)."""
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
 def get_custom_kernels():
     """The native module (oslo/fused_kernels_utils.py:219-232). Nothing is
     compiled here: the library is built ahead of time and only loaded.
@@ -232,35 +239,49 @@ class FusedScaleMaskSoftmax(object):
     def apply(input, pad_mask, scale, use_triang_mask):
         bsz, np, sq, sk = input.size()
         scale = scale if scale is not None else 1.0
+        grad = _needs_grad(input)
 
         if use_triang_mask:
-            if pad_mask is None:
+            pad_add = None if pad_mask is None else _pad_additive_f32(pad_mask, bsz, sk)
+            if not grad:
+                return get_custom_kernels().causal_softmax_forward(input, pad_add, scale)
+            if pad_add is None:
                 return ScaledUpperTriangMaskedSoftmaxFunction.apply(
                     input.view(-1, sq, sk), scale
                 ).view(bsz, np, sq, sk)
-            return _CausalSoftmaxWithPad.apply(input, _pad_additive_f32(pad_mask, bsz, sk), scale)
+            return _CausalSoftmaxWithPad.apply(input, pad_add, scale)
 
-        if pad_mask is None:
-            return _KeyMaskedSoftmax.apply(input, None, scale)
-        return _KeyMaskedSoftmax.apply(input, _key_mask_bytes(pad_mask), scale)
+        mask = None if pad_mask is None else _key_mask_bytes(pad_mask)
+        if not grad:
+            return get_custom_kernels().masked_softmax_forward(input, mask, scale, kernels.MASK_ADD)
+        return _KeyMaskedSoftmax.apply(input, mask, scale)
 
     @staticmethod
     def is_available(dtype, bsz, np, sq, sk, use_triang_mask):
         """Integer gate of oslo/fused_kernels_utils.py:461-479, widened: true
         wherever the reference's is true."""
-        kernels_ = get_custom_kernels()
+        get_custom_kernels()  # raises if the library is missing, as the reference's gate does
         if dtype not in (torch.half, torch.bfloat16, torch.float32):
             return False
-        if sk <= 0 or sk > _lib.load().oslo_softmax_max_cols():
+        if sk <= 0 or sk > _max_cols():
             return False
         if bsz <= 0 or np <= 0 or sq <= 0:
             return False
-        # kept for parity of side effects: the reference computes this number
-        # to test divisibility; no kernel here needs it
-        kernels_.get_batch_per_block(sq, sk, bsz, np)
+        # the reference also tests divisibility by get_batch_per_block here; no
+        # kernel of this library needs it
         if use_triang_mask:
             return sq == sk
         return True
+
+
+_softmax_max_cols = None
+
+
+def _max_cols():
+    global _softmax_max_cols
+    if _softmax_max_cols is None:
+        _softmax_max_cols = _lib.load().oslo_softmax_max_cols()
+    return _softmax_max_cols
 
 
 class FusedScaleMaskWindowSoftmax(object):
@@ -279,6 +300,8 @@ class FusedScaleMaskWindowSoftmax(object):
         bsz, np, sq, sk = input.size()
         scale = scale if scale is not None else 1.0
         pad_add = None if pad_mask is None else _pad_additive_f32(pad_mask, bsz, sk)
+        if not _needs_grad(input):
+            return get_custom_kernels().causal_window_softmax_forward(input, pad_add, scale, window)
         return _CausalWindowSoftmax.apply(input, pad_add, scale, window)
 
     @staticmethod
@@ -306,7 +329,7 @@ class FusedScaleMaskSoftmaxDropout(object):
         p = float(drop_prop) if training else 0.0
         if not (use_triang_mask and 0.0 < p < 1.0):
             y = FusedScaleMaskSoftmax.apply(input, pad_mask, scale, use_triang_mask)
-            return torch.nn.functional.dropout(y, p=p, training=training)
+            return y if p == 0.0 else torch.nn.functional.dropout(y, p=p, training=training)
         bsz, np, sq, sk = input.size()
         scale = scale if scale is not None else 1.0
         pad_add = None if pad_mask is None else _pad_additive_f32(pad_mask, bsz, sk)
@@ -352,6 +375,8 @@ class FusedRotaryPositionEmbedding(object):
     @staticmethod
     def apply(query, key, value, sincos, rotary_dim, offset=0):
         sin, cos = sincos
+        if not _needs_grad(query, key, value):
+            return get_custom_kernels().rotary_qkv_forward(query, key, value, sin, cos, rotary_dim, offset)
         return _RotaryQKV.apply(query, key, value, sin, cos, rotary_dim, offset)
 
     @staticmethod
@@ -381,6 +406,8 @@ class FusedMergeHeads(object):
     @staticmethod
     def apply(x):
         b, h, s, d = x.shape
+        if not _needs_grad(x):
+            return get_custom_kernels().rotary_qkv_backward(None, None, x, None, None, 0)[2].view(b, s, h * d)
         return _MergeHeads.apply(x).view(b, s, h * d)
 
 
@@ -402,6 +429,8 @@ class FusedSplitHeads(object):
 
     @staticmethod
     def apply(qkv, heads):
+        if not _needs_grad(qkv):
+            return get_custom_kernels().split_heads_packed_forward(qkv, heads)
         return _SplitHeadsPacked.apply(qkv, heads)
 
     @staticmethod
@@ -450,6 +479,8 @@ class FusedBiasActivation(object):
     @staticmethod
     def apply(x, bias, act):
         if "gelu" in act:
+            if not _needs_grad(x, bias):
+                return get_custom_kernels().bias_gelu_forward(x, bias)
             return FusedBiasGeLU.apply(x, bias)
         else:
             return _act2fn(act)(x + bias)
@@ -506,6 +537,9 @@ def _bias_dropout_add(x, bias, residual, training, drop_prop):
         return out if residual is None else out + residual
     if p == 0.0 and bias is None and residual is None:
         return x  # nothing to add and nothing to drop
+    if not _needs_grad(x, bias, residual):
+        seed, offset = _next_philox(x.device) if p > 0.0 else (0, 0)
+        return get_custom_kernels().bias_dropout_add_forward(x, bias, residual, p, seed, offset)
     return _BiasDropoutAdd.apply(x, bias, residual, p)
 
 

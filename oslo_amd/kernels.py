@@ -37,8 +37,33 @@ def _device_tensor(t, what, like=None):
         _require(t.device == like.device, f"{what} is on {t.device}, the input on {like.device}")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t):
+    """torch's current stream on t's device, as the library's stream argument."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(t.device.index))
     return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+class _NoSwitch(object):
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(t):
+    """Context that makes t's device current for the launch; nothing to do (and
+    nothing to pay) when it already is."""
+    if t.device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(t.device)
 
 
 def _ptr(t):
@@ -76,7 +101,7 @@ def scaled_upper_triang_masked_softmax_backward(output_grads, softmax_results, s
     _require(sq == sk, "causal softmax needs square score matrices")
     g = output_grads.contiguous()
     y = softmax_results.contiguous()
-    with torch.cuda.device(g.device):
+    with _on_device(g):
         _lib.check(_lib.load().oslo_softmax_causal_bwd(
             _ptr(g), _ptr(g), _ptr(y), float(scale_factor), bh, sk, code, _stream(g)))
     return g
@@ -105,7 +130,7 @@ def scaled_masked_softmax_backward(output_grads, softmax_results, scale_factor):
     y = softmax_results.contiguous()
     sk = g.shape[-1]
     rows = g.numel() // sk if sk else 0
-    with torch.cuda.device(g.device):
+    with _on_device(g):
         _lib.check(_lib.load().oslo_softmax_masked_bwd(
             _ptr(g), _ptr(g), _ptr(y), float(scale_factor), rows, sk, code, _stream(g)))
     return g
@@ -126,7 +151,7 @@ def ngram_repeat_block_forward(tokens, lprobs, bsz, step, beam_size, no_repeat_n
     rows = bsz * beam_size
     _require(tokens.shape[0] == rows and lprobs.shape[0] == rows,
              "tokens and lprobs must have bsz * beam_size rows")
-    with torch.cuda.device(lprobs.device):
+    with _on_device(lprobs):
         _lib.check(_lib.load().oslo_ngram_repeat_block(
             _ptr(lprobs), _ptr(tokens), rows, tokens.shape[1], int(step), lprobs.shape[1],
             int(no_repeat_ngram_size), _stream(lprobs)))
@@ -151,7 +176,7 @@ def causal_softmax_forward(input, pad_add, scale_factor):
                  "pad_add must be fp32 [batch, S]")
         pad_add = pad_add.contiguous()
     y = torch.empty_like(x, requires_grad=False)
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         _lib.check(_lib.load().oslo_softmax_causal_fwd(
             _ptr(y), _ptr(x), _ptr(pad_add), float(scale_factor), b, h, sk, code, _stream(x)))
     return y
@@ -167,7 +192,7 @@ def causal_window_softmax_forward(input, pad_add, scale_factor, window):
     x = input.contiguous()
     pad_add = _pad_add_arg(pad_add, b, sk, input)
     y = torch.empty_like(x, requires_grad=False)
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         _lib.check(_lib.load().oslo_softmax_causal_window_fwd(
             _ptr(y), _ptr(x), _ptr(pad_add), float(scale_factor), int(window), b, h, sk, code, _stream(x)))
     return y
@@ -184,7 +209,7 @@ def causal_window_softmax_backward(output_grads, softmax_results, scale_factor, 
     b, h, s, _ = output_grads.shape
     g = output_grads.contiguous()
     y = softmax_results.contiguous()
-    with torch.cuda.device(g.device):
+    with _on_device(g):
         _lib.check(_lib.load().oslo_softmax_causal_window_bwd(
             _ptr(g), _ptr(g), _ptr(y), float(scale_factor), int(window), b * h, s, code, _stream(g)))
     return g
@@ -213,7 +238,7 @@ def causal_softmax_dropout_forward(input, pad_add, scale_factor, p, seed, offset
     pad_add = _pad_add_arg(pad_add, b, sk, input)
     yd = torch.empty_like(x, requires_grad=False)
     stats = torch.empty((b, h, sq, 2), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         _lib.check(_lib.load().oslo_softmax_causal_dropout_fwd(
             _ptr(yd), _ptr(stats), _ptr(x), _ptr(pad_add), float(scale_factor), float(p),
             int(seed), int(offset), b, h, sk, code, _stream(x)))
@@ -238,7 +263,7 @@ def causal_softmax_dropout_backward(output_grads, input, row_stats, pad_add, sca
     g = output_grads.contiguous()
     x = input.contiguous()
     pad_add = _pad_add_arg(pad_add, b, s, output_grads)
-    with torch.cuda.device(g.device):
+    with _on_device(g):
         _lib.check(_lib.load().oslo_softmax_causal_dropout_bwd(
             _ptr(g), _ptr(g), _ptr(x), _ptr(row_stats), _ptr(pad_add), float(scale_factor), float(p),
             int(seed), int(offset), b, h, s, code, _stream(g)))
@@ -269,7 +294,7 @@ def masked_softmax_forward(input, mask, scale_factor, mask_mode=MASK_ADD):
         msb = mq * mk if mb == b and b > 1 else 0
         msq = mk if mq == sq and sq > 1 else 0
     y = torch.empty_like(x, requires_grad=False)
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         _lib.check(_lib.load().oslo_softmax_masked_fwd(
             _ptr(y), _ptr(x), _ptr(mask), msb, msq, int(mask_mode), float(scale_factor),
             b, h, sq, sk, code, _stream(x)))
@@ -299,7 +324,7 @@ def bias_gelu_forward(y, bias):
     y = y.contiguous()
     bias = bias.contiguous()
     out = torch.empty_like(y, requires_grad=False)
-    with torch.cuda.device(y.device):
+    with _on_device(y):
         _lib.check(_lib.load().oslo_bias_gelu_fwd(
             _ptr(out), _ptr(y), _ptr(bias), rows, cols, code, _stream(y)))
     return out
@@ -316,7 +341,7 @@ def bias_gelu_backward(grad, y, bias, want_dbias=True):
     dy = torch.empty_like(y, requires_grad=False)
     dbias = torch.empty_like(bias, requires_grad=False) if want_dbias else None
     ws = _workspace(rows, cols, y.device) if want_dbias else None
-    with torch.cuda.device(y.device):
+    with _on_device(y):
         _lib.check(_lib.load().oslo_bias_gelu_bwd(
             _ptr(dy), _ptr(dbias), _ptr(ws), _ptr(grad), _ptr(y), _ptr(bias),
             rows, cols, code, _stream(y)))
@@ -334,7 +359,7 @@ def bias_dropout_add_forward(x, bias, residual, p, seed, offset):
                  "residual and input differ in shape or dtype")
         residual = residual.contiguous()
     out = torch.empty_like(x, requires_grad=False)
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         _lib.check(_lib.load().oslo_bias_dropout_add_fwd(
             _ptr(out), _ptr(x), _ptr(bias), _ptr(residual), float(p), int(seed), int(offset),
             rows, cols, code, _stream(x)))
@@ -348,7 +373,7 @@ def bias_dropout_add_backward(grad, p, seed, offset, want_dbias=True):
     dx = torch.empty_like(grad, requires_grad=False)
     dbias = torch.empty(cols, dtype=grad.dtype, device=grad.device) if want_dbias else None
     ws = _workspace(rows, cols, grad.device) if want_dbias else None
-    with torch.cuda.device(grad.device):
+    with _on_device(grad):
         _lib.check(_lib.load().oslo_bias_dropout_add_bwd(
             _ptr(dx), _ptr(dbias), _ptr(ws), _ptr(grad), float(p), int(seed), int(offset),
             rows, cols, code, _stream(grad)))
@@ -392,7 +417,7 @@ def _rotary_call(tensors, sin, cos, rotary_dim, offset, inverse):
         positions = sin.shape[0]
     else:
         sin = cos = None
-    with torch.cuda.device(first.device):
+    with _on_device(first):
         _lib.check(_lib.load().oslo_rotary_qkv(
             _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _ptr(ins[0]), _ptr(ins[1]), _ptr(ins[2]),
             _ptr(sin), _ptr(cos), positions, b, s, h, d, 0, int(rotary_dim), int(offset),
@@ -429,7 +454,7 @@ def split_heads_packed_forward(qkv, heads):
     outs = [torch.empty((b, heads, s, d), dtype=qkv.dtype, device=qkv.device) for _ in range(3)]
     step = e * qkv.element_size()
     ins = [ctypes.c_void_p(qkv.data_ptr() + i * step) for i in range(3)]
-    with torch.cuda.device(qkv.device):
+    with _on_device(qkv):
         _lib.check(_lib.load().oslo_rotary_qkv(
             _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), ins[0], ins[1], ins[2], None, None, 0,
             b, s, heads, d, e3, 0, 0, 0, code, _stream(qkv)))
@@ -451,7 +476,7 @@ def split_heads_packed_backward(grad_query, grad_key, grad_value):
     out = torch.empty((b, s, 3 * e), dtype=grad_query.dtype, device=grad_query.device)
     step = e * out.element_size()
     outs = [ctypes.c_void_p(out.data_ptr() + i * step) for i in range(3)]
-    with torch.cuda.device(out.device):
+    with _on_device(out):
         _lib.check(_lib.load().oslo_rotary_qkv(
             outs[0], outs[1], outs[2], _ptr(grads[0]), _ptr(grads[1]), _ptr(grads[2]), None, None, 0,
             b, s, h, d, 3 * e, 0, 0, 1, code, _stream(out)))
