@@ -374,6 +374,25 @@ def gptj_forward(torch, dev, layers=28, batch=8, seq=2048, reps=5):
             torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps * 1e3
 
+    def graphed_decode_ms(context=1024, steps=20):
+        """The same step over preallocated caches, replayed as one HIP graph."""
+        from oslo_amd.generation_utils import StaticDecoder
+
+        with torch.no_grad():
+            decoder = StaticDecoder(model, context + steps + 8, graph=True)
+            seq_ids = ids[:1, :context]
+            decoder.step(seq_ids)
+            for n in range(3):  # the first of these captures
+                seq_ids = torch.cat([seq_ids, ids[:1, n:n + 1]], dim=1)
+                decoder.step(seq_ids)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for n in range(steps):
+                seq_ids = torch.cat([seq_ids, ids[:1, n:n + 1]], dim=1)
+                decoder.step(seq_ids)
+            torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
     t_unfused = timed()
     ref_logits = run().float()
     d_unfused = decode_ms()
@@ -381,6 +400,7 @@ def gptj_forward(torch, dev, layers=28, batch=8, seq=2048, reps=5):
     t_fused = timed()
     diff = (run().float() - ref_logits).abs().max().item()
     d_fused = decode_ms()
+    d_graph = graphed_decode_ms()
     del model, ref_logits
     torch.cuda.empty_cache()
     tokens = batch * seq
@@ -390,7 +410,8 @@ def gptj_forward(torch, dev, layers=28, batch=8, seq=2048, reps=5):
             "unfused_ms": round(t_unfused * 1e3, 2), "fused_ms": round(t_fused * 1e3, 2),
             "speedup": round(t_unfused / t_fused, 3), "max_abs_logit_diff": round(diff, 4),
             "decode_step_batch1_context1024": {"unfused_ms": round(d_unfused, 2), "fused_ms": round(d_fused, 2),
-                                               "speedup": round(d_unfused / d_fused, 3)}}
+                                               "speedup": round(d_unfused / d_fused, 3),
+                                               "fused_graph_replay_ms": round(d_graph, 2)}}
 
 
 def gptj_train_step(torch, dev, layers=4, batch=8, seq=2048, reps=3):
@@ -539,7 +560,42 @@ def cpu_baseline(torch):
     return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": f"unfused fp32 fwd+bwd on [1,4,2048,2048] x {reps} reps, "
                       f"{dt * 1e3:.1f} ms each, bytes counted at the workload's fp16 size",
-            "gpt2_small_fwd": gpt2_small_forward(torch)}
+            "gpt2_small_fwd": gpt2_small_forward(torch), "gpt2_small_generate": gpt2_small_generate(torch)}
+
+
+def gpt2_small_generate(torch):
+    """The reference's kernel-fusion test (tests/gpt2/gpt2_test_kernel_fusion.py:
+    26-49) on random weights: GPT-2 small, fp32, one prompt of 12 tokens, beam
+    search with 5 beams to exactly 200 tokens, no 4-gram twice. Seconds per
+    generate() before fuse(), after it, with the fused n-gram ban, and with each
+    step replayed as a HIP graph (capture included)."""
+    from oslo_amd import GPT2Config, GPT2LMHeadModel
+
+    torch.manual_seed(0)
+    model = GPT2LMHeadModel(GPT2Config(resid_pdrop=0.0, embd_pdrop=0.0, attn_pdrop=0.0)).eval().to("cuda:0")
+    ids = torch.randint(0, 50257, (1, 12), generator=torch.Generator().manual_seed(1)).to("cuda:0")
+    kw = dict(max_length=200, min_length=200, num_beams=5, no_repeat_ngram_size=4)
+
+    def run(**extra):
+        for _ in range(2):
+            model.generate(ids, **kw, **extra)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = model.generate(ids, **kw, **extra)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, out
+
+    t_before, want = run()
+    model = model.fuse()
+    t_after, out_after = run()
+    t_ban, out_ban = run(fused_no_repeat_ngram_blocking=True)
+    t_graph, out_graph = run(fused_no_repeat_ngram_blocking=True, graph=True)
+    return {"config": "GPT-2 small fp32 random weights, prompt 12 tokens, max_length=min_length=200, num_beams=5, "
+                      "no_repeat_ngram_size=4",
+            "before_fuse_s": round(t_before, 3), "after_fuse_s": round(t_after, 3),
+            "after_fuse_fused_ngram_ban_s": round(t_ban, 3), "after_fuse_graph_replay_s": round(t_graph, 3),
+            "same_tokens": bool(torch.equal(want, out_after) and torch.equal(want, out_ban)
+                                and torch.equal(want, out_graph))}
 
 
 def gpt2_small_forward(torch):

@@ -20,9 +20,11 @@ from .fused_kernels_utils import (  # noqa: F401
     ScaledUpperTriangMaskedSoftmaxFunction,
     get_custom_kernels,
 )
+from .generation_utils import DynamicDecoder, GenerationMixin, StaticDecoder  # noqa: F401
 from .graphs import GraphedForward  # noqa: F401
 from .modeling_gpt2 import GPT2Config, GPT2LMHeadModel  # noqa: F401
 from .modeling_gpt_neo import GPTNeoConfig, GPTNeoForCausalLM  # noqa: F401
 from .modeling_gptj import GPTJConfig, GPTJForCausalLM  # noqa: F401
+from .modeling_utils import DecodeState, StaticKV  # noqa: F401
 
 __version__ = "0.1.0"

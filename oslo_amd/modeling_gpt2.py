@@ -15,8 +15,8 @@ from torch import nn
 
 from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedMergeHeads, FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedSplitHeads)
-from .modeling_utils import (ACT2FN, Conv1D, LayerPolicy, PreTrainedModel, additive_attention_mask,
-                             causal_lm_loss)
+from .modeling_utils import (ACT2FN, Conv1D, LayerPolicy, PreTrainedModel, StaticKV, additive_attention_mask,
+                             append_kv, causal_lm_loss, static_cache_mask)
 
 
 @dataclass
@@ -90,14 +90,14 @@ class GPT2Attention(nn.Module):
             scale *= 1 / float(self.layer_idx + 1)
         return scale
 
-    def _attn(self, query, key, value, attention_mask=None, head_mask=None):
+    def _attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
         """The unfused path: scale, where(causal, w, -1e4), + mask, softmax, dropout."""
         w = torch.matmul(query, key.transpose(-1, -2))
         if self.scale_attn_weights:
             w = w / (float(value.size(-1)) ** 0.5)
         if self.scale_attn_by_inverse_layer_idx:
             w = w / float(self.layer_idx + 1)
-        if not self.is_cross_attention:
+        if causal and not self.is_cross_attention:
             sq, sk = query.size(-2), key.size(-2)
             causal = self.bias[:, :, sk - sq:sk, :sk].bool()
             w = torch.where(causal, w, self.masked_bias.to(w.dtype))
@@ -120,10 +120,7 @@ class GPT2Attention(nn.Module):
         query = self._split_heads(query, self.num_heads, self.head_dim)
         key = self._split_heads(key, self.num_heads, self.head_dim)
         value = self._split_heads(value, self.num_heads, self.head_dim)
-        if layer_past is not None:
-            key = torch.cat((layer_past[0], key), dim=-2)
-            value = torch.cat((layer_past[1], value), dim=-2)
-        present = (key, value) if use_cache else None
+        key, value, present = append_kv(layer_past, key, value, use_cache)
         return query, key, value, present
 
     def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None,
@@ -132,7 +129,10 @@ class GPT2Attention(nn.Module):
         query, key, value, present = self._project_qkv(hidden_states, layer_past, encoder_hidden_states, use_cache)
         if encoder_hidden_states is not None:
             attention_mask = encoder_attention_mask
-        out, w = self._attn(query, key, value, attention_mask, head_mask)
+        static = isinstance(layer_past, StaticKV)
+        if static:
+            attention_mask = static_cache_mask(layer_past, attention_mask, fused=False)
+        out, w = self._attn(query, key, value, attention_mask, head_mask, causal=not static)
         out = self._merge_heads(out, self.num_heads, self.head_dim)
         out = self.resid_dropout(self.c_proj(out))
         return (out, present, w) if output_attentions else (out, present)
@@ -152,10 +152,7 @@ class FusedGPT2Attention(GPT2Attention):
                 hidden_states.is_cuda and FusedSplitHeads.is_available(hidden_states.dtype, self.head_dim)):
             return super()._project_qkv(hidden_states, layer_past, encoder_hidden_states, use_cache)
         query, key, value = FusedSplitHeads.apply(self.c_attn(hidden_states), self.num_heads)
-        if layer_past is not None:
-            key = torch.cat((layer_past[0], key), dim=-2)
-            value = torch.cat((layer_past[1], value), dim=-2)
-        present = (key, value) if use_cache else None
+        key, value, present = append_kv(layer_past, key, value, use_cache)
         return query, key, value, present
 
     def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
@@ -176,10 +173,14 @@ class FusedGPT2Attention(GPT2Attention):
         # a single query over a key/value cache (a decoding step) sees every key:
         # the causal mask is empty and the key-mask kernel applies
         causal = not self.is_cross_attention and sq > 1
-        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal):
+        static = isinstance(layer_past, StaticKV)
+        fused = FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal)
+        if static:
+            attention_mask = static_cache_mask(layer_past, attention_mask, fused)
+        if fused:
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)
         else:
-            out, w = self._attn(query, key, value, attention_mask, head_mask)
+            out, w = self._attn(query, key, value, attention_mask, head_mask, causal=not static)
         if out.is_cuda and FusedSplitHeads.is_available(out.dtype, self.head_dim):
             out = FusedMergeHeads.apply(out)
         else:
@@ -246,8 +247,11 @@ class GPT2Model(nn.Module):
         self.ln_f = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_epsilon)
 
     def forward(self, input_ids, attention_mask=None, past_key_values=None, use_cache=False):
-        past_len = 0 if past_key_values is None else past_key_values[0][0].size(-2)
-        pos = torch.arange(past_len, past_len + input_ids.size(-1), device=input_ids.device)
+        if past_key_values is not None and isinstance(past_key_values[0], StaticKV):
+            pos = past_key_values[0].state.pos
+        else:
+            past_len = 0 if past_key_values is None else past_key_values[0][0].size(-2)
+            pos = torch.arange(past_len, past_len + input_ids.size(-1), device=input_ids.device)
         h = self.drop(self.wte(input_ids) + self.wpe(pos)[None])
         mask = additive_attention_mask(attention_mask, h.dtype)
         presents = []

@@ -19,7 +19,8 @@ from torch import nn
 from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedMergeHeads,
                                  FusedRotaryPositionEmbedding, FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedScaleMaskWindowSoftmax)
-from .modeling_utils import ACT2FN, LayerPolicy, PreTrainedModel, additive_attention_mask, causal_lm_loss
+from .modeling_utils import (ACT2FN, LayerPolicy, PreTrainedModel, StaticKV, additive_attention_mask, append_kv,
+                             causal_lm_loss, static_cache_mask)
 
 
 @dataclass
@@ -58,6 +59,7 @@ class GPTNeoSelfAttention(nn.Module):
         self.embed_dim = config.hidden_size
         self.num_heads = config.num_heads
         self.head_dim = self.embed_dim // self.num_heads
+        self.config_window = config.window_size
         if self.head_dim * self.num_heads != self.embed_dim:
             raise ValueError("embed_dim must be divisible by num_heads")
         self.k_proj = nn.Linear(self.embed_dim, self.embed_dim, bias=False)
@@ -72,12 +74,12 @@ class GPTNeoSelfAttention(nn.Module):
         t = t.permute(0, 2, 1, 3).contiguous()
         return t.view(t.size()[:-2] + (self.num_heads * self.head_dim,))
 
-    def _attn(self, query, key, value, attention_mask=None, head_mask=None):
+    def _attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
         """The unfused path: fp32 scores (no scaling), where(mask, w, -1e9), + mask, softmax."""
         w = torch.matmul(query.to(torch.float32), key.to(torch.float32).transpose(-1, -2))
-        sq, sk = query.size(-2), key.size(-2)
-        causal = self.bias[:, :, sk - sq:sk, :sk].bool()
-        w = torch.where(causal, w, self.masked_bias.to(w.dtype))
+        if causal:
+            sq, sk = query.size(-2), key.size(-2)
+            w = torch.where(self.bias[:, :, sk - sq:sk, :sk].bool(), w, self.masked_bias.to(w.dtype))
         if attention_mask is not None:
             w = w + attention_mask
         w = nn.functional.softmax(w, dim=-1).to(value.dtype)
@@ -90,16 +92,20 @@ class GPTNeoSelfAttention(nn.Module):
         query = self._split_heads(self.q_proj(hidden_states))
         key = self._split_heads(self.k_proj(hidden_states))
         value = self._split_heads(self.v_proj(hidden_states))
-        if layer_past is not None:
-            key = torch.cat((layer_past[0], key), dim=-2)
-            value = torch.cat((layer_past[1], value), dim=-2)
-        present = (key, value) if use_cache else None
+        key, value, present = append_kv(layer_past, key, value, use_cache)
         return query, key, value, present
+
+    def _window(self):
+        """Keys a query sees counting back from itself; None: all of them."""
+        return self.config_window if isinstance(self, GPTNeoLocalSelfAttention) else None
 
     def forward(self, hidden_states, attention_mask=None, layer_past=None, head_mask=None,
                 use_cache=False, output_attentions=False):
         query, key, value, present = self._project_qkv(hidden_states, layer_past, use_cache)
-        out, w = self._attn(query, key, value, attention_mask, head_mask)
+        static = isinstance(layer_past, StaticKV)
+        if static:
+            attention_mask = static_cache_mask(layer_past, attention_mask, fused=False, window=self._window())
+        out, w = self._attn(query, key, value, attention_mask, head_mask, causal=not static)
         out = self.resid_dropout(self.out_proj(self._merge_heads(out)))
         return (out, present, w) if output_attentions else (out, present)
 
@@ -125,10 +131,7 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
         query, key, value = FusedRotaryPositionEmbedding.apply(
             self.q_proj(hidden_states).view(shape), self.k_proj(hidden_states).view(shape),
             self.v_proj(hidden_states).view(shape), (None, None), 0)
-        if layer_past is not None:
-            key = torch.cat((layer_past[0], key), dim=-2)
-            value = torch.cat((layer_past[1], value), dim=-2)
-        present = (key, value) if use_cache else None
+        key, value, present = append_kv(layer_past, key, value, use_cache)
         return query, key, value, present
 
     def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
@@ -148,11 +151,18 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
         # a single query over a key/value cache (a decoding step) sees every key
         # of a global layer: the causal mask is empty and the key-mask kernel
         # applies. A local layer still has its window and stays unfused then.
-        causal = sq > 1 or isinstance(self, GPTNeoLocalSelfAttention)
-        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal):
+        # With a static cache the window, too, is part of the step's key mask.
+        static = isinstance(layer_past, StaticKV)
+        causal = not static and (sq > 1 or isinstance(self, GPTNeoLocalSelfAttention))
+        fused = FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal)
+        if static:
+            attention_mask = static_cache_mask(layer_past, attention_mask, fused, window=self._window())
+        if fused and static:
+            out, w = FusedGPTNeoSelfAttention._fused_attn(self, query, key, value, attention_mask, head_mask, False)
+        elif fused:
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)
         else:
-            out, w = self._attn(query, key, value, attention_mask, head_mask)
+            out, w = self._attn(query, key, value, attention_mask, head_mask, causal=not static)
         out = FusedMergeHeads.apply(out) if self._transposes_fused(out) else self._merge_heads(out)
         out = out @ self.out_proj.weight.t()
         out = FusedBiasDropout.apply(out, self.out_proj.bias, self.training, self.resid_dropout.p)
@@ -247,8 +257,11 @@ class GPTNeoModel(nn.Module):
         self.ln_f = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_epsilon)
 
     def forward(self, input_ids, attention_mask=None, past_key_values=None, use_cache=False):
-        past_len = 0 if past_key_values is None else past_key_values[0][0].size(-2)
-        pos = torch.arange(past_len, past_len + input_ids.size(-1), device=input_ids.device)
+        if past_key_values is not None and isinstance(past_key_values[0], StaticKV):
+            pos = past_key_values[0].state.pos
+        else:
+            past_len = 0 if past_key_values is None else past_key_values[0][0].size(-2)
+            pos = torch.arange(past_len, past_len + input_ids.size(-1), device=input_ids.device)
         h = self.drop(self.wte(input_ids) + self.wpe(pos)[None])
         mask = additive_attention_mask(attention_mask, h.dtype)
         presents = []

@@ -21,7 +21,8 @@ from torch import nn
 from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedMergeHeads,
                                  FusedRotaryPositionEmbedding,
                                  FusedScaleMaskSoftmax, FusedScaleMaskSoftmaxDropout)
-from .modeling_utils import ACT2FN, LayerPolicy, PreTrainedModel, additive_attention_mask, causal_lm_loss
+from .modeling_utils import (ACT2FN, LayerPolicy, PreTrainedModel, StaticKV, additive_attention_mask, append_kv,
+                             causal_lm_loss, static_cache_mask)
 
 
 @dataclass
@@ -71,6 +72,19 @@ def rotary_tables(dim, seq_len, device):
     return tables
 
 
+def rotary_for_step(layer_past, dim, seq_len, device):
+    """(sin, cos, offset) for ``seq_len`` new tokens after the cached ones. With
+    a static cache the position lives on the device: the one table row of the
+    step is gathered there and the offset into it is 0."""
+    if isinstance(layer_past, StaticKV):
+        sin, cos = rotary_tables(dim, layer_past.state.capacity, device)
+        pos = layer_past.state.pos
+        return sin.index_select(0, pos), cos.index_select(0, pos), 0
+    offset = 0 if layer_past is None else layer_past[0].shape[-2]
+    sin, cos = rotary_tables(dim, seq_len + offset, device)
+    return sin, cos, offset
+
+
 def apply_rotary(x, sin, cos, offset=0):
     """x [B, S, H, D]: rotates consecutive feature pairs (2i, 2i+1) by the angle
     of position offset+s."""
@@ -106,12 +120,12 @@ class GPTJAttention(nn.Module):
         t = t.permute(0, 2, 1, 3).contiguous()
         return t.view(t.size()[:-2] + (self.num_attention_heads * self.head_dim,))
 
-    def _attn(self, query, key, value, attention_mask=None, head_mask=None):
+    def _attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
         """The unfused path: fp32 scores, where(causal, w, -1e9), / sqrt(d), + mask, softmax."""
-        sq, sk = query.size(-2), key.size(-2)
-        causal = self.bias[:, :, sk - sq:sk, :sk].bool()
         w = torch.matmul(query.to(torch.float32), key.to(torch.float32).transpose(-1, -2))
-        w = torch.where(causal, w, self.masked_bias.to(w.dtype))
+        if causal:
+            sq, sk = query.size(-2), key.size(-2)
+            w = torch.where(self.bias[:, :, sk - sq:sk, :sk].bool(), w, self.masked_bias.to(w.dtype))
         w = w / self.scale_attn
         if attention_mask is not None:
             w = w + attention_mask
@@ -127,9 +141,8 @@ class GPTJAttention(nn.Module):
         query = self.q_proj(hidden_states).view(shape)
         key = self.k_proj(hidden_states).view(shape)
         value = self.v_proj(hidden_states).view(shape).permute(0, 2, 1, 3)
-        offset = 0 if layer_past is None else layer_past[0].shape[-2]
         rot = self.rotary_dim if self.rotary_dim is not None else self.head_dim
-        sin, cos = rotary_tables(rot, s + offset, hidden_states.device)
+        sin, cos, offset = rotary_for_step(layer_past, rot, s, hidden_states.device)
         if rot < self.head_dim:
             key = torch.cat([apply_rotary(key[..., :rot], sin, cos, offset), key[..., rot:]], dim=-1)
             query = torch.cat([apply_rotary(query[..., :rot], sin, cos, offset), query[..., rot:]], dim=-1)
@@ -138,16 +151,16 @@ class GPTJAttention(nn.Module):
             query = apply_rotary(query, sin, cos, offset)
         key = key.to(value.dtype).permute(0, 2, 1, 3)
         query = query.to(value.dtype).permute(0, 2, 1, 3)
-        if layer_past is not None:
-            key = torch.cat((layer_past[0], key), dim=-2)
-            value = torch.cat((layer_past[1], value), dim=-2)
-        present = (key, value) if use_cache else None
+        key, value, present = append_kv(layer_past, key, value, use_cache)
         return query, key, value, present
 
     def forward(self, hidden_states, attention_mask=None, layer_past=None, head_mask=None,
                 use_cache=False, output_attentions=False):
         query, key, value, present = self._project_qkv(hidden_states, layer_past, use_cache)
-        out, w = self._attn(query, key, value, attention_mask, head_mask)
+        static = isinstance(layer_past, StaticKV)
+        if static:
+            attention_mask = static_cache_mask(layer_past, attention_mask, fused=False)
+        out, w = self._attn(query, key, value, attention_mask, head_mask, causal=not static)
         out = self.resid_dropout(self.out_proj(self._merge_heads(out)))
         return (out, present, w) if output_attentions else (out, present)
 
@@ -164,15 +177,11 @@ class FusedGPTJAttention(GPTJAttention):
             return super()._project_qkv(hidden_states, layer_past, use_cache)
         b, s, _ = hidden_states.shape
         shape = (b, s, self.num_attention_heads, self.head_dim)
-        offset = 0 if layer_past is None else layer_past[0].shape[-2]
-        sincos = rotary_tables(rot, s + offset, hidden_states.device)
+        sin, cos, offset = rotary_for_step(layer_past, rot, s, hidden_states.device)
         query, key, value = FusedRotaryPositionEmbedding.apply(
             self.q_proj(hidden_states).view(shape), self.k_proj(hidden_states).view(shape),
-            self.v_proj(hidden_states).view(shape), sincos, rot, offset)
-        if layer_past is not None:
-            key = torch.cat((layer_past[0], key), dim=-2)
-            value = torch.cat((layer_past[1], value), dim=-2)
-        present = (key, value) if use_cache else None
+            self.v_proj(hidden_states).view(shape), (sin, cos), rot, offset)
+        key, value, present = append_kv(layer_past, key, value, use_cache)
         return query, key, value, present
 
     def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
@@ -192,10 +201,14 @@ class FusedGPTJAttention(GPTJAttention):
         # a single query over a key/value cache (a decoding step) sees every key:
         # the causal mask is empty and the key-mask kernel applies
         causal = sq > 1
-        if FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal):
+        static = isinstance(layer_past, StaticKV)
+        fused = FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal)
+        if static:
+            attention_mask = static_cache_mask(layer_past, attention_mask, fused)
+        if fused:
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)
         else:
-            out, w = self._attn(query, key, value, attention_mask, head_mask)
+            out, w = self._attn(query, key, value, attention_mask, head_mask, causal=not static)
         # out_proj has no bias: the epilogue kernel runs with the bias term
         # dropped (in training; it is skipped when there is nothing to drop)
         vec_ok = FusedRotaryPositionEmbedding.is_available(out.dtype, self.head_dim, 0)

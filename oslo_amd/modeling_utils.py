@@ -14,6 +14,7 @@ import torch
 from torch import nn
 
 from .fused_kernels_utils import FusedKernelMixin
+from .generation_utils import GenerationMixin
 
 
 class Conv1D(nn.Module):
@@ -66,10 +67,10 @@ class LayerPolicy(object):
         raise NotImplementedError
 
 
-class PreTrainedModel(nn.Module, FusedKernelMixin):
-    """Random-initialised model with ``fuse()``. Sub-classes set ``is_fusable``
-    and ``get_layer_policies()`` as the reference's model classes do
-    (oslo/models/gpt2/modeling_gpt2.py:496, :521-523)."""
+class PreTrainedModel(nn.Module, FusedKernelMixin, GenerationMixin):
+    """Random-initialised model with ``fuse()`` and ``generate()``. Sub-classes
+    set ``is_fusable`` and ``get_layer_policies()`` as the reference's model
+    classes do (oslo/models/gpt2/modeling_gpt2.py:496, :521-523)."""
 
     is_fusable = False
 
@@ -91,6 +92,97 @@ class PreTrainedModel(nn.Module, FusedKernelMixin):
             elif isinstance(m, nn.LayerNorm):
                 nn.init.ones_(m.weight)
                 nn.init.zeros_(m.bias)
+
+
+class DecodeState(object):
+    """What the layers' static caches share while one token is decoded at a
+    time: ``pos``, the index of the token being fed (a device tensor, so that
+    a step can be replayed as a HIP graph while it advances), and the key masks
+    that hide the slots past it."""
+
+    def __init__(self, capacity, device, dtype):
+        self.capacity = int(capacity)
+        self.dtype = dtype
+        self.pos = torch.zeros(1, dtype=torch.long, device=device)
+        self.slots = torch.arange(self.capacity, device=device)
+        self._hidden = {}  # window (None: all earlier keys) -> bool [1,1,1,capacity], True = hidden
+
+    def begin_step(self):
+        """Recomputes the masks from ``pos``; called once per step, before the
+        model's forward (inside the graph when the step is captured)."""
+        for window, mask in self._hidden.items():
+            mask.copy_(self._compute(window))
+
+    def _compute(self, window):
+        hidden = self.slots > self.pos
+        if window is not None:
+            hidden = hidden | (self.slots <= self.pos - window)
+        return hidden.view(1, 1, 1, -1)
+
+    def hidden_keys(self, window=None):
+        """bool [1,1,1,capacity]: True where the query at ``pos`` must not look
+        (slots not written yet; for a sliding window also keys too far back)."""
+        mask = self._hidden.get(window)
+        if mask is None:
+            mask = self._hidden[window] = self._compute(window).clone()
+        return mask
+
+
+class StaticKV(object):
+    """One layer's key/value cache as two preallocated [rows, heads, capacity,
+    head_dim] buffers. Passed where the models take ``layer_past``: the new key
+    and value are written at ``state.pos`` and attention runs over the whole
+    buffers under ``state.hidden_keys()``. Shapes never change from step to
+    step, which is what capturing a step as a graph needs."""
+
+    def __init__(self, state, k, v):
+        if k.shape != v.shape or k.dim() != 4 or k.size(2) != state.capacity:
+            raise ValueError("StaticKV: buffers must be two [rows, heads, capacity, head_dim] tensors")
+        self.state, self.k, self.v = state, k, v
+
+    @classmethod
+    def allocate(cls, state, layers, rows, heads, head_dim, dtype, device):
+        """The caches of ``layers`` layers as views of one [layers, 2, rows,
+        heads, capacity, head_dim] tensor, which is returned with them: beam
+        search reorders all of them with one gather along its rows."""
+        store = torch.zeros((layers, 2, rows, heads, state.capacity, head_dim), dtype=dtype, device=device)
+        return store, tuple(cls(state, store[i, 0], store[i, 1]) for i in range(layers))
+
+    def fill(self, key, value):
+        """Takes over the keys/values of a prompt ([rows, heads, n, head_dim])."""
+        n = key.size(-2)
+        self.k[:, :, :n].copy_(key)
+        self.v[:, :, :n].copy_(value)
+
+    def update(self, key, value):
+        if key.size(-2) != 1:
+            raise RuntimeError("StaticKV: a static cache takes one token per step")
+        self.k.index_copy_(2, self.state.pos, key)
+        self.v.index_copy_(2, self.state.pos, value)
+        return self.k, self.v
+
+
+def append_kv(layer_past, key, value, use_cache):
+    """key/value of this call joined to the cache -> (key, value, present)."""
+    if isinstance(layer_past, StaticKV):
+        key, value = layer_past.update(key, value)
+        return key, value, layer_past
+    if layer_past is not None:
+        key = torch.cat((layer_past[0], key), dim=-2)
+        value = torch.cat((layer_past[1], value), dim=-2)
+    return key, value, ((key, value) if use_cache else None)
+
+
+def static_cache_mask(layer_past, attention_mask, fused, window=None):
+    """With a static cache the mask of a step comes from the decode state: a
+    bool key mask for the fused key-mask kernel, an additive one (0 / -10000,
+    the convention of ``additive_attention_mask``) for the unfused attention."""
+    if attention_mask is not None:
+        raise RuntimeError("a static key/value cache does not combine with an attention_mask")
+    hidden = layer_past.state.hidden_keys(window)
+    if fused:
+        return hidden
+    return hidden.to(layer_past.state.dtype) * -10000.0
 
 
 def additive_attention_mask(attention_mask, dtype):
