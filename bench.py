@@ -164,10 +164,11 @@ def main():
     t_fwd = time_launches(fwd, args.steps, 5)
     t_bwd = time_launches(bwd, args.steps, 5)
 
-    def roof(name, nbytes, seconds, elements):
-        """elements: scores or activations the launch produces."""
+    def roof(name, nbytes, seconds, elements, buffer_sets=1):
+        """elements: scores or activations the launch produces; buffer_sets:
+        how many sets of tensors the timed launches took in turn."""
         gbps = nbytes / seconds / 1e9
-        return {"kernel": name, "elements_per_s": round(elements / seconds, 1), "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
+        return {"kernel": name, "buffer_sets": buffer_sets, "elements_per_s": round(elements / seconds, 1), "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "us": round(seconds * 1e6, 1),
                 "algorithmic_bytes": nbytes, "traffic": MEASURED_TRAFFIC.get(name)}
 
@@ -279,35 +280,53 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
     res.append(roof("masked_bwd bf16 [16,16,1024,1024]", 6 * x.numel(), t, x.numel()))
     del x, y, g, dxm
 
+    def rotating(sets, call):
+        """fn() that runs call(set) on the next of `sets` each time: a shape
+        whose tensors fit the 256 MB last-level cache is timed on four sets of
+        buffers in turn, so that no launch finds its input left there by the
+        previous one."""
+        turn = [0]
+
+        def fn():
+            call(sets[turn[0] % len(sets)])
+            turn[0] += 1
+        return fn
+
     # bias-GeLU and bias-dropout-residual, bf16
     for rows, cols in ((16384, 16384), (16384, 4096)):
-        a = randn((rows, cols), 0, 1.0, torch.bfloat16)
-        r = randn((rows, cols), 1, 1.0, torch.bfloat16)
+        n_el = rows * cols
+        n_sets = 1 if 6 * n_el >= (1 << 30) else 4
+        sets = [(randn((rows, cols), 10 * i, 1.0, torch.bfloat16), randn((rows, cols), 10 * i + 1, 1.0, torch.bfloat16),
+                 torch.empty((rows, cols), dtype=torch.bfloat16, device=dev)) for i in range(n_sets)]
         bias = randn((cols,), 3, 0.02, torch.bfloat16)
-        o = torch.empty_like(a)
         db = torch.empty_like(bias)
         ws = torch.empty(lib.oslo_colsum_workspace_bytes(rows, cols) // 4, dtype=torch.float32, device=dev)
-        n_el = rows * cols
         shape = f"bf16 [{rows},{cols}]"
-        t = time_launches(lambda: check(lib.oslo_bias_gelu_fwd(P(o), P(a), P(bias), rows, cols, BF16, st)), n, 3)
-        res.append(roof(f"bias_gelu_fwd {shape}", 4 * n_el, t, n_el))
-        t = time_launches(lambda: check(lib.oslo_bias_gelu_bwd(P(o), P(db), P(ws), P(r), P(a), P(bias), rows, cols, BF16, st)), n, 3)
-        res.append(roof(f"bias_gelu_bwd+dbias {shape}", 6 * n_el, t, n_el))
-        t = time_launches(lambda: check(lib.oslo_bias_dropout_add_fwd(P(o), P(a), P(bias), P(r), 0.1, 1234, 0, rows, cols, BF16, st)), n, 3)
-        res.append(roof(f"bias_dropout_add_fwd p=0.1 {shape}", 6 * n_el, t, n_el))
-        t = time_launches(lambda: check(lib.oslo_bias_dropout_add_bwd(P(o), P(db), P(ws), P(r), 0.1, 1234, 0, rows, cols, BF16, st)), n, 3)
-        res.append(roof(f"bias_dropout_add_bwd+dbias p=0.1 {shape}", 4 * n_el, t, n_el))
-        del a, r, o, ws
+        t = time_launches(rotating(sets, lambda b: check(lib.oslo_bias_gelu_fwd(
+            P(b[2]), P(b[0]), P(bias), rows, cols, BF16, st))), n, 3)
+        res.append(roof(f"bias_gelu_fwd {shape}", 4 * n_el, t, n_el, n_sets))
+        t = time_launches(rotating(sets, lambda b: check(lib.oslo_bias_gelu_bwd(
+            P(b[2]), P(db), P(ws), P(b[1]), P(b[0]), P(bias), rows, cols, BF16, st))), n, 3)
+        res.append(roof(f"bias_gelu_bwd+dbias {shape}", 6 * n_el, t, n_el, n_sets))
+        t = time_launches(rotating(sets, lambda b: check(lib.oslo_bias_dropout_add_fwd(
+            P(b[2]), P(b[0]), P(bias), P(b[1]), 0.1, 1234, 0, rows, cols, BF16, st))), n, 3)
+        res.append(roof(f"bias_dropout_add_fwd p=0.1 {shape}", 6 * n_el, t, n_el, n_sets))
+        t = time_launches(rotating(sets, lambda b: check(lib.oslo_bias_dropout_add_bwd(
+            P(b[2]), P(db), P(ws), P(b[1]), 0.1, 1234, 0, rows, cols, BF16, st))), n, 3)
+        res.append(roof(f"bias_dropout_add_bwd+dbias p=0.1 {shape}", 4 * n_el, t, n_el, n_sets))
+        del sets, ws
 
     # rotary embedding + split heads of q, k, v at the GPT-J-6B shape
     B, S, H, D, rot = 8, 2048, 16, 256, 64
-    q, k, v = (randn((B, S, H, D), 10 + i, 1.0, torch.bfloat16) for i in range(3))
-    qo, ko, vo = (torch.empty((B, H, S, D), dtype=torch.bfloat16, device=dev) for _ in range(3))
+    sets = [tuple(randn((B, S, H, D), 10 + 3 * j + i, 1.0, torch.bfloat16) for i in range(3)) +
+            tuple(torch.empty((B, H, S, D), dtype=torch.bfloat16, device=dev) for _ in range(3)) for j in range(4)]
     from oslo_amd.modeling_gptj import rotary_tables
     sin, cos = rotary_tables(rot, S, dev)
-    t = time_launches(lambda: check(lib.oslo_rotary_qkv(P(qo), P(ko), P(vo), P(q), P(k), P(v), P(sin), P(cos),
-                                                        S, B, S, H, D, 0, rot, 0, 0, BF16, st)), n, 3)
-    res.append(roof("rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64", 3 * 4 * q.numel(), t, 3 * q.numel()))
+    t = time_launches(rotating(sets, lambda b: check(lib.oslo_rotary_qkv(
+        P(b[3]), P(b[4]), P(b[5]), P(b[0]), P(b[1]), P(b[2]), P(sin), P(cos),
+        S, B, S, H, D, 0, rot, 0, 0, BF16, st))), n, 3)
+    n_el = B * S * H * D
+    res.append(roof("rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64", 3 * 4 * n_el, t, 3 * n_el, len(sets)))
     return res
 
 
