@@ -375,6 +375,10 @@ class FusedRotaryPositionEmbedding(object):
     @staticmethod
     def apply(query, key, value, sincos, rotary_dim, offset=0):
         sin, cos = sincos
+        if rotary_dim == 0 and query.size(1) == 1 and all(t.is_contiguous() for t in (query, key, value)):
+            # one position and nothing to rotate: [B,1,H,D] and [B,H,1,D] are the same memory
+            b, _, h, d = query.shape
+            return query.view(b, h, 1, d), key.view(b, h, 1, d), value.view(b, h, 1, d)
         if not _needs_grad(query, key, value):
             return get_custom_kernels().rotary_qkv_forward(query, key, value, sin, cos, rotary_dim, offset)
         return _RotaryQKV.apply(query, key, value, sin, cos, rotary_dim, offset)
@@ -406,6 +410,8 @@ class FusedMergeHeads(object):
     @staticmethod
     def apply(x):
         b, h, s, d = x.shape
+        if s == 1 and x.is_contiguous():  # one position: the permute moves nothing
+            return x.view(b, 1, h * d)
         if not _needs_grad(x):
             return get_custom_kernels().rotary_qkv_backward(None, None, x, None, None, 0)[2].view(b, s, h * d)
         return _MergeHeads.apply(x).view(b, s, h * d)
@@ -429,6 +435,10 @@ class FusedSplitHeads(object):
 
     @staticmethod
     def apply(qkv, heads):
+        if qkv.dim() == 3 and qkv.size(1) == 1 and qkv.size(2) % (3 * heads) == 0:
+            # one position: the three head-major tensors are strided views of the packed row
+            b, e = qkv.size(0), qkv.size(2) // 3
+            return tuple(qkv[:, :, i * e:(i + 1) * e].reshape(b, heads, 1, e // heads) for i in range(3))
         if not _needs_grad(qkv):
             return get_custom_kernels().split_heads_packed_forward(qkv, heads)
         return _SplitHeadsPacked.apply(qkv, heads)

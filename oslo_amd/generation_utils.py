@@ -52,7 +52,8 @@ class StaticDecoder(object):
     """Steps over static caches; optionally each step is one graph replay."""
 
     def __init__(self, model, capacity, graph):
-        self.model, self.capacity, self.graph = model, capacity, graph
+        # whole 64-key vectors: the key-mask softmax then takes its vector path
+        self.model, self.capacity, self.graph = model, -(-int(capacity) // 64) * 64, graph
         self.caches = None
         self._captured = None
 

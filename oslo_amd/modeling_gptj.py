@@ -77,9 +77,12 @@ def rotary_for_step(layer_past, dim, seq_len, device):
     a static cache the position lives on the device: the one table row of the
     step is gathered there and the offset into it is 0."""
     if isinstance(layer_past, StaticKV):
-        sin, cos = rotary_tables(dim, layer_past.state.capacity, device)
-        pos = layer_past.state.pos
-        return sin.index_select(0, pos), cos.index_select(0, pos), 0
+        state = layer_past.state
+        row = state.step_values.get(("rotary", dim))
+        if row is None:  # the first layer of a step gathers the row, the others reuse it
+            sin, cos = rotary_tables(dim, state.capacity, device)
+            row = state.step_values[("rotary", dim)] = (sin.index_select(0, state.pos), cos.index_select(0, state.pos))
+        return row[0], row[1], 0
     offset = 0 if layer_past is None else layer_past[0].shape[-2]
     sin, cos = rotary_tables(dim, seq_len + offset, device)
     return sin, cos, offset

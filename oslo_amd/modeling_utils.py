@@ -106,10 +106,12 @@ class DecodeState(object):
         self.pos = torch.zeros(1, dtype=torch.long, device=device)
         self.slots = torch.arange(self.capacity, device=device)
         self._hidden = {}  # window (None: all earlier keys) -> bool [1,1,1,capacity], True = hidden
+        self.step_values = {}  # what layers share within one step (the rotary table row of ``pos``)
 
     def begin_step(self):
         """Recomputes the masks from ``pos``; called once per step, before the
         model's forward (inside the graph when the step is captured)."""
+        self.step_values.clear()
         for window, mask in self._hidden.items():
             mask.copy_(self._compute(window))
 
