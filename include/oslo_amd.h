@@ -291,6 +291,38 @@ int oslo_rotary_qkv(void *q_out, void *k_out, void *v_out, const void *q_in,
                     int64_t row_stride, int64_t rotary_dim, int64_t offset,
                     int inverse, int dtype, oslo_stream_t stream);
 
+/* Linear layer of a decoding step -------------------------------------------- */
+
+enum oslo_epilogue {
+  OSLO_EPILOGUE_NONE = 0,     /* out = x.w + bias                                 */
+  OSLO_EPILOGUE_GELU_TANH = 1 /* out = gelu_tanh(x.w + bias), oslo_bias_gelu_fwd's */
+};
+
+/* Most input rows oslo_linear_rows_fwd accepts. */
+int oslo_linear_rows_max(void);
+
+/*
+ * out[i, j] = epilogue( sum_c x[i, c] * weight[j, c] + bias[j] ) for a few
+ * input rows: x [m, k], weight [n, k] (the layout of torch.nn.Linear.weight),
+ * bias NULL or [n], out [m, n]; 0 <= m <= oslo_linear_rows_max(). Sums and the
+ * epilogue are fp32, rounded once to the storage type. The kernel streams the
+ * weight once (it is bound by HBM, like a GEMV); for more rows a GEMM library
+ * is the right tool and the call returns OSLO_E_UNSUPPORTED. k*sizeof(dtype)
+ * must be a multiple of 16, x and weight 16-byte aligned, the weight smaller
+ * than 2 GiB; out must not alias x or weight.
+ * Replaces, for the one-token-per-sequence steps of generation, the pair
+ *   x = torch.matmul(x, self.fc_in.weight.t())
+ *   x = FusedBiasActivation.apply(x, self.fc_in.bias, act)
+ * of the fused feed-forward module (oslo/models/gptj/modeling_gptj.py:1049-1054,
+ * oslo/models/gpt_neo/modeling_gpt_neo.py:1086-1091) with epilogue GELU_TANH,
+ * its second projection and bias (modeling_gptj.py:1057-1065) and the bias-free
+ * projections of the attention (q_proj, k_proj, v_proj, out_proj,
+ * modeling_gptj.py:968-970, :1031) with epilogue NONE.
+ */
+int oslo_linear_rows_fwd(void *out, const void *x, const void *weight,
+                         const void *bias, int64_t m, int64_t n, int64_t k,
+                         int epilogue, int dtype, oslo_stream_t stream);
+
 /* Repeated n-gram blocking (beam search) ------------------------------------ */
 
 /*

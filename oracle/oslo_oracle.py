@@ -34,6 +34,11 @@ root):
 * rotary_tables / rotary_split_heads: oslo/models/gptj/modeling_gptj.py:49-80
   and :205-233 (pinned by complex multiplication in float64, the adjoint
   identity and the torch operators of the unfused attention);
+* linear_rows: the projection of the fused feed-forward and attention modules
+  with its bias and activation, oslo/models/gptj/modeling_gptj.py:1049-1065
+  (x @ weight.t(), then bias_gelu_fwd or + bias), written as explicit
+  multiply-and-sum (pinned by a pure-Python float64 loop, numpy's matmul and
+  torch.nn.functional.linear + gelu(approximate="tanh"));
 * build_sample_idx / build_blending_indices:
   oslo/fused_kernels/bindings/pybind_datasets.cpp:35-160 (pinned by the closed
   form "sample k starts at token k*seq_length", the share bound of the
@@ -163,6 +168,15 @@ def bias_gelu_fwd(y, bias, dtype=np.float32):
     t = _acc(dtype)
     x = np.asarray(y, dtype=dtype) + np.asarray(bias, dtype=dtype)
     return x * t(0.5) * (t(1.0) + np.tanh(t(0.79788456) * x * (t(1) + t(0.044715) * x * x)))
+
+
+def linear_rows(x, weight, bias=None, gelu=False, dtype=np.float64):
+    """x [m, k], weight [n, k] -> act(x . weight^T + bias) [m, n]."""
+    x = np.asarray(x, dtype=dtype)
+    w = np.asarray(weight, dtype=dtype)
+    out = (x[:, None, :] * w[None, :, :]).sum(axis=-1)
+    b = np.zeros(w.shape[0], dtype=dtype) if bias is None else np.asarray(bias, dtype=dtype)
+    return bias_gelu_fwd(out, b, dtype=dtype) if gelu else out + b
 
 
 def bias_gelu_bwd(g, y, bias, dtype=np.float32):

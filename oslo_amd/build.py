@@ -27,6 +27,7 @@ SOURCES = [
     "bias_dropout_add.hip",
     "ngram_repeat_block.hip",
     "rotary.hip",
+    "linear_rows.hip",
     "dataset_index.hip",
 ]
 

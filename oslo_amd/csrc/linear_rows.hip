@@ -1,0 +1,296 @@
+// Linear layer for a handful of input rows: out[m, n] = act(x[m, :] . w[n, :] +
+// bias[n]) with 1 <= m <= 8, as in a decoding step, where the projections of a
+// transformer block read every weight once for one token per sequence. That is
+// a stream over the weight matrix, bound by HBM like the other kernels of this
+// library, not a contraction for the matrix cores: the weight bytes are the
+// algorithmic bytes.
+//
+// A wave owns R output features (rows of w, each k contiguous elements) and
+// walks along k in chunks of 64 lanes x one 128-bit vector, U chunks (so R*U
+// loads per lane) in flight. One or two input rows come through the vector
+// cache, which every wave of the CU shares; three to eight are staged in LDS
+// by the block, a segment of k at a time, because their loads would otherwise
+// queue behind the weight loads of the same wave and there are m of them per
+// weight vector. Products accumulate in fp32, pairs of
+// 16-bit elements through v_dot2c_f32_{f16,bf16}. The bias and the tanh-form
+// GeLU of the feed-forward layer are applied to the fp32 sums before the one
+// rounding to the storage type: this is the reference's
+//   x = torch.matmul(x, weight.t()); x = FusedBiasActivation.apply(x, bias, act)
+// (oslo/models/gptj/modeling_gptj.py:1049-1053) without the rounded
+// intermediate.
+
+#include "common.hpp"
+#include "gelu.hpp"
+
+namespace oslo {
+namespace {
+
+constexpr uint32_t kOutside = 0x80000000u; // past any descriptor used here
+constexpr int kMaxRows = 8;
+
+template <typename T, int VEC>
+__device__ __forceinline__ float dot_acc(float acc, const RawVec<T, VEC> &w,
+                                         const RawVec<T, VEC> &x) {
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc = __builtin_fmaf(w[j], x[j], acc);
+  } else {
+    struct Pairs {
+      RawVec<T, 2> p[VEC / 2];
+    };
+    const Pairs wp = __builtin_bit_cast(Pairs, w);
+    const Pairs xp = __builtin_bit_cast(Pairs, x);
+#pragma unroll
+    for (int j = 0; j < VEC / 2; ++j) {
+      if constexpr (__is_same(T, bf16))
+        acc = __builtin_amdgcn_fdot2_f32_bf16(wp.p[j], xp.p[j], acc, false);
+      else
+        acc = __builtin_amdgcn_fdot2(wp.p[j], xp.p[j], acc, false);
+    }
+  }
+  return acc;
+}
+
+// MT: input rows the kernel is compiled for (m <= MT; the rows past m read as
+// zeros and are not stored).
+template <typename T, int VEC, int MT, int R, int U>
+__global__ __launch_bounds__(kBlockThreads) void linear_rows_kernel(
+    T *__restrict__ out, const T *__restrict__ x, const T *__restrict__ w,
+    const T *__restrict__ bias, int m, int64_t n, int64_t k, int chunks,
+    int gelu) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t row0 = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * R;
+  if (row0 >= n) return; // no barrier in this kernel
+  const BufRsrc wrs = make_rsrc(w, (uint32_t)(n * k * (int64_t)sizeof(T)));
+  const BufRsrc xrs = make_rsrc(x, (uint32_t)((int64_t)m * k * (int64_t)sizeof(T)));
+  const uint32_t row_bytes = (uint32_t)(k * (int64_t)sizeof(T));
+
+  float acc[R][MT];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[r][i] = 0.f;
+
+  for (int c0 = 0; c0 < chunks; c0 += U) {
+    uint32_t col[U]; // byte offset of the lane's vector inside a row
+    bool col_ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t e = ((int64_t)(c0 + u) * kWave + lane) * VEC;
+      col_ok[u] = e < k; // k is a multiple of VEC: a vector is inside or outside
+      col[u] = (uint32_t)(e * (int64_t)sizeof(T));
+    }
+    RawVec<T, VEC> wv[R][U];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const bool ok = col_ok[u] && row0 + r < n;
+        wv[r][u] = buffer_load_raw<T, VEC, true>(
+            wrs, ok ? (uint32_t)(row0 + r) * row_bytes + col[u] : kOutside);
+      }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const bool ok = col_ok[u] && i < m;
+        const RawVec<T, VEC> xv = buffer_load_raw<T, VEC, false>(
+            xrs, ok ? (uint32_t)i * row_bytes + col[u] : kOutside);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          acc[r][i] = dot_acc<T, VEC>(acc[r][i], wv[r][u], xv);
+      }
+  }
+
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[r][i] = wave_allreduce(acc[r][i], OpAdd());
+  if (lane == 0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (row0 + r >= n) break;
+      const float b = bias != nullptr ? static_cast<float>(bias[row0 + r]) : 0.f;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        if (i >= m) break;
+        float v = acc[r][i] + b;
+        if (gelu) v = gelu_fwd(v);
+        out[(int64_t)i * n + row0 + r] = static_cast<T>(v);
+      }
+    }
+  }
+}
+
+// The same with the input rows in LDS. The block stages a segment of
+// kSegBytes / MT bytes of each of the MT rows (so 32 KiB in all), its four
+// waves walk their weight rows over that segment, and so on along k. Rows past
+// m and vectors past k are staged as zeros. Every wave stays to the end: there
+// are barriers in the loop.
+constexpr int kSegBytes = 32768;
+
+template <typename T, int VEC, int MT, int R, int U>
+__global__ __launch_bounds__(kBlockThreads) void linear_rows_lds_kernel(
+    T *__restrict__ out, const T *__restrict__ x, const T *__restrict__ w,
+    const T *__restrict__ bias, int m, int64_t n, int64_t k, int gelu) {
+  using Vec = RawVec<T, VEC>;
+  constexpr int kSegVecs = kSegBytes / 16 / MT;  // vectors of one row per segment
+  constexpr int kSegChunks = kSegVecs / kWave;   // chunks of 64 vectors
+  static_assert(kSegChunks % U == 0, "a segment is whole unrolled spans");
+  __shared__ Vec xs[MT * kSegVecs];
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t row0 = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * R;
+  const BufRsrc wrs = make_rsrc(w, (uint32_t)(n * k * (int64_t)sizeof(T)));
+  const BufRsrc xrs = make_rsrc(x, (uint32_t)((int64_t)m * k * (int64_t)sizeof(T)));
+  const uint32_t row_bytes = (uint32_t)(k * (int64_t)sizeof(T));
+  const int kvec = (int)(k / VEC); // vectors per row
+
+  float acc[R][MT];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[r][i] = 0.f;
+
+  for (int v0 = 0; v0 < kvec; v0 += kSegVecs) {
+    if (v0 > 0) __syncthreads(); // the previous segment has been read
+    constexpr int kPasses = MT * kSegVecs / kBlockThreads;
+    Vec stage[kPasses];
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) {
+      const int idx = p * kBlockThreads + threadIdx.x;
+      const int i = idx / kSegVecs, v = v0 + idx % kSegVecs;
+      const bool ok = i < m && v < kvec;
+      stage[p] = buffer_load_raw<T, VEC, false>(
+          xrs, ok ? (uint32_t)i * row_bytes + (uint32_t)v * 16u : kOutside);
+    }
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) xs[p * kBlockThreads + threadIdx.x] = stage[p];
+    __syncthreads();
+
+#pragma unroll 1
+    for (int c0 = 0; c0 < kSegChunks; c0 += U) {
+      Vec wv[R][U];
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int v = v0 + (c0 + u) * kWave + lane;
+          const bool ok = v < kvec && row0 + r < n;
+          wv[r][u] = buffer_load_raw<T, VEC, true>(
+              wrs, ok ? (uint32_t)(row0 + r) * row_bytes + (uint32_t)v * 16u : kOutside);
+        }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+          const Vec xv = xs[i * kSegVecs + (c0 + u) * kWave + lane];
+#pragma unroll
+          for (int r = 0; r < R; ++r)
+            acc[r][i] = dot_acc<T, VEC>(acc[r][i], wv[r][u], xv);
+        }
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[r][i] = wave_allreduce(acc[r][i], OpAdd());
+  if (lane == 0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (row0 + r >= n) break;
+      const float b = bias != nullptr ? static_cast<float>(bias[row0 + r]) : 0.f;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        if (i >= m) break;
+        float v = acc[r][i] + b;
+        if (gelu) v = gelu_fwd(v);
+        out[(int64_t)i * n + row0 + r] = static_cast<T>(v);
+      }
+    }
+  }
+}
+
+template <typename T, int MT, int R, int U>
+int launch_lds(void *out, const void *x, const void *w, const void *bias, int m,
+               int64_t n, int64_t k, int gelu, hipStream_t stream) {
+  constexpr int VEC = Io<T>::kVec;
+  const int64_t rows_per_block = (int64_t)kWavesPerBlock * R;
+  const int64_t blocks = (n + rows_per_block - 1) / rows_per_block;
+  linear_rows_lds_kernel<T, VEC, MT, R, U>
+      <<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(
+          static_cast<T *>(out), static_cast<const T *>(x),
+          static_cast<const T *>(w), static_cast<const T *>(bias), m, n, k, gelu);
+  return check_launch("oslo_linear_rows_fwd");
+}
+
+template <typename T, int MT, int R, int U>
+int launch(void *out, const void *x, const void *w, const void *bias, int m,
+           int64_t n, int64_t k, int gelu, hipStream_t stream) {
+  constexpr int VEC = Io<T>::kVec;
+  const int chunks = (int)((k + (int64_t)kWave * VEC - 1) / ((int64_t)kWave * VEC));
+  const int64_t rows_per_block = (int64_t)kWavesPerBlock * R;
+  const int64_t blocks = (n + rows_per_block - 1) / rows_per_block;
+  linear_rows_kernel<T, VEC, MT, R, U>
+      <<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(
+          static_cast<T *>(out), static_cast<const T *>(x),
+          static_cast<const T *>(w), static_cast<const T *>(bias), m, n, k,
+          chunks, gelu);
+  return check_launch("oslo_linear_rows_fwd");
+}
+
+} // namespace
+} // namespace oslo
+
+extern "C" int oslo_linear_rows_max(void) { return oslo::kMaxRows; }
+
+extern "C" int oslo_linear_rows_fwd(void *out, const void *x, const void *weight,
+                                    const void *bias, int64_t m, int64_t n,
+                                    int64_t k, int epilogue, int dtype,
+                                    oslo_stream_t stream) {
+  using namespace oslo;
+  if (m < 0 || n < 0 || k < 0)
+    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: negative size");
+  if (epilogue != OSLO_EPILOGUE_NONE && epilogue != OSLO_EPILOGUE_GELU_TANH)
+    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: unknown epilogue %d", epilogue);
+  if (dtype != OSLO_F32 && dtype != OSLO_F16 && dtype != OSLO_BF16)
+    return fail(OSLO_E_BAD_ARG, "unknown dtype %d", dtype);
+  if (m > kMaxRows)
+    return fail(OSLO_E_UNSUPPORTED,
+                "oslo_linear_rows_fwd: %lld input rows, at most %d (use a GEMM)",
+                (long long)m, kMaxRows);
+  if (m == 0 || n == 0) return OSLO_OK;
+  if (!out || !x || !weight)
+    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: null pointer");
+  const int64_t es = dtype == OSLO_F32 ? 4 : 2;
+  if (k == 0 || (k * es) % 16 != 0)
+    return fail(OSLO_E_UNSUPPORTED,
+                "oslo_linear_rows_fwd: rows of %lld elements are not whole 16-byte vectors",
+                (long long)k);
+  if (!aligned16(x) || !aligned16(weight))
+    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: x and weight must be 16-byte aligned");
+  if (n > (int64_t)0x7fffffff / (k * es) || m > (int64_t)0x7fffffff / (k * es))
+    return fail(OSLO_E_UNSUPPORTED,
+                "oslo_linear_rows_fwd: weight of 2 GiB or more (32-bit offsets)");
+  if (out == x || out == weight)
+    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: out must not alias an input");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int gelu = epilogue == OSLO_EPILOGUE_GELU_TANH;
+  const int mi = (int)m;
+  OSLO_DISPATCH_DTYPE(dtype, {
+    if (mi == 1) return launch<T, 1, 1, 8>(out, x, weight, bias, mi, n, k, gelu, s);
+    if (mi == 2) return launch<T, 2, 1, 8>(out, x, weight, bias, mi, n, k, gelu, s);
+    // two weight rows per wave halve the LDS reads per weight byte, but leave
+    // too few blocks when there are few output features
+    const bool few = n < 8192;
+    if (mi <= 4)
+      return few ? launch_lds<T, 4, 1, 8>(out, x, weight, bias, mi, n, k, gelu, s)
+                 : launch_lds<T, 4, 2, 4>(out, x, weight, bias, mi, n, k, gelu, s);
+    return few ? launch_lds<T, 8, 1, 4>(out, x, weight, bias, mi, n, k, gelu, s)
+               : launch_lds<T, 8, 2, 4>(out, x, weight, bias, mi, n, k, gelu, s);
+  });
+  return OSLO_OK;
+}

@@ -496,6 +496,55 @@ class FusedBiasActivation(object):
             return _act2fn(act)(x + bias)
 
 
+class FusedLinearRows(object):
+    """
+    Kernel fusion function: Linear + Bias + Activation for a decoding step
+
+    Before fusion: matmul(x, weight.t()) -> (Bias Addition -> Activation)
+    After fusion: one pass over the weight, bias and activation on the fp32 sums
+
+    Not in the reference, whose fused modules keep ``torch.matmul`` and fuse
+    only what follows it (oslo/models/gptj/modeling_gptj.py:1049-1065). With
+    one token per sequence the matmul of a projection is a stream over the
+    weight matrix for a handful of input rows, which the GEMM library runs at
+    a quarter to a half of the memory bandwidth; ``apply`` runs it as such a
+    stream. Inference only (``is_available`` is False when autograd would
+    record the call), at most ``kernels.LINEAR_ROWS_MAX`` rows, weights in the
+    [out_features, in_features] layout of ``nn.Linear``.
+    """
+
+    @staticmethod
+    def is_available(x, weight, bias=None):
+        if not (isinstance(x, torch.Tensor) and x.is_cuda and weight.is_cuda) or x.dim() < 1 or weight.dim() != 2:
+            return False
+        n, k = weight.shape
+        if k == 0 or x.shape[-1] != k or x.dtype != weight.dtype:
+            return False
+        if x.dtype not in (torch.half, torch.bfloat16, torch.float32) or not weight.is_contiguous():
+            return False
+        rows = x.numel() // k
+        es = x.element_size()
+        if not 0 < rows <= kernels.LINEAR_ROWS_MAX or (k * es) % 16 or n * k * es >= 2 ** 31:
+            return False
+        return not _needs_grad(x, weight, bias)
+
+    @staticmethod
+    def apply(x, weight, bias=None, act=None):
+        gelu = act is not None and "gelu" in act
+        out = get_custom_kernels().linear_rows_forward(x, weight, bias, gelu)
+        if act is not None and not gelu:
+            out = _act2fn(act)(out)
+        return out
+
+    @staticmethod
+    def project(module, x):
+        """``module(x)`` for an ``nn.Linear``, through the few-row kernel
+        where it applies."""
+        if FusedLinearRows.is_available(x, module.weight, module.bias):
+            return FusedLinearRows.apply(x, module.weight, module.bias)
+        return module(x)
+
+
 # ---------------------------------------------------------------------------
 # bias + dropout (+ residual)
 # ---------------------------------------------------------------------------

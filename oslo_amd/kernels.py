@@ -17,6 +17,9 @@ from . import _lib
 _DTYPE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 MASK_ADD = 0
 MASK_REPLACE = 1
+EPILOGUE_NONE = 0
+EPILOGUE_GELU_TANH = 1
+LINEAR_ROWS_MAX = 8  # oslo_linear_rows_max()
 
 
 def _require(cond, msg):
@@ -423,6 +426,35 @@ def _rotary_call(tensors, sin, cos, rotary_dim, offset, inverse):
             _ptr(sin), _ptr(cos), positions, b, s, h, d, 0, int(rotary_dim), int(offset),
             1 if inverse else 0, code, _stream(first)))
     return tuple(outs)
+
+
+def linear_rows_forward(x, weight, bias=None, gelu=False):
+    """x [..., K] with at most LINEAR_ROWS_MAX rows in all, weight [N, K] (the
+    layout of nn.Linear), bias None or [N] -> act(x @ weight.t() + bias) as
+    [..., N], act = tanh-form GeLU if ``gelu``. One pass over the weight; sums
+    and the epilogue in fp32 (oslo/models/gptj/modeling_gptj.py:1049-1065 for a
+    decoding step)."""
+    _device_tensor(x, "x")
+    _device_tensor(weight, "weight", x)
+    code = _dtype_code(x, "x")
+    _require(weight.dim() == 2, "weight must be [out_features, in_features]")
+    _require(weight.dtype == x.dtype, "weight and x differ in dtype")
+    n, k = weight.shape
+    _require(x.dim() >= 1 and x.shape[-1] == k, "x must be [..., in_features]")
+    m = x.numel() // k if k else 0
+    if bias is not None:
+        _device_tensor(bias, "bias", x)
+        _require(bias.dim() == 1 and bias.shape[0] == n and bias.dtype == x.dtype,
+                 "bias must be [out_features] of the input's dtype")
+        bias = bias.contiguous()
+    x2 = x.contiguous()
+    w = weight.contiguous()
+    out = torch.empty(x.shape[:-1] + (n,), dtype=x.dtype, device=x.device)
+    with _on_device(x):
+        _lib.check(_lib.load().oslo_linear_rows_fwd(
+            _ptr(out), _ptr(x2), _ptr(w), _ptr(bias), m, n, k,
+            EPILOGUE_GELU_TANH if gelu else EPILOGUE_NONE, code, _stream(x)))
+    return out
 
 
 def rotary_qkv_forward(query, key, value, sin, cos, rotary_dim, offset=0):

@@ -16,7 +16,7 @@ from typing import List, Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedMergeHeads,
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedLinearRows, FusedMergeHeads,
                                  FusedRotaryPositionEmbedding, FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedScaleMaskWindowSoftmax)
 from .modeling_utils import (ACT2FN, LayerPolicy, PreTrainedModel, StaticKV, additive_attention_mask, append_kv,
@@ -128,9 +128,10 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
             return super()._project_qkv(hidden_states, layer_past, use_cache)
         b, s, _ = hidden_states.shape
         shape = (b, s, self.num_heads, self.head_dim)
+        project = FusedLinearRows.project  # a decoding step streams the weights
         query, key, value = FusedRotaryPositionEmbedding.apply(
-            self.q_proj(hidden_states).view(shape), self.k_proj(hidden_states).view(shape),
-            self.v_proj(hidden_states).view(shape), (None, None), 0)
+            project(self.q_proj, hidden_states).view(shape), project(self.k_proj, hidden_states).view(shape),
+            project(self.v_proj, hidden_states).view(shape), (None, None), 0)
         key, value, present = append_kv(layer_past, key, value, use_cache)
         return query, key, value, present
 
@@ -164,8 +165,12 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
         else:
             out, w = self._attn(query, key, value, attention_mask, head_mask, causal=not static)
         out = FusedMergeHeads.apply(out) if self._transposes_fused(out) else self._merge_heads(out)
-        out = out @ self.out_proj.weight.t()
-        out = FusedBiasDropout.apply(out, self.out_proj.bias, self.training, self.resid_dropout.p)
+        if FusedLinearRows.is_available(out, self.out_proj.weight) and not (
+                self.training and self.resid_dropout.p > 0.0):
+            out = FusedLinearRows.apply(out, self.out_proj.weight, self.out_proj.bias)
+        else:
+            out = out @ self.out_proj.weight.t()
+            out = FusedBiasDropout.apply(out, self.out_proj.bias, self.training, self.resid_dropout.p)
         return (out, present, w) if output_attentions else (out, present)
 
 
@@ -215,9 +220,17 @@ class FusedGPTNeoMLP(GPTNeoMLP):
     """oslo/models/gpt_neo/modeling_gpt_neo.py:1078-1102."""
 
     def forward(self, x):
-        x = x @ self.c_fc.weight.t()
-        x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
-        x = x @ self.c_proj.weight.t()
+        if FusedLinearRows.is_available(x, self.c_fc.weight, self.c_fc.bias):
+            # a decoding step: each projection is one pass over its weight with
+            # the bias (and the activation) applied to the fp32 sums
+            x = FusedLinearRows.apply(x, self.c_fc.weight, self.c_fc.bias, self.config.activation_function)
+            if not (self.training and self.dropout.p > 0.0):
+                return FusedLinearRows.apply(x, self.c_proj.weight, self.c_proj.bias)
+            x = FusedLinearRows.apply(x, self.c_proj.weight)
+        else:
+            x = x @ self.c_fc.weight.t()
+            x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
+            x = x @ self.c_proj.weight.t()
         return FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
 
 

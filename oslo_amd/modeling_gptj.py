@@ -18,7 +18,7 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedMergeHeads,
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedLinearRows, FusedMergeHeads,
                                  FusedRotaryPositionEmbedding,
                                  FusedScaleMaskSoftmax, FusedScaleMaskSoftmaxDropout)
 from .modeling_utils import (ACT2FN, LayerPolicy, PreTrainedModel, StaticKV, additive_attention_mask, append_kv,
@@ -181,9 +181,10 @@ class FusedGPTJAttention(GPTJAttention):
         b, s, _ = hidden_states.shape
         shape = (b, s, self.num_attention_heads, self.head_dim)
         sin, cos, offset = rotary_for_step(layer_past, rot, s, hidden_states.device)
+        project = FusedLinearRows.project  # a decoding step streams the weights
         query, key, value = FusedRotaryPositionEmbedding.apply(
-            self.q_proj(hidden_states).view(shape), self.k_proj(hidden_states).view(shape),
-            self.v_proj(hidden_states).view(shape), (sin, cos), rot, offset)
+            project(self.q_proj, hidden_states).view(shape), project(self.k_proj, hidden_states).view(shape),
+            project(self.v_proj, hidden_states).view(shape), (sin, cos), rot, offset)
         key, value, present = append_kv(layer_past, key, value, use_cache)
         return query, key, value, present
 
@@ -216,7 +217,8 @@ class FusedGPTJAttention(GPTJAttention):
         # dropped (in training; it is skipped when there is nothing to drop)
         vec_ok = FusedRotaryPositionEmbedding.is_available(out.dtype, self.head_dim, 0)
         out = FusedMergeHeads.apply(out) if out.is_cuda and vec_ok else self._merge_heads(out)
-        out = FusedBiasDropout.apply(self.out_proj(out), None, self.training, self.resid_dropout.p)
+        out = FusedBiasDropout.apply(FusedLinearRows.project(self.out_proj, out), None, self.training,
+                                     self.resid_dropout.p)
         return (out, present, w) if output_attentions else (out, present)
 
 
@@ -236,9 +238,17 @@ class FusedGPTJMLP(GPTJMLP):
     """oslo/models/gptj/modeling_gptj.py:1041-1065."""
 
     def forward(self, x):
-        x = x @ self.fc_in.weight.t()
-        x = FusedBiasActivation.apply(x, self.fc_in.bias, self.config.activation_function)
-        x = x @ self.fc_out.weight.t()
+        if FusedLinearRows.is_available(x, self.fc_in.weight, self.fc_in.bias):
+            # a decoding step: each projection is one pass over its weight with
+            # the bias (and the activation) applied to the fp32 sums
+            x = FusedLinearRows.apply(x, self.fc_in.weight, self.fc_in.bias, self.config.activation_function)
+            if not (self.training and self.dropout.p > 0.0):
+                return FusedLinearRows.apply(x, self.fc_out.weight, self.fc_out.bias)
+            x = FusedLinearRows.apply(x, self.fc_out.weight)
+        else:
+            x = x @ self.fc_in.weight.t()
+            x = FusedBiasActivation.apply(x, self.fc_in.bias, self.config.activation_function)
+            x = x @ self.fc_out.weight.t()
         return FusedBiasDropout.apply(x, self.fc_out.bias, self.training, self.dropout.p)
 
 

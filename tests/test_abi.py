@@ -103,6 +103,17 @@ def test_argument_screening_without_a_device(lib):
     assert lib.oslo_rotary_qkv(one, null, null, two, null, null, one, one, 8, 1, 8, 2, 16, 24, 4, 0, 0, 1, null) == -1
     assert b"row_stride" in lib.oslo_last_error()      # smaller than heads*head_dim
     assert lib.oslo_rotary_qkv(null, null, null, null, null, null, null, null, 0, 1, 8, 2, 16, 0, 4, 0, 0, 1, null) == 0
+    # few-row linear layer: too many rows, ragged rows, unknown epilogue, aliasing, misalignment
+    three = ctypes.c_void_p(48)
+    assert lib.oslo_linear_rows_max() == 8
+    assert lib.oslo_linear_rows_fwd(one, two, three, null, 9, 4, 8, 0, 1, null) == -2
+    assert lib.oslo_linear_rows_fwd(one, two, three, null, 1, 4, 12, 0, 1, null) == -2
+    assert lib.oslo_linear_rows_fwd(one, two, three, null, 1, 4, 8, 5, 1, null) == -1
+    assert lib.oslo_linear_rows_fwd(two, two, three, null, 1, 4, 8, 0, 1, null) == -1
+    assert lib.oslo_linear_rows_fwd(one, ctypes.c_void_p(40), three, null, 1, 4, 8, 0, 1, null) == -1
+    assert lib.oslo_linear_rows_fwd(one, two, three, null, 1, 1 << 30, 8, 0, 1, null) == -2
+    assert lib.oslo_linear_rows_fwd(one, two, null, null, 1, 4, 8, 0, 1, null) == -1
+    assert lib.oslo_linear_rows_fwd(null, null, null, null, 0, 4, 8, 0, 1, null) == 0
     # n-gram blocking
     assert lib.oslo_ngram_repeat_block(one, one, 2, 4, 3, 8, 0, null) == -1
     assert lib.oslo_ngram_repeat_block(null, one, 2, 4, 3, 8, 2, null) == -1

@@ -405,3 +405,23 @@ def test_window_softmax_is_torch_softmax_over_the_local_attention_band():
     (gx,) = torch.autograd.grad(y, xt, go)
     got_dx = orc.softmax_bwd(go.numpy(), y.detach().numpy(), 0.7, causal=True, dtype=np.float64, window=window)
     np.testing.assert_allclose(got_dx, gx.numpy(), atol=1e-12)
+
+
+def test_linear_rows_against_loops_and_library():
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((3, 7))
+    w = rng.standard_normal((5, 7))
+    b = rng.standard_normal(5)
+    got = orc.linear_rows(x, w, b)
+    for i in range(3):
+        for j in range(5):
+            acc = 0.0
+            for c in range(7):
+                acc += float(x[i, c]) * float(w[j, c])
+            assert abs(got[i, j] - (acc + b[j])) < 1e-12
+    assert np.allclose(orc.linear_rows(x, w), x @ w.T, atol=1e-12)
+    # a transposed operand or a dropped bias would show here
+    want = torch.nn.functional.gelu(
+        torch.nn.functional.linear(torch.from_numpy(x), torch.from_numpy(w), torch.from_numpy(b)), approximate="tanh")
+    assert np.allclose(orc.linear_rows(x, w, b, gelu=True), want.numpy(), atol=1e-7)
+    assert orc.linear_rows(x, w, b).shape == (3, 5)
