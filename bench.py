@@ -327,6 +327,22 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         S, B, S, H, D, 0, rot, 0, 0, BF16, st))), n, 3)
     n_el = B * S * H * D
     res.append(roof("rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64", 3 * 4 * n_el, t, 3 * n_el, len(sets)))
+    del sets
+
+    # the projections of a decoding step at the GPT-J-6B shape: the weight is the traffic
+    for n_out, k_in, gelu, what in ((16384, 4096, 1, "fc_in + bias + gelu"), (4096, 16384, 0, "fc_out + bias"),
+                                    (4096, 4096, 0, "attention projection")):
+        n_sets = max(2, (1 << 30) // (n_out * k_in * 2))
+        weights = [randn((n_out, k_in), 20 + i, 0.02, torch.bfloat16) for i in range(n_sets)]
+        bias = randn((n_out,), 4, 0.02, torch.bfloat16)
+        for m in (1, 8):
+            xin = randn((m, k_in), 5, 1.0, torch.bfloat16)
+            o = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
+            t = time_launches(rotating(weights, lambda wt: check(lib.oslo_linear_rows_fwd(
+                P(o), P(xin), P(wt), P(bias), m, n_out, k_in, gelu, BF16, st))), n, 3)
+            res.append(roof(f"linear_rows {what} bf16 {m} x [{n_out},{k_in}]",
+                            2 * (n_out * k_in + m * k_in + m * n_out + n_out), t, m * n_out, n_sets))
+        del weights
     return res
 
 
