@@ -323,6 +323,20 @@ int oslo_linear_rows_fwd(void *out, const void *x, const void *weight,
                          const void *bias, int64_t m, int64_t n, int64_t k,
                          int epilogue, int dtype, oslo_stream_t stream);
 
+/*
+ * The same for `count` (1 to 3) layers of one shape applied to the same x in
+ * one launch: out[j] = epilogue(x . weight[j]^T + bias[j]). out, weight and
+ * bias are host arrays of `count` device pointers; bias may be NULL (no layer
+ * has a bias) or hold NULL entries (that layer has none). The query, key and
+ * value projections of a decoding step
+ * (oslo/models/gptj/modeling_gptj.py:968-970) are such a triple.
+ */
+int oslo_linear_rows_fwd_multi(void *const *out, const void *x,
+                               const void *const *weight,
+                               const void *const *bias, int count, int64_t m,
+                               int64_t n, int64_t k, int epilogue, int dtype,
+                               oslo_stream_t stream);
+
 /* Repeated n-gram blocking (beam search) ------------------------------------ */
 
 /*

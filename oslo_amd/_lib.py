@@ -51,6 +51,8 @@ PROTOTYPES = {
                    _c.c_int, _c.c_int, _P]),
     "oslo_linear_rows_max": (_c.c_int, []),
     "oslo_linear_rows_fwd": (_c.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _c.c_int, _c.c_int, _P]),
+    "oslo_linear_rows_fwd_multi": (
+        _c.c_int, [_P, _P, _P, _P, _c.c_int, _I64, _I64, _I64, _c.c_int, _c.c_int, _P]),
     "oslo_ngram_repeat_block": (
         _c.c_int, [_P, _P, _I64, _I64, _I64, _I64, _c.c_int, _P]),
     "oslo_sample_idx_rows": (_I64, [_c.c_int32, _c.c_int32, _I64]),

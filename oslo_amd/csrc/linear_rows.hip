@@ -27,6 +27,16 @@ namespace {
 
 constexpr uint32_t kOutside = 0x80000000u; // past any descriptor used here
 constexpr int kMaxRows = 8;
+constexpr int kMaxJobs = 3;
+
+// Up to three layers of the same shape applied to the same input in one launch
+// (blockIdx.y picks the layer): the query, key and value projections.
+template <typename T>
+struct LinearJobs {
+  T *out[kMaxJobs];
+  const T *w[kMaxJobs];
+  const T *bias[kMaxJobs];
+};
 
 template <typename T, int VEC>
 __device__ __forceinline__ float dot_acc(float acc, const RawVec<T, VEC> &w,
@@ -55,9 +65,11 @@ __device__ __forceinline__ float dot_acc(float acc, const RawVec<T, VEC> &w,
 // zeros and are not stored).
 template <typename T, int VEC, int MT, int R, int U>
 __global__ __launch_bounds__(kBlockThreads) void linear_rows_kernel(
-    T *__restrict__ out, const T *__restrict__ x, const T *__restrict__ w,
-    const T *__restrict__ bias, int m, int64_t n, int64_t k, int chunks,
-    int gelu) {
+    LinearJobs<T> jobs, const T *__restrict__ x, int m, int64_t n, int64_t k,
+    int chunks, int gelu) {
+  T *__restrict__ out = jobs.out[blockIdx.y];
+  const T *__restrict__ w = jobs.w[blockIdx.y];
+  const T *__restrict__ bias = jobs.bias[blockIdx.y];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int64_t row0 = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * R;
@@ -132,8 +144,11 @@ constexpr int kSegBytes = 32768;
 
 template <typename T, int VEC, int MT, int R, int U>
 __global__ __launch_bounds__(kBlockThreads) void linear_rows_lds_kernel(
-    T *__restrict__ out, const T *__restrict__ x, const T *__restrict__ w,
-    const T *__restrict__ bias, int m, int64_t n, int64_t k, int gelu) {
+    LinearJobs<T> jobs, const T *__restrict__ x, int m, int64_t n, int64_t k,
+    int gelu) {
+  T *__restrict__ out = jobs.out[blockIdx.y];
+  const T *__restrict__ w = jobs.w[blockIdx.y];
+  const T *__restrict__ bias = jobs.bias[blockIdx.y];
   using Vec = RawVec<T, VEC>;
   constexpr int kSegVecs = kSegBytes / 16 / MT;  // vectors of one row per segment
   constexpr int kSegChunks = kSegVecs / kWave;   // chunks of 64 vectors
@@ -214,44 +229,47 @@ __global__ __launch_bounds__(kBlockThreads) void linear_rows_lds_kernel(
   }
 }
 
+template <typename T>
+LinearJobs<T> make_jobs(void *const *out, const void *const *w,
+                        const void *const *bias, int count) {
+  LinearJobs<T> jobs;
+  for (int j = 0; j < kMaxJobs; ++j) {
+    const int s = j < count ? j : 0;
+    jobs.out[j] = static_cast<T *>(out[s]);
+    jobs.w[j] = static_cast<const T *>(w[s]);
+    jobs.bias[j] = bias ? static_cast<const T *>(bias[s]) : nullptr;
+  }
+  return jobs;
+}
+
 template <typename T, int MT, int R, int U>
-int launch_lds(void *out, const void *x, const void *w, const void *bias, int m,
+int launch_lds(const LinearJobs<T> &jobs, int count, const void *x, int m,
                int64_t n, int64_t k, int gelu, hipStream_t stream) {
   constexpr int VEC = Io<T>::kVec;
   const int64_t rows_per_block = (int64_t)kWavesPerBlock * R;
   const int64_t blocks = (n + rows_per_block - 1) / rows_per_block;
   linear_rows_lds_kernel<T, VEC, MT, R, U>
-      <<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(
-          static_cast<T *>(out), static_cast<const T *>(x),
-          static_cast<const T *>(w), static_cast<const T *>(bias), m, n, k, gelu);
+      <<<dim3((unsigned)blocks, count), dim3(kBlockThreads), 0, stream>>>(
+          jobs, static_cast<const T *>(x), m, n, k, gelu);
   return check_launch("oslo_linear_rows_fwd");
 }
 
 template <typename T, int MT, int R, int U>
-int launch(void *out, const void *x, const void *w, const void *bias, int m,
-           int64_t n, int64_t k, int gelu, hipStream_t stream) {
+int launch(const LinearJobs<T> &jobs, int count, const void *x, int m, int64_t n,
+           int64_t k, int gelu, hipStream_t stream) {
   constexpr int VEC = Io<T>::kVec;
   const int chunks = (int)((k + (int64_t)kWave * VEC - 1) / ((int64_t)kWave * VEC));
   const int64_t rows_per_block = (int64_t)kWavesPerBlock * R;
   const int64_t blocks = (n + rows_per_block - 1) / rows_per_block;
   linear_rows_kernel<T, VEC, MT, R, U>
-      <<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream>>>(
-          static_cast<T *>(out), static_cast<const T *>(x),
-          static_cast<const T *>(w), static_cast<const T *>(bias), m, n, k,
-          chunks, gelu);
+      <<<dim3((unsigned)blocks, count), dim3(kBlockThreads), 0, stream>>>(
+          jobs, static_cast<const T *>(x), m, n, k, chunks, gelu);
   return check_launch("oslo_linear_rows_fwd");
 }
 
-} // namespace
-} // namespace oslo
-
-extern "C" int oslo_linear_rows_max(void) { return oslo::kMaxRows; }
-
-extern "C" int oslo_linear_rows_fwd(void *out, const void *x, const void *weight,
-                                    const void *bias, int64_t m, int64_t n,
-                                    int64_t k, int epilogue, int dtype,
-                                    oslo_stream_t stream) {
-  using namespace oslo;
+int linear_rows(void *const *out, const void *x, const void *const *weight,
+                const void *const *bias, int count, int64_t m, int64_t n,
+                int64_t k, int epilogue, int dtype, hipStream_t s) {
   if (m < 0 || n < 0 || k < 0)
     return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: negative size");
   if (epilogue != OSLO_EPILOGUE_NONE && epilogue != OSLO_EPILOGUE_GELU_TANH)
@@ -263,34 +281,73 @@ extern "C" int oslo_linear_rows_fwd(void *out, const void *x, const void *weight
                 "oslo_linear_rows_fwd: %lld input rows, at most %d (use a GEMM)",
                 (long long)m, kMaxRows);
   if (m == 0 || n == 0) return OSLO_OK;
-  if (!out || !x || !weight)
-    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: null pointer");
+  if (!x) return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: null pointer");
   const int64_t es = dtype == OSLO_F32 ? 4 : 2;
   if (k == 0 || (k * es) % 16 != 0)
     return fail(OSLO_E_UNSUPPORTED,
                 "oslo_linear_rows_fwd: rows of %lld elements are not whole 16-byte vectors",
                 (long long)k);
-  if (!aligned16(x) || !aligned16(weight))
-    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: x and weight must be 16-byte aligned");
   if (n > (int64_t)0x7fffffff / (k * es) || m > (int64_t)0x7fffffff / (k * es))
     return fail(OSLO_E_UNSUPPORTED,
                 "oslo_linear_rows_fwd: weight of 2 GiB or more (32-bit offsets)");
-  if (out == x || out == weight)
-    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: out must not alias an input");
-  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (!aligned16(x))
+    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: x and weight must be 16-byte aligned");
+  for (int j = 0; j < count; ++j) {
+    if (!out[j] || !weight[j])
+      return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: null pointer");
+    if (!aligned16(weight[j]))
+      return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: x and weight must be 16-byte aligned");
+    if (out[j] == x || out[j] == weight[j])
+      return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: out must not alias an input");
+    for (int i = 0; i < j; ++i)
+      if (out[i] == out[j])
+        return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: two layers share an output");
+  }
   const int gelu = epilogue == OSLO_EPILOGUE_GELU_TANH;
   const int mi = (int)m;
   OSLO_DISPATCH_DTYPE(dtype, {
-    if (mi == 1) return launch<T, 1, 1, 8>(out, x, weight, bias, mi, n, k, gelu, s);
-    if (mi == 2) return launch<T, 2, 1, 8>(out, x, weight, bias, mi, n, k, gelu, s);
+    const LinearJobs<T> jobs = make_jobs<T>(out, weight, bias, count);
+    if (mi == 1) return launch<T, 1, 1, 8>(jobs, count, x, mi, n, k, gelu, s);
+    if (mi == 2) return launch<T, 2, 1, 8>(jobs, count, x, mi, n, k, gelu, s);
     // two weight rows per wave halve the LDS reads per weight byte, but leave
     // too few blocks when there are few output features
-    const bool few = n < 8192;
+    const bool few = n * count < 8192;
     if (mi <= 4)
-      return few ? launch_lds<T, 4, 1, 8>(out, x, weight, bias, mi, n, k, gelu, s)
-                 : launch_lds<T, 4, 2, 4>(out, x, weight, bias, mi, n, k, gelu, s);
-    return few ? launch_lds<T, 8, 1, 4>(out, x, weight, bias, mi, n, k, gelu, s)
-               : launch_lds<T, 8, 2, 4>(out, x, weight, bias, mi, n, k, gelu, s);
+      return few ? launch_lds<T, 4, 1, 8>(jobs, count, x, mi, n, k, gelu, s)
+                 : launch_lds<T, 4, 2, 4>(jobs, count, x, mi, n, k, gelu, s);
+    return few ? launch_lds<T, 8, 1, 4>(jobs, count, x, mi, n, k, gelu, s)
+               : launch_lds<T, 8, 2, 4>(jobs, count, x, mi, n, k, gelu, s);
   });
   return OSLO_OK;
+}
+
+} // namespace
+} // namespace oslo
+
+extern "C" int oslo_linear_rows_max(void) { return oslo::kMaxRows; }
+
+extern "C" int oslo_linear_rows_fwd(void *out, const void *x, const void *weight,
+                                    const void *bias, int64_t m, int64_t n,
+                                    int64_t k, int epilogue, int dtype,
+                                    oslo_stream_t stream) {
+  void *const outs[1] = {out};
+  const void *const weights[1] = {weight};
+  const void *const biases[1] = {bias};
+  return oslo::linear_rows(outs, x, weights, biases, 1, m, n, k, epilogue, dtype,
+                           static_cast<hipStream_t>(stream));
+}
+
+extern "C" int oslo_linear_rows_fwd_multi(void *const *out, const void *x,
+                                          const void *const *weight,
+                                          const void *const *bias, int count,
+                                          int64_t m, int64_t n, int64_t k,
+                                          int epilogue, int dtype,
+                                          oslo_stream_t stream) {
+  if (count < 1 || count > oslo::kMaxJobs)
+    return oslo::fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd_multi: %d layers, 1 to %d are taken",
+                      count, oslo::kMaxJobs);
+  if (!out || !weight)
+    return oslo::fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd_multi: null pointer table");
+  return oslo::linear_rows(out, x, weight, bias, count, m, n, k, epilogue, dtype,
+                           static_cast<hipStream_t>(stream));
 }

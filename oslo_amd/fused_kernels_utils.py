@@ -544,6 +544,18 @@ class FusedLinearRows(object):
             return FusedLinearRows.apply(x, module.weight, module.bias)
         return module(x)
 
+    @staticmethod
+    def project_many(modules, x):
+        """``[m(x) for m in modules]`` for up to three ``nn.Linear`` of one
+        shape (the query, key and value projections), in one launch where the
+        few-row kernel applies."""
+        first = modules[0]
+        if (len(modules) <= 3 and all(m.weight.shape == first.weight.shape for m in modules)
+                and all(FusedLinearRows.is_available(x, m.weight, m.bias) for m in modules)):
+            return get_custom_kernels().linear_rows_forward_multi(
+                x, [m.weight for m in modules], [m.bias for m in modules])
+        return [m(x) for m in modules]
+
 
 # ---------------------------------------------------------------------------
 # bias + dropout (+ residual)

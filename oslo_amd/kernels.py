@@ -434,27 +434,47 @@ def linear_rows_forward(x, weight, bias=None, gelu=False):
     [..., N], act = tanh-form GeLU if ``gelu``. One pass over the weight; sums
     and the epilogue in fp32 (oslo/models/gptj/modeling_gptj.py:1049-1065 for a
     decoding step)."""
+    return linear_rows_forward_multi(x, (weight,), (bias,), gelu)[0]
+
+
+def linear_rows_forward_multi(x, weights, biases=None, gelu=False):
+    """One to three layers of the same shape applied to the same x in one
+    launch (the query, key and value projections): a list of outputs."""
+    count = len(weights)
+    _require(1 <= count <= 3, "one to three layers per launch")
+    biases = (None,) * count if biases is None else tuple(biases)
+    _require(len(biases) == count, "one bias (or None) per weight")
     _device_tensor(x, "x")
-    _device_tensor(weight, "weight", x)
     code = _dtype_code(x, "x")
-    _require(weight.dim() == 2, "weight must be [out_features, in_features]")
-    _require(weight.dtype == x.dtype, "weight and x differ in dtype")
-    n, k = weight.shape
+    n, k = weights[0].shape if weights[0].dim() == 2 else (0, 0)
     _require(x.dim() >= 1 and x.shape[-1] == k, "x must be [..., in_features]")
     m = x.numel() // k if k else 0
-    if bias is not None:
-        _device_tensor(bias, "bias", x)
-        _require(bias.dim() == 1 and bias.shape[0] == n and bias.dtype == x.dtype,
-                 "bias must be [out_features] of the input's dtype")
-        bias = bias.contiguous()
+    ws, bs = [], []
+    for w, b in zip(weights, biases):
+        _device_tensor(w, "weight", x)
+        _require(w.dim() == 2 and tuple(w.shape) == (n, k), "weights must be [out_features, in_features], all alike")
+        _require(w.dtype == x.dtype, "weight and x differ in dtype")
+        ws.append(w.contiguous())
+        if b is not None:
+            _device_tensor(b, "bias", x)
+            _require(b.dim() == 1 and b.shape[0] == n and b.dtype == x.dtype,
+                     "bias must be [out_features] of the input's dtype")
+            b = b.contiguous()
+        bs.append(b)
     x2 = x.contiguous()
-    w = weight.contiguous()
-    out = torch.empty(x.shape[:-1] + (n,), dtype=x.dtype, device=x.device)
+    outs = [torch.empty(x.shape[:-1] + (n,), dtype=x.dtype, device=x.device) for _ in range(count)]
+    epilogue = EPILOGUE_GELU_TANH if gelu else EPILOGUE_NONE
     with _on_device(x):
-        _lib.check(_lib.load().oslo_linear_rows_fwd(
-            _ptr(out), _ptr(x2), _ptr(w), _ptr(bias), m, n, k,
-            EPILOGUE_GELU_TANH if gelu else EPILOGUE_NONE, code, _stream(x)))
-    return out
+        if count == 1:
+            _lib.check(_lib.load().oslo_linear_rows_fwd(
+                _ptr(outs[0]), _ptr(x2), _ptr(ws[0]), _ptr(bs[0]), m, n, k, epilogue, code, _stream(x)))
+        else:
+            table = ctypes.c_void_p * count
+            _lib.check(_lib.load().oslo_linear_rows_fwd_multi(
+                table(*(o.data_ptr() for o in outs)), _ptr(x2), table(*(w.data_ptr() for w in ws)),
+                table(*(None if b is None else b.data_ptr() for b in bs)), count, m, n, k, epilogue, code,
+                _stream(x)))
+    return outs
 
 
 def rotary_qkv_forward(query, key, value, sin, cos, rotary_dim, offset=0):

@@ -128,10 +128,10 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
             return super()._project_qkv(hidden_states, layer_past, use_cache)
         b, s, _ = hidden_states.shape
         shape = (b, s, self.num_heads, self.head_dim)
-        project = FusedLinearRows.project  # a decoding step streams the weights
+        # (a decoding step streams the three weights in one launch)
+        query, key, value = FusedLinearRows.project_many((self.q_proj, self.k_proj, self.v_proj), hidden_states)
         query, key, value = FusedRotaryPositionEmbedding.apply(
-            project(self.q_proj, hidden_states).view(shape), project(self.k_proj, hidden_states).view(shape),
-            project(self.v_proj, hidden_states).view(shape), (None, None), 0)
+            query.view(shape), key.view(shape), value.view(shape), (None, None), 0)
         key, value, present = append_kv(layer_past, key, value, use_cache)
         return query, key, value, present
 

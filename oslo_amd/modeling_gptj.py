@@ -181,10 +181,10 @@ class FusedGPTJAttention(GPTJAttention):
         b, s, _ = hidden_states.shape
         shape = (b, s, self.num_attention_heads, self.head_dim)
         sin, cos, offset = rotary_for_step(layer_past, rot, s, hidden_states.device)
-        project = FusedLinearRows.project  # a decoding step streams the weights
+        # (a decoding step streams the three weights in one launch)
+        query, key, value = FusedLinearRows.project_many((self.q_proj, self.k_proj, self.v_proj), hidden_states)
         query, key, value = FusedRotaryPositionEmbedding.apply(
-            project(self.q_proj, hidden_states).view(shape), project(self.k_proj, hidden_states).view(shape),
-            project(self.v_proj, hidden_states).view(shape), (sin, cos), rot, offset)
+            query.view(shape), key.view(shape), value.view(shape), (sin, cos), rot, offset)
         key, value, present = append_kv(layer_past, key, value, use_cache)
         return query, key, value, present
 

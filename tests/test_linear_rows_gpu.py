@@ -47,6 +47,24 @@ def test_linear_rows_matches_oracle(m, n, k, dtype):
         check(out, x, w, bias, gelu, dtype, f"{m}x{n}x{k} bias={bias is not None} gelu={gelu}")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("m,n,k", [(1, 64, 512), (3, 130, 1032), (8, 4096, 1024)])
+def test_linear_rows_three_layers_in_one_launch(m, n, k, dtype):
+    """The multi-layer launch gives, bit for bit, what three single launches give."""
+    x = randn((m, k), dtype, seed=1).to(DEV)
+    ws = [randn((n, k), dtype, seed=10 + j, std=0.05).to(DEV) for j in range(3)]
+    bs = [randn((n,), dtype, seed=20, std=0.5).to(DEV), None, randn((n,), dtype, seed=22, std=0.5).to(DEV)]
+    outs = kernels.linear_rows_forward_multi(x, ws, bs)
+    for w, b, out in zip(ws, bs, outs):
+        assert torch.equal(out, kernels.linear_rows_forward(x, w, b))
+    two = kernels.linear_rows_forward_multi(x, ws[:2], None, gelu=True)
+    assert torch.equal(two[1], kernels.linear_rows_forward(x, ws[1], None, gelu=True))
+    with pytest.raises(RuntimeError):
+        kernels.linear_rows_forward_multi(x, ws + ws[:1])
+    with pytest.raises(RuntimeError):
+        kernels.linear_rows_forward_multi(x, [ws[0], ws[1][:-1]])
+
+
 def test_linear_rows_leading_dims_and_torch_agreement():
     """[B, 1, K] inputs as the modules pass them; against torch's own linear +
     gelu on the device, within bf16 rounding of the two-step path."""
