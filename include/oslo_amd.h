@@ -337,6 +337,38 @@ int oslo_linear_rows_fwd_multi(void *const *out, const void *x,
                                int64_t n, int64_t k, int epilogue, int dtype,
                                oslo_stream_t stream);
 
+/* Attention of a decoding step ----------------------------------------------- */
+
+/*
+ * One query per (sequence, head) over a key/value cache:
+ *   out[i, :] = sum_s softmax_s( scale * q[i, :] . k[i, s, :] ) * v[i, s, :]
+ * over the visible keys s: first <= s <= last, where last is *pos_dev (if
+ * pos_dev is not NULL: an int64 in device memory, read by the kernel, so that a
+ * captured launch follows a position that advances) or else pos, and first is
+ * last - window + 1 for window > 0 (a sliding window, as in GPT-Neo's local
+ * layers), else 0. q, out: [rows_heads, head_dim]; k, v: [rows_heads, capacity,
+ * head_dim] (a [batch, heads, capacity, head_dim] cache); 0 <= last < capacity.
+ * Keys outside the visible range are not read. workspace: fp32, at least
+ * oslo_attention_decode_workspace_bytes(...) bytes, contents irrelevant before
+ * and after. head_dim * sizeof(dtype) must be 128, 256, 512 or 1024 bytes.
+ * Arithmetic in fp32 throughout (scores, softmax, weighted sum), one rounding
+ * at the end.
+ * Replaces, for a query length of 1, the sequence matmul(q, k^T) ->
+ * FusedScaleMaskSoftmax.apply -> matmul(probs, v) of the fused attention
+ * (oslo/models/gptj/modeling_gptj.py:936-951,
+ *  oslo/models/gpt_neo/modeling_gpt_neo.py:993-1008,
+ *  oslo/models/gpt2/modeling_gpt2.py:1435-1459).
+ */
+size_t oslo_attention_decode_workspace_bytes(int64_t rows_heads,
+                                             int64_t capacity, int64_t head_dim,
+                                             int dtype);
+int oslo_attention_decode_fwd(void *out, const void *q, const void *k,
+                              const void *v, float *workspace,
+                              const int64_t *pos_dev, int64_t pos,
+                              int64_t window, float scale, int64_t rows_heads,
+                              int64_t capacity, int64_t head_dim, int dtype,
+                              oslo_stream_t stream);
+
 /* Repeated n-gram blocking (beam search) ------------------------------------ */
 
 /*

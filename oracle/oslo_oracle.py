@@ -39,6 +39,12 @@ root):
   (x @ weight.t(), then bias_gelu_fwd or + bias), written as explicit
   multiply-and-sum (pinned by a pure-Python float64 loop, numpy's matmul and
   torch.nn.functional.linear + gelu(approximate="tanh"));
+* attention_decode: the attention of one query over cached keys and values,
+  oslo/models/gptj/modeling_gptj.py:151-191 with a query length of 1 (scores,
+  scale, the keys past the query hidden, softmax, weighted sum of the values),
+  in float64 (pinned by softmax_masked of this file composed with numpy
+  matmuls, by torch.nn.functional.scaled_dot_product_attention, and by the
+  closed form for equal scores: the mean of the visible values);
 * build_sample_idx / build_blending_indices:
   oslo/fused_kernels/bindings/pybind_datasets.cpp:35-160 (pinned by the closed
   form "sample k starts at token k*seq_length", the share bound of the
@@ -177,6 +183,20 @@ def linear_rows(x, weight, bias=None, gelu=False, dtype=np.float64):
     out = (x[:, None, :] * w[None, :, :]).sum(axis=-1)
     b = np.zeros(w.shape[0], dtype=dtype) if bias is None else np.asarray(bias, dtype=dtype)
     return bias_gelu_fwd(out, b, dtype=dtype) if gelu else out + b
+
+
+def attention_decode(q, k, v, last, scale, window=0, dtype=np.float64):
+    """q [n, d]; k, v [n, capacity, d]; keys first..last visible -> [n, d]."""
+    q, k, v = (np.asarray(t, dtype=dtype) for t in (q, k, v))
+    first = max(0, last - window + 1) if window > 0 else 0
+    out = np.zeros_like(q)
+    for i in range(q.shape[0]):
+        scores = np.array([scale * np.dot(q[i], k[i, s]) for s in range(first, last + 1)], dtype=dtype)
+        e = np.exp(scores - scores.max())
+        p = e / e.sum()
+        for j, s in enumerate(range(first, last + 1)):
+            out[i] += p[j] * v[i, s]
+    return out
 
 
 def bias_gelu_bwd(g, y, bias, dtype=np.float32):

@@ -8,6 +8,7 @@ from .fused_kernels_utils import (  # noqa: F401
     FusedBiasDropout,
     FusedBiasDropoutResidual,
     FusedBiasGeLU,
+    FusedDecodeAttention,
     FusedKernelMixin,
     FusedLinearRows,
     FusedMergeHeads,

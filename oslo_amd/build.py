@@ -28,6 +28,7 @@ SOURCES = [
     "ngram_repeat_block.hip",
     "rotary.hip",
     "linear_rows.hip",
+    "attention_decode.hip",
     "dataset_index.hip",
 ]
 

@@ -496,6 +496,41 @@ class FusedBiasActivation(object):
             return _act2fn(act)(x + bias)
 
 
+class FusedDecodeAttention(object):
+    """
+    Kernel fusion function: the attention of a decoding step
+
+    Before fusion: Matmul (q * K^T) -> (Scale + Mask + Softmax) -> Matmul (Score * V)
+    After fusion: one pass over the visible keys and values
+
+    Not in the reference, whose fused attention keeps both matmuls
+    (oslo/models/gptj/modeling_gptj.py:936-951) and, its gate wanting
+    ``sq == sk``, runs decoding steps unfused altogether. ``apply`` takes the
+    one query per head [B, H, 1, D], the key and value caches [B, H, L, D], the
+    index of the last visible key (an int, or an int64 device tensor that the
+    kernel reads, for steps replayed as a graph) and an optional sliding
+    window. Inference only.
+    """
+
+    @staticmethod
+    def is_available(query, key, training=False, dropout_p=0.0):
+        if not (query.is_cuda and query.dim() == 4 and key.dim() == 4 and query.size(2) == 1):
+            return False
+        if query.dtype not in (torch.half, torch.bfloat16, torch.float32) or key.dtype != query.dtype:
+            return False
+        if training and dropout_p > 0.0:
+            return False
+        head_bytes = query.size(3) * query.element_size()
+        if head_bytes not in (128, 256, 512, 1024) or key.size(2) * head_bytes >= 2 ** 31:
+            return False
+        return not _needs_grad(query, key)
+
+    @staticmethod
+    def apply(query, key, value, pos, scale, window=None):
+        scale = 1.0 if scale is None else scale
+        return get_custom_kernels().attention_decode_forward(query, key, value, pos, scale, window or 0)
+
+
 class FusedLinearRows(object):
     """
     Kernel fusion function: Linear + Bias + Activation for a decoding step

@@ -477,6 +477,43 @@ def linear_rows_forward_multi(x, weights, biases=None, gelu=False):
     return outs
 
 
+def attention_decode_forward(query, key, value, pos, scale, window=0):
+    """query [B, H, 1, D]; key, value [B, H, L, D] caches; attends keys
+    first..last, last = ``pos`` (an int, or an int64 device tensor of one
+    element that the kernel reads), first = last - window + 1 for window > 0,
+    else 0. Returns softmax(scale * q k^T) v as [B, H, 1, D]
+    (oslo/models/gptj/modeling_gptj.py:936-951 for a query length of 1)."""
+    _device_tensor(query, "query")
+    _device_tensor(key, "key", query)
+    _device_tensor(value, "value", query)
+    code = _dtype_code(query, "query")
+    _require(query.dim() == 4 and key.dim() == 4 and value.dim() == 4, "expected 4D tensors")
+    b, h, sq, d = query.shape
+    _require(sq == 1, "one query per sequence and head")
+    _require(key.shape == value.shape and tuple(key.shape[:2]) == (b, h) and key.shape[3] == d,
+             "key and value must be [B, H, L, D] caches of the query's heads")
+    _require(key.dtype == query.dtype and value.dtype == query.dtype, "query, key and value differ in dtype")
+    cap = key.shape[2]
+    q, k, v = query.contiguous(), key.contiguous(), value.contiguous()
+    pos_dev, pos_host = None, 0
+    if isinstance(pos, torch.Tensor):
+        _device_tensor(pos, "pos", query)
+        _require(pos.dtype == torch.int64 and pos.numel() == 1, "pos must be one int64")
+        pos_dev = pos
+    else:
+        pos_host = int(pos)
+    lib = _lib.load()
+    nbytes = lib.oslo_attention_decode_workspace_bytes(b * h, cap, d, code)
+    _require(nbytes > 0 or b * h == 0, f"attention_decode: heads of {d} x {query.dtype} are not supported")
+    ws = torch.empty(nbytes // 4, dtype=torch.float32, device=query.device)
+    out = torch.empty_like(q)
+    with _on_device(q):
+        _lib.check(lib.oslo_attention_decode_fwd(
+            _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(ws), _ptr(pos_dev), pos_host, int(window),
+            float(scale), b * h, cap, d, code, _stream(q)))
+    return out
+
+
 def rotary_qkv_forward(query, key, value, sin, cos, rotary_dim, offset=0):
     """query, key, value: [B, S, H, D] (any may be None); sin, cos: fp32
     [positions, rotary_dim/2]. Returns the three tensors as [B, H, S, D], query

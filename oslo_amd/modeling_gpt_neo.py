@@ -16,7 +16,8 @@ from typing import List, Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedLinearRows, FusedMergeHeads,
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedDecodeAttention, FusedLinearRows,
+                                 FusedMergeHeads,
                                  FusedRotaryPositionEmbedding, FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedScaleMaskWindowSoftmax)
 from .modeling_utils import (ACT2FN, LayerPolicy, PreTrainedModel, StaticKV, additive_attention_mask, append_kv,
@@ -156,9 +157,17 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
         static = isinstance(layer_past, StaticKV)
         causal = not static and (sq > 1 or isinstance(self, GPTNeoLocalSelfAttention))
         fused = FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal)
-        if static:
+        one_pass = (sq == 1 and attention_mask is None and head_mask is None and not output_attentions
+                    and FusedDecodeAttention.is_available(query, key, self.training, self.attn_dropout.p))
+        if static and not one_pass:
             attention_mask = static_cache_mask(layer_past, attention_mask, fused, window=self._window())
-        if fused and static:
+        if one_pass:
+            # a decoding step: scores, softmax and weighted sum in one pass over the
+            # cache, the window of a local layer included
+            out = FusedDecodeAttention.apply(query, key, value, layer_past.state.pos if static else sk - 1,
+                                             None, self._window())
+            w = None
+        elif fused and static:
             out, w = FusedGPTNeoSelfAttention._fused_attn(self, query, key, value, attention_mask, head_mask, False)
         elif fused:
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)

@@ -18,7 +18,8 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedLinearRows, FusedMergeHeads,
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedDecodeAttention, FusedLinearRows,
+                                 FusedMergeHeads,
                                  FusedRotaryPositionEmbedding,
                                  FusedScaleMaskSoftmax, FusedScaleMaskSoftmaxDropout)
 from .modeling_utils import (ACT2FN, LayerPolicy, PreTrainedModel, StaticKV, additive_attention_mask, append_kv,
@@ -207,9 +208,16 @@ class FusedGPTJAttention(GPTJAttention):
         causal = sq > 1
         static = isinstance(layer_past, StaticKV)
         fused = FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal)
-        if static:
+        one_pass = (sq == 1 and attention_mask is None and head_mask is None and not output_attentions
+                    and FusedDecodeAttention.is_available(query, key, self.training, self.attn_dropout.p))
+        if static and not one_pass:
             attention_mask = static_cache_mask(layer_past, attention_mask, fused)
-        if fused:
+        if one_pass:
+            # a decoding step: scores, softmax and weighted sum in one pass over the cache
+            out = FusedDecodeAttention.apply(query, key, value, layer_past.state.pos if static else sk - 1,
+                                             1.0 / self.scale_attn)
+            w = None
+        elif fused:
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)
         else:
             out, w = self._attn(query, key, value, attention_mask, head_mask, causal=not static)

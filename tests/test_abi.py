@@ -118,6 +118,14 @@ def test_argument_screening_without_a_device(lib):
     assert lib.oslo_linear_rows_fwd_multi(table, one, table, null, 4, 1, 4, 8, 0, 1, null) == -1     # four layers
     assert lib.oslo_linear_rows_fwd_multi(null, one, table, null, 2, 1, 4, 8, 0, 1, null) == -1
     assert lib.oslo_linear_rows_fwd_multi(table, ctypes.c_void_p(64), table, null, 3, 1, 4, 8, 0, 1, null) == -1  # out[j] is weight[j]
+    # attention of a decoding step: head size, position, null pointers, workspace size
+    assert lib.oslo_attention_decode_fwd(one, two, three, three, one, null, 0, 0, 1.0, 4, 64, 48, 1, null) == -2
+    assert lib.oslo_attention_decode_fwd(one, two, three, three, one, null, 64, 0, 1.0, 4, 64, 64, 1, null) == -1
+    assert lib.oslo_attention_decode_fwd(one, two, three, three, null, null, 3, 0, 1.0, 4, 64, 64, 1, null) == -1
+    assert lib.oslo_attention_decode_fwd(one, two, three, three, one, null, 3, -1, 1.0, 4, 64, 64, 1, null) == -1
+    assert lib.oslo_attention_decode_fwd(null, null, null, null, null, null, 0, 0, 1.0, 0, 64, 64, 1, null) == 0
+    assert lib.oslo_attention_decode_workspace_bytes(16, 1152, 256, 2) == 16 * 18 * 258 * 4
+    assert lib.oslo_attention_decode_workspace_bytes(16, 1152, 48, 2) == 0
     # n-gram blocking
     assert lib.oslo_ngram_repeat_block(one, one, 2, 4, 3, 8, 0, null) == -1
     assert lib.oslo_ngram_repeat_block(null, one, 2, 4, 3, 8, 2, null) == -1

@@ -425,3 +425,23 @@ def test_linear_rows_against_loops_and_library():
         torch.nn.functional.linear(torch.from_numpy(x), torch.from_numpy(w), torch.from_numpy(b)), approximate="tanh")
     assert np.allclose(orc.linear_rows(x, w, b, gelu=True), want.numpy(), atol=1e-7)
     assert orc.linear_rows(x, w, b).shape == (3, 5)
+
+
+def test_attention_decode_against_library_and_closed_form():
+    rng = np.random.default_rng(9)
+    n, cap, d, last = 3, 12, 8, 7
+    q, k, v = rng.standard_normal((n, d)), rng.standard_normal((n, cap, d)), rng.standard_normal((n, cap, d))
+    got = orc.attention_decode(q, k, v, last, 0.3)
+    # torch's attention over the visible keys only
+    tq, tk, tv = (torch.from_numpy(t) for t in (q[:, None, :], k[:, :last + 1], v[:, :last + 1]))
+    want = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, scale=0.3)[:, 0].numpy()
+    assert np.allclose(got, want, atol=1e-12)
+    # this file's masked softmax (keys past `last` masked) composed with matmuls
+    scores = np.einsum("nd,nsd->ns", q, k)[:, None, None, :]
+    mask = (np.arange(cap) > last)[None, None, None, :].repeat(n, 0)
+    probs = orc.softmax_masked(scores, mask, 0.3, mode="add", dtype=np.float64)[:, 0, 0]
+    assert np.allclose(got, np.einsum("ns,nsd->nd", probs, v), atol=1e-9)
+    # a sliding window of 3 sees keys 5, 6, 7; equal scores give the mean of their values
+    win = orc.attention_decode(np.zeros((n, d)), k, v, last, 1.0, window=3)
+    assert np.allclose(win, v[:, 5:8].mean(axis=1), atol=1e-12)
+    assert np.allclose(orc.attention_decode(q, k, v, 0, 1.0), v[:, 0], atol=1e-12)   # one visible key
