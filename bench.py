@@ -343,6 +343,22 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
             res.append(roof(f"linear_rows {what} bf16 {m} x [{n_out},{k_in}]",
                             2 * (n_out * k_in + m * k_in + m * n_out + n_out), t, m * n_out, n_sets))
         del weights
+
+    # the attention of a decoding step at the GPT-J head shape: 1024 visible keys of a 1152-slot cache
+    H, cap, D, last = 16, 1152, 256, 1023
+    for rows in (1, 8):
+        n_sets = 8
+        caches = [(randn((rows * H, cap, D), 30 + i, 1.0, torch.bfloat16), randn((rows * H, cap, D), 40 + i, 1.0, torch.bfloat16))
+                  for i in range(n_sets)]
+        qd = randn((rows * H, D), 6, 1.0, torch.bfloat16)
+        od = torch.empty_like(qd)
+        wsd = torch.empty(lib.oslo_attention_decode_workspace_bytes(rows * H, cap, D, BF16) // 4,
+                          dtype=torch.float32, device=dev)
+        t = time_launches(rotating(caches, lambda kv: check(lib.oslo_attention_decode_fwd(
+            P(od), P(qd), P(kv[0]), P(kv[1]), P(wsd), None, last, 0, 1 / 16.0, rows * H, cap, D, BF16, st))), n, 3)
+        res.append(roof(f"attention_decode bf16 {rows} x 16 heads, 1024 of 1152 keys, head 256 (two launches)",
+                        2 * 2 * rows * H * (last + 1) * D, t, rows * H * D, n_sets))
+        del caches
     return res
 
 
