@@ -348,7 +348,11 @@ int oslo_linear_rows_fwd_multi(void *const *out, const void *x,
  * last - window + 1 for window > 0 (a sliding window, as in GPT-Neo's local
  * layers), else 0. q, out: [rows_heads, head_dim]; k, v: [rows_heads, capacity,
  * head_dim] (a [batch, heads, capacity, head_dim] cache); 0 <= last < capacity.
- * Keys outside the visible range are not read. workspace: fp32, at least
+ * Keys outside the visible range are not read. k_new, v_new: both NULL, or
+ * [rows_heads, head_dim]: the key and value of position `last`, which are then
+ * used from there and written into slot `last` of k and v by the kernel (the
+ * append to the cache and the attention in one launch); the other slots of k
+ * and v are only read. workspace: fp32, at least
  * oslo_attention_decode_workspace_bytes(...) bytes, contents irrelevant before
  * and after. head_dim * sizeof(dtype) must be 128, 256, 512 or 1024 bytes.
  * Arithmetic in fp32 throughout (scores, softmax, weighted sum), one rounding
@@ -362,8 +366,9 @@ int oslo_linear_rows_fwd_multi(void *const *out, const void *x,
 size_t oslo_attention_decode_workspace_bytes(int64_t rows_heads,
                                              int64_t capacity, int64_t head_dim,
                                              int dtype);
-int oslo_attention_decode_fwd(void *out, const void *q, const void *k,
-                              const void *v, float *workspace,
+int oslo_attention_decode_fwd(void *out, const void *q, void *k, void *v,
+                              const void *k_new, const void *v_new,
+                              float *workspace,
                               const int64_t *pos_dev, int64_t pos,
                               int64_t window, float scale, int64_t rows_heads,
                               int64_t capacity, int64_t head_dim, int dtype,

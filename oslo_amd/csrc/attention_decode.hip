@@ -51,10 +51,10 @@ struct DecodeTile {
 // domain), sum of exponentials, accumulator.
 template <typename T, int LPK>
 __global__ __launch_bounds__(kBlockThreads) void attention_decode_partial_kernel(
-    float *__restrict__ ws, const T *__restrict__ q, const T *__restrict__ k,
-    const T *__restrict__ v, const int64_t *__restrict__ pos_dev,
-    int64_t pos_host, int window, float scale_log2e, int capacity,
-    int head_dim, int splits, int tiles) {
+    float *__restrict__ ws, const T *__restrict__ q, T *k, T *v,
+    const T *__restrict__ k_new, const T *__restrict__ v_new,
+    const int64_t *__restrict__ pos_dev, int64_t pos_host, int window,
+    float scale_log2e, int capacity, int head_dim, int splits, int tiles) {
   constexpr int VEC = Io<T>::kVec;
   using Tile = DecodeTile<LPK>;
   constexpr int U = Tile::kLoads;
@@ -91,6 +91,15 @@ __global__ __launch_bounds__(kBlockThreads) void attention_decode_partial_kernel
   const BufRsrc qrs = make_rsrc(q + bh * (int64_t)head_dim, key_bytes);
   float qf[VEC];
   raw_to_f32<T, VEC>(qf, buffer_load_raw<T, VEC, false>(qrs, (uint32_t)dl * 16u));
+  // The key and value of the query's own position may still be outside the
+  // cache: they are used from where they are and written into their slot by
+  // the one wave that owns it.
+  const bool fresh = k_new != nullptr;
+  RawVec<T, VEC> knew, vnew;
+  if (fresh) {
+    knew = buffer_load_raw<T, VEC, false>(make_rsrc(k_new + bh * (int64_t)head_dim, key_bytes), (uint32_t)dl * 16u);
+    vnew = buffer_load_raw<T, VEC, false>(make_rsrc(v_new + bh * (int64_t)head_dim, key_bytes), (uint32_t)dl * 16u);
+  }
 
   // running maximum, sum and accumulator of the wave (over its tiles)
   float m = -INFINITY, l = 0.f;
@@ -108,9 +117,23 @@ __global__ __launch_bounds__(kBlockThreads) void attention_decode_partial_kernel
     for (int u = 0; u < U; ++u) {
       const int s = key0 + u * Tile::kKeysPerLoad + sub;
       vis[u] = s >= first && s <= last;
-      const uint32_t off = vis[u] ? (uint32_t)s * key_bytes + (uint32_t)dl * 16u : kOutside;
+      const bool from_cache = vis[u] && !(fresh && s == last);
+      const uint32_t off = from_cache ? (uint32_t)s * key_bytes + (uint32_t)dl * 16u : kOutside;
       kraw[u] = buffer_load_raw<T, VEC, true>(krs, off);
       vraw[u] = buffer_load_raw<T, VEC, true>(vrs, off);
+    }
+    if (fresh) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int s = key0 + u * Tile::kKeysPerLoad + sub;
+        if (s == last) {
+          kraw[u] = knew;
+          vraw[u] = vnew;
+          const int64_t slot = (bh * capacity + s) * (int64_t)head_dim + dl * VEC;
+          *reinterpret_cast<RawVec<T, VEC> *>(k + slot) = knew;
+          *reinterpret_cast<RawVec<T, VEC> *>(v + slot) = vnew;
+        }
+      }
     }
 
     // scores of the tile's keys, in log2 units; every lane of a key gets its score
@@ -237,8 +260,8 @@ __global__ __launch_bounds__(kMergeThreads) void attention_decode_merge_kernel(
 }
 
 template <typename T, int LPK>
-int launch(void *out, const void *q, const void *k, const void *v, float *ws,
-           const int64_t *pos_dev, int64_t pos, int window, float scale,
+int launch(void *out, const void *q, void *k, void *v, const void *k_new,
+           const void *v_new, float *ws, const int64_t *pos_dev, int64_t pos, int window, float scale,
            int64_t rows_heads, int capacity, int head_dim, hipStream_t stream) {
   // As many splits as fill the device (about four blocks per CU), not more:
   // every split is a partial result the merge has to read. A block then covers
@@ -250,9 +273,9 @@ int launch(void *out, const void *q, const void *k, const void *v, float *ws,
   splits = (most + tiles - 1) / tiles;
   attention_decode_partial_kernel<T, LPK>
       <<<dim3((unsigned)(rows_heads * splits)), dim3(kBlockThreads), 0, stream>>>(
-          ws, static_cast<const T *>(q), static_cast<const T *>(k),
-          static_cast<const T *>(v), pos_dev, pos, window, scale * kLog2e,
-          capacity, head_dim, splits, tiles);
+          ws, static_cast<const T *>(q), static_cast<T *>(k), static_cast<T *>(v),
+          static_cast<const T *>(k_new), static_cast<const T *>(v_new), pos_dev,
+          pos, window, scale * kLog2e, capacity, head_dim, splits, tiles);
   attention_decode_merge_kernel<T>
       <<<dim3((unsigned)rows_heads), dim3(kMergeThreads), 0, stream>>>(
           static_cast<T *>(out), ws, head_dim, splits);
@@ -294,8 +317,9 @@ extern "C" size_t oslo_attention_decode_workspace_bytes(int64_t rows_heads,
   return (size_t)rows_heads * (size_t)splits * (size_t)(2 + head_dim) * sizeof(float);
 }
 
-extern "C" int oslo_attention_decode_fwd(void *out, const void *q, const void *k,
-                                         const void *v, float *workspace,
+extern "C" int oslo_attention_decode_fwd(void *out, const void *q, void *k,
+                                         void *v, const void *k_new,
+                                         const void *v_new, float *workspace,
                                          const int64_t *pos_dev, int64_t pos,
                                          int64_t window, float scale,
                                          int64_t rows_heads, int64_t capacity,
@@ -328,16 +352,18 @@ extern "C" int oslo_attention_decode_fwd(void *out, const void *q, const void *k
                 (long long)pos, (long long)capacity);
   if (!out || !q || !k || !v || !workspace)
     return fail(OSLO_E_BAD_ARG, "oslo_attention_decode_fwd: null pointer");
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v))
-    return fail(OSLO_E_BAD_ARG, "oslo_attention_decode_fwd: q, k and v must be 16-byte aligned");
+  if ((k_new == nullptr) != (v_new == nullptr))
+    return fail(OSLO_E_BAD_ARG, "oslo_attention_decode_fwd: k_new and v_new go together");
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(k_new) || !aligned16(v_new))
+    return fail(OSLO_E_BAD_ARG, "oslo_attention_decode_fwd: q, k, v, k_new and v_new must be 16-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int win = window > capacity ? (int)capacity : (int)window;
   OSLO_DISPATCH_DTYPE(dtype, {
     switch (lpk) {
-    case 8: return launch<T, 8>(out, q, k, v, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
-    case 16: return launch<T, 16>(out, q, k, v, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
-    case 32: return launch<T, 32>(out, q, k, v, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
-    default: return launch<T, 64>(out, q, k, v, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
+    case 8: return launch<T, 8>(out, q, k, v, k_new, v_new, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
+    case 16: return launch<T, 16>(out, q, k, v, k_new, v_new, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
+    case 32: return launch<T, 32>(out, q, k, v, k_new, v_new, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
+    default: return launch<T, 64>(out, q, k, v, k_new, v_new, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
     }
   });
   return OSLO_OK;

@@ -526,9 +526,13 @@ class FusedDecodeAttention(object):
         return not _needs_grad(query, key)
 
     @staticmethod
-    def apply(query, key, value, pos, scale, window=None):
+    def apply(query, key, value, pos, scale, window=None, new_key=None, new_value=None):
+        """``new_key``, ``new_value``: the key and value of position ``pos``
+        when they are not in the caches yet; the kernel then also writes them
+        into slot ``pos`` of ``key`` and ``value``."""
         scale = 1.0 if scale is None else scale
-        return get_custom_kernels().attention_decode_forward(query, key, value, pos, scale, window or 0)
+        return get_custom_kernels().attention_decode_forward(query, key, value, pos, scale, window or 0,
+                                                             new_key, new_value)
 
 
 class FusedLinearRows(object):

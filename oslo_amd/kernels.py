@@ -477,12 +477,15 @@ def linear_rows_forward_multi(x, weights, biases=None, gelu=False):
     return outs
 
 
-def attention_decode_forward(query, key, value, pos, scale, window=0):
+def attention_decode_forward(query, key, value, pos, scale, window=0, new_key=None, new_value=None):
     """query [B, H, 1, D]; key, value [B, H, L, D] caches; attends keys
     first..last, last = ``pos`` (an int, or an int64 device tensor of one
     element that the kernel reads), first = last - window + 1 for window > 0,
     else 0. Returns softmax(scale * q k^T) v as [B, H, 1, D]
-    (oslo/models/gptj/modeling_gptj.py:936-951 for a query length of 1)."""
+    (oslo/models/gptj/modeling_gptj.py:936-951 for a query length of 1).
+    ``new_key``, ``new_value`` [B, H, 1, D]: the key and value of position
+    ``pos``, not yet in the caches; the kernel uses them and writes them into
+    slot ``pos`` of ``key`` and ``value``, which must then be contiguous."""
     _device_tensor(query, "query")
     _device_tensor(key, "key", query)
     _device_tensor(value, "value", query)
@@ -495,6 +498,13 @@ def attention_decode_forward(query, key, value, pos, scale, window=0):
     _require(key.dtype == query.dtype and value.dtype == query.dtype, "query, key and value differ in dtype")
     cap = key.shape[2]
     q, k, v = query.contiguous(), key.contiguous(), value.contiguous()
+    _require((new_key is None) == (new_value is None), "new_key and new_value go together")
+    if new_key is not None:
+        _require(key.is_contiguous() and value.is_contiguous(), "caches that take a new key must be contiguous")
+        for t, what in ((new_key, "new_key"), (new_value, "new_value")):
+            _device_tensor(t, what, query)
+            _require(t.shape == query.shape and t.dtype == query.dtype, f"{what} must be like the query")
+        new_key, new_value = new_key.contiguous(), new_value.contiguous()
     pos_dev, pos_host = None, 0
     if isinstance(pos, torch.Tensor):
         _device_tensor(pos, "pos", query)
@@ -509,7 +519,8 @@ def attention_decode_forward(query, key, value, pos, scale, window=0):
     out = torch.empty_like(q)
     with _on_device(q):
         _lib.check(lib.oslo_attention_decode_fwd(
-            _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(ws), _ptr(pos_dev), pos_host, int(window),
+            _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(new_key), _ptr(new_value), _ptr(ws), _ptr(pos_dev),
+            pos_host, int(window),
             float(scale), b * h, cap, d, code, _stream(q)))
     return out
 

@@ -153,7 +153,7 @@ class FusedGPT2Attention(GPT2Attention):
                 hidden_states.is_cuda and FusedSplitHeads.is_available(hidden_states.dtype, self.head_dim)):
             return super()._project_qkv(hidden_states, layer_past, encoder_hidden_states, use_cache)
         query, key, value = FusedSplitHeads.apply(self.c_attn(hidden_states), self.num_heads)
-        key, value, present = append_kv(layer_past, key, value, use_cache)
+        key, value, present = append_kv(layer_past, key, value, use_cache, defer=True)
         return query, key, value, present
 
     def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
@@ -179,12 +179,17 @@ class FusedGPT2Attention(GPT2Attention):
         one_pass = (sq == 1 and not self.is_cross_attention and attention_mask is None and head_mask is None
                     and not output_attentions
                     and FusedDecodeAttention.is_available(query, key, self.training, self.attn_dropout.p))
+        fresh = (None, None)  # the step's key and value, if not yet in a static cache
+        if static and one_pass and layer_past.pending_is_dense():
+            fresh = layer_past.take_pending()  # the kernel below writes them into their slot
+        elif static:
+            layer_past.flush()
         if static and not one_pass:
             attention_mask = static_cache_mask(layer_past, attention_mask, fused)
         if one_pass:
             # a decoding step: scores, softmax and weighted sum in one pass over the cache
             out = FusedDecodeAttention.apply(query, key, value, layer_past.state.pos if static else sk - 1,
-                                             self._attention_scale(value))
+                                             self._attention_scale(value), None, *fresh)
             w = None
         elif fused:
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)

@@ -186,7 +186,7 @@ class FusedGPTJAttention(GPTJAttention):
         query, key, value = FusedLinearRows.project_many((self.q_proj, self.k_proj, self.v_proj), hidden_states)
         query, key, value = FusedRotaryPositionEmbedding.apply(
             query.view(shape), key.view(shape), value.view(shape), (sin, cos), rot, offset)
-        key, value, present = append_kv(layer_past, key, value, use_cache)
+        key, value, present = append_kv(layer_past, key, value, use_cache, defer=True)
         return query, key, value, present
 
     def _fused_attn(self, query, key, value, attention_mask=None, head_mask=None, causal=True):
@@ -210,12 +210,17 @@ class FusedGPTJAttention(GPTJAttention):
         fused = FusedScaleMaskSoftmax.is_available(query.dtype, bsz, np_, sq, sk, use_triang_mask=causal)
         one_pass = (sq == 1 and attention_mask is None and head_mask is None and not output_attentions
                     and FusedDecodeAttention.is_available(query, key, self.training, self.attn_dropout.p))
+        fresh = (None, None)  # the step's key and value, if not yet in a static cache
+        if static and one_pass and layer_past.pending_is_dense():
+            fresh = layer_past.take_pending()  # the kernel below writes them into their slot
+        elif static:
+            layer_past.flush()
         if static and not one_pass:
             attention_mask = static_cache_mask(layer_past, attention_mask, fused)
         if one_pass:
             # a decoding step: scores, softmax and weighted sum in one pass over the cache
             out = FusedDecodeAttention.apply(query, key, value, layer_past.state.pos if static else sk - 1,
-                                             1.0 / self.scale_attn)
+                                             1.0 / self.scale_attn, None, *fresh)
             w = None
         elif fused:
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)

@@ -141,6 +141,7 @@ class StaticKV(object):
         if k.shape != v.shape or k.dim() != 4 or k.size(2) != state.capacity:
             raise ValueError("StaticKV: buffers must be two [rows, heads, capacity, head_dim] tensors")
         self.state, self.k, self.v = state, k, v
+        self.pending = None  # (key, value) of the step, handed over but not yet in the buffers
 
     @classmethod
     def allocate(cls, state, layers, rows, heads, head_dim, dtype, device):
@@ -156,18 +157,39 @@ class StaticKV(object):
         self.k[:, :, :n].copy_(key)
         self.v[:, :, :n].copy_(value)
 
-    def update(self, key, value):
+    def update(self, key, value, defer=False):
+        """The step's key and value join the buffers at ``state.pos``. With
+        ``defer`` they are only kept: the caller then either passes them to the
+        one-pass attention kernel, which writes them into their slot itself
+        (``take_pending``), or has them written before it reads the buffers
+        (``flush``)."""
         if key.size(-2) != 1:
             raise RuntimeError("StaticKV: a static cache takes one token per step")
-        self.k.index_copy_(2, self.state.pos, key)
-        self.v.index_copy_(2, self.state.pos, value)
+        self.pending = (key, value)
+        if not defer:
+            self.flush()
         return self.k, self.v
 
+    def pending_is_dense(self):
+        """A key/value pair is waiting and the kernel can read it as it lies."""
+        return self.pending is not None and all(t.is_contiguous() for t in self.pending)
 
-def append_kv(layer_past, key, value, use_cache):
-    """key/value of this call joined to the cache -> (key, value, present)."""
+    def take_pending(self):
+        pending, self.pending = self.pending, None
+        return pending
+
+    def flush(self):
+        if self.pending is not None:
+            key, value = self.take_pending()
+            self.k.index_copy_(2, self.state.pos, key)
+            self.v.index_copy_(2, self.state.pos, value)
+
+
+def append_kv(layer_past, key, value, use_cache, defer=False):
+    """key/value of this call joined to the cache -> (key, value, present).
+    ``defer``: see StaticKV.update (no effect on other caches)."""
     if isinstance(layer_past, StaticKV):
-        key, value = layer_past.update(key, value)
+        key, value = layer_past.update(key, value, defer)
         return key, value, layer_past
     if layer_past is not None:
         key = torch.cat((layer_past[0], key), dim=-2)

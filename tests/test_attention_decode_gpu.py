@@ -93,6 +93,27 @@ def test_attention_decode_against_the_three_step_path():
     assert (out.float() - want.float()).abs().max() <= 2e-2 * want.float().abs().max()
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("cap,last,window", [(64, 0, 0), (100, 37, 0), (300, 299, 0), (300, 150, 16)])
+def test_attention_decode_appends_the_new_key(cap, last, window, dtype):
+    """The key and value of the query's position handed over outside the cache:
+    same result, bit for bit, as with them in the cache, and afterwards they
+    are in their slot and no other slot has changed."""
+    b, h, d = 2, 3, 64
+    q = randn((b, h, 1, d), dtype, seed=1).to(DEV)
+    k = randn((b, h, cap, d), dtype, seed=2).to(DEV)
+    v = randn((b, h, cap, d), dtype, seed=3).to(DEV)
+    want = kernels.attention_decode_forward(q, k, v, last, 0.25, window)
+    k2, v2 = k.clone(), v.clone()
+    k2[:, :, last] = 7.0            # the slot holds something else until the kernel fills it
+    v2[:, :, last] = -7.0
+    pos = torch.tensor([last], dtype=torch.int64, device=DEV)
+    got = kernels.attention_decode_forward(q, k2, v2, pos, 0.25, window,
+                                           k[:, :, last:last + 1].contiguous(), v[:, :, last:last + 1].contiguous())
+    assert torch.equal(got, want)
+    assert torch.equal(k2, k) and torch.equal(v2, v)
+
+
 def test_attention_decode_errors():
     q = torch.zeros(1, 2, 1, 64, device=DEV)
     kv = torch.zeros(1, 2, 16, 64, device=DEV)
