@@ -48,14 +48,32 @@ class DynamicDecoder(object):
         return out["logits"][:, -1, :]
 
 
+def _model_fingerprint(model):
+    """What a captured step depends on besides its inputs: the classes of the
+    modules (``fuse()`` changes them), the storage of every parameter and
+    buffer (``.half()`` or loading weights replaces it) and the mode."""
+    return (model.training,
+            tuple(id(type(m)) for m in model.modules()),
+            tuple(t.data_ptr() for t in model.parameters()),
+            tuple(t.data_ptr() for t in model.buffers()))
+
+
 class StaticDecoder(object):
-    """Steps over static caches; optionally each step is one graph replay."""
+    """Steps over static caches; optionally each step is one graph replay. The
+    first ``step`` takes the whole prompt (an ordinary forward whose keys and
+    values fill the caches), every later one the sequences grown by one token.
+    ``restart()`` makes the next ``step`` a first one again: the buffers and
+    the captured graphs are kept as long as the shapes stay the same."""
 
     def __init__(self, model, capacity, graph):
         # whole 64-key vectors: the key-mask softmax then takes its vector path
         self.model, self.capacity, self.graph = model, -(-int(capacity) // 64) * 64, graph
         self.caches = None
-        self._captured = None
+        self._captured = {}  # reorder flag -> (graph, logits)
+        self._started = False
+
+    def restart(self):
+        self._started = False
 
     def _prefill(self, ids):
         from .modeling_utils import DecodeState, StaticKV
@@ -63,14 +81,22 @@ class StaticDecoder(object):
         out = self.model(ids, use_cache=True)
         presents = out["past_key_values"]
         k0 = presents[0][0]
-        self.state = DecodeState(self.capacity, ids.device, k0.dtype)
-        self.store, self.caches = StaticKV.allocate(self.state, len(presents), k0.size(0), k0.size(1), k0.size(3),
-                                                    k0.dtype, k0.device)
+        shape = (len(presents), 2, k0.size(0), k0.size(1), self.capacity, k0.size(3))
+        if self.caches is None or tuple(self.store.shape) != shape or self.store.dtype != k0.dtype \
+                or self.store.device != k0.device:
+            self.state = DecodeState(self.capacity, ids.device, k0.dtype)
+            self.store, self.caches = StaticKV.allocate(self.state, len(presents), k0.size(0), k0.size(1), k0.size(3),
+                                                        k0.dtype, k0.device)
+            self.token = ids[:, -1:].clone()
+            self.beam_idx = torch.arange(ids.size(0), device=ids.device)
+            self._captured = {}
+        # slots past the prompt may hold an earlier sequence: they are hidden
+        # until a step writes them
         for cache, (key, value) in zip(self.caches, presents):
+            cache.pending = None
             cache.fill(key, value)
         self.state.pos.fill_(ids.size(1))
-        self.token = ids[:, -1:].clone()
-        self.beam_idx = torch.arange(ids.size(0), device=ids.device)
+        self._started = True
         return out["logits"][:, -1, :]
 
     def _run(self, reorder):
@@ -102,7 +128,7 @@ class StaticDecoder(object):
         return graph, logits
 
     def step(self, ids, beam_idx=None):
-        if self.caches is None:
+        if not self._started:
             return self._prefill(ids)
         if int(ids.size(1)) > self.capacity:
             raise RuntimeError("generate: the static cache is full")
@@ -112,9 +138,9 @@ class StaticDecoder(object):
         reorder = beam_idx is not None
         if not self.graph:
             return self._run(reorder)
-        if self._captured is None:
-            self._captured = self._capture(reorder)
-        graph, logits = self._captured
+        if reorder not in self._captured:
+            self._captured[reorder] = self._capture(reorder)
+        graph, logits = self._captured[reorder]
         graph.replay()
         return logits
 
@@ -189,7 +215,7 @@ class GenerationMixin(object):
         if static_cache and not use_cache:
             raise ValueError("generate: static_cache=True contradicts use_cache=False")
         if static_cache:
-            decoder = StaticDecoder(self, max_length, graph)
+            decoder = self._static_decoder(max_length, graph)
         else:
             decoder = DynamicDecoder(self, use_cache)
 
@@ -212,6 +238,20 @@ class GenerationMixin(object):
             return self._greedy_search(input_ids, max_length, scores_of, eos_token_id, pad_token_id, decoder)
         return self._beam_search(input_ids, max_length, min_length, num_beams, scores_of, eos_token_id,
                                  pad_token_id, length_penalty, decoder)
+
+    def _static_decoder(self, max_length, graph):
+        """The decoder of the previous call when nothing it captured has
+        changed (the graph of a step is worth keeping: capturing it costs as
+        much as some twenty steps), else a new one."""
+        if not graph:
+            return StaticDecoder(self, max_length, False)
+        key = (-(-int(max_length) // 64) * 64, _model_fingerprint(self))
+        kept = self.__dict__.get("_kept_decoder")
+        if kept is None or kept[0] != key:
+            kept = (key, StaticDecoder(self, max_length, True))
+            self.__dict__["_kept_decoder"] = kept
+        kept[1].restart()
+        return kept[1]
 
     @staticmethod
     def _greedy_search(ids, max_length, scores_of, eos_token_id, pad_token_id, decoder):

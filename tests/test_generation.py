@@ -151,9 +151,21 @@ def test_graphed_decoding_same_tokens(family):
         for extra in (dict(static_cache=True), dict(graph=True)):
             got = model.generate(ids, **kw, **extra)
             assert got.shape == w.shape and torch.equal(got, w), (kw, extra)
+    # a second prompt reuses the captured steps of the first (same shapes); another batch size does not
+    kept = model._kept_decoder[1]
+    ids2 = torch.randint(1, 211, (2, 6), generator=torch.Generator().manual_seed(5)).cuda()
+    ids3 = torch.randint(1, 211, (3, 9), generator=torch.Generator().manual_seed(6)).cuda()
+    for other in (ids2, ids3, ids):
+        for kw in DECODING[:2]:
+            assert torch.equal(model.generate(other, graph=True, **kw), model.generate(other, **kw)), kw
+        assert model._kept_decoder[1] is kept
     # the fused ban reads the growing token tensor outside the graph
     kw = dict(max_length=50, min_length=50, num_beams=3, no_repeat_ngram_size=2)
     assert torch.equal(model.generate(ids, graph=True, fused_no_repeat_ngram_blocking=True, **kw), want[1])
+    # new storage for the weights: the kept graph would read the old one, so it is dropped
+    model = model.double().float()
+    assert torch.equal(model.generate(ids, graph=True, **DECODING[1]), want[1])
+    assert model._kept_decoder[1] is not kept
     model.train()
     with pytest.raises(RuntimeError):
         model.generate(ids, max_length=20, graph=True)
