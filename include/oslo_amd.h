@@ -337,6 +337,19 @@ int oslo_linear_rows_fwd_multi(void *const *out, const void *x,
                                int64_t n, int64_t k, int epilogue, int dtype,
                                oslo_stream_t stream);
 
+/*
+ * The same layer with the weight stored [k, n] (input features major), the
+ * layout of GPT-2's Conv1D (transformers' pytorch_utils.Conv1D, y = x @ w + b):
+ * out[i, j] = epilogue( sum_c x[i, c] * weight[c, j] + bias[j] ). Both k and n
+ * times sizeof(dtype) must be multiples of 16. Replaces, for a decoding step,
+ * self.c_attn(hidden_states), `attn_output @= self.c_proj.weight` + bias and the
+ * two projections of the fused feed-forward module with FusedBiasActivation
+ * (oslo/models/gpt2/modeling_gpt2.py:1485, :1523-1536, :1553-1567).
+ */
+int oslo_linear_rows_kn_fwd(void *out, const void *x, const void *weight,
+                            const void *bias, int64_t m, int64_t n, int64_t k,
+                            int epilogue, int dtype, oslo_stream_t stream);
+
 /* Attention of a decoding step ----------------------------------------------- */
 
 /*

@@ -195,6 +195,17 @@ __device__ __forceinline__ float wave_allreduce(float v, Op op) {
   return op(lo, hi);
 }
 
+// Sum over the 16 lanes of a DPP row (lane / 16 equal), left in every one of
+// them: four DPP steps in the vector ALU, the first four of wave_allreduce. A
+// ds_bpermute shuffle would take each value through the LDS crossbar instead.
+__device__ __forceinline__ float sum_over_row(float v) {
+  v += dpp_move<0xB1>(v);  // lane ^ 1
+  v += dpp_move<0x4E>(v);  // lane ^ 2
+  v += dpp_move<0x141>(v); // row_half_mirror: the other quad of 8
+  v += dpp_move<0x140>(v); // row_mirror: the other half of 16
+  return v;
+}
+
 // ---------------------------------------------------------------------------
 // Host side: status + per-thread error text.
 // ---------------------------------------------------------------------------

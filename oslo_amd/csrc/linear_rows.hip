@@ -321,8 +321,165 @@ int linear_rows(void *const *out, const void *x, const void *const *weight,
   return OSLO_OK;
 }
 
+// The same layer with the weight stored [k, n] (in_features major), the layout
+// of GPT-2's Conv1D: out[i, j] = sum_c x[i, c] * w[c, j]. Here a row of w holds
+// one input feature for all outputs, so the lanes go along j: a block owns a
+// strip of 4 lanes x one vector of output features (64 bytes of every weight
+// row; narrow, because these matrices have few output features and every strip
+// is a block) and its 16 waves share the k rows. A wave-wide load covers 16
+// rows of the strip; a lane takes VEC consecutive rows per step, so that its
+// inputs x[i, c..c+VEC) are one vector load per input row. The 16 row groups
+// of a wave are the 16 lanes of a DPP row (lane % 16), so that their sums meet
+// by DPP in the vector ALU; the 16 waves then meet in LDS.
+// These matrices are small (a few MB): the launch is bound by latency, and one
+// block per strip keeps it to a single launch with a fixed summation order.
+constexpr int kKnThreads = 1024;
+constexpr int kKnWaves = kKnThreads / kWave;
+constexpr int kStripLanes = 4; // lanes along the output features
+
+template <typename T, int VEC, int MT>
+__global__ __launch_bounds__(kKnThreads) void linear_rows_kn_kernel(
+    T *__restrict__ out, const T *__restrict__ x, const T *__restrict__ w,
+    const T *__restrict__ bias, int m, int64_t n, int64_t k, int gelu) {
+  constexpr int kRowGroups = kWave / kStripLanes; // 16 rows per load instruction
+  constexpr int kStrip = kStripLanes * VEC;       // output features per block
+  __shared__ float red[kKnWaves][MT][kStrip];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int group = lane % kRowGroups, cl = lane / kRowGroups; // rows by lane % 16, features by lane / 16
+  const int64_t col = (int64_t)blockIdx.x * kStrip + cl * VEC;
+  const bool col_ok = col < n; // n is a multiple of VEC
+  const BufRsrc wrs = make_rsrc(w, (uint32_t)(n * k * (int64_t)sizeof(T)));
+  const BufRsrc xrs = make_rsrc(x, (uint32_t)((int64_t)m * k * (int64_t)sizeof(T)));
+  const uint32_t wrow_bytes = (uint32_t)(n * (int64_t)sizeof(T));
+  const uint32_t xrow_bytes = (uint32_t)(k * (int64_t)sizeof(T));
+
+  float acc[MT][VEC];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[i][j] = 0.f;
+
+  constexpr int kRowsPerWave = kRowGroups * VEC; // rows of one wave per step
+  for (int64_t k0 = (int64_t)wave * kRowsPerWave; k0 < k; k0 += (int64_t)kKnWaves * kRowsPerWave) {
+    const int64_t row = k0 + group * VEC; // the lane's VEC consecutive rows (k is a multiple of VEC)
+    const bool row_ok = row < k;
+    RawVec<T, VEC> wv[VEC];
+#pragma unroll
+    for (int u = 0; u < VEC; ++u)
+      wv[u] = buffer_load_raw<T, VEC, true>(
+          wrs, row_ok && col_ok ? (uint32_t)(row + u) * wrow_bytes + (uint32_t)col * (uint32_t)sizeof(T) : kOutside);
+    RawVec<T, VEC> xv[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+      xv[i] = buffer_load_raw<T, VEC, false>(
+          xrs, row_ok && i < m ? (uint32_t)i * xrow_bytes + (uint32_t)row * (uint32_t)sizeof(T) : kOutside);
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) {
+      float wf[VEC];
+      raw_to_f32<T, VEC>(wf, wv[u]);
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const float xi = static_cast<float>(xv[i][u]);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[i][j] = __builtin_fmaf(xi, wf[j], acc[i][j]);
+      }
+    }
+  }
+
+  // the 16 row groups of the wave, then the 16 waves
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      static_assert(kRowGroups == 16, "the row groups are the 16 lanes of a DPP row");
+      acc[i][j] = sum_over_row(acc[i][j]);
+    }
+  if (group == 0) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) red[wave][i][cl * VEC + j] = acc[i][j];
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < m * kStrip; t += kKnThreads) {
+    const int i = t / kStrip, c = t % kStrip;
+    const int64_t j = (int64_t)blockIdx.x * kStrip + c;
+    if (j >= n) continue;
+    float v = 0.f;
+#pragma unroll
+    for (int wv_ = 0; wv_ < kKnWaves; ++wv_) v += red[wv_][i][c];
+    if (bias != nullptr) v += static_cast<float>(bias[j]);
+    if (gelu) v = gelu_fwd(v);
+    out[(int64_t)i * n + j] = static_cast<T>(v);
+  }
+}
+
+template <typename T, int MT>
+int launch_kn(void *out, const void *x, const void *w, const void *bias, int m,
+              int64_t n, int64_t k, int gelu, hipStream_t stream) {
+  constexpr int VEC = Io<T>::kVec;
+  constexpr int kStrip = kStripLanes * VEC;
+  const int64_t blocks = (n + kStrip - 1) / kStrip;
+  linear_rows_kn_kernel<T, VEC, MT>
+      <<<dim3((unsigned)blocks), dim3(kKnThreads), 0, stream>>>(
+          static_cast<T *>(out), static_cast<const T *>(x),
+          static_cast<const T *>(w), static_cast<const T *>(bias), m, n, k, gelu);
+  return check_launch("oslo_linear_rows_kn_fwd");
+}
+
 } // namespace
 } // namespace oslo
+
+extern "C" int oslo_linear_rows_kn_fwd(void *out, const void *x, const void *weight,
+                                       const void *bias, int64_t m, int64_t n,
+                                       int64_t k, int epilogue, int dtype,
+                                       oslo_stream_t stream) {
+  using namespace oslo;
+  if (m < 0 || n < 0 || k < 0)
+    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_kn_fwd: negative size");
+  if (epilogue != OSLO_EPILOGUE_NONE && epilogue != OSLO_EPILOGUE_GELU_TANH)
+    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_kn_fwd: unknown epilogue %d", epilogue);
+  if (dtype != OSLO_F32 && dtype != OSLO_F16 && dtype != OSLO_BF16)
+    return fail(OSLO_E_BAD_ARG, "unknown dtype %d", dtype);
+  if (m > kMaxRows)
+    return fail(OSLO_E_UNSUPPORTED,
+                "oslo_linear_rows_kn_fwd: %lld input rows, at most %d (use a GEMM)",
+                (long long)m, kMaxRows);
+  if (m == 0 || n == 0) return OSLO_OK;
+  if (!out || !x || !weight)
+    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_kn_fwd: null pointer");
+  const int64_t es = dtype == OSLO_F32 ? 4 : 2;
+  if (k == 0 || (k * es) % 16 != 0 || (n * es) % 16 != 0)
+    return fail(OSLO_E_UNSUPPORTED,
+                "oslo_linear_rows_kn_fwd: %lld x %lld: rows of x and of the weight must be whole 16-byte vectors",
+                (long long)k, (long long)n);
+  if (!aligned16(x) || !aligned16(weight))
+    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_kn_fwd: x and weight must be 16-byte aligned");
+  if (n > (int64_t)0x7fffffff / (k * es) || m > (int64_t)0x7fffffff / (k * es))
+    return fail(OSLO_E_UNSUPPORTED,
+                "oslo_linear_rows_kn_fwd: weight of 2 GiB or more (32-bit offsets)");
+  if (out == x || out == weight)
+    return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_kn_fwd: out must not alias an input");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int gelu = epilogue == OSLO_EPILOGUE_GELU_TANH;
+  const int mi = (int)m;
+  OSLO_DISPATCH_DTYPE(dtype, {
+    // compiled for the exact row count: a block does all the arithmetic of its
+    // strip, and rows padded up to a power of two showed in the time
+    switch (mi) {
+    case 1: return launch_kn<T, 1>(out, x, weight, bias, mi, n, k, gelu, s);
+    case 2: return launch_kn<T, 2>(out, x, weight, bias, mi, n, k, gelu, s);
+    case 3: return launch_kn<T, 3>(out, x, weight, bias, mi, n, k, gelu, s);
+    case 4: return launch_kn<T, 4>(out, x, weight, bias, mi, n, k, gelu, s);
+    case 5: return launch_kn<T, 5>(out, x, weight, bias, mi, n, k, gelu, s);
+    case 6: return launch_kn<T, 6>(out, x, weight, bias, mi, n, k, gelu, s);
+    case 7: return launch_kn<T, 7>(out, x, weight, bias, mi, n, k, gelu, s);
+    default: return launch_kn<T, 8>(out, x, weight, bias, mi, n, k, gelu, s);
+    }
+  });
+  return OSLO_OK;
+}
 
 extern "C" int oslo_linear_rows_max(void) { return oslo::kMaxRows; }
 

@@ -548,15 +548,16 @@ class FusedLinearRows(object):
     weight matrix for a handful of input rows, which the GEMM library runs at
     a quarter to a half of the memory bandwidth; ``apply`` runs it as such a
     stream. Inference only (``is_available`` is False when autograd would
-    record the call), at most ``kernels.LINEAR_ROWS_MAX`` rows, weights in the
-    [out_features, in_features] layout of ``nn.Linear``.
+    record the call), at most ``kernels.LINEAR_ROWS_MAX`` rows. Weights in the
+    [out_features, in_features] layout of ``nn.Linear``, or with ``conv1d``
+    in the [in_features, out_features] layout of GPT-2's ``Conv1D``.
     """
 
     @staticmethod
-    def is_available(x, weight, bias=None):
+    def is_available(x, weight, bias=None, conv1d=False):
         if not (isinstance(x, torch.Tensor) and x.is_cuda and weight.is_cuda) or x.dim() < 1 or weight.dim() != 2:
             return False
-        n, k = weight.shape
+        n, k = (weight.shape[1], weight.shape[0]) if conv1d else weight.shape
         if k == 0 or x.shape[-1] != k or x.dtype != weight.dtype:
             return False
         if x.dtype not in (torch.half, torch.bfloat16, torch.float32) or not weight.is_contiguous():
@@ -565,12 +566,15 @@ class FusedLinearRows(object):
         es = x.element_size()
         if not 0 < rows <= kernels.LINEAR_ROWS_MAX or (k * es) % 16 or n * k * es >= 2 ** 31:
             return False
+        if conv1d and (n * es) % 16:
+            return False
         return not _needs_grad(x, weight, bias)
 
     @staticmethod
-    def apply(x, weight, bias=None, act=None):
+    def apply(x, weight, bias=None, act=None, conv1d=False):
         gelu = act is not None and "gelu" in act
-        out = get_custom_kernels().linear_rows_forward(x, weight, bias, gelu)
+        forward = get_custom_kernels().linear_rows_kn_forward if conv1d else get_custom_kernels().linear_rows_forward
+        out = forward(x, weight, bias, gelu)
         if act is not None and not gelu:
             out = _act2fn(act)(out)
         return out
@@ -581,6 +585,14 @@ class FusedLinearRows(object):
         where it applies."""
         if FusedLinearRows.is_available(x, module.weight, module.bias):
             return FusedLinearRows.apply(x, module.weight, module.bias)
+        return module(x)
+
+    @staticmethod
+    def project_conv1d(module, x):
+        """``module(x)`` for a GPT-2 ``Conv1D``, through the few-row kernel
+        where it applies."""
+        if FusedLinearRows.is_available(x, module.weight, module.bias, conv1d=True):
+            return FusedLinearRows.apply(x, module.weight, module.bias, conv1d=True)
         return module(x)
 
     @staticmethod

@@ -437,6 +437,32 @@ def linear_rows_forward(x, weight, bias=None, gelu=False):
     return linear_rows_forward_multi(x, (weight,), (bias,), gelu)[0]
 
 
+def linear_rows_kn_forward(x, weight, bias=None, gelu=False):
+    """The same with the weight stored [K, N], the layout of GPT-2's Conv1D:
+    act(x @ weight + bias) (oslo/models/gpt2/modeling_gpt2.py:1553-1567 for a
+    decoding step)."""
+    _device_tensor(x, "x")
+    _device_tensor(weight, "weight", x)
+    code = _dtype_code(x, "x")
+    _require(weight.dim() == 2, "weight must be [in_features, out_features]")
+    _require(weight.dtype == x.dtype, "weight and x differ in dtype")
+    k, n = weight.shape
+    _require(x.dim() >= 1 and x.shape[-1] == k, "x must be [..., in_features]")
+    m = x.numel() // k if k else 0
+    if bias is not None:
+        _device_tensor(bias, "bias", x)
+        _require(bias.dim() == 1 and bias.shape[0] == n and bias.dtype == x.dtype,
+                 "bias must be [out_features] of the input's dtype")
+        bias = bias.contiguous()
+    x2, w = x.contiguous(), weight.contiguous()
+    out = torch.empty(x.shape[:-1] + (n,), dtype=x.dtype, device=x.device)
+    with _on_device(x):
+        _lib.check(_lib.load().oslo_linear_rows_kn_fwd(
+            _ptr(out), _ptr(x2), _ptr(w), _ptr(bias), m, n, k,
+            EPILOGUE_GELU_TANH if gelu else EPILOGUE_NONE, code, _stream(x)))
+    return out
+
+
 def linear_rows_forward_multi(x, weights, biases=None, gelu=False):
     """One to three layers of the same shape applied to the same x in one
     launch (the query, key and value projections): a list of outputs."""

@@ -13,7 +13,8 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedDecodeAttention, FusedMergeHeads,
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedDecodeAttention, FusedLinearRows,
+                                 FusedMergeHeads,
                                  FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedSplitHeads)
 from .modeling_utils import (ACT2FN, Conv1D, LayerPolicy, PreTrainedModel, StaticKV, additive_attention_mask,
@@ -152,7 +153,9 @@ class FusedGPT2Attention(GPT2Attention):
         if encoder_hidden_states is not None or not (
                 hidden_states.is_cuda and FusedSplitHeads.is_available(hidden_states.dtype, self.head_dim)):
             return super()._project_qkv(hidden_states, layer_past, encoder_hidden_states, use_cache)
-        query, key, value = FusedSplitHeads.apply(self.c_attn(hidden_states), self.num_heads)
+        # (a decoding step streams the weight in one pass, bias included)
+        query, key, value = FusedSplitHeads.apply(FusedLinearRows.project_conv1d(self.c_attn, hidden_states),
+                                                  self.num_heads)
         key, value, present = append_kv(layer_past, key, value, use_cache, defer=True)
         return query, key, value, present
 
@@ -199,8 +202,12 @@ class FusedGPT2Attention(GPT2Attention):
             out = FusedMergeHeads.apply(out)
         else:
             out = self._merge_heads(out, self.num_heads, self.head_dim)
-        out = out @ self.c_proj.weight  # projection without its bias ...
-        out = FusedBiasDropout.apply(out, self.c_proj.bias, self.training, self.resid_dropout.p)  # ... fused here
+        if FusedLinearRows.is_available(out, self.c_proj.weight, self.c_proj.bias, conv1d=True) and not (
+                self.training and self.resid_dropout.p > 0.0):
+            out = FusedLinearRows.apply(out, self.c_proj.weight, self.c_proj.bias, conv1d=True)  # a decoding step
+        else:
+            out = out @ self.c_proj.weight  # projection without its bias ...
+            out = FusedBiasDropout.apply(out, self.c_proj.bias, self.training, self.resid_dropout.p)  # ... fused here
         return (out, present, w) if output_attentions else (out, present)
 
 
@@ -220,9 +227,18 @@ class FusedGPT2MLP(GPT2MLP):
     """oslo/models/gpt2/modeling_gpt2.py:1545-1569."""
 
     def forward(self, x):
-        x = x @ self.c_fc.weight
-        x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
-        x = x @ self.c_proj.weight
+        if FusedLinearRows.is_available(x, self.c_fc.weight, self.c_fc.bias, conv1d=True):
+            # a decoding step: each projection is one pass over its weight with
+            # the bias (and the activation) applied to the fp32 sums
+            x = FusedLinearRows.apply(x, self.c_fc.weight, self.c_fc.bias, self.config.activation_function,
+                                      conv1d=True)
+            if not (self.training and self.dropout.p > 0.0):
+                return FusedLinearRows.apply(x, self.c_proj.weight, self.c_proj.bias, conv1d=True)
+            x = FusedLinearRows.apply(x, self.c_proj.weight, conv1d=True)
+        else:
+            x = x @ self.c_fc.weight
+            x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
+            x = x @ self.c_proj.weight
         return FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
 
 

@@ -47,6 +47,26 @@ def test_linear_rows_matches_oracle(m, n, k, dtype):
         check(out, x, w, bias, gelu, dtype, f"{m}x{n}x{k} bias={bias is not None} gelu={gelu}")
 
 
+# weight stored [k, n] (Conv1D): n and k multiples of the vector; ragged strips (n not a multiple of
+# 8 vectors), k below / past what 16 waves cover in one step
+KN_SHAPES = [(1, 8, 8), (2, 24, 64), (3, 2304, 768), (5, 768, 3072), (8, 136, 1032), (4, 3072, 768), (7, 40, 4104)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("m,n,k", KN_SHAPES)
+def test_linear_rows_conv1d_layout_matches_oracle(m, n, k, dtype):
+    x = randn((m, k), dtype, seed=m * 11 + k)
+    w = randn((k, n), dtype, seed=n * 13 + k, std=0.05)       # [in, out]
+    b = randn((n,), dtype, seed=n, std=0.5)
+    for bias, gelu in ((None, False), (b, False), (b, True)):
+        out = kernels.linear_rows_kn_forward(x.to(DEV), w.to(DEV), None if bias is None else bias.to(DEV), gelu)
+        assert out.shape == (m, n) and out.dtype == dtype
+        check(out, x, w.t().contiguous(), bias, gelu, dtype, f"kn {m}x{n}x{k} bias={bias is not None} gelu={gelu}")
+    if n != k:
+        with pytest.raises(RuntimeError):
+            kernels.linear_rows_kn_forward(x.to(DEV), w.t().contiguous().to(DEV))   # the other layout
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
 @pytest.mark.parametrize("m,n,k", [(1, 64, 512), (3, 130, 1032), (8, 4096, 1024)])
 def test_linear_rows_three_layers_in_one_launch(m, n, k, dtype):
