@@ -146,8 +146,7 @@ __global__ __launch_bounds__(kBlockThreads) void attention_decode_partial_kernel
       float d = 0.f;
 #pragma unroll
       for (int j = 0; j < VEC; ++j) d = __builtin_fmaf(kf[j], qf[j], d);
-#pragma unroll
-      for (int s = 1; s < LPK; s <<= 1) d += lane_xor(d, s);
+      d = sum_over_lanes<LPK>(d); // the lanes of the key
       score[u] = vis[u] ? d * scale_log2e : -INFINITY;
       mt = fmaxf(mt, score[u]);
     }

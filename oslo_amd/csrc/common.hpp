@@ -206,6 +206,25 @@ __device__ __forceinline__ float sum_over_row(float v) {
   return v;
 }
 
+// Sum over an aligned group of N lanes (N = 8, 16, 32 or 64), left in every
+// lane of the group: DPP inside a row of 16, one ds_swizzle for lane ^ 16, two
+// v_readlane for the halves of the wave (the steps of wave_allreduce).
+template <int N>
+__device__ __forceinline__ float sum_over_lanes(float v) {
+  static_assert(N == 8 || N == 16 || N == 32 || N == 64, "aligned lane groups");
+  if constexpr (N == 64) {
+    return wave_allreduce(v, OpAdd());
+  } else {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    if constexpr (N >= 16) v += dpp_move<0x140>(v);
+    if constexpr (N >= 32)
+      v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+    return v;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Host side: status + per-thread error text.
 // ---------------------------------------------------------------------------
