@@ -366,7 +366,7 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         wsd = torch.empty(lib.oslo_attention_decode_workspace_bytes(rows * H, cap, D, BF16) // 4,
                           dtype=torch.float32, device=dev)
         t = time_launches(rotating(caches, lambda kv: check(lib.oslo_attention_decode_fwd(
-            P(od), P(qd), P(kv[0]), P(kv[1]), None, None, P(wsd), None, last, 0, 1 / 16.0, rows * H, cap, D, BF16, st))), n, 3)
+            P(od), P(qd), P(kv[0]), P(kv[1]), None, None, 0, 0, P(wsd), None, last, 0, 1 / 16.0, rows * H, cap, D, BF16, st))), n, 3)
         res.append(roof(f"attention_decode bf16 {rows} x 16 heads, 1024 of 1152 keys, head 256 (two launches)",
                         2 * 2 * rows * H * (last + 1) * D, t, rows * H * D, n_sets))
         del caches

@@ -362,10 +362,12 @@ int oslo_linear_rows_kn_fwd(void *out, const void *x, const void *weight,
  * layers), else 0. q, out: [rows_heads, head_dim]; k, v: [rows_heads, capacity,
  * head_dim] (a [batch, heads, capacity, head_dim] cache); 0 <= last < capacity.
  * Keys outside the visible range are not read. k_new, v_new: both NULL, or
- * [rows_heads, head_dim]: the key and value of position `last`, which are then
- * used from there and written into slot `last` of k and v by the kernel (the
- * append to the cache and the attention in one launch); the other slots of k
- * and v are only read. workspace: fp32, at least
+ * the key and value of position `last` as [rows_heads / heads, heads, head_dim]
+ * with new_seq_stride elements between sequences (0: dense; 3*heads*head_dim
+ * for the slices of GPT-2's packed c_attn output), which are then used from
+ * there and written into slot `last` of k and v by the kernel (the append to
+ * the cache and the attention in one launch); the other slots of k and v are
+ * only read. heads is used only with k_new. workspace: fp32, at least
  * oslo_attention_decode_workspace_bytes(...) bytes, contents irrelevant before
  * and after. head_dim * sizeof(dtype) must be 128, 256, 512 or 1024 bytes.
  * Arithmetic in fp32 throughout (scores, softmax, weighted sum), one rounding
@@ -381,6 +383,7 @@ size_t oslo_attention_decode_workspace_bytes(int64_t rows_heads,
                                              int dtype);
 int oslo_attention_decode_fwd(void *out, const void *q, void *k, void *v,
                               const void *k_new, const void *v_new,
+                              int64_t heads, int64_t new_seq_stride,
                               float *workspace,
                               const int64_t *pos_dev, int64_t pos,
                               int64_t window, float scale, int64_t rows_heads,

@@ -52,9 +52,10 @@ struct DecodeTile {
 template <typename T, int LPK>
 __global__ __launch_bounds__(kBlockThreads) void attention_decode_partial_kernel(
     float *__restrict__ ws, const T *__restrict__ q, T *k, T *v,
-    const T *__restrict__ k_new, const T *__restrict__ v_new,
-    const int64_t *__restrict__ pos_dev, int64_t pos_host, int window,
-    float scale_log2e, int capacity, int head_dim, int splits, int tiles) {
+    const T *__restrict__ k_new, const T *__restrict__ v_new, int heads,
+    int64_t new_seq_stride, const int64_t *__restrict__ pos_dev,
+    int64_t pos_host, int window, float scale_log2e, int capacity,
+    int head_dim, int splits, int tiles) {
   constexpr int VEC = Io<T>::kVec;
   using Tile = DecodeTile<LPK>;
   constexpr int U = Tile::kLoads;
@@ -97,8 +98,11 @@ __global__ __launch_bounds__(kBlockThreads) void attention_decode_partial_kernel
   const bool fresh = k_new != nullptr;
   RawVec<T, VEC> knew, vnew;
   if (fresh) {
-    knew = buffer_load_raw<T, VEC, false>(make_rsrc(k_new + bh * (int64_t)head_dim, key_bytes), (uint32_t)dl * 16u);
-    vnew = buffer_load_raw<T, VEC, false>(make_rsrc(v_new + bh * (int64_t)head_dim, key_bytes), (uint32_t)dl * 16u);
+    // [sequence, head, head_dim] with a stride between sequences (dense, or
+    // slices of a packed q|k|v projection)
+    const int64_t at = (bh / heads) * new_seq_stride + (bh % heads) * (int64_t)head_dim;
+    knew = buffer_load_raw<T, VEC, false>(make_rsrc(k_new + at, key_bytes), (uint32_t)dl * 16u);
+    vnew = buffer_load_raw<T, VEC, false>(make_rsrc(v_new + at, key_bytes), (uint32_t)dl * 16u);
   }
 
   // running maximum, sum and accumulator of the wave (over its tiles)
@@ -260,7 +264,8 @@ __global__ __launch_bounds__(kMergeThreads) void attention_decode_merge_kernel(
 
 template <typename T, int LPK>
 int launch(void *out, const void *q, void *k, void *v, const void *k_new,
-           const void *v_new, float *ws, const int64_t *pos_dev, int64_t pos, int window, float scale,
+           const void *v_new, int heads, int64_t new_seq_stride, float *ws,
+           const int64_t *pos_dev, int64_t pos, int window, float scale,
            int64_t rows_heads, int capacity, int head_dim, hipStream_t stream) {
   // As many splits as fill the device (about four blocks per CU), not more:
   // every split is a partial result the merge has to read. A block then covers
@@ -273,8 +278,9 @@ int launch(void *out, const void *q, void *k, void *v, const void *k_new,
   attention_decode_partial_kernel<T, LPK>
       <<<dim3((unsigned)(rows_heads * splits)), dim3(kBlockThreads), 0, stream>>>(
           ws, static_cast<const T *>(q), static_cast<T *>(k), static_cast<T *>(v),
-          static_cast<const T *>(k_new), static_cast<const T *>(v_new), pos_dev,
-          pos, window, scale * kLog2e, capacity, head_dim, splits, tiles);
+          static_cast<const T *>(k_new), static_cast<const T *>(v_new), heads,
+          new_seq_stride, pos_dev, pos, window, scale * kLog2e, capacity,
+          head_dim, splits, tiles);
   attention_decode_merge_kernel<T>
       <<<dim3((unsigned)rows_heads), dim3(kMergeThreads), 0, stream>>>(
           static_cast<T *>(out), ws, head_dim, splits);
@@ -318,7 +324,9 @@ extern "C" size_t oslo_attention_decode_workspace_bytes(int64_t rows_heads,
 
 extern "C" int oslo_attention_decode_fwd(void *out, const void *q, void *k,
                                          void *v, const void *k_new,
-                                         const void *v_new, float *workspace,
+                                         const void *v_new, int64_t heads,
+                                         int64_t new_seq_stride,
+                                         float *workspace,
                                          const int64_t *pos_dev, int64_t pos,
                                          int64_t window, float scale,
                                          int64_t rows_heads, int64_t capacity,
@@ -353,16 +361,27 @@ extern "C" int oslo_attention_decode_fwd(void *out, const void *q, void *k,
     return fail(OSLO_E_BAD_ARG, "oslo_attention_decode_fwd: null pointer");
   if ((k_new == nullptr) != (v_new == nullptr))
     return fail(OSLO_E_BAD_ARG, "oslo_attention_decode_fwd: k_new and v_new go together");
+  if (k_new != nullptr) {
+    if (heads <= 0 || rows_heads % heads != 0)
+      return fail(OSLO_E_BAD_ARG, "oslo_attention_decode_fwd: %lld heads do not divide %lld rows",
+                  (long long)heads, (long long)rows_heads);
+    if (new_seq_stride == 0) new_seq_stride = heads * head_dim;
+    if (new_seq_stride < heads * head_dim || (new_seq_stride * es) % 16 != 0)
+      return fail(OSLO_E_BAD_ARG, "oslo_attention_decode_fwd: new_seq_stride %lld (whole 16-byte vectors, at least heads*head_dim)",
+                  (long long)new_seq_stride);
+  } else {
+    heads = 1;
+  }
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(k_new) || !aligned16(v_new))
     return fail(OSLO_E_BAD_ARG, "oslo_attention_decode_fwd: q, k, v, k_new and v_new must be 16-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int win = window > capacity ? (int)capacity : (int)window;
   OSLO_DISPATCH_DTYPE(dtype, {
     switch (lpk) {
-    case 8: return launch<T, 8>(out, q, k, v, k_new, v_new, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
-    case 16: return launch<T, 16>(out, q, k, v, k_new, v_new, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
-    case 32: return launch<T, 32>(out, q, k, v, k_new, v_new, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
-    default: return launch<T, 64>(out, q, k, v, k_new, v_new, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
+    case 8: return launch<T, 8>(out, q, k, v, k_new, v_new, (int)heads, new_seq_stride, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
+    case 16: return launch<T, 16>(out, q, k, v, k_new, v_new, (int)heads, new_seq_stride, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
+    case 32: return launch<T, 32>(out, q, k, v, k_new, v_new, (int)heads, new_seq_stride, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
+    default: return launch<T, 64>(out, q, k, v, k_new, v_new, (int)heads, new_seq_stride, workspace, pos_dev, pos, win, scale, rows_heads, (int)capacity, (int)head_dim, s);
     }
   });
   return OSLO_OK;

@@ -503,6 +503,12 @@ def linear_rows_forward_multi(x, weights, biases=None, gelu=False):
     return outs
 
 
+def _heads_side_by_side(t):
+    """[B, H, 1, D] whose heads of one sequence are consecutive runs of D elements."""
+    b, h, _, d = t.shape
+    return t.stride(3) == 1 and (h == 1 or t.stride(1) == d) and (b == 1 or t.stride(0) >= h * d)
+
+
 def attention_decode_forward(query, key, value, pos, scale, window=0, new_key=None, new_value=None):
     """query [B, H, 1, D]; key, value [B, H, L, D] caches; attends keys
     first..last, last = ``pos`` (an int, or an int64 device tensor of one
@@ -511,7 +517,9 @@ def attention_decode_forward(query, key, value, pos, scale, window=0, new_key=No
     (oslo/models/gptj/modeling_gptj.py:936-951 for a query length of 1).
     ``new_key``, ``new_value`` [B, H, 1, D]: the key and value of position
     ``pos``, not yet in the caches; the kernel uses them and writes them into
-    slot ``pos`` of ``key`` and ``value``, which must then be contiguous."""
+    slot ``pos`` of ``key`` and ``value``, which must then be contiguous. They
+    may be strided between sequences (views of a packed projection) as long as
+    a sequence's heads lie side by side."""
     _device_tensor(query, "query")
     _device_tensor(key, "key", query)
     _device_tensor(value, "value", query)
@@ -530,7 +538,10 @@ def attention_decode_forward(query, key, value, pos, scale, window=0, new_key=No
         for t, what in ((new_key, "new_key"), (new_value, "new_value")):
             _device_tensor(t, what, query)
             _require(t.shape == query.shape and t.dtype == query.dtype, f"{what} must be like the query")
-        new_key, new_value = new_key.contiguous(), new_value.contiguous()
+        if not (_heads_side_by_side(new_key) and _heads_side_by_side(new_value)
+                and (b == 1 or new_key.stride(0) == new_value.stride(0))):
+            new_key, new_value = new_key.contiguous(), new_value.contiguous()
+        new_stride = new_key.stride(0) if b > 1 else 0
     pos_dev, pos_host = None, 0
     if isinstance(pos, torch.Tensor):
         _device_tensor(pos, "pos", query)
@@ -545,8 +556,8 @@ def attention_decode_forward(query, key, value, pos, scale, window=0, new_key=No
     out = torch.empty_like(q)
     with _on_device(q):
         _lib.check(lib.oslo_attention_decode_fwd(
-            _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(new_key), _ptr(new_value), _ptr(ws), _ptr(pos_dev),
-            pos_host, int(window),
+            _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(new_key), _ptr(new_value), h,
+            new_stride if new_key is not None else 0, _ptr(ws), _ptr(pos_dev), pos_host, int(window),
             float(scale), b * h, cap, d, code, _stream(q)))
     return out
 

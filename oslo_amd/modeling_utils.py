@@ -171,8 +171,17 @@ class StaticKV(object):
         return self.k, self.v
 
     def pending_is_dense(self):
-        """A key/value pair is waiting and the kernel can read it as it lies."""
-        return self.pending is not None and all(t.is_contiguous() for t in self.pending)
+        """A key/value pair is waiting and the kernel can read it as it lies:
+        the heads of a sequence side by side (sequences may be strided, as the
+        slices of a packed projection are)."""
+        if self.pending is None:
+            return False
+        key, value = self.pending
+        b, h, _, d = key.shape
+
+        def ok(t):
+            return t.stride(3) == 1 and (h == 1 or t.stride(1) == d) and (b == 1 or t.stride(0) >= h * d)
+        return ok(key) and ok(value) and (b == 1 or key.stride(0) == value.stride(0))
 
     def take_pending(self):
         pending, self.pending = self.pending, None

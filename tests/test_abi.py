@@ -123,12 +123,14 @@ def test_argument_screening_without_a_device(lib):
     assert lib.oslo_linear_rows_fwd_multi(null, one, table, null, 2, 1, 4, 8, 0, 1, null) == -1
     assert lib.oslo_linear_rows_fwd_multi(table, ctypes.c_void_p(64), table, null, 3, 1, 4, 8, 0, 1, null) == -1  # out[j] is weight[j]
     # attention of a decoding step: head size, position, null pointers, workspace size
-    assert lib.oslo_attention_decode_fwd(one, two, three, three, null, null, one, null, 0, 0, 1.0, 4, 64, 48, 1, null) == -2
-    assert lib.oslo_attention_decode_fwd(one, two, three, three, null, null, one, null, 64, 0, 1.0, 4, 64, 64, 1, null) == -1
-    assert lib.oslo_attention_decode_fwd(one, two, three, three, null, null, null, null, 3, 0, 1.0, 4, 64, 64, 1, null) == -1
-    assert lib.oslo_attention_decode_fwd(one, two, three, three, null, null, one, null, 3, -1, 1.0, 4, 64, 64, 1, null) == -1
-    assert lib.oslo_attention_decode_fwd(null, null, null, null, null, null, null, null, 0, 0, 1.0, 0, 64, 64, 1, null) == 0
-    assert lib.oslo_attention_decode_fwd(one, two, three, three, one, null, one, null, 3, 0, 1.0, 4, 64, 64, 1, null) == -1  # k_new alone
+    assert lib.oslo_attention_decode_fwd(one, two, three, three, null, null, 0, 0, one, null, 0, 0, 1.0, 4, 64, 48, 1, null) == -2
+    assert lib.oslo_attention_decode_fwd(one, two, three, three, null, null, 0, 0, one, null, 64, 0, 1.0, 4, 64, 64, 1, null) == -1
+    assert lib.oslo_attention_decode_fwd(one, two, three, three, null, null, 0, 0, null, null, 3, 0, 1.0, 4, 64, 64, 1, null) == -1
+    assert lib.oslo_attention_decode_fwd(one, two, three, three, null, null, 0, 0, one, null, 3, -1, 1.0, 4, 64, 64, 1, null) == -1
+    assert lib.oslo_attention_decode_fwd(null, null, null, null, null, null, 0, 0, null, null, 0, 0, 1.0, 0, 64, 64, 1, null) == 0
+    assert lib.oslo_attention_decode_fwd(one, two, three, three, one, null, 2, 0, one, null, 3, 0, 1.0, 4, 64, 64, 1, null) == -1  # k_new alone
+    assert lib.oslo_attention_decode_fwd(one, two, three, three, one, one, 3, 0, one, null, 3, 0, 1.0, 4, 64, 64, 1, null) == -1  # 3 heads, 4 rows
+    assert lib.oslo_attention_decode_fwd(one, two, three, three, one, one, 2, 100, one, null, 3, 0, 1.0, 4, 64, 64, 1, null) == -1  # stride below heads*head_dim
     assert lib.oslo_attention_decode_workspace_bytes(16, 1152, 256, 2) == 16 * 18 * 258 * 4
     assert lib.oslo_attention_decode_workspace_bytes(16, 1152, 48, 2) == 0
     # n-gram blocking

@@ -112,6 +112,18 @@ def test_attention_decode_appends_the_new_key(cap, last, window, dtype):
                                            k[:, :, last:last + 1].contiguous(), v[:, :, last:last + 1].contiguous())
     assert torch.equal(got, want)
     assert torch.equal(k2, k) and torch.equal(v2, v)
+    # the same from the slices of a packed q|k|v row per sequence (GPT-2's c_attn output)
+    packed = torch.zeros((b, 1, 3 * h * d), dtype=dtype, device=DEV)
+    packed[:, 0, h * d:2 * h * d] = k[:, :, last].reshape(b, h * d)
+    packed[:, 0, 2 * h * d:] = v[:, :, last].reshape(b, h * d)
+    nk = packed[:, :, h * d:2 * h * d].reshape(b, h, 1, d)
+    nv = packed[:, :, 2 * h * d:].reshape(b, h, 1, d)
+    assert not nk.is_contiguous()
+    k3, v3 = k.clone(), v.clone()
+    k3[:, :, last] = 7.0
+    v3[:, :, last] = -7.0
+    assert torch.equal(kernels.attention_decode_forward(q, k3, v3, pos, 0.25, window, nk, nv), want)
+    assert torch.equal(k3, k) and torch.equal(v3, v)
 
 
 def test_attention_decode_errors():
