@@ -136,14 +136,16 @@ __global__ __launch_bounds__(kBlockThreads) void linear_rows_kernel(
 }
 
 // The same with the input rows in LDS. The block stages a segment of
-// kSegBytes / MT bytes of each of the MT rows (so 32 KiB in all), its four
+// kSegBytes / MT bytes of each of the MT rows (so 32 KiB in all), its eight
 // waves walk their weight rows over that segment, and so on along k. Rows past
 // m and vectors past k are staged as zeros. Every wave stays to the end: there
 // are barriers in the loop.
 constexpr int kSegBytes = 32768;
+constexpr int kLdsThreads = 512; // 8 waves share one staged segment
+constexpr int kLdsWaves = kLdsThreads / kWave;
 
 template <typename T, int VEC, int MT, int R, int U>
-__global__ __launch_bounds__(kBlockThreads) void linear_rows_lds_kernel(
+__global__ __launch_bounds__(kLdsThreads) void linear_rows_lds_kernel(
     LinearJobs<T> jobs, const T *__restrict__ x, int m, int64_t n, int64_t k,
     int gelu) {
   T *__restrict__ out = jobs.out[blockIdx.y];
@@ -157,7 +159,7 @@ __global__ __launch_bounds__(kBlockThreads) void linear_rows_lds_kernel(
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
-  const int64_t row0 = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * R;
+  const int64_t row0 = ((int64_t)blockIdx.x * kLdsWaves + wave) * R;
   const BufRsrc wrs = make_rsrc(w, (uint32_t)(n * k * (int64_t)sizeof(T)));
   const BufRsrc xrs = make_rsrc(x, (uint32_t)((int64_t)m * k * (int64_t)sizeof(T)));
   const uint32_t row_bytes = (uint32_t)(k * (int64_t)sizeof(T));
@@ -171,18 +173,18 @@ __global__ __launch_bounds__(kBlockThreads) void linear_rows_lds_kernel(
 
   for (int v0 = 0; v0 < kvec; v0 += kSegVecs) {
     if (v0 > 0) __syncthreads(); // the previous segment has been read
-    constexpr int kPasses = MT * kSegVecs / kBlockThreads;
+    constexpr int kPasses = MT * kSegVecs / kLdsThreads;
     Vec stage[kPasses];
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
-      const int idx = p * kBlockThreads + threadIdx.x;
+      const int idx = p * kLdsThreads + threadIdx.x;
       const int i = idx / kSegVecs, v = v0 + idx % kSegVecs;
       const bool ok = i < m && v < kvec;
       stage[p] = buffer_load_raw<T, VEC, false>(
           xrs, ok ? (uint32_t)i * row_bytes + (uint32_t)v * 16u : kOutside);
     }
 #pragma unroll
-    for (int p = 0; p < kPasses; ++p) xs[p * kBlockThreads + threadIdx.x] = stage[p];
+    for (int p = 0; p < kPasses; ++p) xs[p * kLdsThreads + threadIdx.x] = stage[p];
     __syncthreads();
 
 #pragma unroll 1
@@ -246,10 +248,10 @@ template <typename T, int MT, int R, int U>
 int launch_lds(const LinearJobs<T> &jobs, int count, const void *x, int m,
                int64_t n, int64_t k, int gelu, hipStream_t stream) {
   constexpr int VEC = Io<T>::kVec;
-  const int64_t rows_per_block = (int64_t)kWavesPerBlock * R;
+  const int64_t rows_per_block = (int64_t)kLdsWaves * R;
   const int64_t blocks = (n + rows_per_block - 1) / rows_per_block;
   linear_rows_lds_kernel<T, VEC, MT, R, U>
-      <<<dim3((unsigned)blocks, count), dim3(kBlockThreads), 0, stream>>>(
+      <<<dim3((unsigned)blocks, count), dim3(kLdsThreads), 0, stream>>>(
           jobs, static_cast<const T *>(x), m, n, k, gelu);
   return check_launch("oslo_linear_rows_fwd");
 }
