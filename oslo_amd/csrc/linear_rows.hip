@@ -144,7 +144,7 @@ constexpr int kSegBytes = 32768;
 constexpr int kLdsThreads = 512; // 8 waves share one staged segment
 constexpr int kLdsWaves = kLdsThreads / kWave;
 
-template <typename T, int VEC, int MT, int R, int U>
+template <typename T, int VEC, int MT, int R, int U, bool EARLY>
 __global__ __launch_bounds__(kLdsThreads) void linear_rows_lds_kernel(
     LinearJobs<T> jobs, const T *__restrict__ x, int m, int64_t n, int64_t k,
     int gelu) {
@@ -171,8 +171,24 @@ __global__ __launch_bounds__(kLdsThreads) void linear_rows_lds_kernel(
 #pragma unroll
     for (int i = 0; i < MT; ++i) acc[r][i] = 0.f;
 
+  // the weight vectors of U chunks starting at chunk c0 of the segment at v0
+  auto load_weights = [&](Vec (&wv)[R][U], int v0, int c0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int v = v0 + (c0 + u) * kWave + lane;
+        const bool ok = v < kvec && row0 + r < n;
+        wv[r][u] = buffer_load_raw<T, VEC, true>(
+            wrs, ok ? (uint32_t)(row0 + r) * row_bytes + (uint32_t)v * 16u : kOutside);
+      }
+  };
+
   for (int v0 = 0; v0 < kvec; v0 += kSegVecs) {
-    if (v0 > 0) __syncthreads(); // the previous segment has been read
+    // The loads of the segment's inputs go out first and the first weight loads
+    // right behind them, before any barrier: loads return in order, so the
+    // wait for the inputs leaves the weight loads, whose latency is the long
+    // one, in flight across the staging.
     constexpr int kPasses = MT * kSegVecs / kLdsThreads;
     Vec stage[kPasses];
 #pragma unroll
@@ -183,22 +199,16 @@ __global__ __launch_bounds__(kLdsThreads) void linear_rows_lds_kernel(
       stage[p] = buffer_load_raw<T, VEC, false>(
           xrs, ok ? (uint32_t)i * row_bytes + (uint32_t)v * 16u : kOutside);
     }
+    Vec wv[R][U];
+    if constexpr (EARLY) load_weights(wv, v0, 0);
+    if (v0 > 0) __syncthreads(); // the previous segment has been read
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) xs[p * kLdsThreads + threadIdx.x] = stage[p];
     __syncthreads();
 
 #pragma unroll 1
     for (int c0 = 0; c0 < kSegChunks; c0 += U) {
-      Vec wv[R][U];
-#pragma unroll
-      for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int v = v0 + (c0 + u) * kWave + lane;
-          const bool ok = v < kvec && row0 + r < n;
-          wv[r][u] = buffer_load_raw<T, VEC, true>(
-              wrs, ok ? (uint32_t)(row0 + r) * row_bytes + (uint32_t)v * 16u : kOutside);
-        }
+      if (!EARLY || c0 > 0) load_weights(wv, v0, c0);
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -244,13 +254,13 @@ LinearJobs<T> make_jobs(void *const *out, const void *const *w,
   return jobs;
 }
 
-template <typename T, int MT, int R, int U>
+template <typename T, int MT, int R, int U, bool EARLY = true>
 int launch_lds(const LinearJobs<T> &jobs, int count, const void *x, int m,
                int64_t n, int64_t k, int gelu, hipStream_t stream) {
   constexpr int VEC = Io<T>::kVec;
   const int64_t rows_per_block = (int64_t)kLdsWaves * R;
   const int64_t blocks = (n + rows_per_block - 1) / rows_per_block;
-  linear_rows_lds_kernel<T, VEC, MT, R, U>
+  linear_rows_lds_kernel<T, VEC, MT, R, U, EARLY>
       <<<dim3((unsigned)blocks, count), dim3(kLdsThreads), 0, stream>>>(
           jobs, static_cast<const T *>(x), m, n, k, gelu);
   return check_launch("oslo_linear_rows_fwd");
@@ -317,8 +327,10 @@ int linear_rows(void *const *out, const void *x, const void *const *weight,
     if (mi <= 4)
       return few ? launch_lds<T, 4, 1, 8>(jobs, count, x, mi, n, k, gelu, s)
                  : launch_lds<T, 4, 2, 4>(jobs, count, x, mi, n, k, gelu, s);
+    // (with 8 input rows and two weight rows per wave the early weight loads
+    // measured 6-11 % slower than loading inside the loop: that one keeps them there)
     return few ? launch_lds<T, 8, 1, 4>(jobs, count, x, mi, n, k, gelu, s)
-               : launch_lds<T, 8, 2, 4>(jobs, count, x, mi, n, k, gelu, s);
+               : launch_lds<T, 8, 2, 4, false>(jobs, count, x, mi, n, k, gelu, s);
   });
   return OSLO_OK;
 }
