@@ -17,7 +17,8 @@
 // rounding to the storage type: this is the reference's
 //   x = torch.matmul(x, weight.t()); x = FusedBiasActivation.apply(x, bias, act)
 // (oslo/models/gptj/modeling_gptj.py:1049-1053) without the rounded
-// intermediate.
+// intermediate. A second kernel at the end of this file takes the weight in
+// GPT-2's [k, n] layout.
 
 #include "common.hpp"
 #include "gelu.hpp"
@@ -139,7 +140,8 @@ __global__ __launch_bounds__(kBlockThreads) void linear_rows_kernel(
 // kSegBytes / MT bytes of each of the MT rows (so 32 KiB in all), its eight
 // waves walk their weight rows over that segment, and so on along k. Rows past
 // m and vectors past k are staged as zeros. Every wave stays to the end: there
-// are barriers in the loop.
+// are barriers in the loop. EARLY: the first weight loads of a segment go out
+// before its staging and barriers (the launcher says per tile where that paid).
 constexpr int kSegBytes = 32768;
 constexpr int kLdsThreads = 512; // 8 waves share one staged segment
 constexpr int kLdsWaves = kLdsThreads / kWave;
