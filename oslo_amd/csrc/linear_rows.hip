@@ -146,22 +146,22 @@ constexpr int kSegBytes = 32768;
 constexpr int kLdsThreads = 512; // 8 waves share one staged segment
 constexpr int kLdsWaves = kLdsThreads / kWave;
 
-template <typename T, int VEC, int MT, int R, int U, bool EARLY>
-__global__ __launch_bounds__(kLdsThreads) void linear_rows_lds_kernel(
+template <typename T, int VEC, int MT, int R, int U, bool EARLY, int THREADS, int SEGBYTES>
+__global__ __launch_bounds__(THREADS) void linear_rows_lds_kernel(
     LinearJobs<T> jobs, const T *__restrict__ x, int m, int64_t n, int64_t k,
     int gelu) {
   T *__restrict__ out = jobs.out[blockIdx.y];
   const T *__restrict__ w = jobs.w[blockIdx.y];
   const T *__restrict__ bias = jobs.bias[blockIdx.y];
   using Vec = RawVec<T, VEC>;
-  constexpr int kSegVecs = kSegBytes / 16 / MT;  // vectors of one row per segment
+  constexpr int kSegVecs = SEGBYTES / 16 / MT;  // vectors of one row per segment
   constexpr int kSegChunks = kSegVecs / kWave;   // chunks of 64 vectors
   static_assert(kSegChunks % U == 0, "a segment is whole unrolled spans");
   __shared__ Vec xs[MT * kSegVecs];
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
-  const int64_t row0 = ((int64_t)blockIdx.x * kLdsWaves + wave) * R;
+  const int64_t row0 = ((int64_t)blockIdx.x * (THREADS / kWave) + wave) * R;
   const BufRsrc wrs = make_rsrc(w, (uint32_t)(n * k * (int64_t)sizeof(T)));
   const BufRsrc xrs = make_rsrc(x, (uint32_t)((int64_t)m * k * (int64_t)sizeof(T)));
   const uint32_t row_bytes = (uint32_t)(k * (int64_t)sizeof(T));
@@ -191,11 +191,11 @@ __global__ __launch_bounds__(kLdsThreads) void linear_rows_lds_kernel(
     // right behind them, before any barrier: loads return in order, so the
     // wait for the inputs leaves the weight loads, whose latency is the long
     // one, in flight across the staging.
-    constexpr int kPasses = MT * kSegVecs / kLdsThreads;
+    constexpr int kPasses = MT * kSegVecs / THREADS;
     Vec stage[kPasses];
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
-      const int idx = p * kLdsThreads + threadIdx.x;
+      const int idx = p * THREADS + threadIdx.x;
       const int i = idx / kSegVecs, v = v0 + idx % kSegVecs;
       const bool ok = i < m && v < kvec;
       stage[p] = buffer_load_raw<T, VEC, false>(
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(kLdsThreads) void linear_rows_lds_kernel(
     if constexpr (EARLY) load_weights(wv, v0, 0);
     if (v0 > 0) __syncthreads(); // the previous segment has been read
 #pragma unroll
-    for (int p = 0; p < kPasses; ++p) xs[p * kLdsThreads + threadIdx.x] = stage[p];
+    for (int p = 0; p < kPasses; ++p) xs[p * THREADS + threadIdx.x] = stage[p];
     __syncthreads();
 
 #pragma unroll 1
@@ -256,14 +256,14 @@ LinearJobs<T> make_jobs(void *const *out, const void *const *w,
   return jobs;
 }
 
-template <typename T, int MT, int R, int U, bool EARLY = true>
+template <typename T, int MT, int R, int U, bool EARLY = true, int THREADS = kLdsThreads, int SEGBYTES = kSegBytes>
 int launch_lds(const LinearJobs<T> &jobs, int count, const void *x, int m,
                int64_t n, int64_t k, int gelu, hipStream_t stream) {
   constexpr int VEC = Io<T>::kVec;
-  const int64_t rows_per_block = (int64_t)kLdsWaves * R;
+  const int64_t rows_per_block = (int64_t)(THREADS / kWave) * R;
   const int64_t blocks = (n + rows_per_block - 1) / rows_per_block;
-  linear_rows_lds_kernel<T, VEC, MT, R, U, EARLY>
-      <<<dim3((unsigned)blocks, count), dim3(kLdsThreads), 0, stream>>>(
+  linear_rows_lds_kernel<T, VEC, MT, R, U, EARLY, THREADS, SEGBYTES>
+      <<<dim3((unsigned)blocks, count), dim3(THREADS), 0, stream>>>(
           jobs, static_cast<const T *>(x), m, n, k, gelu);
   return check_launch("oslo_linear_rows_fwd");
 }
