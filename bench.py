@@ -350,7 +350,7 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
             xin = randn((m, k_in), 5, 1.0, torch.bfloat16)
             o = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
             t = time_launches(rotating(weights, lambda wt: check(lib.oslo_linear_rows_fwd(
-                P(o), P(xin), P(wt), P(bias), m, n_out, k_in, gelu, BF16, st))), n, 3)
+                P(o), P(xin), P(wt), P(bias), None, m, n_out, k_in, gelu, BF16, st))), n, 3)
             res.append(roof(f"linear_rows {what} bf16 {m} x [{n_out},{k_in}]",
                             2 * (n_out * k_in + m * k_in + m * n_out + n_out), t, m * n_out, n_sets))
         del weights

@@ -302,10 +302,13 @@ enum oslo_epilogue {
 int oslo_linear_rows_max(void);
 
 /*
- * out[i, j] = epilogue( sum_c x[i, c] * weight[j, c] + bias[j] ) for a few
+ * out[i, j] = epilogue( sum_c x[i, c] * weight[j, c] + bias[j] ) + residual[i, j] for a few
  * input rows: x [m, k], weight [n, k] (the layout of torch.nn.Linear.weight),
- * bias NULL or [n], out [m, n]; 0 <= m <= oslo_linear_rows_max(). Sums and the
- * epilogue are fp32, rounded once to the storage type. The kernel streams the
+ * bias NULL or [n], out [m, n]; 0 <= m <= oslo_linear_rows_max(). residual:
+ * NULL or [m, n], added after the epilogue (the residual connection around the
+ * attention or the feed-forward module, oslo/models/gpt2/modeling_gpt2.py:444,
+ * :474); out may alias it. Sums and the epilogue are fp32, rounded once to the
+ * storage type. The kernel streams the
  * weight once (it is bound by HBM, like a GEMV); for more rows a GEMM library
  * is the right tool and the call returns OSLO_E_UNSUPPORTED. k*sizeof(dtype)
  * must be a multiple of 16, x and weight 16-byte aligned, the weight smaller
@@ -320,8 +323,9 @@ int oslo_linear_rows_max(void);
  * modeling_gptj.py:968-970, :1031) with epilogue NONE.
  */
 int oslo_linear_rows_fwd(void *out, const void *x, const void *weight,
-                         const void *bias, int64_t m, int64_t n, int64_t k,
-                         int epilogue, int dtype, oslo_stream_t stream);
+                         const void *bias, const void *residual, int64_t m,
+                         int64_t n, int64_t k, int epilogue, int dtype,
+                         oslo_stream_t stream);
 
 /*
  * The same for `count` (1 to 3) layers of one shape applied to the same x in
@@ -340,15 +344,17 @@ int oslo_linear_rows_fwd_multi(void *const *out, const void *x,
 /*
  * The same layer with the weight stored [k, n] (input features major), the
  * layout of GPT-2's Conv1D (transformers' pytorch_utils.Conv1D, y = x @ w + b):
- * out[i, j] = epilogue( sum_c x[i, c] * weight[c, j] + bias[j] ). Both k and n
+ * out[i, j] = epilogue( sum_c x[i, c] * weight[c, j] + bias[j] ) + residual[i, j].
+ * Both k and n
  * times sizeof(dtype) must be multiples of 16. Replaces, for a decoding step,
  * self.c_attn(hidden_states), `attn_output @= self.c_proj.weight` + bias and the
  * two projections of the fused feed-forward module with FusedBiasActivation
  * (oslo/models/gpt2/modeling_gpt2.py:1485, :1523-1536, :1553-1567).
  */
 int oslo_linear_rows_kn_fwd(void *out, const void *x, const void *weight,
-                            const void *bias, int64_t m, int64_t n, int64_t k,
-                            int epilogue, int dtype, oslo_stream_t stream);
+                            const void *bias, const void *residual, int64_t m,
+                            int64_t n, int64_t k, int epilogue, int dtype,
+                            oslo_stream_t stream);
 
 /* Attention of a decoding step ----------------------------------------------- */
 

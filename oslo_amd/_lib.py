@@ -50,8 +50,8 @@ PROTOTYPES = {
         _c.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                    _c.c_int, _c.c_int, _P]),
     "oslo_linear_rows_max": (_c.c_int, []),
-    "oslo_linear_rows_fwd": (_c.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _c.c_int, _c.c_int, _P]),
-    "oslo_linear_rows_kn_fwd": (_c.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _c.c_int, _c.c_int, _P]),
+    "oslo_linear_rows_fwd": (_c.c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _c.c_int, _c.c_int, _P]),
+    "oslo_linear_rows_kn_fwd": (_c.c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _c.c_int, _c.c_int, _P]),
     "oslo_linear_rows_fwd_multi": (
         _c.c_int, [_P, _P, _P, _P, _c.c_int, _I64, _I64, _I64, _c.c_int, _c.c_int, _P]),
     "oslo_attention_decode_workspace_bytes": (_c.c_size_t, [_I64, _I64, _I64, _c.c_int]),

@@ -37,6 +37,7 @@ struct LinearJobs {
   T *out[kMaxJobs];
   const T *w[kMaxJobs];
   const T *bias[kMaxJobs];
+  const T *residual; // [m, n], added after the activation; for one layer only
 };
 
 template <typename T, int VEC>
@@ -130,7 +131,9 @@ __global__ __launch_bounds__(kBlockThreads) void linear_rows_kernel(
         if (i >= m) break;
         float v = acc[r][i] + b;
         if (gelu) v = gelu_fwd(v);
-        out[(int64_t)i * n + row0 + r] = static_cast<T>(v);
+        const int64_t at = (int64_t)i * n + row0 + r;
+        if (jobs.residual != nullptr) v += static_cast<float>(jobs.residual[at]);
+        out[at] = static_cast<T>(v);
       }
     }
   }
@@ -237,7 +240,9 @@ __global__ __launch_bounds__(THREADS) void linear_rows_lds_kernel(
         if (i >= m) break;
         float v = acc[r][i] + b;
         if (gelu) v = gelu_fwd(v);
-        out[(int64_t)i * n + row0 + r] = static_cast<T>(v);
+        const int64_t at = (int64_t)i * n + row0 + r;
+        if (jobs.residual != nullptr) v += static_cast<float>(jobs.residual[at]);
+        out[at] = static_cast<T>(v);
       }
     }
   }
@@ -245,7 +250,8 @@ __global__ __launch_bounds__(THREADS) void linear_rows_lds_kernel(
 
 template <typename T>
 LinearJobs<T> make_jobs(void *const *out, const void *const *w,
-                        const void *const *bias, int count) {
+                        const void *const *bias, const void *residual,
+                        int count) {
   LinearJobs<T> jobs;
   for (int j = 0; j < kMaxJobs; ++j) {
     const int s = j < count ? j : 0;
@@ -253,6 +259,7 @@ LinearJobs<T> make_jobs(void *const *out, const void *const *w,
     jobs.w[j] = static_cast<const T *>(w[s]);
     jobs.bias[j] = bias ? static_cast<const T *>(bias[s]) : nullptr;
   }
+  jobs.residual = static_cast<const T *>(residual);
   return jobs;
 }
 
@@ -282,8 +289,9 @@ int launch(const LinearJobs<T> &jobs, int count, const void *x, int m, int64_t n
 }
 
 int linear_rows(void *const *out, const void *x, const void *const *weight,
-                const void *const *bias, int count, int64_t m, int64_t n,
-                int64_t k, int epilogue, int dtype, hipStream_t s) {
+                const void *const *bias, const void *residual, int count,
+                int64_t m, int64_t n, int64_t k, int epilogue, int dtype,
+                hipStream_t s) {
   if (m < 0 || n < 0 || k < 0)
     return fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd: negative size");
   if (epilogue != OSLO_EPILOGUE_NONE && epilogue != OSLO_EPILOGUE_GELU_TANH)
@@ -320,7 +328,7 @@ int linear_rows(void *const *out, const void *x, const void *const *weight,
   const int gelu = epilogue == OSLO_EPILOGUE_GELU_TANH;
   const int mi = (int)m;
   OSLO_DISPATCH_DTYPE(dtype, {
-    const LinearJobs<T> jobs = make_jobs<T>(out, weight, bias, count);
+    const LinearJobs<T> jobs = make_jobs<T>(out, weight, bias, residual, count);
     if (mi == 1) return launch<T, 1, 1, 8>(jobs, count, x, mi, n, k, gelu, s);
     if (mi == 2) return launch<T, 2, 1, 8>(jobs, count, x, mi, n, k, gelu, s);
     // two weight rows per wave halve the LDS reads per weight byte, but leave
@@ -356,7 +364,8 @@ constexpr int kStripLanes = 4; // lanes along the output features
 template <typename T, int VEC, int MT>
 __global__ __launch_bounds__(kKnThreads) void linear_rows_kn_kernel(
     T *__restrict__ out, const T *__restrict__ x, const T *__restrict__ w,
-    const T *__restrict__ bias, int m, int64_t n, int64_t k, int gelu) {
+    const T *__restrict__ bias, const T *residual, int m, int64_t n, int64_t k,
+    int gelu) {
   constexpr int kRowGroups = kWave / kStripLanes; // 16 rows per load instruction
   constexpr int kStrip = kStripLanes * VEC;       // output features per block
   __shared__ float red[kKnWaves][MT][kStrip];
@@ -427,20 +436,23 @@ __global__ __launch_bounds__(kKnThreads) void linear_rows_kn_kernel(
     for (int wv_ = 0; wv_ < kKnWaves; ++wv_) v += red[wv_][i][c];
     if (bias != nullptr) v += static_cast<float>(bias[j]);
     if (gelu) v = gelu_fwd(v);
+    if (residual != nullptr) v += static_cast<float>(residual[(int64_t)i * n + j]);
     out[(int64_t)i * n + j] = static_cast<T>(v);
   }
 }
 
 template <typename T, int MT>
-int launch_kn(void *out, const void *x, const void *w, const void *bias, int m,
-              int64_t n, int64_t k, int gelu, hipStream_t stream) {
+int launch_kn(void *out, const void *x, const void *w, const void *bias,
+              const void *residual, int m, int64_t n, int64_t k, int gelu,
+              hipStream_t stream) {
   constexpr int VEC = Io<T>::kVec;
   constexpr int kStrip = kStripLanes * VEC;
   const int64_t blocks = (n + kStrip - 1) / kStrip;
   linear_rows_kn_kernel<T, VEC, MT>
       <<<dim3((unsigned)blocks), dim3(kKnThreads), 0, stream>>>(
           static_cast<T *>(out), static_cast<const T *>(x),
-          static_cast<const T *>(w), static_cast<const T *>(bias), m, n, k, gelu);
+          static_cast<const T *>(w), static_cast<const T *>(bias),
+          static_cast<const T *>(residual), m, n, k, gelu);
   return check_launch("oslo_linear_rows_kn_fwd");
 }
 
@@ -448,8 +460,9 @@ int launch_kn(void *out, const void *x, const void *w, const void *bias, int m,
 } // namespace oslo
 
 extern "C" int oslo_linear_rows_kn_fwd(void *out, const void *x, const void *weight,
-                                       const void *bias, int64_t m, int64_t n,
-                                       int64_t k, int epilogue, int dtype,
+                                       const void *bias, const void *residual,
+                                       int64_t m, int64_t n, int64_t k,
+                                       int epilogue, int dtype,
                                        oslo_stream_t stream) {
   using namespace oslo;
   if (m < 0 || n < 0 || k < 0)
@@ -484,14 +497,14 @@ extern "C" int oslo_linear_rows_kn_fwd(void *out, const void *x, const void *wei
     // compiled for the exact row count: a block does all the arithmetic of its
     // strip, and rows padded up to a power of two showed in the time
     switch (mi) {
-    case 1: return launch_kn<T, 1>(out, x, weight, bias, mi, n, k, gelu, s);
-    case 2: return launch_kn<T, 2>(out, x, weight, bias, mi, n, k, gelu, s);
-    case 3: return launch_kn<T, 3>(out, x, weight, bias, mi, n, k, gelu, s);
-    case 4: return launch_kn<T, 4>(out, x, weight, bias, mi, n, k, gelu, s);
-    case 5: return launch_kn<T, 5>(out, x, weight, bias, mi, n, k, gelu, s);
-    case 6: return launch_kn<T, 6>(out, x, weight, bias, mi, n, k, gelu, s);
-    case 7: return launch_kn<T, 7>(out, x, weight, bias, mi, n, k, gelu, s);
-    default: return launch_kn<T, 8>(out, x, weight, bias, mi, n, k, gelu, s);
+    case 1: return launch_kn<T, 1>(out, x, weight, bias, residual, mi, n, k, gelu, s);
+    case 2: return launch_kn<T, 2>(out, x, weight, bias, residual, mi, n, k, gelu, s);
+    case 3: return launch_kn<T, 3>(out, x, weight, bias, residual, mi, n, k, gelu, s);
+    case 4: return launch_kn<T, 4>(out, x, weight, bias, residual, mi, n, k, gelu, s);
+    case 5: return launch_kn<T, 5>(out, x, weight, bias, residual, mi, n, k, gelu, s);
+    case 6: return launch_kn<T, 6>(out, x, weight, bias, residual, mi, n, k, gelu, s);
+    case 7: return launch_kn<T, 7>(out, x, weight, bias, residual, mi, n, k, gelu, s);
+    default: return launch_kn<T, 8>(out, x, weight, bias, residual, mi, n, k, gelu, s);
     }
   });
   return OSLO_OK;
@@ -500,14 +513,14 @@ extern "C" int oslo_linear_rows_kn_fwd(void *out, const void *x, const void *wei
 extern "C" int oslo_linear_rows_max(void) { return oslo::kMaxRows; }
 
 extern "C" int oslo_linear_rows_fwd(void *out, const void *x, const void *weight,
-                                    const void *bias, int64_t m, int64_t n,
-                                    int64_t k, int epilogue, int dtype,
-                                    oslo_stream_t stream) {
+                                    const void *bias, const void *residual,
+                                    int64_t m, int64_t n, int64_t k, int epilogue,
+                                    int dtype, oslo_stream_t stream) {
   void *const outs[1] = {out};
   const void *const weights[1] = {weight};
   const void *const biases[1] = {bias};
-  return oslo::linear_rows(outs, x, weights, biases, 1, m, n, k, epilogue, dtype,
-                           static_cast<hipStream_t>(stream));
+  return oslo::linear_rows(outs, x, weights, biases, residual, 1, m, n, k,
+                           epilogue, dtype, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int oslo_linear_rows_fwd_multi(void *const *out, const void *x,
@@ -521,6 +534,6 @@ extern "C" int oslo_linear_rows_fwd_multi(void *const *out, const void *x,
                       count, oslo::kMaxJobs);
   if (!out || !weight)
     return oslo::fail(OSLO_E_BAD_ARG, "oslo_linear_rows_fwd_multi: null pointer table");
-  return oslo::linear_rows(out, x, weight, bias, count, m, n, k, epilogue, dtype,
-                           static_cast<hipStream_t>(stream));
+  return oslo::linear_rows(out, x, weight, bias, nullptr, count, m, n, k, epilogue,
+                           dtype, static_cast<hipStream_t>(stream));
 }

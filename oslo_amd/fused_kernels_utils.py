@@ -571,13 +571,15 @@ class FusedLinearRows(object):
         return not _needs_grad(x, weight, bias)
 
     @staticmethod
-    def apply(x, weight, bias=None, act=None, conv1d=False):
+    def apply(x, weight, bias=None, act=None, conv1d=False, residual=None):
+        """``residual``: a tensor of the output's shape added last (the residual
+        connection around the module), inside the same launch."""
         gelu = act is not None and "gelu" in act
         forward = get_custom_kernels().linear_rows_kn_forward if conv1d else get_custom_kernels().linear_rows_forward
-        out = forward(x, weight, bias, gelu)
         if act is not None and not gelu:
-            out = _act2fn(act)(out)
-        return out
+            out = _act2fn(act)(forward(x, weight, bias, False))
+            return out if residual is None else out + residual
+        return forward(x, weight, bias, gelu, residual)
 
     @staticmethod
     def project(module, x):
@@ -785,4 +787,7 @@ class FusedKernelMixin(object):
                 model_module.__class__ = fused_modules[cls]
                 setattr(model_module, "config", self.config)
 
+        # beyond the reference: with everything fused, a decoding step also
+        # streams the output head's weight through the few-row kernel
+        self.fused_lm_head = user_modules is None
         return self

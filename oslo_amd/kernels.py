@@ -428,19 +428,28 @@ def _rotary_call(tensors, sin, cos, rotary_dim, offset, inverse):
     return tuple(outs)
 
 
-def linear_rows_forward(x, weight, bias=None, gelu=False):
+def linear_rows_forward(x, weight, bias=None, gelu=False, residual=None):
     """x [..., K] with at most LINEAR_ROWS_MAX rows in all, weight [N, K] (the
     layout of nn.Linear), bias None or [N] -> act(x @ weight.t() + bias) as
-    [..., N], act = tanh-form GeLU if ``gelu``. One pass over the weight; sums
-    and the epilogue in fp32 (oslo/models/gptj/modeling_gptj.py:1049-1065 for a
-    decoding step)."""
-    return linear_rows_forward_multi(x, (weight,), (bias,), gelu)[0]
+    [..., N], act = tanh-form GeLU if ``gelu``; ``residual`` [..., N] is added
+    last. One pass over the weight; sums and the epilogue in fp32
+    (oslo/models/gptj/modeling_gptj.py:1049-1065 for a decoding step)."""
+    return linear_rows_forward_multi(x, (weight,), (bias,), gelu, residual)[0]
 
 
-def linear_rows_kn_forward(x, weight, bias=None, gelu=False):
+def _residual_like(residual, shape, x):
+    if residual is None:
+        return None
+    _device_tensor(residual, "residual", x)
+    _require(tuple(residual.shape) == tuple(shape) and residual.dtype == x.dtype,
+             "residual must have the output's shape and dtype")
+    return residual.contiguous()
+
+
+def linear_rows_kn_forward(x, weight, bias=None, gelu=False, residual=None):
     """The same with the weight stored [K, N], the layout of GPT-2's Conv1D:
-    act(x @ weight + bias) (oslo/models/gpt2/modeling_gpt2.py:1553-1567 for a
-    decoding step)."""
+    act(x @ weight + bias) + residual (oslo/models/gpt2/modeling_gpt2.py
+    :1553-1567 for a decoding step)."""
     _device_tensor(x, "x")
     _device_tensor(weight, "weight", x)
     code = _dtype_code(x, "x")
@@ -456,17 +465,20 @@ def linear_rows_kn_forward(x, weight, bias=None, gelu=False):
         bias = bias.contiguous()
     x2, w = x.contiguous(), weight.contiguous()
     out = torch.empty(x.shape[:-1] + (n,), dtype=x.dtype, device=x.device)
+    residual = _residual_like(residual, out.shape, x)
     with _on_device(x):
         _lib.check(_lib.load().oslo_linear_rows_kn_fwd(
-            _ptr(out), _ptr(x2), _ptr(w), _ptr(bias), m, n, k,
+            _ptr(out), _ptr(x2), _ptr(w), _ptr(bias), _ptr(residual), m, n, k,
             EPILOGUE_GELU_TANH if gelu else EPILOGUE_NONE, code, _stream(x)))
     return out
 
 
-def linear_rows_forward_multi(x, weights, biases=None, gelu=False):
+def linear_rows_forward_multi(x, weights, biases=None, gelu=False, residual=None):
     """One to three layers of the same shape applied to the same x in one
-    launch (the query, key and value projections): a list of outputs."""
+    launch (the query, key and value projections): a list of outputs.
+    ``residual`` goes with a single layer only."""
     count = len(weights)
+    _require(residual is None or count == 1, "a residual goes with one layer")
     _require(1 <= count <= 3, "one to three layers per launch")
     biases = (None,) * count if biases is None else tuple(biases)
     _require(len(biases) == count, "one bias (or None) per weight")
@@ -490,10 +502,12 @@ def linear_rows_forward_multi(x, weights, biases=None, gelu=False):
     x2 = x.contiguous()
     outs = [torch.empty(x.shape[:-1] + (n,), dtype=x.dtype, device=x.device) for _ in range(count)]
     epilogue = EPILOGUE_GELU_TANH if gelu else EPILOGUE_NONE
+    residual = _residual_like(residual, outs[0].shape, x)
     with _on_device(x):
         if count == 1:
             _lib.check(_lib.load().oslo_linear_rows_fwd(
-                _ptr(outs[0]), _ptr(x2), _ptr(ws[0]), _ptr(bs[0]), m, n, k, epilogue, code, _stream(x)))
+                _ptr(outs[0]), _ptr(x2), _ptr(ws[0]), _ptr(bs[0]), _ptr(residual), m, n, k, epilogue, code,
+                _stream(x)))
         else:
             table = ctypes.c_void_p * count
             _lib.check(_lib.load().oslo_linear_rows_fwd_multi(

@@ -169,7 +169,9 @@ class FusedGPT2Attention(GPT2Attention):
 
     def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None,
                 encoder_hidden_states=None, encoder_attention_mask=None, use_cache=False,
-                output_attentions=False):
+                output_attentions=False, residual=None):
+        """``residual``: added to the output (the residual connection of the
+        block, which a decoding step takes into the projection's launch)."""
         query, key, value, present = self._project_qkv(hidden_states, layer_past, encoder_hidden_states, use_cache)
         if encoder_hidden_states is not None:
             attention_mask = encoder_attention_mask
@@ -204,10 +206,13 @@ class FusedGPT2Attention(GPT2Attention):
             out = self._merge_heads(out, self.num_heads, self.head_dim)
         if FusedLinearRows.is_available(out, self.c_proj.weight, self.c_proj.bias, conv1d=True) and not (
                 self.training and self.resid_dropout.p > 0.0):
-            out = FusedLinearRows.apply(out, self.c_proj.weight, self.c_proj.bias, conv1d=True)  # a decoding step
+            out = FusedLinearRows.apply(out, self.c_proj.weight, self.c_proj.bias, conv1d=True,
+                                        residual=residual)  # a decoding step
         else:
             out = out @ self.c_proj.weight  # projection without its bias ...
             out = FusedBiasDropout.apply(out, self.c_proj.bias, self.training, self.resid_dropout.p)  # ... fused here
+            if residual is not None:
+                out = out + residual
         return (out, present, w) if output_attentions else (out, present)
 
 
@@ -226,20 +231,23 @@ class GPT2MLP(nn.Module):
 class FusedGPT2MLP(GPT2MLP):
     """oslo/models/gpt2/modeling_gpt2.py:1545-1569."""
 
-    def forward(self, x):
+    def forward(self, x, residual=None):
+        """``residual``: added to the output (the residual connection of the block)."""
         if FusedLinearRows.is_available(x, self.c_fc.weight, self.c_fc.bias, conv1d=True):
             # a decoding step: each projection is one pass over its weight with
-            # the bias (and the activation) applied to the fp32 sums
+            # the bias (and the activation, and the residual) applied to the fp32 sums
             x = FusedLinearRows.apply(x, self.c_fc.weight, self.c_fc.bias, self.config.activation_function,
                                       conv1d=True)
             if not (self.training and self.dropout.p > 0.0):
-                return FusedLinearRows.apply(x, self.c_proj.weight, self.c_proj.bias, conv1d=True)
+                return FusedLinearRows.apply(x, self.c_proj.weight, self.c_proj.bias, conv1d=True,
+                                             residual=residual)
             x = FusedLinearRows.apply(x, self.c_proj.weight, conv1d=True)
         else:
             x = x @ self.c_fc.weight
             x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
             x = x @ self.c_proj.weight
-        return FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
+        x = FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
+        return x if residual is None else x + residual
 
 
 class GPT2Block(nn.Module):
@@ -259,12 +267,28 @@ class GPT2Block(nn.Module):
         return hidden_states, a[1]
 
 
+class FusedGPT2Block(GPT2Block):
+    """The block with its two residual additions handed to the fused modules,
+    which take them into their last projection's launch in a decoding step.
+    No counterpart in the reference, which fuses attention and MLP only
+    (oslo/models/gpt2/configuration_gpt2.py:272-284); the arithmetic is that
+    of oslo/models/gpt2/modeling_gpt2.py:420-481."""
+
+    def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None, use_cache=False):
+        if not (isinstance(self.attn, FusedGPT2Attention) and isinstance(self.mlp, FusedGPT2MLP)):
+            return super().forward(hidden_states, layer_past, attention_mask, head_mask, use_cache)
+        a = self.attn(self.ln_1(hidden_states), layer_past=layer_past, attention_mask=attention_mask,
+                      head_mask=head_mask, use_cache=use_cache, residual=hidden_states)
+        hidden_states = self.mlp(self.ln_2(a[0]), residual=a[0])
+        return hidden_states, a[1]
+
+
 class GPT2LayerPolicy(LayerPolicy):
     """oslo/models/gpt2/configuration_gpt2.py:272-284."""
 
     @staticmethod
     def fused_modules():
-        return {GPT2Attention: FusedGPT2Attention, GPT2MLP: FusedGPT2MLP}
+        return {GPT2Attention: FusedGPT2Attention, GPT2MLP: FusedGPT2MLP, GPT2Block: FusedGPT2Block}
 
 
 class GPT2Model(nn.Module):
@@ -307,6 +331,7 @@ class GPT2LMHeadModel(PreTrainedModel):
 
     def forward(self, input_ids, attention_mask=None, past_key_values=None, use_cache=False, labels=None):
         h, presents = self.transformer(input_ids, attention_mask, past_key_values, use_cache)
-        logits = self.lm_head(h)
+        fused_head = getattr(self, "fused_lm_head", False) and not self.training
+        logits = FusedLinearRows.project(self.lm_head, h) if fused_head else self.lm_head(h)
         loss = causal_lm_loss(logits, labels) if labels is not None else None
         return {"loss": loss, "logits": logits, "past_key_values": presents}

@@ -147,7 +147,9 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
         return torch.matmul(w, value), w
 
     def forward(self, hidden_states, attention_mask=None, layer_past=None, head_mask=None,
-                use_cache=False, output_attentions=False):
+                use_cache=False, output_attentions=False, residual=None):
+        """``residual``: added to the output (the residual connection of the
+        block, which a decoding step takes into the projection's launch)."""
         query, key, value, present = self._project_qkv(hidden_states, layer_past, use_cache)
         (bsz, np_, sq, _), sk = query.size(), key.size(-2)
         # a single query over a key/value cache (a decoding step) sees every key
@@ -181,10 +183,12 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
         out = FusedMergeHeads.apply(out) if self._transposes_fused(out) else self._merge_heads(out)
         if FusedLinearRows.is_available(out, self.out_proj.weight) and not (
                 self.training and self.resid_dropout.p > 0.0):
-            out = FusedLinearRows.apply(out, self.out_proj.weight, self.out_proj.bias)
+            out = FusedLinearRows.apply(out, self.out_proj.weight, self.out_proj.bias, residual=residual)
         else:
             out = out @ self.out_proj.weight.t()
             out = FusedBiasDropout.apply(out, self.out_proj.bias, self.training, self.resid_dropout.p)
+            if residual is not None:
+                out = out + residual
         return (out, present, w) if output_attentions else (out, present)
 
 
@@ -233,19 +237,21 @@ class GPTNeoMLP(nn.Module):
 class FusedGPTNeoMLP(GPTNeoMLP):
     """oslo/models/gpt_neo/modeling_gpt_neo.py:1078-1102."""
 
-    def forward(self, x):
+    def forward(self, x, residual=None):
+        """``residual``: added to the output (the residual connection of the block)."""
         if FusedLinearRows.is_available(x, self.c_fc.weight, self.c_fc.bias):
             # a decoding step: each projection is one pass over its weight with
-            # the bias (and the activation) applied to the fp32 sums
+            # the bias (and the activation, and the residual) applied to the fp32 sums
             x = FusedLinearRows.apply(x, self.c_fc.weight, self.c_fc.bias, self.config.activation_function)
             if not (self.training and self.dropout.p > 0.0):
-                return FusedLinearRows.apply(x, self.c_proj.weight, self.c_proj.bias)
+                return FusedLinearRows.apply(x, self.c_proj.weight, self.c_proj.bias, residual=residual)
             x = FusedLinearRows.apply(x, self.c_proj.weight)
         else:
             x = x @ self.c_fc.weight.t()
             x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
             x = x @ self.c_proj.weight.t()
-        return FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
+        x = FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
+        return x if residual is None else x + residual
 
 
 class GPTNeoBlock(nn.Module):
@@ -265,13 +271,30 @@ class GPTNeoBlock(nn.Module):
         return hidden_states, a[1]
 
 
+class FusedGPTNeoBlock(GPTNeoBlock):
+    """The block with its two residual additions handed to the fused modules,
+    which take them into their last projection's launch in a decoding step.
+    No counterpart in the reference, which fuses attention and MLP only
+    (oslo/models/gpt_neo/configuration_gpt_neo.py:330-342); the arithmetic is
+    that of oslo/models/gpt_neo/modeling_gpt_neo.py:333-380."""
+
+    def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None, use_cache=False):
+        inner = self.attn.attention
+        if not (isinstance(inner, FusedGPTNeoSelfAttention) and isinstance(self.mlp, FusedGPTNeoMLP)):
+            return super().forward(hidden_states, layer_past, attention_mask, head_mask, use_cache)
+        a = inner(self.ln_1(hidden_states), attention_mask=attention_mask, layer_past=layer_past,
+                  head_mask=head_mask, use_cache=use_cache, residual=hidden_states)
+        hidden_states = self.mlp(self.ln_2(a[0]), residual=a[0])
+        return hidden_states, a[1]
+
+
 class GPTNeoLayerPolicy(LayerPolicy):
     """oslo/models/gpt_neo/configuration_gpt_neo.py:330-342."""
 
     @staticmethod
     def fused_modules():
         return {GPTNeoSelfAttention: FusedGPTNeoSelfAttention, GPTNeoMLP: FusedGPTNeoMLP,
-                GPTNeoLocalSelfAttention: FusedGPTNeoLocalSelfAttention}
+                GPTNeoLocalSelfAttention: FusedGPTNeoLocalSelfAttention, GPTNeoBlock: FusedGPTNeoBlock}
 
 
 class GPTNeoModel(nn.Module):
@@ -314,6 +337,7 @@ class GPTNeoForCausalLM(PreTrainedModel):
 
     def forward(self, input_ids, attention_mask=None, past_key_values=None, use_cache=False, labels=None):
         h, presents = self.transformer(input_ids, attention_mask, past_key_values, use_cache)
-        logits = self.lm_head(h)
+        fused_head = getattr(self, "fused_lm_head", False) and not self.training
+        logits = FusedLinearRows.project(self.lm_head, h) if fused_head else self.lm_head(h)
         loss = causal_lm_loss(logits, labels) if labels is not None else None
         return {"loss": loss, "logits": logits, "past_key_values": presents}

@@ -200,7 +200,9 @@ class FusedGPTJAttention(GPTJAttention):
         return torch.matmul(w, value), w
 
     def forward(self, hidden_states, attention_mask=None, layer_past=None, head_mask=None,
-                use_cache=False, output_attentions=False):
+                use_cache=False, output_attentions=False, residual=None):
+        """``residual``: added to the output (the residual connection of the
+        block, which a decoding step takes into the projection's launch)."""
         query, key, value, present = self._project_qkv(hidden_states, layer_past, use_cache)
         (bsz, np_, sq, _), sk = query.size(), key.size(-2)
         # a single query over a key/value cache (a decoding step) sees every key:
@@ -230,8 +232,14 @@ class FusedGPTJAttention(GPTJAttention):
         # dropped (in training; it is skipped when there is nothing to drop)
         vec_ok = FusedRotaryPositionEmbedding.is_available(out.dtype, self.head_dim, 0)
         out = FusedMergeHeads.apply(out) if out.is_cuda and vec_ok else self._merge_heads(out)
-        out = FusedBiasDropout.apply(FusedLinearRows.project(self.out_proj, out), None, self.training,
-                                     self.resid_dropout.p)
+        if residual is not None and FusedLinearRows.is_available(out, self.out_proj.weight) and not (
+                self.training and self.resid_dropout.p > 0.0):
+            out = FusedLinearRows.apply(out, self.out_proj.weight, residual=residual)  # a decoding step
+        else:
+            out = FusedBiasDropout.apply(FusedLinearRows.project(self.out_proj, out), None, self.training,
+                                         self.resid_dropout.p)
+            if residual is not None:
+                out = out + residual
         return (out, present, w) if output_attentions else (out, present)
 
 
@@ -250,19 +258,21 @@ class GPTJMLP(nn.Module):
 class FusedGPTJMLP(GPTJMLP):
     """oslo/models/gptj/modeling_gptj.py:1041-1065."""
 
-    def forward(self, x):
+    def forward(self, x, residual=None):
+        """``residual``: added to the output (the residual connection of the block)."""
         if FusedLinearRows.is_available(x, self.fc_in.weight, self.fc_in.bias):
             # a decoding step: each projection is one pass over its weight with
-            # the bias (and the activation) applied to the fp32 sums
+            # the bias (and the activation, and the residual) applied to the fp32 sums
             x = FusedLinearRows.apply(x, self.fc_in.weight, self.fc_in.bias, self.config.activation_function)
             if not (self.training and self.dropout.p > 0.0):
-                return FusedLinearRows.apply(x, self.fc_out.weight, self.fc_out.bias)
+                return FusedLinearRows.apply(x, self.fc_out.weight, self.fc_out.bias, residual=residual)
             x = FusedLinearRows.apply(x, self.fc_out.weight)
         else:
             x = x @ self.fc_in.weight.t()
             x = FusedBiasActivation.apply(x, self.fc_in.bias, self.config.activation_function)
             x = x @ self.fc_out.weight.t()
-        return FusedBiasDropout.apply(x, self.fc_out.bias, self.training, self.dropout.p)
+        x = FusedBiasDropout.apply(x, self.fc_out.bias, self.training, self.dropout.p)
+        return x if residual is None else x + residual
 
 
 class GPTJBlock(nn.Module):
@@ -282,12 +292,30 @@ class GPTJBlock(nn.Module):
         return hidden_states, a[1]
 
 
+class FusedGPTJBlock(GPTJBlock):
+    """The block with its residual additions handed to the fused modules,
+    which take them into their last projection's launch in a decoding step:
+    attention output + residual first, then the feed-forward output on top (the
+    unfused block adds attention, feed-forward and residual in that order,
+    oslo/models/gptj/modeling_gptj.py:306-327). No counterpart in the
+    reference, which fuses attention and MLP only
+    (oslo/models/gptj/configuration_gptj.py:155-167)."""
+
+    def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None, use_cache=False):
+        if not (isinstance(self.attn, FusedGPTJAttention) and isinstance(self.mlp, FusedGPTJMLP)):
+            return super().forward(hidden_states, layer_past, attention_mask, head_mask, use_cache)
+        normed = self.ln_1(hidden_states)
+        a = self.attn(normed, layer_past=layer_past, attention_mask=attention_mask, head_mask=head_mask,
+                      use_cache=use_cache, residual=hidden_states)
+        return self.mlp(normed, residual=a[0]), a[1]
+
+
 class GPTJLayerPolicy(LayerPolicy):
     """oslo/models/gptj/configuration_gptj.py:155-167."""
 
     @staticmethod
     def fused_modules():
-        return {GPTJAttention: FusedGPTJAttention, GPTJMLP: FusedGPTJMLP}
+        return {GPTJAttention: FusedGPTJAttention, GPTJMLP: FusedGPTJMLP, GPTJBlock: FusedGPTJBlock}
 
 
 class GPTJModel(nn.Module):
@@ -323,6 +351,7 @@ class GPTJForCausalLM(PreTrainedModel):
 
     def forward(self, input_ids, attention_mask=None, past_key_values=None, use_cache=False, labels=None):
         h, presents = self.transformer(input_ids, attention_mask, past_key_values, use_cache)
-        logits = self.lm_head(h)
+        fused_head = getattr(self, "fused_lm_head", False) and not self.training
+        logits = FusedLinearRows.project(self.lm_head, h) if fused_head else self.lm_head(h)
         loss = causal_lm_loss(logits, labels) if labels is not None else None
         return {"loss": loss, "logits": logits, "past_key_values": presents}

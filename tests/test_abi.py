@@ -106,18 +106,18 @@ def test_argument_screening_without_a_device(lib):
     # few-row linear layer: too many rows, ragged rows, unknown epilogue, aliasing, misalignment
     three = ctypes.c_void_p(48)
     assert lib.oslo_linear_rows_max() == 8
-    assert lib.oslo_linear_rows_fwd(one, two, three, null, 9, 4, 8, 0, 1, null) == -2
-    assert lib.oslo_linear_rows_fwd(one, two, three, null, 1, 4, 12, 0, 1, null) == -2
-    assert lib.oslo_linear_rows_fwd(one, two, three, null, 1, 4, 8, 5, 1, null) == -1
-    assert lib.oslo_linear_rows_fwd(two, two, three, null, 1, 4, 8, 0, 1, null) == -1
-    assert lib.oslo_linear_rows_fwd(one, ctypes.c_void_p(40), three, null, 1, 4, 8, 0, 1, null) == -1
-    assert lib.oslo_linear_rows_fwd(one, two, three, null, 1, 1 << 30, 8, 0, 1, null) == -2
-    assert lib.oslo_linear_rows_fwd(one, two, null, null, 1, 4, 8, 0, 1, null) == -1
-    assert lib.oslo_linear_rows_fwd(null, null, null, null, 0, 4, 8, 0, 1, null) == 0
-    assert lib.oslo_linear_rows_kn_fwd(one, two, three, null, 9, 8, 8, 0, 1, null) == -2
-    assert lib.oslo_linear_rows_kn_fwd(one, two, three, null, 1, 12, 8, 0, 1, null) == -2     # ragged weight rows
-    assert lib.oslo_linear_rows_kn_fwd(one, two, three, null, 1, 8, 8, 0, 7, null) == -1
-    assert lib.oslo_linear_rows_kn_fwd(null, null, null, null, 0, 8, 8, 0, 1, null) == 0
+    assert lib.oslo_linear_rows_fwd(one, two, three, null, null, 9, 4, 8, 0, 1, null) == -2
+    assert lib.oslo_linear_rows_fwd(one, two, three, null, null, 1, 4, 12, 0, 1, null) == -2
+    assert lib.oslo_linear_rows_fwd(one, two, three, null, null, 1, 4, 8, 5, 1, null) == -1
+    assert lib.oslo_linear_rows_fwd(two, two, three, null, null, 1, 4, 8, 0, 1, null) == -1
+    assert lib.oslo_linear_rows_fwd(one, ctypes.c_void_p(40), three, null, null, 1, 4, 8, 0, 1, null) == -1
+    assert lib.oslo_linear_rows_fwd(one, two, three, null, null, 1, 1 << 30, 8, 0, 1, null) == -2
+    assert lib.oslo_linear_rows_fwd(one, two, null, null, null, 1, 4, 8, 0, 1, null) == -1
+    assert lib.oslo_linear_rows_fwd(null, null, null, null, null, 0, 4, 8, 0, 1, null) == 0
+    assert lib.oslo_linear_rows_kn_fwd(one, two, three, null, null, 9, 8, 8, 0, 1, null) == -2
+    assert lib.oslo_linear_rows_kn_fwd(one, two, three, null, null, 1, 12, 8, 0, 1, null) == -2     # ragged weight rows
+    assert lib.oslo_linear_rows_kn_fwd(one, two, three, null, null, 1, 8, 8, 0, 7, null) == -1
+    assert lib.oslo_linear_rows_kn_fwd(null, null, null, null, null, 0, 8, 8, 0, 1, null) == 0
     table = (ctypes.c_void_p * 3)(16, 32, 48)
     assert lib.oslo_linear_rows_fwd_multi(table, one, table, null, 4, 1, 4, 8, 0, 1, null) == -1     # four layers
     assert lib.oslo_linear_rows_fwd_multi(null, one, table, null, 2, 1, 4, 8, 0, 1, null) == -1

@@ -124,6 +124,28 @@ def test_fuse_modules_filter_and_errors():
         Plain(None).fuse()
 
 
+def test_blocks_are_fused_unless_the_reference_selection_is_asked_for():
+    """fuse() also swaps the blocks (their residual additions go into the fused
+    modules); the reference's own selection leaves them alone, and so does a
+    partial one, whose unfused child the fused block could not hand a residual."""
+    for make, block, fused_block, selection in (
+            (tiny_gpt2, modeling_gpt2.GPT2Block, modeling_gpt2.FusedGPT2Block,
+             [modeling_gpt2.GPT2Attention, modeling_gpt2.GPT2MLP]),
+            (tiny_gptj, modeling_gptj.GPTJBlock, modeling_gptj.FusedGPTJBlock,
+             [modeling_gptj.GPTJAttention, modeling_gptj.GPTJMLP]),
+            (tiny_neo, modeling_gpt_neo.GPTNeoBlock, modeling_gpt_neo.FusedGPTNeoBlock,
+             [modeling_gpt_neo.GPTNeoSelfAttention, modeling_gpt_neo.GPTNeoMLP])):
+        m = make().fuse()
+        assert all(type(b) is fused_block for b in m.transformer.h) and m.fused_lm_head
+        m = make().fuse(modules=selection)
+        assert all(type(b) is block for b in m.transformer.h) and not m.fused_lm_head
+        # a fused block may sit over an unfused child (it then runs the plain block's code)
+        m = make().fuse(modules=[selection[1], block])
+        assert all(type(b) is fused_block for b in m.transformer.h)
+        assert not any(type(x) in (modeling_gpt2.FusedGPT2Attention, modeling_gptj.FusedGPTJAttention,
+                                   modeling_gpt_neo.FusedGPTNeoSelfAttention) for x in m.modules())
+
+
 def test_gpt_neo_local_attention_has_a_fused_class_of_its_own():
     m = tiny_neo().fuse()
     kinds = [type(b.attn.attention) for b in m.transformer.h]

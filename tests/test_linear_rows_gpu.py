@@ -85,6 +85,29 @@ def test_linear_rows_three_layers_in_one_launch(m, n, k, dtype):
         kernels.linear_rows_forward_multi(x, [ws[0], ws[1][:-1]])
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("m,n,k", [(1, 72, 512), (3, 136, 1032), (8, 264, 2048)])
+def test_linear_rows_residual_epilogue(m, n, k, dtype):
+    """act(x.w + b) + residual in one launch, both weight layouts: one rounding
+    of the float64 value; in place over the residual too."""
+    x = randn((m, k), dtype, seed=1)
+    w = randn((n, k), dtype, seed=2, std=0.05)
+    b = randn((n,), dtype, seed=3, std=0.5)
+    res = randn((m, n), dtype, seed=4, std=2.0)
+    for gelu in (False, True):
+        want = orc.linear_rows(f32(x), f32(w), f32(b), gelu) + f32(res).astype(np.float64)
+        mass = (np.abs(f32(x)).astype(np.float64) @ np.abs(f32(w)).astype(np.float64).T) + np.abs(f32(res))
+        tol = EPS[dtype] * np.abs(want) + 1e-6 * mass + 1e-30
+        nk = kernels.linear_rows_forward(x.to(DEV), w.to(DEV), b.to(DEV), gelu, res.to(DEV))
+        kn = kernels.linear_rows_kn_forward(x.to(DEV), w.t().contiguous().to(DEV), b.to(DEV), gelu, res.to(DEV))
+        for out in (nk, kn):
+            assert np.max(np.abs(f32(out).astype(np.float64) - want) / tol) <= 1.0
+    with pytest.raises(RuntimeError):
+        kernels.linear_rows_forward(x.to(DEV), w.to(DEV), None, False, res[:, :-1].to(DEV))
+    with pytest.raises(RuntimeError):
+        kernels.linear_rows_forward_multi(x.to(DEV), [w.to(DEV), w.to(DEV)], None, False, res.to(DEV))
+
+
 def test_linear_rows_leading_dims_and_torch_agreement():
     """[B, 1, K] inputs as the modules pass them; against torch's own linear +
     gelu on the device, within bf16 rounding of the two-step path."""

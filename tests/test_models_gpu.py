@@ -56,6 +56,31 @@ def test_fused_model_matches_unfused(family, dtype, padded):
 
 
 @pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
+def test_partial_fusion_selections_compute_the_same(family):
+    """Attention and MLP only (the reference's selection), a fused block over an
+    unfused attention, and everything: the same logits within fp32 rounding,
+    in a full forward and in a decoding step over a cache."""
+    from oslo_amd import modeling_gpt2 as g2, modeling_gpt_neo as neo, modeling_gptj as gj
+    parts = {"gpt2": (g2.GPT2Attention, g2.GPT2MLP, g2.GPT2Block),
+             "gptj": (gj.GPTJAttention, gj.GPTJMLP, gj.GPTJBlock),
+             "gpt_neo": (neo.GPTNeoSelfAttention, neo.GPTNeoMLP, neo.GPTNeoBlock)}[family]
+    ids = torch.randint(0, 512, (2, 40), device=DEV)
+    outs = []
+    for selection in (None, [parts[0], parts[1]], [parts[1], parts[2]], "unfused"):
+        torch.manual_seed(0)
+        m = models()[family]().to(DEV).eval()
+        if selection != "unfused":
+            m.fuse(modules=selection)
+        with torch.no_grad():
+            full = m(ids, use_cache=True)
+            step = m(ids[:, :1], past_key_values=full["past_key_values"], use_cache=True)["logits"]
+        outs.append((full["logits"], step))
+    for full, step in outs[:-1]:
+        assert (full - outs[-1][0]).abs().max() <= 2e-4
+        assert (step - outs[-1][1]).abs().max() <= 2e-4
+
+
+@pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
 def test_fused_model_backward_matches_unfused(family):
     torch.manual_seed(1)
     m = models()[family]().to(DEV).train()            # fp32, every dropout p = 0
