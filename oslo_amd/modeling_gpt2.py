@@ -13,7 +13,8 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedDecodeAttention, FusedLinearRows,
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedBiasDropoutResidual,
+                                 FusedDecodeAttention, FusedLinearRows,
                                  FusedMergeHeads,
                                  FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedSplitHeads)
@@ -209,10 +210,12 @@ class FusedGPT2Attention(GPT2Attention):
             out = FusedLinearRows.apply(out, self.c_proj.weight, self.c_proj.bias, conv1d=True,
                                         residual=residual)  # a decoding step
         else:
-            out = out @ self.c_proj.weight  # projection without its bias ...
-            out = FusedBiasDropout.apply(out, self.c_proj.bias, self.training, self.resid_dropout.p)  # ... fused here
-            if residual is not None:
-                out = out + residual
+            out = out @ self.c_proj.weight  # projection without its bias, which is fused here:
+            if residual is None:
+                out = FusedBiasDropout.apply(out, self.c_proj.bias, self.training, self.resid_dropout.p)
+            else:  # with the block's residual addition in the same pass
+                out = FusedBiasDropoutResidual.apply(out, self.c_proj.bias, residual, self.training,
+                                                     self.resid_dropout.p)
         return (out, present, w) if output_attentions else (out, present)
 
 
@@ -246,8 +249,10 @@ class FusedGPT2MLP(GPT2MLP):
             x = x @ self.c_fc.weight
             x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
             x = x @ self.c_proj.weight
-        x = FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
-        return x if residual is None else x + residual
+        if residual is None:
+            return FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
+        # bias, dropout and the block's residual addition in one pass
+        return FusedBiasDropoutResidual.apply(x, self.c_proj.bias, residual, self.training, self.dropout.p)
 
 
 class GPT2Block(nn.Module):

@@ -16,7 +16,8 @@ from typing import List, Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedDecodeAttention, FusedLinearRows,
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedBiasDropoutResidual,
+                                 FusedDecodeAttention, FusedLinearRows,
                                  FusedMergeHeads,
                                  FusedRotaryPositionEmbedding, FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedScaleMaskWindowSoftmax)
@@ -186,9 +187,11 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
             out = FusedLinearRows.apply(out, self.out_proj.weight, self.out_proj.bias, residual=residual)
         else:
             out = out @ self.out_proj.weight.t()
-            out = FusedBiasDropout.apply(out, self.out_proj.bias, self.training, self.resid_dropout.p)
-            if residual is not None:
-                out = out + residual
+            if residual is None:
+                out = FusedBiasDropout.apply(out, self.out_proj.bias, self.training, self.resid_dropout.p)
+            else:  # bias, dropout and the block's residual addition in one pass
+                out = FusedBiasDropoutResidual.apply(out, self.out_proj.bias, residual, self.training,
+                                                     self.resid_dropout.p)
         return (out, present, w) if output_attentions else (out, present)
 
 
@@ -250,8 +253,10 @@ class FusedGPTNeoMLP(GPTNeoMLP):
             x = x @ self.c_fc.weight.t()
             x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
             x = x @ self.c_proj.weight.t()
-        x = FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
-        return x if residual is None else x + residual
+        if residual is None:
+            return FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)
+        # bias, dropout and the block's residual addition in one pass
+        return FusedBiasDropoutResidual.apply(x, self.c_proj.bias, residual, self.training, self.dropout.p)
 
 
 class GPTNeoBlock(nn.Module):

@@ -18,7 +18,8 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedDecodeAttention, FusedLinearRows,
+from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedBiasDropoutResidual,
+                                 FusedDecodeAttention, FusedLinearRows,
                                  FusedMergeHeads,
                                  FusedRotaryPositionEmbedding,
                                  FusedScaleMaskSoftmax, FusedScaleMaskSoftmaxDropout)
@@ -236,10 +237,11 @@ class FusedGPTJAttention(GPTJAttention):
                 self.training and self.resid_dropout.p > 0.0):
             out = FusedLinearRows.apply(out, self.out_proj.weight, residual=residual)  # a decoding step
         else:
-            out = FusedBiasDropout.apply(FusedLinearRows.project(self.out_proj, out), None, self.training,
-                                         self.resid_dropout.p)
-            if residual is not None:
-                out = out + residual
+            out = FusedLinearRows.project(self.out_proj, out)
+            if residual is None:
+                out = FusedBiasDropout.apply(out, None, self.training, self.resid_dropout.p)
+            else:  # dropout and the block's residual addition in one pass
+                out = FusedBiasDropoutResidual.apply(out, None, residual, self.training, self.resid_dropout.p)
         return (out, present, w) if output_attentions else (out, present)
 
 
@@ -271,8 +273,10 @@ class FusedGPTJMLP(GPTJMLP):
             x = x @ self.fc_in.weight.t()
             x = FusedBiasActivation.apply(x, self.fc_in.bias, self.config.activation_function)
             x = x @ self.fc_out.weight.t()
-        x = FusedBiasDropout.apply(x, self.fc_out.bias, self.training, self.dropout.p)
-        return x if residual is None else x + residual
+        if residual is None:
+            return FusedBiasDropout.apply(x, self.fc_out.bias, self.training, self.dropout.p)
+        # bias, dropout and the block's residual addition in one pass
+        return FusedBiasDropoutResidual.apply(x, self.fc_out.bias, residual, self.training, self.dropout.p)
 
 
 class GPTJBlock(nn.Module):
