@@ -147,7 +147,6 @@ __global__ __launch_bounds__(kBlockThreads) void linear_rows_kernel(
 // before its staging and barriers (the launcher says per tile where that paid).
 constexpr int kSegBytes = 32768;
 constexpr int kLdsThreads = 512; // 8 waves share one staged segment
-constexpr int kLdsWaves = kLdsThreads / kWave;
 
 template <typename T, int VEC, int MT, int R, int U, bool EARLY, int THREADS, int SEGBYTES>
 __global__ __launch_bounds__(THREADS) void linear_rows_lds_kernel(
