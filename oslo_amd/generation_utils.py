@@ -110,15 +110,20 @@ class StaticDecoder(object):
     def _capture(self, reorder):
         device = self.token.device
         pos = self.state.pos.clone()
+        beam_idx = self.beam_idx.clone()
         # warm-up on a side stream: lazy initialisation must not happen inside
-        # the capture. The warm-up steps write slots that the real steps
-        # overwrite; the position is put back afterwards.
+        # the capture. The warm-up steps really run: they write the slot of the
+        # step, which the real step writes again, and advance the position,
+        # which is put back; they reorder the caches by the identity, because
+        # the step's own reordering must be applied once, by the replay.
         side = torch.cuda.Stream(device=device)
         side.wait_stream(torch.cuda.current_stream(device))
         with torch.cuda.stream(side):
+            self.beam_idx.copy_(torch.arange(beam_idx.numel(), device=device))
             for _ in range(2):
                 self._run(reorder)
                 self.state.pos.copy_(pos)
+            self.beam_idx.copy_(beam_idx)
         torch.cuda.current_stream(device).wait_stream(side)
         torch.cuda.synchronize(device)
         graph = torch.cuda.CUDAGraph()

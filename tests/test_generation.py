@@ -159,6 +159,18 @@ def test_graphed_decoding_same_tokens(family):
         for kw in DECODING[:2]:
             assert torch.equal(model.generate(other, graph=True, **kw), model.generate(other, **kw)), kw
         assert model._kept_decoder[1] is kept
+    # the step that is captured may carry any beam permutation: it is applied once
+    from oslo_amd import DynamicDecoder, StaticDecoder
+    rows = ids.repeat_interleave(3, dim=0)
+    with torch.no_grad():
+        dyn, sta = DynamicDecoder(model, True), StaticDecoder(model, 64, True)
+        assert torch.allclose(dyn.step(rows), sta.step(rows), atol=1e-5)
+        perm = torch.tensor([2, 0, 1, 5, 3, 4], device=rows.device)
+        grown = torch.cat([rows[perm], rows[:, :1]], dim=1)
+        for _ in range(3):
+            want_logits, got_logits = dyn.step(grown, perm), sta.step(grown, perm)
+            assert torch.allclose(want_logits, got_logits, atol=1e-4)
+            grown = torch.cat([grown[perm], grown[:, :1]], dim=1)
     # the fused ban reads the growing token tensor outside the graph
     kw = dict(max_length=50, min_length=50, num_beams=3, no_repeat_ngram_size=2)
     assert torch.equal(model.generate(ids, graph=True, fused_no_repeat_ngram_blocking=True, **kw), want[1])
