@@ -258,6 +258,12 @@ class GenerationMixin(object):
         kept[1].restart()
         return kept[1]
 
+    def release_decoder(self):
+        """Drops the decoder ``generate(graph=True)`` keeps between calls (its
+        key/value buffers and captured graphs), e.g. before the model is
+        pickled or to give the memory back."""
+        self.__dict__.pop("_kept_decoder", None)
+
     @staticmethod
     def _greedy_search(ids, max_length, scores_of, eos_token_id, pad_token_id, decoder):
         unfinished = None if eos_token_id is None else torch.ones(ids.size(0), dtype=torch.bool, device=ids.device)

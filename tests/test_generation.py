@@ -174,6 +174,10 @@ def test_graphed_decoding_same_tokens(family):
     # the fused ban reads the growing token tensor outside the graph
     kw = dict(max_length=50, min_length=50, num_beams=3, no_repeat_ngram_size=2)
     assert torch.equal(model.generate(ids, graph=True, fused_no_repeat_ngram_blocking=True, **kw), want[1])
+    model.release_decoder()
+    assert "_kept_decoder" not in model.__dict__
+    assert torch.equal(model.generate(ids, graph=True, **DECODING[1]), want[1])
+    kept = model._kept_decoder[1]
     # new storage for the weights: the kept graph would read the old one, so it is dropped
     model = model.double().float()
     assert torch.equal(model.generate(ids, graph=True, **DECODING[1]), want[1])
