@@ -39,16 +39,16 @@ HBM_PEAK_GBPS = 8000.0
 # profiles/bench_kernels_hbm_traffic.md and, for the two kernels of the step,
 # profiles/causal_softmax_fp16_8x16x2048x2048_hbm_traffic.md.
 MEASURED_TRAFFIC = {
-    "linear_rows fc_in + bias + gelu bf16 1 x [16384,4096]": 134714368,
-    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135668121,
-    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134616985,
-    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136735846,
-    "linear_rows attention projection bf16 1 x [4096,4096]": 33756160,
-    "linear_rows attention projection bf16 8 x [4096,4096]": 34499584,
-    "attention_decode bf16 1 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 17570816,
-    "attention_decode bf16 8 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 136474624,
+    "linear_rows fc_in + bias + gelu bf16 1 x [16384,4096]": 134699008,
+    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135284940,
+    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134601216,
+    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136613376,
+    "linear_rows attention projection bf16 1 x [4096,4096]": 33740800,
+    "linear_rows attention projection bf16 8 x [4096,4096]": 34370560,
+    "attention_decode bf16 1 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 17573888,
+    "attention_decode bf16 8 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 136477696,
     "causal_fwd fp16 [8,16,2048,2048]": 1627472076,
-    "causal_bwd fp16 [8,16,2048,2048]": 2181120000,
+    "causal_bwd fp16 [8,16,2048,2048]": 2181120204,
     "causal_fwd bf16 [8,16,2048,2048]": 1627472076,
     "causal_bwd bf16 [8,16,2048,2048] (in place)": 2181120204,
     "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635890995,
@@ -58,15 +58,15 @@ MEASURED_TRAFFIC = {
     "causal_fwd bf16 [1,16,8192,8192]": 3229695590,
     "masked_fwd bf16 [16,16,1024,1024] key mask": 1073948672,
     "masked_bwd bf16 [16,16,1024,1024]": 1610650624,
-    "bias_gelu_fwd bf16 [16384,16384]": 1073872486,
-    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677933363,
+    "bias_gelu_fwd bf16 [16384,16384]": 1073872076,
+    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677933158,
     "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610758758,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141059584,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141059174,
     "bias_gelu_fwd bf16 [16384,4096]": 268489523,
-    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419568025,
+    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419568230,
     "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402726502,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285348249,
-    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807947468,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285348454,
+    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807983308,
     "causal_fwd bf16 [8,16,2048,2048] with padding mask": 1628013772,
     "causal_window_fwd window 256 bf16 [8,16,2048,2048]": 1230656716,
     "causal_window_bwd window 256 bf16 [8,16,2048,2048] (in place)": 1387504640,
