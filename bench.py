@@ -285,6 +285,13 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
     mask = (torch.arange(S, device=dev)[None, :] >= lens[:, None]).contiguous().view(torch.uint8)
     t = time_launches(lambda: check(lib.oslo_softmax_masked_fwd(P(y), P(x), P(mask), S, 0, 0, 0.125, B, H, S, S, BF16, st)), n, 3)
     res.append(roof("masked_fwd bf16 [16,16,1024,1024] key mask", 4 * x.numel() + mask.numel(), t, x.numel()))
+    # the same with a [B,1,Sq,Sk] mask whose query rows past the sample's length are fully masked
+    full_mask = (mask.view(B, 1, 1, S).bool() | (torch.arange(S, device=dev)[None, :] >= lens[:, None]).view(B, 1, S, 1))
+    full_mask = full_mask.contiguous().view(torch.uint8)
+    t = time_launches(lambda: check(lib.oslo_softmax_masked_fwd(P(y), P(x), P(full_mask), S * S, S, 0, 0.125, B, H, S, S, BF16, st)), n, 3)
+    res.append(roof("masked_fwd bf16 [16,16,1024,1024] full [B,1,Sq,Sk] mask, fully masked tail rows",
+                    4 * x.numel() + full_mask.numel(), t, x.numel()))
+    del full_mask
     g = randn((B, H, S, S), 1, 1.0, torch.bfloat16)
     dxm = torch.empty_like(g)
     t = time_launches(lambda: check(lib.oslo_softmax_masked_bwd(P(dxm), P(g), P(y), 0.125, B * H * S, S, BF16, st)), n, 3)
