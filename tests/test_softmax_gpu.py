@@ -195,6 +195,60 @@ def test_causal_full_size_properties(dtype):
     assert torch.count_nonzero(torch.triu(dx[::9], 1)) == 0
 
 
+def test_padded_full_size_properties():
+    """The padded benchmark configuration, bf16 [16,16,1024,1024] with valid
+    lengths uniform in [128,1024]: properties on the whole tensor, the oracle on
+    slabs; then the same scores under a [B,1,Sq,Sk] mask whose query rows past
+    the length are fully masked (additive semantics: such a row is the plain
+    softmax of its scores), forward and backward."""
+    dtype = torch.bfloat16
+    b, h, s = 16, 16, 1024
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x = (torch.randn((b, h, s, s), generator=g, device=DEV, dtype=torch.float32) * 8 ** 0.5).to(dtype)
+    g.manual_seed(2)
+    lens = torch.randint(128, 1025, (b,), generator=g, device=DEV)
+    key_mask = (torch.arange(s, device=DEV)[None, :] >= lens[:, None]).view(b, 1, 1, s)
+    y = kernels.masked_softmax_forward(x, key_mask, 0.125, kernels.MASK_ADD)
+    assert torch.count_nonzero(y * key_mask) == 0                       # masked keys get exactly 0
+    sums = y.sum(-1, dtype=torch.float32)
+    assert float((sums - 1).abs().max()) <= 1e-3 + 2.0 ** -8
+    assert torch.equal(y, kernels.masked_softmax_forward(x, key_mask, 0.125, kernels.MASK_ADD))
+    for bi, hi in [(0, 0), (9, 7), (15, 15)]:
+        want = orc.softmax_masked(f32(x[bi:bi + 1, hi:hi + 1]), key_mask[bi:bi + 1].cpu().numpy(), 0.125, "add")
+        assert_close(y[bi:bi + 1, hi:hi + 1], want, dtype, f"slab {bi},{hi}")
+        check_rowsums(y[bi:bi + 1, hi:hi + 1], dtype, want)
+    full_mask = key_mask | (torch.arange(s, device=DEV)[None, :] >= lens[:, None]).view(b, 1, s, 1)
+    yf = kernels.masked_softmax_forward(x, full_mask, 0.125, kernels.MASK_ADD)
+    bi = int(torch.argmin(lens))                                        # the sample with the longest masked tail
+    n = int(lens[bi])
+    assert torch.equal(yf[bi, :, :n], y[bi, :, :n])                     # rows inside the length: as under the key mask
+    plain = orc.softmax_masked(f32(x[bi:bi + 1, 3:4, n:]), None, 0.125, "add")
+    assert_close(yf[bi:bi + 1, 3:4, n:], plain, dtype, "fully masked rows")
+    go = torch.randn((b, h, s, s), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+    want_dx = orc.softmax_bwd(f32(go[bi, 3]), f32(yf[bi, 3]), 0.125)
+    dx = kernels.scaled_masked_softmax_backward(go, yf, 0.125)
+    assert_close(dx[bi, 3], want_dx, dtype, "bwd slab")
+    assert torch.count_nonzero(dx[bi, :, :n] * key_mask[bi]) == 0       # no gradient into masked keys
+
+
+def test_long_row_full_size_properties():
+    """The long-row benchmark configuration, bf16 [1,16,8192,8192], scale 1/16:
+    zeros above the diagonal, row sums, determinism on the whole tensor, the
+    oracle on one head."""
+    dtype = torch.bfloat16
+    h, s = 16, 8192
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x = torch.randn((1, h, s, s), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+    y = kernels.causal_softmax_forward(x, None, 1 / 16)
+    assert torch.count_nonzero(torch.triu(y[0, ::5], 1)) == 0
+    sums = y.sum(-1, dtype=torch.float32)
+    assert float((sums - 1).abs().max()) <= 1e-3 + 2.0 ** -8
+    assert torch.equal(y, kernels.causal_softmax_forward(x, None, 1 / 16))
+    want = orc.softmax_causal(f32(x[:, 11:12]), 1 / 16)
+    assert_close(y[:, 11:12], want, dtype, "head 11")
+    check_rowsums(y[:, 11:12], dtype, want)
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
 @pytest.mark.parametrize("s", [5, 64, 520, 1024, 2048, 2050, 4096])
 @pytest.mark.parametrize("with_pad", [False, True], ids=["nopad", "pad"])
