@@ -141,4 +141,49 @@ def test_random_shapes_against_torch_expressions():
             pos = torch.tensor([last], device=dev) if rng.random() < 0.5 else last
             oa = kernels.attention_decode_forward(q, kk, vv, pos, 0.2, win)
             report("attention_decode", (oa.float() - refa).abs().max().item(), tol * max(1.0, refa.abs().max().item()), (dt, bb, hh, cap, d, last, win))
+        # softmax + dropout in one pass, forward and backward (the mask is read off the output)
+        if S <= 2048:
+            p_drop = rng.choice([0.1, 0.5])
+            seed_s, off_s = rng.randint(0, 2 ** 40), 4 * rng.randint(0, 2 ** 30)
+            yd, stats = kernels.causal_softmax_dropout_forward(x, pad, scale, p_drop, seed_s, off_s)
+            plain = torch.softmax((x.float() * scale + (0 if pad is None else pad[:, None, None, :]))
+                                  .masked_fill(~(i[None, :] <= i[:, None]), float("-inf")), -1)
+            kept = yd != 0
+            report("dropout_softmax_fwd", ((yd.float() - plain * kept / (1 - p_drop)).abs()).max().item(),
+                   tol / (1 - p_drop), (dt, b, h, S, p_drop))
+            # where the mask says "kept" the probability may still have rounded to 0: use the mask of ones
+            ones_keep = kernels.bias_dropout_add_forward(torch.ones(b * h * S, S, device=dev, dtype=dt), None, None,
+                                                         p_drop, seed_s, off_s).view(b, h, S, S) != 0
+            gd = torch.randn(b, h, S, S, device=dev).to(dt)
+            gy = gd.float() * ones_keep / (1 - p_drop)
+            want_dx = scale * plain * (gy - (gy * plain).sum(-1, keepdim=True))
+            dxd = kernels.causal_softmax_dropout_backward(gd.clone(), x, stats, pad, scale, p_drop, seed_s, off_s)
+            report("dropout_softmax_bwd", (dxd.float() - want_dx).abs().max().item(),
+                   2 * tol * max(1.0, want_dx.abs().max().item()), (dt, b, h, S, p_drop))
+        # masked softmax backward and bias-dropout backward
+        gm = torch.randn(b, h, sq, sk, device=dev).to(dt)
+        ymf = ym.float()
+        want_m = scale * ymf * (gm.float() - (gm.float() * ymf).sum(-1, keepdim=True))
+        dxm = kernels.scaled_masked_softmax_backward(gm.clone(), ym, scale)
+        report("masked_bwd", (dxm.float() - want_m).abs().max().item(), tol * max(1.0, want_m.abs().max().item()),
+               (dt, b, h, sq, sk))
+        dxb, dbb = kernels.bias_dropout_add_backward(go, p, seed, off)
+        want_b = go.float() * keep / (1 - p)
+        report("bda_bwd", ((dxb.float() - want_b).abs() / want_b.abs().clamp(min=1)).max().item(), tol, (dt, rows, cols, p))
+        report("bda_dbias", ((dbb.float() - want_b.sum(0)).abs() / (want_b.abs().sum(0) + 1)).max().item(),
+               max(tol, 1e-5), (dt, rows, cols, p))
+        # rotary embedding + split heads against the torch operators
+        from oslo_amd.modeling_gptj import apply_rotary, rotary_tables
+        rb, rs, rh, rd = rng.randint(1, 3), rng.randint(1, 70), rng.randint(1, 5), rng.choice([32, 64, 128])
+        rot = rng.choice([0, 8, 16, rd])
+        roff = rng.randint(0, 20)
+        qkv = [torch.randn(rb, rs, rh, rd, device=dev).to(dt) for _ in range(3)]
+        sin, cos = rotary_tables(max(rot, 2), rs + roff, dev)
+        outs = kernels.rotary_qkv_forward(qkv[0], qkv[1], qkv[2], sin if rot else None, cos if rot else None, rot, roff)
+        for t_in, t_out, rotated in zip(qkv, outs, (True, True, False)):
+            ref = t_in.float()
+            if rotated and rot:
+                ref = torch.cat([apply_rotary(ref[..., :rot], sin, cos, roff), ref[..., rot:]], dim=-1)
+            report("rotary", (t_out.float() - ref.permute(0, 2, 1, 3)).abs().max().item(),
+                   tol * max(1.0, ref.abs().max().item()), (dt, rb, rs, rh, rd, rot, roff))
     assert not failures, failures[:5]
