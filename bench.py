@@ -207,12 +207,21 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    def section(fn, *a):
+        """A model-level section must not cost the line its kernel figures: what
+        goes wrong in one is reported in its place."""
+        try:
+            return fn(*a)
+        except Exception as e:  # noqa: BLE001
+            torch.cuda.empty_cache()
+            return {"error": f"{type(e).__name__}: {e}"[:300]}
+
     if not args.no_gptj:
-        out["gptj_fwd"] = gptj_forward(torch, dev)
-        out["gptj_train_step"] = gptj_train_step(torch, dev)
-        out["other_families_fwd"] = other_families_forward(torch, dev)
+        out["gptj_fwd"] = section(gptj_forward, torch, dev)
+        out["gptj_train_step"] = section(gptj_train_step, torch, dev)
+        out["other_families_fwd"] = section(other_families_forward, torch, dev)
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(torch)
+        out["cpu_baseline"] = cpu_baseline(torch, section)
     print(json.dumps(out))
 
 
@@ -599,7 +608,7 @@ def other_families_forward(torch, dev, reps=5):
     return res
 
 
-def cpu_baseline(torch):
+def cpu_baseline(torch, section=lambda fn, *a: fn(*a)):
     """The unfused arithmetic (scale, where(causal), softmax, autograd backward)
     with torch's CPU operators on the host cores, fp32 (CPU half softmax is not
     representative), on a bounded sample: [1,4,2048,2048] slabs of the same
@@ -629,7 +638,8 @@ def cpu_baseline(torch):
     return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": f"unfused fp32 fwd+bwd on [1,4,2048,2048] x {reps} reps, "
                       f"{dt * 1e3:.1f} ms each, bytes counted at the workload's fp16 size",
-            "gpt2_small_fwd": gpt2_small_forward(torch), "gpt2_small_generate": gpt2_small_generate(torch)}
+            "gpt2_small_fwd": section(gpt2_small_forward, torch),
+            "gpt2_small_generate": section(gpt2_small_generate, torch)}
 
 
 def gpt2_small_generate(torch):
