@@ -130,3 +130,24 @@ def test_graphed_forward_of_a_fused_model(family):
         graphed(ids[:, :50], attention_mask=mask[:, :50])
     with pytest.raises(RuntimeError, match="eval"):
         GraphedForward(model.train(), ids, attention_mask=mask)
+
+
+def test_kernels_follow_torchs_current_stream():
+    """Inside ``torch.cuda.stream(side)`` the launches go to ``side``: the
+    stream handed to the library is the one torch reports, and work queued on
+    that stream before the call (a fill of the input) is seen by the kernel."""
+    from oslo_amd import kernels
+
+    side = torch.cuda.Stream(device=DEV)
+    x = torch.zeros(4, 8, 256, 256, device=DEV, dtype=torch.float16)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        assert kernels._stream(x).value == torch.cuda.current_stream(x.device).cuda_stream == side.cuda_stream
+        for _ in range(20):                       # keep the side stream busy ahead of the fill
+            x.mul_(1.0)
+        x.fill_(3.0)                              # equal scores: every visible key gets 1 / (row + 1)
+        y = kernels.causal_softmax_forward(x, None, 1.0)
+    side.synchronize()
+    row = torch.arange(1, 257, device=DEV, dtype=torch.float32)
+    want = torch.tril(torch.ones(256, 256, device=DEV)) / row[:, None]
+    assert (y[2, 5].float() - want).abs().max() <= 2e-3
