@@ -16,6 +16,70 @@ namespace oslo {
 namespace {
 
 // ---------------------------------------------------------------------------
+// The padding-mask values of a wave's part of a causal row, as raw vectors
+// beside the row's own loads. Every wave of a [batch, heads, S, S] batch reads
+// the same mask row, and two of three vector-memory instructions of an fp16
+// row are mask loads. With STAGE, for rows of 4 vectors per lane on and at
+// least two rows per block, the mask row of the block's batch goes through LDS
+// once per block and each wave takes its part from there. Measured on fp16,
+// forward without dropout: [8,16,2048,2048] 271 -> 245 us, S=1536 181 -> 157,
+// S=4096 544 -> 504. What keeps the direct loads, also measured: shorter rows
+// (they lose to the barrier, S=1024: 66 -> 78 us), one row per block (nothing
+// is shared, S=8192: 1195 -> 1534 us), and the kernels with dropout, where
+// the Philox arithmetic hides the mask loads (S=4096: forward 552 -> 566,
+// backward 711 -> 740 us). Every thread of the block must call it (barrier).
+// ---------------------------------------------------------------------------
+template <int VEC, int NCHUNK, int WPR, bool STAGE>
+__device__ __forceinline__ void load_pad_row(RawVec<float, VEC> (&praw)[NCHUNK],
+                                             const float *__restrict__ pad,
+                                             const RowMap &map, int S, int heads,
+                                             int64_t slab, uint32_t keys, int sub,
+                                             int lane) {
+  using Tile = RowTile<VEC, NCHUNK, WPR>;
+  constexpr bool kStage = STAGE && NCHUNK * WPR >= 4 && Tile::kRowsPerBlock >= 2;
+  const int batch = (int)slab / heads;
+  auto direct = [&]() {
+    const BufRsrc prs =
+        make_rsrc(pad + (int64_t)batch * S, keys * (uint32_t)sizeof(float));
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c)
+      praw[c] = buffer_load_raw<float, VEC, false>(
+          prs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(float));
+  };
+  if constexpr (!kStage) {
+    direct();
+  } else {
+    __shared__ __align__(32) float s_pad[Tile::kMaxCols];
+    // Row slots ascend within a block: the first one names the block's batch,
+    // the last one how far its longest causal row reaches (all of the mask
+    // row if the block runs over the end of its first [S, S] slab). A wave of
+    // another batch (a block across a batch boundary) loads its own.
+    int64_t row0 = mapped_row(map, Tile::kRowsPerBlock, 0);
+    int64_t row1 = mapped_row(map, Tile::kRowsPerBlock, Tile::kRowsPerBlock - 1);
+    if (row0 >= map.total_rows) row0 = map.total_rows - 1;
+    if (row1 >= map.total_rows) row1 = map.total_rows - 1;
+    const int64_t slab0 = row0 / S;
+    const int batch0 = (int)slab0 / heads;
+    const bool staged = batch == batch0; // wave-uniform
+    const int64_t reach = row1 - slab0 * S;
+    const int top = reach >= S ? S : ((int)reach / VEC + 1) * VEC;
+    const BufRsrc srs = make_rsrc(pad + (int64_t)batch0 * S,
+                                  (uint32_t)top * (uint32_t)sizeof(float));
+    for (int i = threadIdx.x * VEC; i < top; i += kBlockThreads * VEC)
+      *reinterpret_cast<RawVec<float, VEC> *>(&s_pad[i]) =
+          buffer_load_raw<float, VEC, false>(srs, (uint32_t)i * (uint32_t)sizeof(float));
+    if (!staged) direct();
+    __syncthreads();
+    if (staged) {
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c)
+        praw[c] = *reinterpret_cast<const RawVec<float, VEC> *>(
+            &s_pad[Tile::col(c, sub, lane)]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Register-resident path: rows up to kSoftmaxMaxCols, S a multiple of VEC.
 // ---------------------------------------------------------------------------
 // DROP: what is written is y * keep / (1-p), the probabilities after attention
@@ -43,7 +107,6 @@ __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
   const int r = (int)(row - slab * S);
   const T *xr = x + row * S;
   T *yr = y + row * S;
-  const float *padr = HAS_PAD ? pad + (slab / heads) * S : nullptr;
 
   // Every load of the row is issued first (raw), conversion comes afterwards.
   // The row is bounded at the vector that holds key r: lanes wholly above the
@@ -56,13 +119,8 @@ __global__ __launch_bounds__(kBlockThreads) void causal_fwd_kernel(
   for (int c = 0; c < NCHUNK; ++c)
     raw[c] = buffer_load_raw<T, VEC, true>(
         xrs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(T));
-  if constexpr (HAS_PAD) {
-    const BufRsrc prs = make_rsrc(padr, keys * (uint32_t)sizeof(float));
-#pragma unroll
-    for (int c = 0; c < NCHUNK; ++c)
-      praw[c] = buffer_load_raw<float, VEC, false>(
-          prs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(float));
-  }
+  if constexpr (HAS_PAD)
+    load_pad_row<VEC, NCHUNK, WPR, !DROP>(praw, pad, map, S, heads, slab, keys, sub, lane);
 
   pin_loaded(raw);
   if constexpr (HAS_PAD) pin_loaded(praw);
@@ -258,14 +316,8 @@ __global__ __launch_bounds__(kBlockThreads) void causal_dropout_bwd_kernel(
     graw[c] = buffer_load_raw<T, VEC, true>(grs, off);
     xraw[c] = buffer_load_raw<T, VEC, true>(xrs, off);
   }
-  if constexpr (HAS_PAD) {
-    const BufRsrc prs =
-        make_rsrc(pad + (slab / heads) * S, keys * (uint32_t)sizeof(float));
-#pragma unroll
-    for (int c = 0; c < NCHUNK; ++c)
-      praw[c] = buffer_load_raw<float, VEC, false>(
-          prs, (uint32_t)Tile::col(c, sub, lane) * (uint32_t)sizeof(float));
-  }
+  if constexpr (HAS_PAD)
+    load_pad_row<VEC, NCHUNK, WPR, false>(praw, pad, map, S, heads, slab, keys, sub, lane);
   const float2 st = *reinterpret_cast<const float2 *>(stats + 2 * row);
   const float m = st.x, inv = st.y;
 
@@ -467,6 +519,8 @@ int launch_causal_fwd(T *y, float *stats, const T *x, const float *pad,
     // the variants with dropout (Philox) or a padding mask (its loads, and one
     // more multiply and add per key) carry more arithmetic per byte and want
     // every wave the registers allow: measured 277 -> 267 us with the mask
+    // read directly, and with the mask staged in LDS a cap at 5 or 6 blocks
+    // per CU still loses (245 -> 299 and 269 us)
     const unsigned lds = (with_dropout || pad)
                              ? 0u
                              : occupancy_pad_bytes(false, S * (int64_t)sizeof(T));
