@@ -32,6 +32,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 
 # HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` and
 # `--pmc WRITE_SIZE` (KiB per dispatch, scaled by the reading of a 1 GiB copy
@@ -386,6 +387,22 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         res.append(roof(f"attention_decode bf16 {rows} x 16 heads, 1024 of 1152 keys, head 256 (two launches)",
                         2 * 2 * rows * H * (last + 1) * D, t, rows * H * D, n_sets))
         del caches
+
+    # causal attention over a whole prompt in one kernel, at the GPT-J shape and a GPT-Neo-sized one:
+    # the one kernel here that is bound by the matrix cores (4 flops per score and feature, lower triangle)
+    import ctypes
+    for (B, Hh, S, D) in ((8, 16, 2048, 256), (8, 16, 2048, 128)):
+        q, k, v = (randn((B, Hh, S, D), 50 + i, 1.0, torch.bfloat16) for i in range(3))
+        o = torch.empty((B, S, Hh, D), dtype=torch.bfloat16, device=dev)
+        strides = (ctypes.c_int64 * 12)(*(3 * [Hh * S * D, S * D, D] + [S * Hh * D, D, Hh * D]))
+        t = time_launches(lambda: check(lib.oslo_attention_prefill_fwd(
+            P(o), P(q), P(k), P(v), None, D ** -0.5, B, Hh, S, D, strides, BF16, st)), max(5, n // 2), 3)
+        flops = 4 * B * Hh * D * (S * (S + 1) // 2)
+        res.append({"kernel": f"attention_prefill bf16 [{B},{Hh},{S},{D}] causal", "bound": "mfma",
+                    "achieved": round(flops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "us": round(t * 1e6, 1),
+                    "algorithmic_flops": flops, "traffic": None})
+        del q, k, v, o
     return res
 
 

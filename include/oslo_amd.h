@@ -396,6 +396,33 @@ int oslo_attention_decode_fwd(void *out, const void *q, void *k, void *v,
                               int64_t capacity, int64_t head_dim, int dtype,
                               oslo_stream_t stream);
 
+/*
+ * Causal attention over a whole prompt without the [S, S] matrix in memory:
+ *   out[b, h, i, :] = sum_{s <= i} softmax_s( scale * q[b,h,i,:] . k[b,h,s,:]
+ *                                             + pad[b, s] ) * v[b,h,s,:]
+ * q, k, v, out: 16-bit (OSLO_F16 or OSLO_BF16), S positions of head_dim (64,
+ * 128 or 256) contiguous features per (batch, head); strides[12] gives, in
+ * elements, the batch, head and position strides of q, k, v and out in that
+ * order, so that split heads ([B, H, S, D]), merged heads ([B, S, H, D]) and
+ * slices of a packed qkv projection are all taken where they lie (multiples
+ * of 8 elements, pointers 16-byte aligned, a (batch, head) slice under 2 GiB).
+ * pad: NULL, or an additive fp32 [batch, S] key mask (then S % 4 == 0).
+ * Products of the 16-bit inputs are accumulated in fp32, the softmax is fp32
+ * under a running maximum, the probabilities are rounded to the storage type
+ * before they multiply v (as the unfused path casts them), the sum over keys
+ * is fp32 and is normalised and rounded once at the end. No workspace.
+ * Replaces, for inference, matmul(q, k^T) -> FusedScaleMaskSoftmax.apply ->
+ * matmul(probs, v) of the fused attention
+ * (oslo/models/gptj/modeling_gptj.py:936-951,
+ *  oslo/models/gpt_neo/modeling_gpt_neo.py:993-1008,
+ *  oslo/models/gpt2/modeling_gpt2.py:1435-1459).
+ */
+int oslo_attention_prefill_fwd(void *out, const void *q, const void *k,
+                               const void *v, const float *pad, float scale,
+                               int64_t batch, int64_t heads, int64_t S,
+                               int64_t head_dim, const int64_t *strides,
+                               int dtype, oslo_stream_t stream);
+
 /* Repeated n-gram blocking (beam search) ------------------------------------ */
 
 /*

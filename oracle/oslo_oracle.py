@@ -45,6 +45,13 @@ root):
   in float64 (pinned by softmax_masked of this file composed with numpy
   matmuls, by torch.nn.functional.scaled_dot_product_attention, and by the
   closed form for equal scores: the mean of the visible values);
+* attention_prefill: the same attention for a whole prompt,
+  oslo/models/gptj/modeling_gptj.py:151-191 (scores, scale, causal where(),
+  additive padding mask, softmax, weighted sum of the values), row by row in
+  float64 (pinned by softmax_causal of this file composed with numpy matmuls,
+  by torch.nn.functional.scaled_dot_product_attention, by the closed form for
+  equal scores -- the running mean of the values -- and by attention_decode
+  on the last row);
 * build_sample_idx / build_blending_indices:
   oslo/fused_kernels/bindings/pybind_datasets.cpp:35-160 (pinned by the closed
   form "sample k starts at token k*seq_length", the share bound of the
@@ -196,6 +203,24 @@ def attention_decode(q, k, v, last, scale, window=0, dtype=np.float64):
         p = e / e.sum()
         for j, s in enumerate(range(first, last + 1)):
             out[i] += p[j] * v[i, s]
+    return out
+
+
+def attention_prefill(q, k, v, scale, pad=None, dtype=np.float64):
+    """q, k, v [n, S, d]; pad None or additive [S] / [n, S] key mask -> [n, S, d]:
+    row i attends keys 0..i."""
+    q, k, v = (np.asarray(t, dtype=dtype) for t in (q, k, v))
+    n, S, _ = q.shape
+    if pad is not None:
+        pad = np.broadcast_to(np.asarray(pad, dtype=dtype), (n, S))
+    out = np.zeros_like(q)
+    for b in range(n):
+        for i in range(S):
+            scores = scale * (k[b, :i + 1] @ q[b, i])
+            if pad is not None:
+                scores = scores + pad[b, :i + 1]
+            e = np.exp(scores - scores.max())
+            out[b, i] = (e / e.sum()) @ v[b, :i + 1]
     return out
 
 

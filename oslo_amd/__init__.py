@@ -9,6 +9,7 @@ from .fused_kernels_utils import (  # noqa: F401
     FusedBiasDropoutResidual,
     FusedBiasGeLU,
     FusedDecodeAttention,
+    FusedPrefillAttention,
     FusedKernelMixin,
     FusedLinearRows,
     FusedMergeHeads,

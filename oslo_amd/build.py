@@ -29,6 +29,7 @@ SOURCES = [
     "rotary.hip",
     "linear_rows.hip",
     "attention_decode.hip",
+    "attention_prefill.hip",
     "dataset_index.hip",
 ]
 

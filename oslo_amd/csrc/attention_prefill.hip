@@ -1,0 +1,372 @@
+// Causal attention over a whole prompt in one kernel (no [S, S] matrix in
+// memory):
+//   out[q, :] = sum_{k <= q} softmax_k(scale * Q[q, :] . K[k, :] + pad[k]) * V[k, :]
+// for every (batch, head), 16-bit inputs, fp32 accumulation. It replaces, for
+// inference, the three launches of the fused attention -- batched matmul
+// Q K^T, the fused scale + mask + softmax, batched matmul P V
+// (oslo/models/gptj/modeling_gptj.py:936-951,
+// oslo/models/gpt_neo/modeling_gpt_neo.py:993-1008,
+// oslo/models/gpt2/modeling_gpt2.py:1435-1459) -- which write the scores,
+// read and write them again in the softmax and read them a fourth time. This
+// is the one kernel of the library that is bound by the matrix cores, not by
+// HBM: 4 * S^2/2 * head_dim flops per head against 4 * S * head_dim elements.
+//
+// One block of four waves takes 128 queries of one head, 32 per wave, and walks
+// the keys in tiles of 64. Everything is computed transposed, so that a query
+// is a lane and not a register index:
+//   S^T[key, q] = K_tile (A operand, rows = keys, from LDS) x Q^T (B operand,
+//                 held in registers for the whole kernel),
+//   O^T[d, q]  += V_tile^T (A operand, rows = features, from LDS) x P^T (B).
+// In the accumulator layout of v_mfma_f32_32x32x16 a lane holds one column
+// (lane % 32 = the query) and 16 rows, so the running maximum, the sum and
+// the rescaling of O are per-lane scalars: the softmax needs one exchange
+// between the two halves of the wave per tile and no LDS. The 16 rows of a
+// lane are keys 8j + 4h + t (j, t = 0..3; h = lane / 32), and a B operand
+// wants, per half, 8 consecutive contraction slots: the probabilities are used
+// where they are, and the contraction order is permuted instead -- V^T is
+// written to LDS with key 8j + 4h + t of each group of 16 at slot 8h + 4j + t.
+// V arrives as [key][feature]; each thread transposes an 8 x 8 block in
+// registers and writes 128-bit rows of V^T. Both LDS tiles are swizzled by
+// 16-byte chunk so that the 128-bit reads of a wave (8 lanes = 8 rows at one
+// chunk) and the writes fall on different banks.
+
+#include "common.hpp"
+
+namespace oslo {
+namespace {
+
+constexpr int kQueriesPerBlock = 128;
+constexpr int kKeysPerTile = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T>
+struct MatrixOp;
+template <>
+struct MatrixOp<bf16> {
+  typedef bf16 Frag __attribute__((ext_vector_type(8)));
+  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct MatrixOp<f16> {
+  typedef f16 Frag __attribute__((ext_vector_type(8)));
+  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+struct PrefillArgs {
+  void *out;
+  const void *q, *k, *v;
+  const float *pad; // [batch, S] additive, or null
+  int64_t q_b, q_h, q_s; // element strides: batch, head, position
+  int64_t k_b, k_h, k_s;
+  int64_t v_b, v_h, v_s;
+  int64_t o_b, o_h, o_s;
+  float scale_log2e;
+  int S;
+  int heads;
+  int batch_heads;
+  int head_groups; // ceil(batch_heads / 8)
+  int query_blocks;
+};
+
+__device__ __forceinline__ float other_half(float v) {
+  return __shfl_xor(v, 32, kWave);
+}
+
+template <typename T, int D, bool HAS_PAD>
+__global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_prefill_kernel(
+    const PrefillArgs a) {
+  using Op = MatrixOp<T>;
+  using Frag = typename Op::Frag;
+  constexpr int kChunks = D / 8;   // 16-byte chunks of a key
+  constexpr int kSteps = D / 16;   // contraction steps of Q K^T
+  constexpr int kBlocksD = D / 32; // 32-row blocks of O^T
+  constexpr int kLoadsK = kKeysPerTile * kChunks / kBlockThreads; // per thread and tile
+  __shared__ __align__(16) T k_lds[kKeysPerTile * D];  // [key][chunk ^ (key & 7)][8]
+  __shared__ __align__(16) T vt_lds[D * kKeysPerTile]; // [d][(slot + d + d/8) & 7][8]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int half = lane >> 5;
+  const int col = lane & 31;
+
+  // All query blocks of a head run on one XCD (blocks go round-robin over
+  // the 8 XCDs), so its keys and values are read from HBM into one L2; the
+  // blocks with the most keys start first.
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  const int bh = xcd + 8 * (slot % a.head_groups);
+  const int qb = a.query_blocks - 1 - slot / a.head_groups;
+  if (bh >= a.batch_heads) return; // the whole block
+  const int b = bh / a.heads;
+  const int hd = bh - b * a.heads;
+  const int S = a.S;
+  const int q0 = qb * kQueriesPerBlock;
+
+  const T *qp = static_cast<const T *>(a.q) + b * a.q_b + hd * a.q_h;
+  const T *kp = static_cast<const T *>(a.k) + b * a.k_b + hd * a.k_h;
+  const T *vp = static_cast<const T *>(a.v) + b * a.v_b + hd * a.v_h;
+  // rows at or past S fall outside the descriptors and read as zeros
+  const BufRsrc qrs = make_rsrc(qp, (uint32_t)(((int64_t)(S - 1) * a.q_s + D) * sizeof(T)));
+  const BufRsrc krs = make_rsrc(kp, (uint32_t)(((int64_t)(S - 1) * a.k_s + D) * sizeof(T)));
+  const BufRsrc vrs = make_rsrc(vp, (uint32_t)(((int64_t)(S - 1) * a.v_s + D) * sizeof(T)));
+  const uint32_t q_row = (uint32_t)a.q_s * sizeof(T);
+  const uint32_t k_row = (uint32_t)a.k_s * sizeof(T);
+  const uint32_t v_row = (uint32_t)a.v_s * sizeof(T);
+
+  // Q^T as B operands: lane (query, half) holds features 16 s + 8 half .. + 7
+  const int wave_q0 = q0 + 32 * wave;
+  const int qrow = wave_q0 + col;
+  Frag qf[kSteps];
+#pragma unroll
+  for (int s = 0; s < kSteps; ++s)
+    qf[s] = __builtin_bit_cast(
+        Frag, __builtin_amdgcn_raw_buffer_load_b128(
+                  qrs, (uint32_t)qrow * q_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0));
+
+  const float *padr = HAS_PAD ? a.pad + (int64_t)b * S : nullptr;
+
+  // A tile travels global -> registers -> LDS; the loads of the next tile are
+  // in flight while this one is computed.
+  // K: thread takes chunk tid % kChunks of rows tid / kChunks + j * (256 / kChunks).
+  // V: a task is 8 keys (one contraction chunk 2u + h of the tile) x 8 features.
+  const int k_ch = tid % kChunks, k_r0 = tid / kChunks;
+  const bool v_task = tid < D;
+  const int v_g = tid % kChunks, v_kg = tid / kChunks;
+  u32x4 kreg[kLoadsK], vreg[8];
+  auto issue_loads = [&](int key0) {
+#pragma unroll
+    for (int j = 0; j < kLoadsK; ++j)
+      kreg[j] = __builtin_amdgcn_raw_buffer_load_b128(
+          krs, (uint32_t)(key0 + k_r0 + j * (kBlockThreads / kChunks)) * k_row + (uint32_t)k_ch * 16u, 0, 0);
+    if (v_task) {
+      const int kbase = key0 + 16 * (v_kg >> 1) + 4 * (v_kg & 1);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        vreg[i] = __builtin_amdgcn_raw_buffer_load_b128(
+            vrs, (uint32_t)(kbase + 8 * (i >> 2) + (i & 3)) * v_row + (uint32_t)v_g * 16u, 0, 0);
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < kLoadsK; ++j) {
+      const int row = k_r0 + j * (kBlockThreads / kChunks);
+      *reinterpret_cast<u32x4 *>(&k_lds[(row * kChunks + (k_ch ^ (row & 7))) * 8]) = kreg[j];
+    }
+    if (v_task) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { // 8 x 8 transposition of 16-bit values
+        u32x4 tr;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t lo = vreg[2 * w][e >> 1], hi = vreg[2 * w + 1][e >> 1];
+          tr[w] = (e & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+        }
+        const int d = 8 * v_g + e;
+        *reinterpret_cast<u32x4 *>(&vt_lds[(d * 8 + ((v_kg + e + v_g) & 7)) * 8]) = tr;
+      }
+    }
+  };
+
+  f32x16 o[kBlocksD];
+#pragma unroll
+  for (int i = 0; i < kBlocksD; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+  float m = -INFINITY; // running maximum of the query's scores, log2 units
+  float l = 0.f;       // this lane's share of the running sum
+
+  const int last_key = (q0 + kQueriesPerBlock < S ? q0 + kQueriesPerBlock : S) - 1;
+  const int tiles = last_key / kKeysPerTile + 1;
+  issue_loads(0);
+  for (int t = 0; t < tiles; ++t) {
+    const int key0 = t * kKeysPerTile;
+    __syncthreads(); // the reads of the previous tile are done
+    store_tile();
+    __syncthreads();
+    if (t + 1 < tiles) issue_loads(key0 + kKeysPerTile);
+
+    // the tile in two steps of 32 keys, each a step of the running softmax:
+    // the matrix products of one step are independent of the other step's
+    // exponentials
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const int keyb = key0 + 32 * kb;
+      if (keyb > wave_q0 + 31) break; // every key is ahead of the wave's queries
+
+      // S^T = K Q^T
+      f32x16 sc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+      const int key = 32 * kb + col;
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) {
+        const Frag kf = *reinterpret_cast<const Frag *>(
+            &k_lds[(key * kChunks + ((2 * s + half) ^ (key & 7))) * 8]);
+        sc = Op::run(kf, qf[s], sc);
+      }
+
+      // causal and padding mask, maximum (log2 units)
+      const bool diagonal = keyb + 31 > wave_q0;
+      float mt = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int kj = keyb + 8 * j + 4 * half;
+        float pv[4] = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (HAS_PAD) {
+          // keys at or past S only meet queries they are masked for
+          const float4 p4 = *reinterpret_cast<const float4 *>(padr + (kj < S ? kj : 0));
+          pv[0] = p4.x * kLog2e, pv[1] = p4.y * kLog2e, pv[2] = p4.z * kLog2e, pv[3] = p4.w * kLog2e;
+        }
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+          float x = sc[4 * j + tt] * a.scale_log2e;
+          if constexpr (HAS_PAD) x += pv[tt];
+          if (diagonal) x = kj + tt <= qrow ? x : -INFINITY;
+          sc[4 * j + tt] = x;
+          mt = fmaxf(mt, x);
+        }
+      }
+      mt = fmaxf(mt, other_half(mt));
+      // key 0 is visible to every query, so the maximum is finite from the
+      // first step on
+      const float m_new = fmaxf(m, mt);
+      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+      m = m_new;
+      float sum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        sc[r] = __builtin_amdgcn_exp2f(sc[r] - m_new);
+        sum += sc[r];
+      }
+      l = l * alpha + sum;
+      if (__any(alpha != 1.0f)) { // wave-uniform: later steps seldom raise the maximum
+#pragma unroll
+        for (int i = 0; i < kBlocksD; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
+      }
+
+      // P^T as B operands, in the storage type like the unfused path's cast
+      Frag pf[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pf[u][i] = static_cast<T>(sc[8 * u + i]);
+
+      // O^T += V^T P^T
+#pragma unroll
+      for (int i = 0; i < kBlocksD; ++i) {
+        const int d = 32 * i + col;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const Frag vf = *reinterpret_cast<const Frag *>(
+              &vt_lds[(d * 8 + ((4 * kb + 2 * u + half + d + (d >> 3)) & 7)) * 8]);
+          o[i] = Op::run(vf, pf[u], o[i]);
+        }
+      }
+    }
+  }
+
+  l += other_half(l);
+  const float inv = 1.0f / l;
+  if (qrow >= S) return;
+  T *op = static_cast<T *>(a.out) + b * a.o_b + hd * a.o_h + (int64_t)qrow * a.o_s;
+  typedef T Out4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+  for (int i = 0; i < kBlocksD; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      Out4 w;
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(o[i][4 * j + tt] * inv);
+      *reinterpret_cast<Out4 *>(op + 32 * i + 8 * j + 4 * half) = w;
+    }
+}
+
+template <typename T, int D>
+void launch_prefill_dim(const PrefillArgs &a, hipStream_t stream) {
+  const dim3 grid((unsigned)(8 * a.head_groups * a.query_blocks));
+  if (a.pad != nullptr)
+    attention_prefill_kernel<T, D, true><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  else
+    attention_prefill_kernel<T, D, false><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+}
+
+template <typename T>
+int launch_prefill(const PrefillArgs &a, int head_dim, hipStream_t stream) {
+  switch (head_dim) {
+    case 64: launch_prefill_dim<T, 64>(a, stream); break;
+    case 128: launch_prefill_dim<T, 128>(a, stream); break;
+    default: launch_prefill_dim<T, 256>(a, stream); break;
+  }
+  return check_launch("attention_prefill_fwd");
+}
+
+} // namespace
+} // namespace oslo
+
+extern "C" int oslo_attention_prefill_fwd(void *out, const void *q, const void *k,
+                                          const void *v, const float *pad,
+                                          float scale, int64_t batch, int64_t heads,
+                                          int64_t S, int64_t head_dim,
+                                          const int64_t *strides, int dtype,
+                                          oslo_stream_t stream) {
+  using namespace oslo;
+  if (batch < 0 || heads < 0 || S < 0 || head_dim < 0)
+    return fail(OSLO_E_BAD_ARG, "oslo_attention_prefill_fwd: negative size");
+  if (dtype != OSLO_F16 && dtype != OSLO_BF16) {
+    if (dtype == OSLO_F32)
+      return fail(OSLO_E_UNSUPPORTED, "oslo_attention_prefill_fwd: fp16 and bf16 are taken, not fp32");
+    return fail(OSLO_E_BAD_ARG, "unknown dtype %d", dtype);
+  }
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+    return fail(OSLO_E_UNSUPPORTED,
+                "oslo_attention_prefill_fwd: heads of %lld features (64, 128 or 256 are taken)",
+                (long long)head_dim);
+  if (batch == 0 || heads == 0 || S == 0) return OSLO_OK;
+  if (!out || !q || !k || !v || !strides)
+    return fail(OSLO_E_BAD_ARG, "oslo_attention_prefill_fwd: null pointer");
+  if (batch * heads > (int64_t)0x7fffffff / 8)
+    return fail(OSLO_E_UNSUPPORTED, "oslo_attention_prefill_fwd: too many heads for one launch");
+  const void *ptrs[4] = {q, k, v, out};
+  for (int i = 0; i < 4; ++i) {
+    if (!aligned16(ptrs[i]))
+      return fail(OSLO_E_UNSUPPORTED, "oslo_attention_prefill_fwd: tensors must be 16-byte aligned");
+    const int64_t sb = strides[3 * i], sh = strides[3 * i + 1], ss = strides[3 * i + 2];
+    if (sb < 0 || sh < 0 || ss < head_dim || sb % 8 || sh % 8 || ss % 8)
+      return fail(OSLO_E_UNSUPPORTED,
+                  "oslo_attention_prefill_fwd: strides must be multiples of 8 elements, "
+                  "the position stride at least head_dim");
+    // byte offsets inside one (batch, head) slice are 32-bit
+    if ((S + kQueriesPerBlock) * ss * 2 > (int64_t)0x7fffffff)
+      return fail(OSLO_E_UNSUPPORTED, "oslo_attention_prefill_fwd: a head's slice exceeds 2 GiB");
+  }
+  if (pad != nullptr && (S % 4 != 0 || !aligned16(pad)))
+    return fail(OSLO_E_UNSUPPORTED,
+                "oslo_attention_prefill_fwd: with a padding mask S must be a multiple of 4 and the mask 16-byte aligned");
+  PrefillArgs a;
+  a.out = out, a.q = q, a.k = k, a.v = v, a.pad = pad;
+  a.q_b = strides[0], a.q_h = strides[1], a.q_s = strides[2];
+  a.k_b = strides[3], a.k_h = strides[4], a.k_s = strides[5];
+  a.v_b = strides[6], a.v_h = strides[7], a.v_s = strides[8];
+  a.o_b = strides[9], a.o_h = strides[10], a.o_s = strides[11];
+  a.scale_log2e = scale * kLog2e;
+  a.S = (int)S;
+  a.heads = (int)heads;
+  a.batch_heads = (int)(batch * heads);
+  a.head_groups = (a.batch_heads + 7) / 8;
+  a.query_blocks = (int)((S + kQueriesPerBlock - 1) / kQueriesPerBlock);
+  if ((int64_t)8 * a.head_groups * a.query_blocks > (int64_t)0x7fffffff)
+    return fail(OSLO_E_UNSUPPORTED, "oslo_attention_prefill_fwd: too many blocks for one launch");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == OSLO_F16) return launch_prefill<f16>(a, (int)head_dim, st);
+  return launch_prefill<bf16>(a, (int)head_dim, st);
+}

@@ -412,6 +412,8 @@ class FusedMergeHeads(object):
         b, h, s, d = x.shape
         if s == 1 and x.is_contiguous():  # one position: the permute moves nothing
             return x.view(b, 1, h * d)
+        if x.stride() == (s * h * d, d, h * d, 1):  # [B, S, H, D] memory already (FusedPrefillAttention)
+            return x.permute(0, 2, 1, 3).view(b, s, h * d)
         if not _needs_grad(x):
             return get_custom_kernels().rotary_qkv_backward(None, None, x, None, None, 0)[2].view(b, s, h * d)
         return _MergeHeads.apply(x).view(b, s, h * d)
@@ -533,6 +535,49 @@ class FusedDecodeAttention(object):
         scale = 1.0 if scale is None else scale
         return get_custom_kernels().attention_decode_forward(query, key, value, pos, scale, window or 0,
                                                              new_key, new_value)
+
+
+class FusedPrefillAttention(object):
+    """
+    Kernel fusion function: causal attention over a whole prompt
+
+    Before fusion: Matmul (Q * K^T) -> (Scale + Mask + Softmax) -> Matmul (Score * V)
+    After fusion: one kernel on the matrix cores; the [S, S] scores stay on chip
+
+    Not in the reference, whose fused attention keeps both matmuls around the
+    softmax kernel (oslo/models/gptj/modeling_gptj.py:936-951). ``apply`` takes
+    query, key and value as [B, H, S, D] (views with any strides), the model's
+    additive padding mask [B, 1, 1, S] or None, and the scale; it returns the
+    attention output shaped [B, H, S, D] over [B, S, H, D] memory, which
+    ``FusedMergeHeads`` turns into [B, S, H*D] without a copy. Inference only
+    (no backward, no attention dropout, no probabilities to return), fp16 and
+    bf16, heads of 64, 128 or 256 features.
+    """
+
+    MIN_LENGTH = 128  # shorter prompts: the three launches are as fast
+
+    @staticmethod
+    def is_available(query, key, attention_mask=None, training=False, dropout_p=0.0):
+        if not (query.is_cuda and query.dim() == 4 and key.dim() == 4 and key.shape == query.shape):
+            return False
+        if query.dtype not in (torch.half, torch.bfloat16) or key.dtype != query.dtype:
+            return False
+        if training and dropout_p > 0.0:
+            return False
+        b, _, s, d = query.shape
+        if d not in (64, 128, 256) or s < FusedPrefillAttention.MIN_LENGTH or s * d * query.element_size() >= 2 ** 30:
+            return False
+        if attention_mask is not None and not (
+                s % 4 == 0 and attention_mask.is_floating_point() and attention_mask.numel() == b * s
+                and tuple(attention_mask.shape) in ((b, 1, 1, s), (b, s))):
+            return False
+        return not _needs_grad(query, key)
+
+    @staticmethod
+    def apply(query, key, value, attention_mask=None, scale=None):
+        b, _, s, _ = query.shape
+        pad = None if attention_mask is None else attention_mask.reshape(b, s).float()
+        return get_custom_kernels().attention_prefill_forward(query, key, value, 1.0 if scale is None else scale, pad)
 
 
 class FusedLinearRows(object):

@@ -576,6 +576,51 @@ def attention_decode_forward(query, key, value, pos, scale, window=0, new_key=No
     return out
 
 
+PREFILL_HEAD_DIMS = (64, 128, 256)
+
+
+def attention_prefill_forward(query, key, value, scale, pad=None):
+    """Causal attention of a whole prompt in one kernel: query, key, value
+    [B, H, S, D] fp16/bf16 views (features contiguous, any batch/head/position
+    strides that are multiples of 8 elements), ``pad`` an optional additive
+    fp32 [B, S] key mask. Returns softmax(scale * q k^T + causal + pad) v,
+    shaped [B, H, S, D] over [B, S, H, D] memory, so that merging the heads
+    afterwards moves nothing (oslo/models/gptj/modeling_gptj.py:936-951 and
+    the ``_merge_heads`` that follows it). The [S, S] scores never reach memory."""
+    _device_tensor(query, "query")
+    _device_tensor(key, "key", query)
+    _device_tensor(value, "value", query)
+    code = _dtype_code(query, "query")
+    _require(query.dtype in (torch.float16, torch.bfloat16), "attention_prefill: fp16 or bf16 tensors")
+    _require(query.dim() == 4 and key.shape == query.shape and value.shape == query.shape,
+             "query, key and value must be [B, H, S, D] alike")
+    _require(key.dtype == query.dtype and value.dtype == query.dtype, "query, key and value differ in dtype")
+    b, h, s, d = query.shape
+    _require(d in PREFILL_HEAD_DIMS, f"attention_prefill: heads of {d} features (64, 128 or 256 are taken)")
+
+    def strided(t):
+        ok = t.stride(3) == 1 and all(st % 8 == 0 for st in t.stride()[:3]) and t.data_ptr() % 16 == 0 \
+            and (s == 1 or t.stride(2) >= d)
+        return t if ok else t.contiguous()
+
+    q, k, v = strided(query), strided(key), strided(value)
+    if pad is not None:
+        _device_tensor(pad, "pad", query)
+        _require(pad.dtype == torch.float32 and tuple(pad.shape) == (b, s), "pad must be fp32 [B, S]")
+        _require(s % 4 == 0, "attention_prefill: with a padding mask S must be a multiple of 4")
+        pad = pad.contiguous()
+    out = torch.empty((b, s, h, d), dtype=query.dtype, device=query.device).permute(0, 2, 1, 3)
+    if out.numel() == 0:
+        return out
+    strides = (ctypes.c_int64 * 12)()
+    for i, t in enumerate((q, k, v, out)):
+        strides[3 * i], strides[3 * i + 1], strides[3 * i + 2] = t.stride(0), t.stride(1), t.stride(2)
+    with _on_device(q):
+        _lib.check(_lib.load().oslo_attention_prefill_fwd(
+            _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(pad), float(scale), b, h, s, d, strides, code, _stream(q)))
+    return out
+
+
 def rotary_qkv_forward(query, key, value, sin, cos, rotary_dim, offset=0):
     """query, key, value: [B, S, H, D] (any may be None); sin, cos: fp32
     [positions, rotary_dim/2]. Returns the three tensors as [B, H, S, D], query

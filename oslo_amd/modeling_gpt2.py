@@ -14,7 +14,7 @@ import torch
 from torch import nn
 
 from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedBiasDropoutResidual,
-                                 FusedDecodeAttention, FusedLinearRows,
+                                 FusedDecodeAttention, FusedLinearRows, FusedPrefillAttention,
                                  FusedMergeHeads,
                                  FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedSplitHeads)
@@ -192,11 +192,18 @@ class FusedGPT2Attention(GPT2Attention):
             layer_past.flush()
         if static and not one_pass:
             attention_mask = static_cache_mask(layer_past, attention_mask, fused)
+        prompt = (causal and not static and head_mask is None and not output_attentions
+                  and FusedPrefillAttention.is_available(query, key, attention_mask, self.training,
+                                                         self.attn_dropout.p))
         if one_pass:
             # a decoding step: scores, softmax and weighted sum in one pass over the cache
             out = FusedDecodeAttention.apply(query, key, value, layer_past.state.pos if static else sk - 1,
                                              self._attention_scale(value), None, *fresh)
             w = None
+        elif prompt:
+            # a whole prompt at inference: one kernel, the scores stay on chip
+            out, w = FusedPrefillAttention.apply(query, key, value, attention_mask,
+                                                 self._attention_scale(value)), None
         elif fused:
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)
         else:

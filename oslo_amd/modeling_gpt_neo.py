@@ -17,7 +17,7 @@ import torch
 from torch import nn
 
 from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedBiasDropoutResidual,
-                                 FusedDecodeAttention, FusedLinearRows,
+                                 FusedDecodeAttention, FusedLinearRows, FusedPrefillAttention,
                                  FusedMergeHeads,
                                  FusedRotaryPositionEmbedding, FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedScaleMaskWindowSoftmax)
@@ -169,12 +169,19 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
             layer_past.flush()
         if static and not one_pass:
             attention_mask = static_cache_mask(layer_past, attention_mask, fused, window=self._window())
+        prompt = (causal and sq > 1 and not isinstance(self, GPTNeoLocalSelfAttention) and head_mask is None
+                  and not output_attentions
+                  and FusedPrefillAttention.is_available(query, key, attention_mask, self.training,
+                                                         self.attn_dropout.p))
         if one_pass:
             # a decoding step: scores, softmax and weighted sum in one pass over the
             # cache, the window of a local layer included
             out = FusedDecodeAttention.apply(query, key, value, layer_past.state.pos if static else sk - 1,
                                              None, self._window(), *fresh)
             w = None
+        elif prompt:
+            # a whole prompt at inference (global layers): one kernel, the scores stay on chip
+            out, w = FusedPrefillAttention.apply(query, key, value, attention_mask, None), None
         elif fused and static:
             out, w = FusedGPTNeoSelfAttention._fused_attn(self, query, key, value, attention_mask, head_mask, False)
         elif fused:

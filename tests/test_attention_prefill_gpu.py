@@ -1,0 +1,146 @@
+"""Causal attention over a whole prompt in one kernel, called through the C
+ABI, against the CPU oracle in float64 (small cases) and against the same
+formula in float64 on the device (large ones). Tolerance: the result is an fp32
+sum rounded once to the storage type (at most REL * |ref|, REL = 2^-8 for bf16,
+2^-11 for fp16), and the probabilities are rounded to the storage type before
+they multiply the values, as the unfused path casts them (at most REL * max|v|
+over a row, whose probabilities sum to one):
+|err| <= REL * (|ref| + max|v|) + 1e-4."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oslo_oracle as orc
+from oslo_amd import FusedMergeHeads, FusedPrefillAttention, kernels
+from tests.util import IDS, f32, randn
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+HALVES = [torch.float16, torch.bfloat16]
+REL = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}
+
+
+def device_reference(q, k, v, scale, pad=None):
+    q, k, v = q.double(), k.double(), v.double()
+    s = q.shape[2]
+    w = q @ k.transpose(-1, -2) * scale
+    if pad is not None:
+        w = w + pad.double()[:, None, None, :]
+    w = w.masked_fill(torch.ones(s, s, device=q.device, dtype=torch.bool).triu(1), float("-inf"))
+    return torch.softmax(w, -1) @ v
+
+
+def check(out, want, dtype, what, vmax=4.0):
+    """``vmax``: the largest value magnitude (4.0 covers the unit-normal inputs here)."""
+    out, want = out.double(), want.double() if isinstance(want, torch.Tensor) else torch.from_numpy(want).to(out.device)
+    excess = ((out - want).abs() - REL[dtype] * (want.abs() + vmax)).max().item()
+    assert excess <= 1e-4, (excess, what)
+
+
+def padding(b, s, seed):
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.randint(max(1, s // 2), s + 1, (b,), generator=g)
+    return torch.where(torch.arange(s)[None, :] < lens[:, None], 0.0, -10000.0).float()
+
+
+# prompts shorter than a key tile, ragged against the 64-key tiles and the 128-query blocks, several blocks
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+@pytest.mark.parametrize("d", [64, 128, 256])
+@pytest.mark.parametrize("s", [1, 8, 63, 64, 65, 128, 200, 332])
+def test_prefill_matches_oracle(s, d, dtype):
+    b, h = 2, 3
+    q, k, v = (randn((b, h, s, d), dtype, seed=7 * s + i) for i in range(3))
+    scale = 1.0 / math.sqrt(d)
+    out = kernels.attention_prefill_forward(q.to(DEV), k.to(DEV), v.to(DEV), scale)
+    assert out.shape == (b, h, s, d) and out.dtype == dtype
+    assert out.permute(0, 2, 1, 3).is_contiguous()  # merged-heads memory
+    want = orc.attention_prefill(f32(q).reshape(b * h, s, d), f32(k).reshape(b * h, s, d),
+                                 f32(v).reshape(b * h, s, d), scale).reshape(b, h, s, d)
+    check(out, want, dtype, (s, d))
+    if s % 4 == 0:
+        pad = padding(b, s, s)
+        out = kernels.attention_prefill_forward(q.to(DEV), k.to(DEV), v.to(DEV), scale, pad.to(DEV))
+        want = orc.attention_prefill(f32(q).reshape(b * h, s, d), f32(k).reshape(b * h, s, d),
+                                     f32(v).reshape(b * h, s, d), scale,
+                                     pad.numpy().repeat(h, axis=0)).reshape(b, h, s, d)
+        check(out, want, dtype, (s, d, "pad"))
+
+
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+@pytest.mark.parametrize("b,h,s,d", [(2, 16, 1024, 64), (1, 9, 1000, 128), (2, 4, 2048, 256), (1, 2, 4100, 128)])
+def test_prefill_long_prompts(b, h, s, d, dtype):
+    q, k, v = (randn((b, h, s, d), dtype, seed=s + i).to(DEV) for i in range(3))
+    pad = padding(b, s, 3).to(DEV)
+    for p in (None, pad):
+        out = kernels.attention_prefill_forward(q, k, v, 0.1, p)
+        check(out, device_reference(q, k, v, 0.1, p), dtype, (b, h, s, d, p is not None))
+
+
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+def test_prefill_large_scores_and_size_independent_properties(dtype):
+    """Scores of several hundred (the maximum is subtracted in fp32: nothing
+    overflows); row 0 is the first value; equal scores give the running mean
+    of the values; the output is linear in the values."""
+    b, h, s, d = 1, 4, 512, 128
+    q, k, v = (randn((b, h, s, d), dtype, seed=20 + i).to(DEV) for i in range(3))
+    out = kernels.attention_prefill_forward(q * 6, k * 6, v, 1.0)
+    assert torch.isfinite(out).all()
+    check(out, device_reference(q * 6, k * 6, v, 1.0), dtype, "large scores")
+    assert torch.equal(out[:, :, 0], v[:, :, 0])
+    flat = kernels.attention_prefill_forward(torch.zeros_like(q), k, v, 1.0)
+    mean = v.double().cumsum(2) / torch.arange(1, s + 1, device=DEV)[None, None, :, None]
+    check(flat, mean, dtype, "running mean")
+    two = kernels.attention_prefill_forward(q, k, v * 2, 0.1)
+    one = kernels.attention_prefill_forward(q, k, v, 0.1)
+    if dtype == torch.bfloat16:
+        assert torch.equal(two, one * 2)  # a power of two: exact
+    else:  # fp16 values under 2^-14 are subnormal and their doubles are not: equal to an ulp
+        assert torch.allclose(two.float(), one.float() * 2, rtol=2.0 ** -10, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+def test_prefill_takes_strided_views(dtype):
+    """Merged-heads memory ([B, S, H, D] viewed as [B, H, S, D]) and the slices of
+    a packed q|k|v projection are read where they lie."""
+    b, h, s, d = 2, 4, 160, 64
+    packed = randn((b, s, 3 * h * d), dtype, seed=5).to(DEV)
+    q, k, v = (packed[:, :, i * h * d:(i + 1) * h * d].view(b, s, h, d).permute(0, 2, 1, 3) for i in range(3))
+    assert not q.is_contiguous()
+    out = kernels.attention_prefill_forward(q, k, v, 0.125)
+    want = kernels.attention_prefill_forward(q.contiguous(), k.contiguous(), v.contiguous(), 0.125)
+    assert torch.equal(out, want)
+    check(out, device_reference(q, k, v, 0.125), dtype, "strided")
+    merged = FusedMergeHeads.apply(out)
+    assert merged.shape == (b, s, h * d) and merged.data_ptr() == out.data_ptr()  # no copy
+    assert torch.equal(merged, out.permute(0, 2, 1, 3).reshape(b, s, h * d))
+
+
+def test_prefill_operator_gate_and_errors():
+    q = randn((1, 2, 256, 64), torch.float16, seed=1).to(DEV)
+    mask = padding(1, 256, 1).to(DEV).view(1, 1, 1, 256).half()
+    assert FusedPrefillAttention.is_available(q, q)
+    assert FusedPrefillAttention.is_available(q, q, mask)
+    assert not FusedPrefillAttention.is_available(q, q, training=True, dropout_p=0.1)
+    assert not FusedPrefillAttention.is_available(q.float(), q.float())
+    assert not FusedPrefillAttention.is_available(q[:, :, :64], q[:, :, :64])      # short prompt
+    assert not FusedPrefillAttention.is_available(q[:, :, :128], q)                # a cache longer than the prompt
+    assert not FusedPrefillAttention.is_available(q[..., :32], q[..., :32])        # head size
+    assert not FusedPrefillAttention.is_available(q.requires_grad_(), q)
+    q = q.detach()
+    out = FusedPrefillAttention.apply(q, q, q, mask, 0.125)
+    check(out, device_reference(q, q, q, 0.125, mask.view(1, 256).float()), torch.float16, "operator")
+    with pytest.raises(RuntimeError):
+        kernels.attention_prefill_forward(q.float(), q.float(), q.float(), 1.0)
+    with pytest.raises(RuntimeError):
+        kernels.attention_prefill_forward(q[..., :32], q[..., :32], q[..., :32], 1.0)
+    with pytest.raises(RuntimeError):
+        kernels.attention_prefill_forward(q, q[:, :, :128], q, 1.0)
+    with pytest.raises(RuntimeError):
+        kernels.attention_prefill_forward(q[:, :, :254], q[:, :, :254], q[:, :, :254], 1.0,
+                                          torch.zeros(1, 254, device=DEV))
+    empty = kernels.attention_prefill_forward(q[:0], q[:0], q[:0], 1.0)
+    assert empty.shape == (0, 2, 256, 64)

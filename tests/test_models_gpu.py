@@ -56,6 +56,52 @@ def test_fused_model_matches_unfused(family, dtype, padded):
 
 
 @pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("padded", [False, True], ids=["nopad", "pad"])
+def test_prompt_attention_runs_as_one_kernel_at_inference(family, dtype, padded, monkeypatch):
+    """Heads of 64 features and a prompt of 160 tokens, no gradient: the fused
+    attention takes the one-kernel prompt attention (GPT-Neo's local layer keeps
+    its window kernel), the logits match the unfused model's, and the cache it
+    returns continues into a decoding step like the unfused one's."""
+    big = {
+        "gpt2": lambda: GPT2LMHeadModel(GPT2Config(vocab_size=512, n_positions=256, n_embd=256, n_layer=2, n_head=4,
+                                                   resid_pdrop=0.0, embd_pdrop=0.0, attn_pdrop=0.0)),
+        "gptj": lambda: GPTJForCausalLM(GPTJConfig(vocab_size=512, n_positions=256, n_embd=256, n_layer=2, n_head=4,
+                                                   rotary_dim=16)),
+        "gpt_neo": lambda: GPTNeoForCausalLM(GPTNeoConfig(vocab_size=512, max_position_embeddings=256,
+                                                          hidden_size=256, num_layers=2, num_heads=4, window_size=32)),
+    }
+    torch.manual_seed(0)
+    m = big[family]().to(DEV, dtype).eval()
+    ids = torch.randint(0, 512, (3, 160), device=DEV)
+    mask = None
+    if padded:
+        mask = torch.ones(3, 160, device=DEV)
+        mask[1, 100:] = 0
+        mask[2, 17:] = 0
+    calls = []
+    real = fku.FusedPrefillAttention.apply
+    monkeypatch.setattr(fku.FusedPrefillAttention, "apply",
+                        staticmethod(lambda *a: (calls.append(tuple(a[0].shape)), real(*a))[1]))
+    with torch.no_grad():
+        want = m(ids, attention_mask=mask, use_cache=True)
+        step_mask = None if mask is None else torch.cat([mask, torch.ones(3, 1, device=DEV)], dim=1)
+        want_step = m(ids[:, :1], attention_mask=step_mask, past_key_values=want["past_key_values"])["logits"]
+        m.fuse()
+        got = m(ids, attention_mask=mask, use_cache=True)
+        got_step = m(ids[:, :1], attention_mask=step_mask, past_key_values=got["past_key_values"])["logits"]
+    assert calls == [(3, 4, 160, 64)] * (1 if family == "gpt_neo" else 2)
+    keep = torch.ones(3, 160, dtype=torch.bool, device=DEV) if mask is None else mask.bool()
+    err = (got["logits"].float() - want["logits"].float()).abs()[keep].max().item()
+    assert err <= LOGIT_TOL[dtype], f"{family} {dtype}: logits differ by {err}"
+    assert (got_step.float() - want_step.float()).abs().max().item() <= LOGIT_TOL[dtype]
+    # with gradients recorded the three-launch path (which has a backward) is taken
+    calls.clear()
+    m(ids, attention_mask=mask)
+    assert calls == []
+
+
+@pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
 def test_partial_fusion_selections_compute_the_same(family):
     """Attention and MLP only (the reference's selection), a fused block over an
     unfused attention, and everything: the same logits within fp32 rounding,

@@ -427,6 +427,35 @@ def test_linear_rows_against_loops_and_library():
     assert orc.linear_rows(x, w, b).shape == (3, 5)
 
 
+def test_attention_prefill_against_library_and_closed_form():
+    rng = np.random.default_rng(10)
+    n, S, d = 2, 11, 8
+    q, k, v = (rng.standard_normal((n, S, d)) for _ in range(3))
+    pad = np.where(rng.random((n, S)) < 0.3, -10000.0, 0.0)
+    pad[:, 0] = 0.0
+    got = orc.attention_prefill(q, k, v, 0.3)
+    tq, tk, tv = (torch.from_numpy(t) for t in (q, k, v))
+    want = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, is_causal=True, scale=0.3).numpy()
+    assert np.allclose(got, want, atol=1e-12)
+    # with the additive key mask: torch's attention given causal + padding as one float mask
+    causal = np.where(np.arange(S)[None, :] > np.arange(S)[:, None], -np.inf, 0.0)
+    mask = torch.from_numpy(causal[None] + pad[:, None, :])
+    want = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, attn_mask=mask, scale=0.3).numpy()
+    got_pad = orc.attention_prefill(q, k, v, 0.3, pad)
+    assert np.allclose(got_pad, want, atol=1e-9)
+    # this file's causal softmax composed with matmuls
+    scores = np.einsum("nid,njd->nij", q, k)[:, None]
+    probs = orc.softmax_causal(scores, 0.3, pad_add=pad, dtype=np.float64)[:, 0]
+    assert np.allclose(got_pad, np.einsum("nij,njd->nid", probs, v), atol=1e-9)
+    # equal scores: the running mean of the values; the last row is a decoding step
+    flat = orc.attention_prefill(np.zeros((n, S, d)), k, v, 1.0)
+    assert np.allclose(flat, np.cumsum(v, axis=1) / np.arange(1, S + 1)[None, :, None], atol=1e-12)
+    assert np.allclose(got[:, -1], orc.attention_decode(q[:, -1], k, v, S - 1, 0.3), atol=1e-12)
+    # a dropped scale, a transposed operand or an off-by-one diagonal would fail the above; so does
+    # attending the future: row 0 is exactly the first value
+    assert np.allclose(got[:, 0], v[:, 0], atol=1e-12)
+
+
 def test_attention_decode_against_library_and_closed_form():
     rng = np.random.default_rng(9)
     n, cap, d, last = 3, 12, 8, 7
