@@ -407,7 +407,7 @@ int oslo_attention_decode_fwd(void *out, const void *q, void *k, void *v,
  * slices of a packed qkv projection are all taken where they lie (multiples
  * of 8 elements, pointers 16-byte aligned, a (batch, head) slice under 2 GiB).
  * pad: NULL, or an additive fp32 [batch, S] key mask (then S % 4 == 0).
- * Products of the 16-bit inputs are accumulated in fp32, the softmax is fp32
+ * scale > 0. Products of the 16-bit inputs are accumulated in fp32, the softmax is fp32
  * under a running maximum, the probabilities are rounded to the storage type
  * before they multiply v (as the unfused path casts them), the sum over keys
  * is fp32 and is normalised and rounded once at the end. No workspace.

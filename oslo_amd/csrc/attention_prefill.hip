@@ -38,6 +38,7 @@ namespace {
 constexpr int kQueriesPerBlock = 128;
 constexpr int kKeysPerTile = 64;
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kSlack = 8.0f; // see the kernel: how far a score may exceed the reference maximum
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -213,7 +214,9 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
         sc = Op::run(kf, qf[s], sc);
       }
 
-      // causal and padding mask, maximum (log2 units)
+      // Causal and padding mask, maximum. Without a padding mask the scores
+      // stay raw: the scale (positive) commutes with the maximum and goes
+      // into the exponent's multiply-add.
       const bool diagonal = keyb + 31 > wave_q0;
       float mt = -INFINITY;
 #pragma unroll
@@ -227,32 +230,43 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
         }
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
-          float x = sc[4 * j + tt] * a.scale_log2e;
-          if constexpr (HAS_PAD) x += pv[tt];
+          float x = sc[4 * j + tt];
+          if constexpr (HAS_PAD) x = x * a.scale_log2e + pv[tt];
           if (diagonal) x = kj + tt <= qrow ? x : -INFINITY;
           sc[4 * j + tt] = x;
           mt = fmaxf(mt, x);
         }
       }
+      if constexpr (!HAS_PAD) mt *= a.scale_log2e;
       mt = fmaxf(mt, other_half(mt));
-      // key 0 is visible to every query, so the maximum is finite from the
-      // first step on
-      const float m_new = fmaxf(m, mt);
-      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
-      m = m_new;
-      float sum = 0.f;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        sc[r] = __builtin_amdgcn_exp2f(sc[r] - m_new);
-        sum += sc[r];
-      }
-      l = l * alpha + sum;
-      if (__any(alpha != 1.0f)) { // wave-uniform: later steps seldom raise the maximum
+      // The reference maximum m only follows the scores when they exceed it by
+      // more than kSlack (log2 units): exponentials up to 2^kSlack are as exact
+      // as those up to 1 in fp32, fp16 and bf16, and the softmax does not
+      // depend on the shift. Rescaling O costs as much as the softmax of a
+      // step, and with an exact running maximum some query of a wave raises it
+      // in most steps; with the slack it happens in the first steps only.
+      // Key 0 is visible to every query: m is finite after the first step.
+      const bool raise = mt > m + kSlack; // true in the first step (m = -inf)
+      if (__any(raise)) { // wave-uniform
+        const float m_new = raise ? mt : m;
+        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+        m = m_new;
+        l *= alpha;
 #pragma unroll
         for (int i = 0; i < kBlocksD; ++i)
 #pragma unroll
           for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
       }
+      float sum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        if constexpr (HAS_PAD)
+          sc[r] = __builtin_amdgcn_exp2f(sc[r] - m);
+        else
+          sc[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[r], a.scale_log2e, -m));
+        sum += sc[r];
+      }
+      l += sum;
 
       // P^T as B operands, in the storage type like the unfused path's cast
       Frag pf[2];
@@ -331,6 +345,8 @@ extern "C" int oslo_attention_prefill_fwd(void *out, const void *q, const void *
     return fail(OSLO_E_UNSUPPORTED,
                 "oslo_attention_prefill_fwd: heads of %lld features (64, 128 or 256 are taken)",
                 (long long)head_dim);
+  if (!(scale > 0.0f))
+    return fail(OSLO_E_BAD_ARG, "oslo_attention_prefill_fwd: the scale must be positive");
   if (batch == 0 || heads == 0 || S == 0) return OSLO_OK;
   if (!out || !q || !k || !v || !strides)
     return fail(OSLO_E_BAD_ARG, "oslo_attention_prefill_fwd: null pointer");
