@@ -89,6 +89,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   constexpr int kSteps = D / 16;   // contraction steps of Q K^T
   constexpr int kBlocksD = D / 32; // 32-row blocks of O^T
   constexpr int kLoadsK = kKeysPerTile * kChunks / kBlockThreads; // per thread and tile
+  constexpr int kSwizzleK = kChunks >= 16 ? 15 : 7;                // rows over which K's chunks rotate
   __shared__ __align__(16) T k_lds[kKeysPerTile * D];  // [key][chunk ^ (key & 7)][8]
   __shared__ __align__(16) T vt_lds[D * kKeysPerTile]; // [d][(slot + d + d/8) & 7][8]
 
@@ -159,7 +160,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
 #pragma unroll
     for (int j = 0; j < kLoadsK; ++j) {
       const int row = k_r0 + j * (kBlockThreads / kChunks);
-      *reinterpret_cast<u32x4 *>(&k_lds[(row * kChunks + (k_ch ^ (row & 7))) * 8]) = kreg[j];
+      *reinterpret_cast<u32x4 *>(&k_lds[(row * kChunks + (k_ch ^ (row & kSwizzleK))) * 8]) = kreg[j];
     }
     if (v_task) {
 #pragma unroll
@@ -210,7 +211,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
 #pragma unroll
       for (int s = 0; s < kSteps; ++s) {
         const Frag kf = *reinterpret_cast<const Frag *>(
-            &k_lds[(key * kChunks + ((2 * s + half) ^ (key & 7))) * 8]);
+            &k_lds[(key * kChunks + ((2 * s + half) ^ (key & kSwizzleK))) * 8]);
         sc = Op::run(kf, qf[s], sc);
       }
 
@@ -232,11 +233,19 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
         for (int tt = 0; tt < 4; ++tt) {
           float x = sc[4 * j + tt];
           if constexpr (HAS_PAD) x = x * a.scale_log2e + pv[tt];
-          if (diagonal) x = kj + tt <= qrow ? x : -INFINITY;
           sc[4 * j + tt] = x;
-          mt = fmaxf(mt, x);
         }
       }
+      if (diagonal) {
+        // a branch of its own (the empty asm keeps it one): the comparisons
+        // run in the last tiles of a block only
+        asm volatile("");
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          sc[r] = keyb + 8 * (r >> 2) + 4 * half + (r & 3) <= qrow ? sc[r] : -INFINITY;
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sc[r]);
       if constexpr (!HAS_PAD) mt *= a.scale_log2e;
       mt = fmaxf(mt, other_half(mt));
       // The reference maximum m only follows the scores when they exceed it by
