@@ -396,7 +396,7 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         o = torch.empty((B, S, Hh, D), dtype=torch.bfloat16, device=dev)
         strides = (ctypes.c_int64 * 12)(*(3 * [Hh * S * D, S * D, D] + [S * Hh * D, D, Hh * D]))
         t = time_launches(lambda: check(lib.oslo_attention_prefill_fwd(
-            P(o), P(q), P(k), P(v), None, D ** -0.5, B, Hh, S, D, strides, BF16, st)), max(5, n // 2), 3)
+            P(o), P(q), P(k), P(v), None, D ** -0.5, B, Hh, S, D, 0, strides, BF16, st)), max(5, n // 2), 3)
         flops = 4 * B * Hh * D * (S * (S + 1) // 2)
         res.append({"kernel": f"attention_prefill bf16 [{B},{Hh},{S},{D}] causal", "bound": "mfma",
                     "achieved": round(flops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",

@@ -406,6 +406,8 @@ int oslo_attention_decode_fwd(void *out, const void *q, void *k, void *v,
  * order, so that split heads ([B, H, S, D]), merged heads ([B, S, H, D]) and
  * slices of a packed qkv projection are all taken where they lie (multiples
  * of 8 elements, pointers 16-byte aligned, a (batch, head) slice under 2 GiB).
+ * window > 0 restricts the sum to the last `window` keys, i - window < s <= i
+ * (GPT-Neo's local attention, oslo/models/gpt_neo/modeling_gpt_neo.py:153-163).
  * pad: NULL, or an additive fp32 [batch, S] key mask (then S % 4 == 0).
  * scale > 0. Products of the 16-bit inputs are accumulated in fp32, the softmax is fp32
  * under a running maximum, the probabilities are rounded to the storage type
@@ -420,8 +422,9 @@ int oslo_attention_decode_fwd(void *out, const void *q, void *k, void *v,
 int oslo_attention_prefill_fwd(void *out, const void *q, const void *k,
                                const void *v, const float *pad, float scale,
                                int64_t batch, int64_t heads, int64_t S,
-                               int64_t head_dim, const int64_t *strides,
-                               int dtype, oslo_stream_t stream);
+                               int64_t head_dim, int64_t window,
+                               const int64_t *strides, int dtype,
+                               oslo_stream_t stream);
 
 /* Repeated n-gram blocking (beam search) ------------------------------------ */
 

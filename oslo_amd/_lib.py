@@ -59,7 +59,7 @@ PROTOTYPES = {
         _c.c_int, [_P, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _I64, _I64, _c.c_float, _I64, _I64, _I64, _c.c_int,
                    _P]),
     "oslo_attention_prefill_fwd": (
-        _c.c_int, [_P, _P, _P, _P, _P, _c.c_float, _I64, _I64, _I64, _I64, _c.POINTER(_c.c_int64), _c.c_int, _P]),
+        _c.c_int, [_P, _P, _P, _P, _P, _c.c_float, _I64, _I64, _I64, _I64, _I64, _c.POINTER(_c.c_int64), _c.c_int, _P]),
     "oslo_ngram_repeat_block": (
         _c.c_int, [_P, _P, _I64, _I64, _I64, _I64, _c.c_int, _P]),
     "oslo_sample_idx_rows": (_I64, [_c.c_int32, _c.c_int32, _I64]),

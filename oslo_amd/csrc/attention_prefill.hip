@@ -74,13 +74,14 @@ struct PrefillArgs {
   int batch_heads;
   int head_groups; // ceil(batch_heads / 8)
   int query_blocks;
+  int window; // 0: every key up to the query; else the last `window` of them
 };
 
 __device__ __forceinline__ float other_half(float v) {
   return __shfl_xor(v, 32, kWave);
 }
 
-template <typename T, int D, bool HAS_PAD>
+template <typename T, int D, bool HAS_PAD, bool HAS_WINDOW>
 __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_prefill_kernel(
     const PrefillArgs a) {
   using Op = MatrixOp<T>;
@@ -134,6 +135,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
                   qrs, (uint32_t)qrow * q_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0));
 
   const float *padr = HAS_PAD ? a.pad + (int64_t)b * S : nullptr;
+  const int behind = HAS_WINDOW ? qrow - a.window : -1; // the last key behind the query's window
 
   // A tile travels global -> registers -> LDS; the loads of the next tile are
   // in flight while this one is computed.
@@ -187,8 +189,12 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
 
   const int last_key = (q0 + kQueriesPerBlock < S ? q0 + kQueriesPerBlock : S) - 1;
   const int tiles = last_key / kKeysPerTile + 1;
-  issue_loads(0);
-  for (int t = 0; t < tiles; ++t) {
+  // with a sliding window the block starts at the tile of its first query's
+  // first visible key
+  const int window = HAS_WINDOW ? a.window : 0;
+  const int first_tile = HAS_WINDOW && q0 - window + 1 > 0 ? (q0 - window + 1) / kKeysPerTile : 0;
+  issue_loads(first_tile * kKeysPerTile);
+  for (int t = first_tile; t < tiles; ++t) {
     const int key0 = t * kKeysPerTile;
     __syncthreads(); // the reads of the previous tile are done
     store_tile();
@@ -202,6 +208,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
     for (int kb = 0; kb < 2; ++kb) {
       const int keyb = key0 + 32 * kb;
       if (keyb > wave_q0 + 31) break; // every key is ahead of the wave's queries
+      if (HAS_WINDOW && keyb + 31 <= wave_q0 - window) continue; // or behind their windows
 
       // S^T = K Q^T
       f32x16 sc;
@@ -218,7 +225,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
       // Causal and padding mask, maximum. Without a padding mask the scores
       // stay raw: the scale (positive) commutes with the maximum and goes
       // into the exponent's multiply-add.
-      const bool diagonal = keyb + 31 > wave_q0;
+      const bool diagonal = keyb + 31 > wave_q0 || (HAS_WINDOW && keyb <= wave_q0 + 31 - window);
       float mt = -INFINITY;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -241,8 +248,10 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
         // run in the last tiles of a block only
         asm volatile("");
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          sc[r] = keyb + 8 * (r >> 2) + 4 * half + (r & 3) <= qrow ? sc[r] : -INFINITY;
+        for (int r = 0; r < 16; ++r) {
+          const int kr = keyb + 8 * (r >> 2) + 4 * half + (r & 3);
+          sc[r] = kr <= qrow && (!HAS_WINDOW || kr > behind) ? sc[r] : -INFINITY;
+        }
       }
 #pragma unroll
       for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sc[r]);
@@ -254,11 +263,14 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
       // depend on the shift. Rescaling O costs as much as the softmax of a
       // step, and with an exact running maximum some query of a wave raises it
       // in most steps; with the slack it happens in the first steps only.
-      // Key 0 is visible to every query: m is finite after the first step.
-      const bool raise = mt > m + kSlack; // true in the first step (m = -inf)
+      // Without a window key 0 is visible to every query and m is finite
+      // after the first step; with one, a query may see nothing in the first
+      // steps of its wave: m stays -inf, nothing is rescaled, and the
+      // exponentials (of -inf) are taken against 0.
+      const bool raise = mt > m + kSlack; // true at the first visible key (m = -inf)
       if (__any(raise)) { // wave-uniform
         const float m_new = raise ? mt : m;
-        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+        const float alpha = !HAS_WINDOW || raise ? __builtin_amdgcn_exp2f(m - m_new) : 1.0f;
         m = m_new;
         l *= alpha;
 #pragma unroll
@@ -267,12 +279,13 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
           for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
       }
       float sum = 0.f;
+      const float shift = HAS_WINDOW && m == -INFINITY ? 0.f : m;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         if constexpr (HAS_PAD)
-          sc[r] = __builtin_amdgcn_exp2f(sc[r] - m);
+          sc[r] = __builtin_amdgcn_exp2f(sc[r] - shift);
         else
-          sc[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[r], a.scale_log2e, -m));
+          sc[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[r], a.scale_log2e, -shift));
         sum += sc[r];
       }
       l += sum;
@@ -317,10 +330,16 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
 template <typename T, int D>
 void launch_prefill_dim(const PrefillArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)(8 * a.head_groups * a.query_blocks));
-  if (a.pad != nullptr)
-    attention_prefill_kernel<T, D, true><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
-  else
-    attention_prefill_kernel<T, D, false><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  auto go = [&]<bool HAS_PAD, bool HAS_WINDOW>() {
+    attention_prefill_kernel<T, D, HAS_PAD, HAS_WINDOW><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+  };
+  if (a.window > 0) {
+    if (a.pad != nullptr) go.template operator()<true, true>();
+    else go.template operator()<false, true>();
+  } else {
+    if (a.pad != nullptr) go.template operator()<true, false>();
+    else go.template operator()<false, false>();
+  }
 }
 
 template <typename T>
@@ -340,10 +359,11 @@ extern "C" int oslo_attention_prefill_fwd(void *out, const void *q, const void *
                                           const void *v, const float *pad,
                                           float scale, int64_t batch, int64_t heads,
                                           int64_t S, int64_t head_dim,
+                                          int64_t window,
                                           const int64_t *strides, int dtype,
                                           oslo_stream_t stream) {
   using namespace oslo;
-  if (batch < 0 || heads < 0 || S < 0 || head_dim < 0)
+  if (batch < 0 || heads < 0 || S < 0 || head_dim < 0 || window < 0)
     return fail(OSLO_E_BAD_ARG, "oslo_attention_prefill_fwd: negative size");
   if (dtype != OSLO_F16 && dtype != OSLO_BF16) {
     if (dtype == OSLO_F32)
@@ -389,6 +409,7 @@ extern "C" int oslo_attention_prefill_fwd(void *out, const void *q, const void *
   a.batch_heads = (int)(batch * heads);
   a.head_groups = (a.batch_heads + 7) / 8;
   a.query_blocks = (int)((S + kQueriesPerBlock - 1) / kQueriesPerBlock);
+  a.window = window >= S ? 0 : (int)window;
   if ((int64_t)8 * a.head_groups * a.query_blocks > (int64_t)0x7fffffff)
     return fail(OSLO_E_UNSUPPORTED, "oslo_attention_prefill_fwd: too many blocks for one launch");
   hipStream_t st = static_cast<hipStream_t>(stream);

@@ -574,10 +574,12 @@ class FusedPrefillAttention(object):
         return not _needs_grad(query, key)
 
     @staticmethod
-    def apply(query, key, value, attention_mask=None, scale=None):
+    def apply(query, key, value, attention_mask=None, scale=None, window=None):
+        """``window``: GPT-Neo's local attention (query i sees keys i - window < s <= i)."""
         b, _, s, _ = query.shape
         pad = None if attention_mask is None else attention_mask.reshape(b, s).float()
-        return get_custom_kernels().attention_prefill_forward(query, key, value, 1.0 if scale is None else scale, pad)
+        return get_custom_kernels().attention_prefill_forward(query, key, value, 1.0 if scale is None else scale, pad,
+                                                              window or 0)
 
 
 class FusedLinearRows(object):

@@ -579,11 +579,12 @@ def attention_decode_forward(query, key, value, pos, scale, window=0, new_key=No
 PREFILL_HEAD_DIMS = (64, 128, 256)
 
 
-def attention_prefill_forward(query, key, value, scale, pad=None):
+def attention_prefill_forward(query, key, value, scale, pad=None, window=0):
     """Causal attention of a whole prompt in one kernel: query, key, value
     [B, H, S, D] fp16/bf16 views (features contiguous, any batch/head/position
     strides that are multiples of 8 elements), ``pad`` an optional additive
-    fp32 [B, S] key mask. Returns softmax(scale * q k^T + causal + pad) v,
+    fp32 [B, S] key mask, ``window`` > 0 a sliding window (query i sees keys
+    i - window < s <= i). Returns softmax(scale * q k^T + causal + pad) v,
     shaped [B, H, S, D] over [B, S, H, D] memory, so that merging the heads
     afterwards moves nothing (oslo/models/gptj/modeling_gptj.py:936-951 and
     the ``_merge_heads`` that follows it). The [S, S] scores never reach memory."""
@@ -617,7 +618,8 @@ def attention_prefill_forward(query, key, value, scale, pad=None):
         strides[3 * i], strides[3 * i + 1], strides[3 * i + 2] = t.stride(0), t.stride(1), t.stride(2)
     with _on_device(q):
         _lib.check(_lib.load().oslo_attention_prefill_fwd(
-            _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(pad), float(scale), b, h, s, d, strides, code, _stream(q)))
+            _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(pad), float(scale), b, h, s, d, int(window), strides, code,
+            _stream(q)))
     return out
 
 

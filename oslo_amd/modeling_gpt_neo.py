@@ -169,8 +169,7 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
             layer_past.flush()
         if static and not one_pass:
             attention_mask = static_cache_mask(layer_past, attention_mask, fused, window=self._window())
-        prompt = (causal and sq > 1 and not isinstance(self, GPTNeoLocalSelfAttention) and head_mask is None
-                  and not output_attentions
+        prompt = (causal and sq > 1 and head_mask is None and not output_attentions
                   and FusedPrefillAttention.is_available(query, key, attention_mask, self.training,
                                                          self.attn_dropout.p))
         if one_pass:
@@ -180,8 +179,9 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
                                              None, self._window(), *fresh)
             w = None
         elif prompt:
-            # a whole prompt at inference (global layers): one kernel, the scores stay on chip
-            out, w = FusedPrefillAttention.apply(query, key, value, attention_mask, None), None
+            # a whole prompt at inference: one kernel, the scores stay on chip (a local
+            # layer's window included)
+            out, w = FusedPrefillAttention.apply(query, key, value, attention_mask, None, self._window()), None
         elif fused and static:
             out, w = FusedGPTNeoSelfAttention._fused_attn(self, query, key, value, attention_mask, head_mask, False)
         elif fused:

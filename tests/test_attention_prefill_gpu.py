@@ -24,14 +24,17 @@ HALVES = [torch.float16, torch.bfloat16]
 REL = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}
 
 
-def device_reference(q, k, v, scale, pad=None):
+def device_reference(q, k, v, scale, pad=None, window=0):
     q, k, v = q.double(), k.double(), v.double()
     s = q.shape[2]
     w = q @ k.transpose(-1, -2) * scale
     if pad is not None:
         w = w + pad.double()[:, None, None, :]
-    w = w.masked_fill(torch.ones(s, s, device=q.device, dtype=torch.bool).triu(1), float("-inf"))
-    return torch.softmax(w, -1) @ v
+    i = torch.arange(s, device=q.device)
+    hidden = i[None, :] > i[:, None]
+    if window:
+        hidden = hidden | (i[None, :] <= i[:, None] - window)
+    return torch.softmax(w.masked_fill(hidden, float("-inf")), -1) @ v
 
 
 def check(out, want, dtype, what, vmax=4.0):
@@ -78,6 +81,27 @@ def test_prefill_long_prompts(b, h, s, d, dtype):
     for p in (None, pad):
         out = kernels.attention_prefill_forward(q, k, v, 0.1, p)
         check(out, device_reference(q, k, v, 0.1, p), dtype, (b, h, s, d, p is not None))
+
+
+# windows shorter than a step of 32 keys, ragged against steps and tiles, longer than a query block,
+# and at least the prompt (no window at all)
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+@pytest.mark.parametrize("window", [1, 5, 32, 33, 64, 100, 256, 300, 700])
+def test_prefill_sliding_window(window, dtype):
+    for (b, h, s, d) in ((2, 3, 520, 64), (1, 2, 700, 256)):
+        q, k, v = (randn((b, h, s, d), dtype, seed=window + i).to(DEV) for i in range(3))
+        pad = padding(b, s, window).to(DEV)
+        for p in (None, pad):
+            out = kernels.attention_prefill_forward(q, k, v, 0.1, p, window)
+            check(out, device_reference(q, k, v, 0.1, p, window), dtype, (b, h, s, d, window, p is not None))
+    # small enough for the oracle: its causal softmax with a window, composed with a matmul
+    b, h, s, d = 1, 2, 96, 64
+    q, k, v = (randn((b, h, s, d), dtype, seed=3 * window + i) for i in range(3))
+    scores = np.einsum("bhid,bhjd->bhij", f32(q).astype(np.float64), f32(k).astype(np.float64))
+    probs = orc.softmax_causal(scores, 0.1, dtype=np.float64, window=window)
+    want = np.einsum("bhij,bhjd->bhid", probs, f32(v).astype(np.float64))
+    out = kernels.attention_prefill_forward(q.to(DEV), k.to(DEV), v.to(DEV), 0.1, None, window)
+    check(out, want, dtype, ("oracle", window))
 
 
 @pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)

@@ -60,8 +60,8 @@ def test_fused_model_matches_unfused(family, dtype, padded):
 @pytest.mark.parametrize("padded", [False, True], ids=["nopad", "pad"])
 def test_prompt_attention_runs_as_one_kernel_at_inference(family, dtype, padded, monkeypatch):
     """Heads of 64 features and a prompt of 160 tokens, no gradient: the fused
-    attention takes the one-kernel prompt attention (GPT-Neo's local layer keeps
-    its window kernel), the logits match the unfused model's, and the cache it
+    attention takes the one-kernel prompt attention (GPT-Neo's local layer with
+    its window), the logits match the unfused model's, and the cache it
     returns continues into a decoding step like the unfused one's."""
     big = {
         "gpt2": lambda: GPT2LMHeadModel(GPT2Config(vocab_size=512, n_positions=256, n_embd=256, n_layer=2, n_head=4,
@@ -90,7 +90,7 @@ def test_prompt_attention_runs_as_one_kernel_at_inference(family, dtype, padded,
         m.fuse()
         got = m(ids, attention_mask=mask, use_cache=True)
         got_step = m(ids[:, :1], attention_mask=step_mask, past_key_values=got["past_key_values"])["logits"]
-    assert calls == [(3, 4, 160, 64)] * (1 if family == "gpt_neo" else 2)
+    assert calls == [(3, 4, 160, 64)] * 2
     keep = torch.ones(3, 160, dtype=torch.bool, device=DEV) if mask is None else mask.bool()
     err = (got["logits"].float() - want["logits"].float()).abs()[keep].max().item()
     assert err <= LOGIT_TOL[dtype], f"{family} {dtype}: logits differ by {err}"

@@ -2,9 +2,9 @@
 seeds and positions drawn from a seeded generator, each result compared on the
 device with the same expression written in torch fp32 (float64 for the
 attention of a decoding step). It complements the oracle tests, which pin
-exact bars on chosen shapes, by covering shapes nobody chose: 250 draws here
-
-the same loop was run for 4500 draws with other seeds without a failure."""
+exact bars on chosen shapes, by covering shapes nobody chose: 250 draws here;
+the same loop was run for 4500 draws with other seeds without a failure (the
+attention over a whole prompt joined later, on a stream of draws of its own)."""
 
 import random
 
@@ -29,13 +29,18 @@ def test_random_shapes_against_torch_expressions():
 
     DT = [torch.float32, torch.float16, torch.bfloat16]
     TOL = {torch.float32: 2e-6, torch.float16: 2e-3, torch.bfloat16: 1.6e-2}
-    def pick_len():
-        r = rng.random()
+    def pick_len_from(r_):
+        r = r_.random()
         if r < 0.3:
-            return rng.randint(1, 70)
+            return r_.randint(1, 70)
         if r < 0.6:
-            return min(8192, rng.choice([64, 128, 256, 512, 1024, 2048, 4096, 8192]) + rng.choice([-8, -1, 0, 0, 1, 8]))
-        return rng.randint(1, 8192)
+            return min(8192, r_.choice([64, 128, 256, 512, 1024, 2048, 4096, 8192]) + r_.choice([-8, -1, 0, 0, 1, 8]))
+        return r_.randint(1, 8192)
+
+    def pick_len():
+        return pick_len_from(rng)
+
+    rng_prompt = random.Random(1)
     for it in range(N):
         dt = rng.choice(DT)
         tol = TOL[dt]
@@ -141,6 +146,33 @@ def test_random_shapes_against_torch_expressions():
             pos = torch.tensor([last], device=dev) if rng.random() < 0.5 else last
             oa = kernels.attention_decode_forward(q, kk, vv, pos, 0.2, win)
             report("attention_decode", (oa.float() - refa).abs().max().item(), tol * max(1.0, refa.abs().max().item()), (dt, bb, hh, cap, d, last, win))
+        # attention over a whole prompt (16-bit only; drawn from a stream of its own, so that the
+        # draws of the other families are the ones the longer runs covered)
+        if dt != torch.float32:
+            pd = rng_prompt.choice([64, 128, 256])
+            ps = max(1, min(pick_len_from(rng_prompt), 3000))
+            pb, ph = rng_prompt.randint(1, 2), rng_prompt.randint(1, 5)
+            pscale = rng_prompt.choice([1.0, 0.125, pd ** -0.5])
+            pq, pk, pvv = (torch.randn(pb, ph, ps, pd, device=dev).to(dt) for _ in range(3))
+            ppad = None
+            if ps % 4 == 0 and rng_prompt.random() < 0.5:
+                plens = torch.randint(1, ps + 1, (pb,), device=dev)
+                ppad = torch.where(torch.arange(ps, device=dev)[None] < plens[:, None], 0.0, -10000.0).float()
+            if rng_prompt.random() < 0.3:  # merged-heads memory viewed as [B, H, S, D]
+                pq, pk, pvv = (t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3) for t in (pq, pk, pvv))
+            w = pq.double() @ pk.double().transpose(-1, -2) * pscale
+            if ppad is not None:
+                w = w + ppad.double()[:, None, None, :]
+            ii = torch.arange(ps, device=dev)
+            pwin = rng_prompt.choice([0, 0, 1, 7, 64, 256])
+            hidden = ii[None, :] > ii[:, None]
+            if pwin:
+                hidden = hidden | (ii[None, :] <= ii[:, None] - pwin)
+            refp = torch.softmax(w.masked_fill(hidden, float("-inf")), -1) @ pvv.double()
+            op = kernels.attention_prefill_forward(pq, pk, pvv, pscale, ppad, pwin)
+            rel = 2.0 ** -11 if dt == torch.float16 else 2.0 ** -8   # output rounding + rounding of the probabilities
+            report("attention_prefill", ((op.double() - refp).abs() - rel * (refp.abs() + pvv.abs().max().item())).max().item(),
+                   1e-4, (dt, pb, ph, ps, pd, pscale, ppad is not None, pwin))
         # softmax + dropout in one pass, forward and backward (the mask is read off the output)
         if S <= 2048:
             p_drop = rng.choice([0.1, 0.5])
