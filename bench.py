@@ -41,34 +41,34 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 # profiles/causal_softmax_fp16_8x16x2048x2048_hbm_traffic.md.
 MEASURED_TRAFFIC = {
     "linear_rows fc_in + bias + gelu bf16 1 x [16384,4096]": 134699008,
-    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135284940,
-    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134601216,
-    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136613376,
+    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135285043,
+    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134601011,
+    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136612249,
     "linear_rows attention projection bf16 1 x [4096,4096]": 33740800,
     "linear_rows attention projection bf16 8 x [4096,4096]": 34370560,
     "attention_decode bf16 1 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 17573888,
     "attention_decode bf16 8 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 136477696,
     "causal_fwd fp16 [8,16,2048,2048]": 1627472076,
     "causal_bwd fp16 [8,16,2048,2048]": 2181120204,
-    "causal_fwd bf16 [8,16,2048,2048]": 1627472076,
+    "causal_fwd bf16 [8,16,2048,2048]": 1627459788,
     "causal_bwd bf16 [8,16,2048,2048] (in place)": 2181120204,
-    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635890995,
+    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635900211,
     "causal_dropout_bwd p=0.1 bf16 [8,16,2048,2048] (in place)": 2214719488,
-    "causal_fwd fp32 [8,16,2048,2048]": 3238062284,
-    "causal_bwd fp32 [8,16,2048,2048] (in place)": 4328582963,
-    "causal_fwd bf16 [1,16,8192,8192]": 3229695590,
-    "masked_fwd bf16 [16,16,1024,1024] key mask": 1073948672,
+    "causal_fwd fp32 [8,16,2048,2048]": 3238067404,
+    "causal_bwd fp32 [8,16,2048,2048] (in place)": 4328580915,
+    "causal_fwd bf16 [1,16,8192,8192]": 3229695795,
+    "masked_fwd bf16 [16,16,1024,1024] key mask": 1082271948,
     "masked_bwd bf16 [16,16,1024,1024]": 1610650624,
-    "bias_gelu_fwd bf16 [16384,16384]": 1073872076,
-    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677933158,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610758758,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141059174,
+    "bias_gelu_fwd bf16 [16384,16384]": 1073874739,
+    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677932953,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610759168,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141059379,
     "bias_gelu_fwd bf16 [16384,4096]": 268489523,
     "bias_gelu_bwd+dbias bf16 [16384,4096]": 419568230,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402726502,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285348454,
-    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807983308,
-    "causal_fwd bf16 [8,16,2048,2048] with padding mask": 1628013772,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402726297,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285347840,
+    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807980441,
+    "causal_fwd bf16 [8,16,2048,2048] with padding mask": 1628022988,
     "causal_window_fwd window 256 bf16 [8,16,2048,2048]": 1230656716,
     "causal_window_bwd window 256 bf16 [8,16,2048,2048] (in place)": 1387504640,
 }
@@ -407,17 +407,25 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
 
 
 def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
-    """--only causal_fwd | causal_bwd | copy: launch one kernel `steps` times
+    """--only causal_fwd | causal_bwd | attention_prefill | copy: launch one kernel `steps` times
     (profiling runs). `copy` is torch's device copy of 1 GiB, the kernel of
     known traffic that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
     if args.only == "copy":
         a = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
         b = torch.empty_like(a)
         fn = lambda: b.copy_(a)
+    elif args.only == "attention_prefill":
+        import ctypes
+        B, Hh, S, D = 8, 16, 2048, 256  # the GPT-J shape of the kernel table
+        q, k, v = (torch.randn(B, Hh, S, D, device=dev).to(torch.bfloat16) for _ in range(3))
+        o = torch.empty((B, S, Hh, D), dtype=torch.bfloat16, device=dev)
+        strides = (ctypes.c_int64 * 12)(*(3 * [Hh * S * D, S * D, D] + [S * Hh * D, D, Hh * D]))
+        fn = lambda: check(lib.oslo_attention_prefill_fwd(
+            P(o), P(q), P(k), P(v), None, D ** -0.5, B, Hh, S, D, 0, strides, 2, st))
     else:
         fn = {"causal_fwd": fwd, "causal_bwd": bwd}.get(args.only)
     if fn is None:
-        sys.exit("--only takes causal_fwd, causal_bwd or copy")
+        sys.exit("--only takes causal_fwd, causal_bwd, attention_prefill or copy")
     if args.only == "causal_bwd":
         fwd()
     t = time_launches(fn, args.steps, args.warmup)
