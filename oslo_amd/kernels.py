@@ -601,7 +601,7 @@ def attention_prefill_forward(query, key, value, scale, pad=None, window=0):
 
     def strided(t):
         ok = t.stride(3) == 1 and all(st % 8 == 0 for st in t.stride()[:3]) and t.data_ptr() % 16 == 0 \
-            and (s == 1 or t.stride(2) >= d)
+            and (s == 1 or t.stride(2) >= d) and (s + 128) * t.stride(2) * 2 < 2 ** 31  # 32-bit offsets in a head
         return t if ok else t.contiguous()
 
     q, k, v = strided(query), strided(key), strided(value)
