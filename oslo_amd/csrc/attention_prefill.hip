@@ -20,15 +20,18 @@
 // In the accumulator layout of v_mfma_f32_32x32x16 a lane holds one column
 // (lane % 32 = the query) and 16 rows, so the running maximum, the sum and
 // the rescaling of O are per-lane scalars: the softmax needs one exchange
-// between the two halves of the wave per tile and no LDS. The 16 rows of a
+// between the two halves of the wave per step and no LDS. The 16 rows of a
 // lane are keys 8j + 4h + t (j, t = 0..3; h = lane / 32), and a B operand
 // wants, per half, 8 consecutive contraction slots: the probabilities are used
 // where they are, and the contraction order is permuted instead -- V^T is
-// written to LDS with key 8j + 4h + t of each group of 16 at slot 8h + 4j + t.
+// written to LDS with key 8j + 4h + t of each group of 16 (j = 0, 1 there) at
+// slot 8h + 4j + t.
 // V arrives as [key][feature]; each thread transposes an 8 x 8 block in
 // registers and writes 128-bit rows of V^T. Both LDS tiles are swizzled by
-// 16-byte chunk so that the 128-bit reads of a wave (8 lanes = 8 rows at one
-// chunk) and the writes fall on different banks.
+// 16-byte chunk so that the 128-bit reads of a wave (the LDS serves 16 lanes
+// at a time: 16 rows at one chunk) and the writes spread over the banks. A
+// tile of keys is taken in two steps of 32, each a step of the running
+// softmax, and the next tile's global loads are in flight meanwhile.
 
 #include "common.hpp"
 
