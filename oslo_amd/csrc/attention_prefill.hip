@@ -300,12 +300,14 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
 #pragma unroll
         for (int i = 0; i < 8; ++i) pf[u][i] = static_cast<T>(sc[8 * u + i]);
 
-      // O^T += V^T P^T
+      // O^T += V^T P^T, the first 16 keys into every block of O^T, then the
+      // other 16: the products of the first half only need the first half of
+      // the exponentials
 #pragma unroll
-      for (int i = 0; i < kBlocksD; ++i) {
-        const int d = 32 * i + col;
+      for (int u = 0; u < 2; ++u) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int i = 0; i < kBlocksD; ++i) {
+          const int d = 32 * i + col;
           const Frag vf = *reinterpret_cast<const Frag *>(
               &vt_lds[(d * 8 + ((4 * kb + 2 * u + half + d + (d >> 3)) & 7)) * 8]);
           o[i] = Op::run(vf, pf[u], o[i]);
