@@ -126,6 +126,28 @@ def test_prefill_large_scores_and_size_independent_properties(dtype):
         assert torch.allclose(two.float(), one.float() * 2, rtol=2.0 ** -10, atol=1e-6)
 
 
+def test_prefill_full_size_properties():
+    """The GPT-J shape of the benchmark, [8, 16, 2048, 256] bf16, where the oracle
+    would take hours: the first row is the first value exactly, equal scores
+    (q = 0) give the running mean of the values, and the result agrees with the
+    library's attention (an independent implementation) within the bound for two
+    bf16 results."""
+    dtype = torch.bfloat16
+    b, h, s, d = 8, 16, 2048, 256
+    g = torch.Generator(device=DEV).manual_seed(0)
+    q, k, v = (torch.randn((b, h, s, d), generator=g, device=DEV).to(dtype) for _ in range(3))
+    out = kernels.attention_prefill_forward(q, k, v, d ** -0.5)
+    assert torch.isfinite(out).all()
+    assert torch.equal(out[:, :, 0], v[:, :, 0])
+    lib = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+    excess = ((out.float() - lib.float()).abs() - 2 * REL[dtype] * (lib.float().abs() + 4.0)).max().item()
+    assert excess <= 1e-4, excess
+    flat = kernels.attention_prefill_forward(torch.zeros_like(q), k, v, 1.0)
+    for bb in range(0, b, 3):  # in slices: float64 of the whole tensor is 1 GiB
+        mean = v[bb].double().cumsum(1) / torch.arange(1, s + 1, device=DEV)[None, :, None]
+        check(flat[bb], mean, dtype, "running mean", vmax=6.0)
+
+
 @pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
 def test_prefill_takes_strided_views(dtype):
     """Merged-heads memory ([B, S, H, D] viewed as [B, H, S, D]) and the slices of
