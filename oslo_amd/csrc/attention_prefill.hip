@@ -94,6 +94,14 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   constexpr int kBlocksD = D / 32; // 32-row blocks of O^T
   constexpr int kLoadsK = kKeysPerTile * kChunks / kBlockThreads; // per thread and tile
   constexpr int kSwizzleK = kChunks >= 16 ? 15 : 7;                // rows over which K's chunks rotate
+  // At head_dim 256 the 64 registers of Q^T are what pushes a wave past its
+  // 256 vector registers: the compiler then parks half of Q^T in the
+  // accumulator file, moves it back before every product and has one buffer
+  // left for the K operand, so that every product waits for its own LDS read.
+  // There Q^T lives in (dynamic) LDS instead, in operand order, each wave its
+  // own 16 KiB, and both operands of S^T = K Q^T are read from LDS.
+  constexpr bool kQInLds = D == 256;
+  extern __shared__ __align__(16) unsigned char dynamic_lds[];
   __shared__ __align__(16) T k_lds[kKeysPerTile * D];  // [key][chunk ^ (key & 7)][8]
   __shared__ __align__(16) T vt_lds[D * kKeysPerTile]; // [d][(slot + d + d/8) & 7][8]
 
@@ -130,12 +138,23 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   // Q^T as B operands: lane (query, half) holds features 16 s + 8 half .. + 7
   const int wave_q0 = q0 + 32 * wave;
   const int qrow = wave_q0 + col;
-  Frag qf[kSteps];
+  Frag qf[kQInLds ? 1 : kSteps];
+  u32x4 *q_lds = reinterpret_cast<u32x4 *>(dynamic_lds) + wave * kSteps * kWave + lane;
+  if constexpr (kQInLds) {
+    u32x4 tmp[kSteps];
 #pragma unroll
-  for (int s = 0; s < kSteps; ++s)
-    qf[s] = __builtin_bit_cast(
-        Frag, __builtin_amdgcn_raw_buffer_load_b128(
-                  qrs, (uint32_t)qrow * q_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0));
+    for (int s = 0; s < kSteps; ++s)
+      tmp[s] = __builtin_amdgcn_raw_buffer_load_b128(
+          qrs, (uint32_t)qrow * q_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0);
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) q_lds[s * kWave] = tmp[s];
+  } else {
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s)
+      qf[s] = __builtin_bit_cast(
+          Frag, __builtin_amdgcn_raw_buffer_load_b128(
+                    qrs, (uint32_t)qrow * q_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0));
+  }
 
   const float *padr = HAS_PAD ? a.pad + (int64_t)b * S : nullptr;
   const int behind = HAS_WINDOW ? qrow - a.window : -1; // the last key behind the query's window
@@ -222,7 +241,24 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
       for (int s = 0; s < kSteps; ++s) {
         const Frag kf = *reinterpret_cast<const Frag *>(
             &k_lds[(key * kChunks + ((2 * s + half) ^ (key & kSwizzleK))) * 8]);
-        sc = Op::run(kf, qf[s], sc);
+        if constexpr (kQInLds)
+          sc = Op::run(kf, __builtin_bit_cast(Frag, q_lds[s * kWave]), sc);
+        else
+          sc = Op::run(kf, qf[s], sc);
+      }
+      // The LDS reads run kAhead steps ahead of the products that use them (left
+      // alone, the scheduler keeps one operand buffer and every product waits
+      // out its own read). 0x100: LDS reads, 0x008: matrix products.
+      {
+        constexpr int kReads = kQInLds ? 2 : 1; // per step
+        constexpr int kAhead = kSteps < 3 ? kSteps : 3;
+        __builtin_amdgcn_sched_group_barrier(0x100, kReads * kAhead, 0);
+#pragma unroll
+        for (int s = 0; s < kSteps - kAhead; ++s) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
       }
 
       // Causal and padding mask, maximum. Without a padding mask the scores
@@ -313,6 +349,17 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
           o[i] = Op::run(vf, pf[u], o[i]);
         }
       }
+      {
+        constexpr int kProducts = 2 * kBlocksD;
+        constexpr int kAhead = kProducts < 3 ? kProducts : 3;
+        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 1);
+#pragma unroll
+        for (int n = 0; n < kProducts - kAhead; ++n) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 1);
+      }
     }
   }
 
@@ -335,8 +382,14 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
 template <typename T, int D>
 void launch_prefill_dim(const PrefillArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)(8 * a.head_groups * a.query_blocks));
+  // head_dim 256 keeps Q^T in dynamic LDS: 128 queries x 256 features
+  constexpr unsigned kDynamic = D == 256 ? kQueriesPerBlock * D * sizeof(T) : 0;
   auto go = [&]<bool HAS_PAD, bool HAS_WINDOW>() {
-    attention_prefill_kernel<T, D, HAS_PAD, HAS_WINDOW><<<grid, dim3(kBlockThreads), 0, stream>>>(a);
+    auto *kernel = attention_prefill_kernel<T, D, HAS_PAD, HAS_WINDOW>;
+    if (kDynamic > 0)
+      (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynamic);
+    kernel<<<grid, dim3(kBlockThreads), kDynamic, stream>>>(a);
   };
   if (a.window > 0) {
     if (a.pad != nullptr) go.template operator()<true, true>();
