@@ -101,6 +101,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   // There Q^T lives in (dynamic) LDS instead, in operand order, each wave its
   // own 16 KiB, and both operands of S^T = K Q^T are read from LDS.
   constexpr bool kQInLds = D == 256;
+  constexpr bool kTwoLoops = D == 256; // see `step` below
   extern __shared__ __align__(16) unsigned char dynamic_lds[];
   __shared__ __align__(16) T k_lds[kKeysPerTile * D];  // [key][chunk ^ (key & 7)][8]
   __shared__ __align__(16) T vt_lds[D * kKeysPerTile]; // [d][(slot + d + d/8) & 7][8]
@@ -215,98 +216,95 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   // first visible key
   const int window = HAS_WINDOW ? a.window : 0;
   const int first_tile = HAS_WINDOW && q0 - window + 1 > 0 ? (q0 - window + 1) / kKeysPerTile : 0;
-  issue_loads(first_tile * kKeysPerTile);
-  for (int t = first_tile; t < tiles; ++t) {
-    const int key0 = t * kKeysPerTile;
-    __syncthreads(); // the reads of the previous tile are done
-    store_tile();
-    __syncthreads();
-    if (t + 1 < tiles) issue_loads(key0 + kKeysPerTile);
+  // One step of 32 keys of the tile in LDS. RESCALE: O may be rescaled to a
+  // higher reference maximum. The loop over the tiles runs the variant without
+  // it and falls back, for a single step, when a query that has already
+  // accumulated something needs a higher reference: with the multiplications
+  // of O in the same loop, the compiler copies all of O's accumulators to
+  // vector registers in every tile (it places the copies that the rare
+  // multiplication needs ahead of the branch), 128 moves and 128 registers at
+  // head_dim 256. Returns false if nothing was done for that reason.
+  auto step = [&]<bool RESCALE>(int key0, int kb) -> bool {
+    const int keyb = key0 + 32 * kb;
+    if (keyb > wave_q0 + 31) return true; // every key is ahead of the wave's queries
+    if (HAS_WINDOW && keyb + 31 <= wave_q0 - window) return true; // or behind their windows
 
-    // the tile in two steps of 32 keys, each a step of the running softmax:
-    // the matrix products of one step are independent of the other step's
-    // exponentials
+    // S^T = K Q^T
+    f32x16 sc;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      const int keyb = key0 + 32 * kb;
-      if (keyb > wave_q0 + 31) break; // every key is ahead of the wave's queries
-      if (HAS_WINDOW && keyb + 31 <= wave_q0 - window) continue; // or behind their windows
+    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+    const int key = 32 * kb + col;
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+      const Frag kf = *reinterpret_cast<const Frag *>(
+          &k_lds[(key * kChunks + ((2 * s + half) ^ (key & kSwizzleK))) * 8]);
+      if constexpr (kQInLds)
+        sc = Op::run(kf, __builtin_bit_cast(Frag, q_lds[s * kWave]), sc);
+      else
+        sc = Op::run(kf, qf[s], sc);
+    }
+    // The LDS reads run kAhead steps ahead of the products that use them (left
+    // alone, the scheduler keeps one operand buffer and every product waits
+    // out its own read). 0x100: LDS reads, 0x008: matrix products.
+    {
+      constexpr int kReads = kQInLds ? 2 : 1; // per step
+      constexpr int kAhead = kSteps < 3 ? kSteps : 3;
+      __builtin_amdgcn_sched_group_barrier(0x100, kReads * kAhead, 0);
+#pragma unroll
+      for (int s = 0; s < kSteps - kAhead; ++s) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+    }
 
-      // S^T = K Q^T
-      f32x16 sc;
+    // Causal and padding mask, maximum. Without a padding mask the scores
+    // stay raw: the scale (positive) commutes with the maximum and goes
+    // into the exponent's multiply-add.
+    const bool diagonal = keyb + 31 > wave_q0 || (HAS_WINDOW && keyb <= wave_q0 + 31 - window);
+    float mt = -INFINITY;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) sc[r] = 0.f;
-      const int key = 32 * kb + col;
-#pragma unroll
-      for (int s = 0; s < kSteps; ++s) {
-        const Frag kf = *reinterpret_cast<const Frag *>(
-            &k_lds[(key * kChunks + ((2 * s + half) ^ (key & kSwizzleK))) * 8]);
-        if constexpr (kQInLds)
-          sc = Op::run(kf, __builtin_bit_cast(Frag, q_lds[s * kWave]), sc);
-        else
-          sc = Op::run(kf, qf[s], sc);
-      }
-      // The LDS reads run kAhead steps ahead of the products that use them (left
-      // alone, the scheduler keeps one operand buffer and every product waits
-      // out its own read). 0x100: LDS reads, 0x008: matrix products.
-      {
-        constexpr int kReads = kQInLds ? 2 : 1; // per step
-        constexpr int kAhead = kSteps < 3 ? kSteps : 3;
-        __builtin_amdgcn_sched_group_barrier(0x100, kReads * kAhead, 0);
-#pragma unroll
-        for (int s = 0; s < kSteps - kAhead; ++s) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
-      }
-
-      // Causal and padding mask, maximum. Without a padding mask the scores
-      // stay raw: the scale (positive) commutes with the maximum and goes
-      // into the exponent's multiply-add.
-      const bool diagonal = keyb + 31 > wave_q0 || (HAS_WINDOW && keyb <= wave_q0 + 31 - window);
-      float mt = -INFINITY;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int kj = keyb + 8 * j + 4 * half;
-        float pv[4] = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (HAS_PAD) {
-          // keys at or past S only meet queries they are masked for
-          const float4 p4 = *reinterpret_cast<const float4 *>(padr + (kj < S ? kj : 0));
-          pv[0] = p4.x * kLog2e, pv[1] = p4.y * kLog2e, pv[2] = p4.z * kLog2e, pv[3] = p4.w * kLog2e;
-        }
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-          float x = sc[4 * j + tt];
-          if constexpr (HAS_PAD) x = x * a.scale_log2e + pv[tt];
-          sc[4 * j + tt] = x;
-        }
-      }
-      if (diagonal) {
-        // a branch of its own (the empty asm keeps it one): the comparisons
-        // run in the last tiles of a block only
-        asm volatile("");
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int kr = keyb + 8 * (r >> 2) + 4 * half + (r & 3);
-          sc[r] = kr <= qrow && (!HAS_WINDOW || kr > behind) ? sc[r] : -INFINITY;
-        }
+    for (int j = 0; j < 4; ++j) {
+      const int kj = keyb + 8 * j + 4 * half;
+      float pv[4] = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (HAS_PAD) {
+        // keys at or past S only meet queries they are masked for
+        const float4 p4 = *reinterpret_cast<const float4 *>(padr + (kj < S ? kj : 0));
+        pv[0] = p4.x * kLog2e, pv[1] = p4.y * kLog2e, pv[2] = p4.z * kLog2e, pv[3] = p4.w * kLog2e;
       }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sc[r]);
-      if constexpr (!HAS_PAD) mt *= a.scale_log2e;
-      mt = fmaxf(mt, other_half(mt));
-      // The reference maximum m only follows the scores when they exceed it by
-      // more than kSlack (log2 units): exponentials up to 2^kSlack are as exact
-      // as those up to 1 in fp32, fp16 and bf16, and the softmax does not
-      // depend on the shift. Rescaling O costs as much as the softmax of a
-      // step, and with an exact running maximum some query of a wave raises it
-      // in most steps; with the slack it happens in the first steps only.
-      // Without a window key 0 is visible to every query and m is finite
-      // after the first step; with one, a query may see nothing in the first
-      // steps of its wave: m stays -inf, nothing is rescaled, and the
-      // exponentials (of -inf) are taken against 0.
-      const bool raise = mt > m + kSlack; // true at the first visible key (m = -inf)
+      for (int tt = 0; tt < 4; ++tt) {
+        float x = sc[4 * j + tt];
+        if constexpr (HAS_PAD) x = x * a.scale_log2e + pv[tt];
+        sc[4 * j + tt] = x;
+      }
+    }
+    if (diagonal) {
+      // a branch of its own (the empty asm keeps it one): the comparisons
+      // run in the last tiles of a block only
+      asm volatile("");
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kr = keyb + 8 * (r >> 2) + 4 * half + (r & 3);
+        sc[r] = kr <= qrow && (!HAS_WINDOW || kr > behind) ? sc[r] : -INFINITY;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sc[r]);
+    if constexpr (!HAS_PAD) mt *= a.scale_log2e;
+    mt = fmaxf(mt, other_half(mt));
+    // The reference maximum m only follows the scores when they exceed it by
+    // more than kSlack (log2 units): exponentials up to 2^kSlack are as exact
+    // as those up to 1 in fp32, fp16 and bf16, and the softmax does not
+    // depend on the shift. Rescaling O costs as much as the softmax of a
+    // step, and with an exact running maximum some query of a wave raises it
+    // in most steps; with the slack it happens in the first steps only.
+    // Without a window key 0 is visible to every query and m is finite
+    // after the first step; with one, a query may see nothing in the first
+    // steps of its wave: m stays -inf, nothing is rescaled, and the
+    // exponentials (of -inf) are taken against 0.
+    const bool raise = mt > m + kSlack; // true at the first visible key (m = -inf)
+    if constexpr (RESCALE) {
       if (__any(raise)) { // wave-uniform
         const float m_new = raise ? mt : m;
         const float alpha = !HAS_WINDOW || raise ? __builtin_amdgcn_exp2f(m - m_new) : 1.0f;
@@ -317,50 +315,93 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
 #pragma unroll
           for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
       }
-      float sum = 0.f;
-      const float shift = HAS_WINDOW && m == -INFINITY ? 0.f : m;
+    } else {
+      // a query that has accumulated nothing yet (m = -inf) takes its
+      // reference maximum without rescaling anything; any other raise is
+      // left to the caller's slow path, before this step has changed anything
+      if (__any(raise && m != -INFINITY)) return false;
+      m = raise ? mt : m;
+    }
+    float sum = 0.f;
+    const float shift = HAS_WINDOW && m == -INFINITY ? 0.f : m;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        if constexpr (HAS_PAD)
-          sc[r] = __builtin_amdgcn_exp2f(sc[r] - shift);
-        else
-          sc[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[r], a.scale_log2e, -shift));
-        sum += sc[r];
-      }
-      l += sum;
+    for (int r = 0; r < 16; ++r) {
+      if constexpr (HAS_PAD)
+        sc[r] = __builtin_amdgcn_exp2f(sc[r] - shift);
+      else
+        sc[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[r], a.scale_log2e, -shift));
+      sum += sc[r];
+    }
+    l += sum;
 
-      // P^T as B operands, in the storage type like the unfused path's cast
-      Frag pf[2];
+    // P^T as B operands, in the storage type like the unfused path's cast
+    Frag pf[2];
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) pf[u][i] = static_cast<T>(sc[8 * u + i]);
+      for (int i = 0; i < 8; ++i) pf[u][i] = static_cast<T>(sc[8 * u + i]);
 
-      // O^T += V^T P^T, the first 16 keys into every block of O^T, then the
-      // other 16: the products of the first half only need the first half of
-      // the exponentials
+    // O^T += V^T P^T, the first 16 keys into every block of O^T, then the
+    // other 16: the products of the first half only need the first half of
+    // the exponentials
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < 2; ++u) {
 #pragma unroll
-        for (int i = 0; i < kBlocksD; ++i) {
-          const int d = 32 * i + col;
-          const Frag vf = *reinterpret_cast<const Frag *>(
-              &vt_lds[(d * 8 + ((4 * kb + 2 * u + half + d + (d >> 3)) & 7)) * 8]);
-          o[i] = Op::run(vf, pf[u], o[i]);
-        }
-      }
-      {
-        constexpr int kProducts = 2 * kBlocksD;
-        constexpr int kAhead = kProducts < 3 ? kProducts : 3;
-        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 1);
-#pragma unroll
-        for (int n = 0; n < kProducts - kAhead; ++n) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 1);
+      for (int i = 0; i < kBlocksD; ++i) {
+        const int d = 32 * i + col;
+        const Frag vf = *reinterpret_cast<const Frag *>(
+            &vt_lds[(d * 8 + ((4 * kb + 2 * u + half + d + (d >> 3)) & 7)) * 8]);
+        o[i] = Op::run(vf, pf[u], o[i]);
       }
     }
+    {
+      constexpr int kProducts = 2 * kBlocksD;
+      constexpr int kAhead = kProducts < 3 ? kProducts : 3;
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 1);
+#pragma unroll
+      for (int n = 0; n < kProducts - kAhead; ++n) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 1);
+    }
+    return true;
+  };
+
+  issue_loads(first_tile * kKeysPerTile);
+  int t = first_tile;
+  if constexpr (!kTwoLoops) {
+    for (; t < tiles; ++t) {
+      const int key0 = t * kKeysPerTile;
+      __syncthreads(); // the reads of the previous tile are done
+      store_tile();
+      __syncthreads();
+      if (t + 1 < tiles) issue_loads(key0 + kKeysPerTile);
+      step.template operator()<true>(key0, 0);
+      step.template operator()<true>(key0, 1);
+    }
+  }
+  while (kTwoLoops && t < tiles) {
+    int redo = -1; // the step of tile t that needs the rescaling variant
+    for (; t < tiles; ++t) {
+      const int key0 = t * kKeysPerTile;
+      __syncthreads(); // the reads of the previous tile are done
+      store_tile();
+      __syncthreads();
+      if (t + 1 < tiles) issue_loads(key0 + kKeysPerTile);
+      if (!step.template operator()<false>(key0, 0)) {
+        redo = 0;
+        break;
+      }
+      if (!step.template operator()<false>(key0, 1)) {
+        redo = 1;
+        break;
+      }
+    }
+    if (redo < 0) break;
+#pragma unroll 1
+    for (int kb = redo; kb < 2; ++kb) step.template operator()<true>(t * kKeysPerTile, kb);
+    ++t;
   }
 
   l += other_half(l);
