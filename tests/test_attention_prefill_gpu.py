@@ -126,6 +126,25 @@ def test_prefill_large_scores_and_size_independent_properties(dtype):
         assert torch.allclose(two.float(), one.float() * 2, rtol=2.0 ** -10, atol=1e-6)
 
 
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_prefill_scores_that_keep_rising(d, dtype):
+    """Every tile of keys scores far above the ones before it (by 46 in log2
+    units per tile, the slack of the reference maximum being 8), so that O is
+    rescaled in every tile; then scores that fall (nothing is ever rescaled
+    after the first tile), and a rise only at the very end."""
+    b, h, s = 1, 2, 700
+    pos = torch.arange(s, dtype=torch.float32)
+    v = randn((b, h, s, d), dtype, seed=d).to(DEV)
+    q = torch.full((b, h, s, d), 0.25).to(dtype).to(DEV)
+    for slope in (lambda j: j / 64.0, lambda j: -j / 64.0, lambda j: (j >= s - 3).float() * 40.0):
+        k = (slope(pos)[None, None, :, None] * torch.ones(d) * (8.0 / d)).to(dtype).to(DEV)  # q.k = 2 * slope
+        k = k.expand(b, h, s, d).contiguous()
+        out = kernels.attention_prefill_forward(q, k, v, 16.0)
+        assert torch.isfinite(out).all()
+        check(out, device_reference(q, k, v, 16.0), dtype, ("slope", d))
+
+
 def test_prefill_full_size_properties():
     """The GPT-J shape of the benchmark, [8, 16, 2048, 256] bf16, where the oracle
     would take hours: the first row is the first value exactly, equal scores
