@@ -577,13 +577,13 @@ def other_families_forward(torch, dev, reps=5):
     at published shapes cut to a few layers: GPT-2 XL blocks (d_model 1600, 25
     heads of 64, 1024 positions) in fp16 and GPT-Neo 2.7B blocks (d_model 2560,
     20 heads of 128, 2048 positions; every second layer is a sliding-window
-    layer, which fusion leaves alone) in fp16, the one dtype the reference's
-    gate admits. GPT-Neo does not scale its scores; with random N(0, 0.02)
-    weights at this width they have a standard deviation of about 11, and the
-    fused attention (the reference's too) takes them from a GEMM in the model
-    dtype where the unfused attention computes them in fp32: the logit
-    difference reported for this family is that quantisation, not the kernels
-    (in fp32 the two paths agree to 2e-4)."""
+    layer) in fp16, the one dtype the reference's gate admits. GPT-Neo does
+    not scale its scores; with random N(0, 0.02) weights at this width they
+    have a standard deviation of about 11, so its softmax is close to a
+    maximum and amplifies the 16-bit roundings that the fused and the unfused
+    modules make at different places (bias and GeLU on fp32 sums against one
+    rounding per operator): the logit difference reported for this family is
+    that sensitivity, not the kernels (in fp32 the two paths agree to 2e-4)."""
     from oslo_amd import GPT2Config, GPT2LMHeadModel, GPTNeoConfig, GPTNeoForCausalLM
 
     cases = [
