@@ -554,7 +554,7 @@ class FusedPrefillAttention(object):
     bf16, heads of 64, 128 or 256 features.
     """
 
-    MIN_LENGTH = 128  # shorter prompts: the three launches are as fast
+    MIN_LENGTH = 2  # one query is a decoding step (FusedDecodeAttention); from two on, one launch beats three
 
     @staticmethod
     def is_available(query, key, attention_mask=None, training=False, dropout_p=0.0):

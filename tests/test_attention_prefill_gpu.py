@@ -191,7 +191,8 @@ def test_prefill_operator_gate_and_errors():
     assert FusedPrefillAttention.is_available(q, q, mask)
     assert not FusedPrefillAttention.is_available(q, q, training=True, dropout_p=0.1)
     assert not FusedPrefillAttention.is_available(q.float(), q.float())
-    assert not FusedPrefillAttention.is_available(q[:, :, :64], q[:, :, :64])      # short prompt
+    assert FusedPrefillAttention.is_available(q[:, :, :5], q[:, :, :5])            # short prompts too
+    assert not FusedPrefillAttention.is_available(q[:, :, :1], q[:, :, :1])        # one query: a decoding step
     assert not FusedPrefillAttention.is_available(q[:, :, :128], q)                # a cache longer than the prompt
     assert not FusedPrefillAttention.is_available(q[..., :32], q[..., :32])        # head size
     assert not FusedPrefillAttention.is_available(q.requires_grad_(), q)
