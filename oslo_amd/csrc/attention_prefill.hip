@@ -421,34 +421,40 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
 }
 
 template <typename T, int D>
-void launch_prefill_dim(const PrefillArgs &a, hipStream_t stream) {
+int launch_prefill_dim(const PrefillArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)(8 * a.head_groups * a.query_blocks));
-  // head_dim 256 keeps Q^T in dynamic LDS: 128 queries x 256 features
+  // head_dim 256 keeps Q^T in dynamic LDS: 128 queries x 256 features. Static
+  // and dynamic LDS together exceed the 64 KiB a kernel gets unasked, so the
+  // limit is raised for the kernel (on the current device; a host-side
+  // setting, not a stream operation) before every launch.
   constexpr unsigned kDynamic = D == 256 ? kQueriesPerBlock * D * sizeof(T) : 0;
-  auto go = [&]<bool HAS_PAD, bool HAS_WINDOW>() {
+  auto go = [&]<bool HAS_PAD, bool HAS_WINDOW>() -> int {
     auto *kernel = attention_prefill_kernel<T, D, HAS_PAD, HAS_WINDOW>;
-    if (kDynamic > 0)
-      (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynamic);
+    if (kDynamic > 0) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynamic);
+      if (e != hipSuccess)
+        return fail(OSLO_E_LAUNCH, "oslo_attention_prefill_fwd: %u bytes of dynamic LDS refused: %s",
+                    kDynamic, hipGetErrorString(e));
+    }
     kernel<<<grid, dim3(kBlockThreads), kDynamic, stream>>>(a);
+    return check_launch("attention_prefill_fwd");
   };
   if (a.window > 0) {
-    if (a.pad != nullptr) go.template operator()<true, true>();
-    else go.template operator()<false, true>();
-  } else {
-    if (a.pad != nullptr) go.template operator()<true, false>();
-    else go.template operator()<false, false>();
+    if (a.pad != nullptr) return go.template operator()<true, true>();
+    return go.template operator()<false, true>();
   }
+  if (a.pad != nullptr) return go.template operator()<true, false>();
+  return go.template operator()<false, false>();
 }
 
 template <typename T>
 int launch_prefill(const PrefillArgs &a, int head_dim, hipStream_t stream) {
   switch (head_dim) {
-    case 64: launch_prefill_dim<T, 64>(a, stream); break;
-    case 128: launch_prefill_dim<T, 128>(a, stream); break;
-    default: launch_prefill_dim<T, 256>(a, stream); break;
+    case 64: return launch_prefill_dim<T, 64>(a, stream);
+    case 128: return launch_prefill_dim<T, 128>(a, stream);
+    default: return launch_prefill_dim<T, 256>(a, stream);
   }
-  return check_launch("attention_prefill_fwd");
 }
 
 } // namespace
