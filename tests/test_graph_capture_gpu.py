@@ -91,6 +91,32 @@ def test_captured_sequence_replays_like_eager():
             assert not torch.isnan(captured[name].float()).any(), f"replay {replay}: {name} not written"
 
 
+@pytest.mark.parametrize("d,padded", [(256, False), (64, True)])
+def test_prompt_attention_captured(d, padded):
+    """The one-kernel prompt attention under capture (at head_dim 256 its launcher
+    also raises the kernel's LDS limit, a host-side setting): replays on new
+    inputs equal the eager results."""
+    from oslo_amd import kernels
+
+    q, k, v = (torch.randn(2, 4, 300, d, device=DEV).bfloat16() for _ in range(3))
+    pad = None
+    if padded:
+        pad = torch.zeros(2, 300, device=DEV)
+        pad[1, 250:] = -10000.0
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = kernels.attention_prefill_forward(q, k, v, 0.0625, pad)
+    for replay in range(3):
+        for t in (q, k, v):
+            t.copy_(torch.randn_like(t))
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = kernels.attention_prefill_forward(q, k, v, 0.0625, pad)   # eager work between replays
+        assert torch.equal(out, eager), f"replay {replay} differs from eager"
+        assert torch.isfinite(out).all()
+
+
 @pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
 def test_graphed_forward_of_a_fused_model(family):
     """The whole fused forward captured once and replayed with new token ids and
