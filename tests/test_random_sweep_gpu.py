@@ -4,7 +4,9 @@ device with the same expression written in torch fp32 (float64 for the
 attention of a decoding step). It complements the oracle tests, which pin
 exact bars on chosen shapes, by covering shapes nobody chose: 250 draws here;
 the same loop was run for 4500 draws with other seeds without a failure (the
-attention over a whole prompt joined later, on a stream of draws of its own)."""
+attention over a whole prompt joined later, on a stream of draws of its own; a
+loop of that family alone, with left and right padding, windows and strided
+layouts, was run for 6900 draws without a failure)."""
 
 import random
 
