@@ -105,6 +105,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   extern __shared__ __align__(16) unsigned char dynamic_lds[];
   __shared__ __align__(16) T k_lds[kKeysPerTile * D];  // [key][chunk ^ (key & 7)][8]
   __shared__ __align__(16) T vt_lds[D * kKeysPerTile]; // [d][(slot + d + d/8) & 7][8]
+  __shared__ __align__(16) float pad_lds[HAS_PAD ? kKeysPerTile : 4]; // the tile's mask values, log2 units
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -168,7 +169,16 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   const bool v_task = tid < D;
   const int v_g = tid % kChunks, v_kg = tid / kChunks;
   u32x4 kreg[kLoadsK], vreg[8];
+  // the padding mask of a tile travels with it: 16 lanes take four keys each
+  // (keys at or past S read as 0; they only meet queries they are masked for)
+  const BufRsrc prs = make_rsrc(padr, HAS_PAD ? (uint32_t)S * (uint32_t)sizeof(float) : 0u);
+  float4 padreg = make_float4(0.f, 0.f, 0.f, 0.f);
   auto issue_loads = [&](int key0) {
+    if constexpr (HAS_PAD) {
+      if (tid < kKeysPerTile / 4)
+        padreg = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                prs, (uint32_t)(key0 + 4 * tid) * (uint32_t)sizeof(float), 0, 0));
+    }
 #pragma unroll
     for (int j = 0; j < kLoadsK; ++j)
       kreg[j] = __builtin_amdgcn_raw_buffer_load_b128(
@@ -182,6 +192,11 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
     }
   };
   auto store_tile = [&]() {
+    if constexpr (HAS_PAD) {
+      if (tid < kKeysPerTile / 4)
+        *reinterpret_cast<float4 *>(&pad_lds[4 * tid]) = make_float4(
+            padreg.x * kLog2e, padreg.y * kLog2e, padreg.z * kLog2e, padreg.w * kLog2e);
+    }
 #pragma unroll
     for (int j = 0; j < kLoadsK; ++j) {
       const int row = k_r0 + j * (kBlockThreads / kChunks);
@@ -265,12 +280,10 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
     float mt = -INFINITY;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int kj = keyb + 8 * j + 4 * half;
       float pv[4] = {0.f, 0.f, 0.f, 0.f};
       if constexpr (HAS_PAD) {
-        // keys at or past S only meet queries they are masked for
-        const float4 p4 = *reinterpret_cast<const float4 *>(padr + (kj < S ? kj : 0));
-        pv[0] = p4.x * kLog2e, pv[1] = p4.y * kLog2e, pv[2] = p4.z * kLog2e, pv[3] = p4.w * kLog2e;
+        const float4 p4 = *reinterpret_cast<const float4 *>(&pad_lds[32 * kb + 8 * j + 4 * half]);
+        pv[0] = p4.x, pv[1] = p4.y, pv[2] = p4.z, pv[3] = p4.w;
       }
 #pragma unroll
       for (int tt = 0; tt < 4; ++tt) {
