@@ -288,7 +288,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
 #pragma unroll
       for (int tt = 0; tt < 4; ++tt) {
         float x = sc[4 * j + tt];
-        if constexpr (HAS_PAD) x = x * a.scale_log2e + pv[tt];
+        if constexpr (HAS_PAD) x = __builtin_fmaf(x, a.scale_log2e, pv[tt]);
         sc[4 * j + tt] = x;
       }
     }
