@@ -395,13 +395,19 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         q, k, v = (randn((B, Hh, S, D), 50 + i, 1.0, torch.bfloat16) for i in range(3))
         o = torch.empty((B, S, Hh, D), dtype=torch.bfloat16, device=dev)
         strides = (ctypes.c_int64 * 12)(*(3 * [Hh * S * D, S * D, D] + [S * Hh * D, D, Hh * D]))
-        t = time_launches(lambda: check(lib.oslo_attention_prefill_fwd(
-            P(o), P(q), P(k), P(v), None, D ** -0.5, B, Hh, S, D, 0, strides, BF16, st)), max(5, n // 2), 3)
         flops = 4 * B * Hh * D * (S * (S + 1) // 2)
-        res.append({"kernel": f"attention_prefill bf16 [{B},{Hh},{S},{D}] causal", "bound": "mfma",
-                    "achieved": round(flops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "us": round(t * 1e6, 1),
-                    "algorithmic_flops": flops, "traffic": None})
+        lens = torch.randint(S // 2, S + 1, (B,), device=dev, generator=torch.Generator(device=dev).manual_seed(2))
+        key_pad = torch.where(torch.arange(S, device=dev)[None, :] < lens[:, None], 0.0, -10000.0).float().contiguous()
+        for what, mask in (("causal", None), ("causal with padding mask", key_pad)):
+            if mask is not None and D != 256:
+                continue
+            t = time_launches(lambda: check(lib.oslo_attention_prefill_fwd(
+                P(o), P(q), P(k), P(v), P(mask) if mask is not None else None, D ** -0.5, B, Hh, S, D, 0, strides,
+                BF16, st)), max(5, n // 2), 3)
+            res.append({"kernel": f"attention_prefill bf16 [{B},{Hh},{S},{D}] {what}", "bound": "mfma",
+                        "achieved": round(flops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                        "frac": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "us": round(t * 1e6, 1),
+                        "algorithmic_flops": flops, "traffic": None})
         del q, k, v, o
     return res
 
