@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   constexpr bool kQInLds = D == 256;
   constexpr bool kTwoLoops = D == 256; // see `step` below
   extern __shared__ __align__(16) unsigned char dynamic_lds[];
-  __shared__ __align__(16) T k_lds[kKeysPerTile * D];  // [key][chunk ^ (key & 7)][8]
+  __shared__ __align__(16) T k_lds[kKeysPerTile * D];  // [key][chunk ^ (key & kSwizzleK)][8]
   __shared__ __align__(16) T vt_lds[D * kKeysPerTile]; // [d][(slot + d + d/8) & 7][8]
   __shared__ __align__(16) float pad_lds[HAS_PAD ? kKeysPerTile : 4]; // the tile's mask values, log2 units
 
