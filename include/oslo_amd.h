@@ -227,6 +227,27 @@ int oslo_bias_gelu_bwd(void *dy, void *dbias, float *workspace, const void *g,
                        const void *y, const void *bias, int64_t rows,
                        int64_t cols, int dtype, oslo_stream_t stream);
 
+/*
+ * oslo_bias_gelu_bwd without the workspace argument: the fp32 partial rows of
+ * dbias go to a buffer of OSLO_STATIC_WORKSPACE_BYTES that is part of the
+ * library's device image (one copy per GPU, held until the process ends), so
+ * the caller needs no device allocation of its own for the call. Results are
+ * bit-identical to oslo_bias_gelu_bwd's. It has no counterpart in the
+ * reference; it is for callers that cannot allocate: code under HIP graph
+ * capture, serving loops and harnesses that forbid hipMalloc.
+ * Fails with OSLO_E_UNSUPPORTED when dbias != NULL and
+ * oslo_colsum_workspace_bytes(rows, cols) exceeds the buffer ([16384, 16384]
+ * is the largest square problem that fits). The first call on a device looks
+ * the buffer's address up (that loads the library's device image if nothing
+ * has yet): make one call, of any size, before a graph capture begins. All
+ * calls on a GPU share the one buffer: calls that may overlap there (different
+ * streams, different threads) race; order them or use oslo_bias_gelu_bwd.
+ */
+#define OSLO_STATIC_WORKSPACE_BYTES (32u << 20)
+int oslo_bias_gelu_bwd_static(void *dy, void *dbias, const void *g,
+                              const void *y, const void *bias, int64_t rows,
+                              int64_t cols, int dtype, oslo_stream_t stream);
+
 /* Bias + dropout (+ residual) ----------------------------------------------- */
 
 /*

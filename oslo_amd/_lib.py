@@ -42,6 +42,8 @@ PROTOTYPES = {
     "oslo_colsum_workspace_bytes": (_c.c_size_t, [_I64, _I64]),
     "oslo_bias_gelu_bwd": (
         _c.c_int, [_P, _P, _P, _P, _P, _P, _I64, _I64, _c.c_int, _P]),
+    "oslo_bias_gelu_bwd_static": (
+        _c.c_int, [_P, _P, _P, _P, _P, _I64, _I64, _c.c_int, _P]),
     "oslo_bias_dropout_add_fwd": (
         _c.c_int, [_P, _P, _P, _P, _c.c_float, _U64, _U64, _I64, _I64, _c.c_int, _P]),
     "oslo_bias_dropout_add_bwd": (

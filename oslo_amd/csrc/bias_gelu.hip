@@ -5,8 +5,18 @@
 // the bias gradient (a column sum), which the reference leaves to a separate
 // full-tensor reduction by autograd (oslo/fused_kernels_utils.py:376-380).
 
+#include <mutex>
+
 #include "elementwise.hpp"
 #include "gelu.hpp"
+
+// Device memory of the entry point that takes no workspace argument
+// (oslo_bias_gelu_bwd_static): the fp32 partial rows of the bias gradient live
+// here instead of in a caller's buffer. Every GPU the library runs on holds its
+// own copy of this array, at its own address, until the process ends. In host
+// code the name is only a handle for hipGetSymbolAddress; kernels get the
+// address that call returns.
+static __device__ __align__(256) float scratch[OSLO_STATIC_WORKSPACE_BYTES / sizeof(float)];
 
 namespace oslo {
 namespace {
@@ -111,6 +121,30 @@ int launch_bwd(T *dy, T *dbias, float *ws, const T *g, const T *y,
   return check_launch("bias_gelu_bwd");
 }
 
+// Address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float *g_scratch_ptr[kMaxDevices];
+
+int static_scratch(float **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return fail(OSLO_E_LAUNCH, "bias_gelu_bwd_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(OSLO_E_UNSUPPORTED, "bias_gelu_bwd_static: device %d, at most %d are tracked", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    float *p = nullptr;
+    e = hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return fail(OSLO_E_LAUNCH, "bias_gelu_bwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return OSLO_OK;
+}
+
 } // namespace
 } // namespace oslo
 
@@ -168,4 +202,27 @@ extern "C" int oslo_bias_gelu_bwd(void *dy, void *dbias, float *workspace,
                : launch_bwd<T, 1>(d, db, workspace, gg, yy, bb, rows, cols, st);
   });
   return OSLO_OK;
+}
+
+extern "C" int oslo_bias_gelu_bwd_static(void *dy, void *dbias, const void *g,
+                                         const void *y, const void *bias,
+                                         int64_t rows, int64_t cols, int dtype,
+                                         oslo_stream_t stream) {
+  using namespace oslo;
+  if (rows < 0 || cols < 0)
+    return fail(OSLO_E_BAD_ARG, "bias_gelu_bwd_static: negative size");
+  const size_t need = dbias ? oslo_colsum_workspace_bytes(rows, cols) : 0;
+  if (need > (size_t)OSLO_STATIC_WORKSPACE_BYTES)
+    return fail(OSLO_E_UNSUPPORTED,
+                "bias_gelu_bwd_static: [%lld, %lld] needs %zu bytes of workspace, the static "
+                "buffer holds %zu; use oslo_bias_gelu_bwd with a workspace of the caller",
+                (long long)rows, (long long)cols, need, (size_t)OSLO_STATIC_WORKSPACE_BYTES);
+  float *ws = nullptr;
+  if (dbias) {
+    const int s = static_scratch(&ws);
+    if (s != OSLO_OK) return s;
+  }
+  // Every partial row the finishing sum reads is written by this call's first
+  // kernel, so nothing in the buffer has to start at zero.
+  return oslo_bias_gelu_bwd(dy, dbias, ws, g, y, bias, rows, cols, dtype, stream);
 }
