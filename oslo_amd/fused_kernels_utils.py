@@ -21,6 +21,7 @@ Differences from the reference, all widening:
 """
 
 import inspect
+import threading
 import weakref
 
 import torch
@@ -197,32 +198,37 @@ def _key_mask_bytes(pad_mask):
     return pad_mask if pad_mask.dtype == torch.bool else pad_mask != 0
 
 
-_pad_cache = None  # (weakref to the mask, its version, the fp32 [B, Sk] form)
+_pad_cache = threading.local()  # .entry = (weakref to the mask, its version, the fp32 [B, Sk] form)
 
 
 def _pad_additive_f32(pad_mask, bsz, sk):
     """[B or 1, 1, 1, Sk] mask (bool/uint8: True = padded -> -10000; float:
     additive as given) -> fp32 [B, Sk]. Every layer of a model passes the same
-    mask tensor, so the last conversion is kept and reused while that tensor is
-    alive and unmodified."""
-    global _pad_cache
-    if _pad_cache is not None:
-        ref, version, converted = _pad_cache
-        if ref() is pad_mask and pad_mask._version == version and tuple(converted.shape) == (bsz, sk):
-            return converted
+    mask tensor, so the calling thread's last conversion is kept and reused
+    while that tensor is alive and unmodified. A tensor created under
+    ``torch.inference_mode()`` has no version counter, so an in-place change
+    of it could not be noticed: such masks are converted on every call."""
     if pad_mask.dim() != 4 or pad_mask.shape[1] != 1 or pad_mask.shape[2] != 1 \
             or pad_mask.shape[3] != sk or pad_mask.shape[0] not in (1, bsz):
         raise RuntimeError(
             "FusedScaleMaskSoftmax: with use_triang_mask the pad_mask must be "
             f"[batch or 1, 1, 1, {sk}], got {tuple(pad_mask.shape)}"
         )
+    cacheable = not pad_mask.is_inference()
+    if cacheable:
+        entry = getattr(_pad_cache, "entry", None)
+        if entry is not None:
+            ref, version, converted = entry
+            if ref() is pad_mask and pad_mask._version == version and tuple(converted.shape) == (bsz, sk):
+                return converted
     m = pad_mask.reshape(pad_mask.shape[0], sk)
     if m.dtype in (torch.bool, torch.uint8):
         m = m.to(torch.float32) * -10000.0
     else:
         m = m.to(torch.float32)
     m = m.expand(bsz, sk).contiguous()
-    _pad_cache = (weakref.ref(pad_mask), pad_mask._version, m)
+    if cacheable:
+        _pad_cache.entry = (weakref.ref(pad_mask), pad_mask._version, m)
     return m
 
 

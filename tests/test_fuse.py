@@ -81,6 +81,36 @@ def test_pad_mask_shape_is_checked():
         FusedScaleMaskSoftmax.apply(torch.randn(2, 2, 8, 8), torch.zeros(2, 1, 8, 8), 1.0, True)
 
 
+def test_pad_mask_conversion_on_the_host():
+    """The [B,1,1,Sk] -> fp32 [B,Sk] conversion needs no device: bool and float
+    forms, broadcasting over the batch, reuse while the tensor is unchanged, a
+    fresh conversion after an in-place change, and masks made under
+    torch.inference_mode(), which have no version counter to consult."""
+    from oslo_amd import fused_kernels_utils as fku
+    m = torch.zeros(2, 1, 1, 8)
+    m[1, :, :, 5:] = -10000.0
+    a = fku._pad_additive_f32(m, 2, 8)
+    assert a.dtype == torch.float32 and torch.equal(a, m.view(2, 8))
+    assert fku._pad_additive_f32(m, 2, 8) is a
+    m[0, :, :, 2:] = -10000.0
+    b = fku._pad_additive_f32(m, 2, 8)
+    assert b is not a and torch.equal(b, m.view(2, 8))
+    bm = torch.zeros(1, 1, 1, 8, dtype=torch.bool)
+    bm[..., 6:] = True
+    c = fku._pad_additive_f32(bm, 3, 8)
+    assert c.shape == (3, 8) and torch.equal(c[2], torch.tensor([0.0] * 6 + [-10000.0] * 2))
+    with torch.inference_mode():
+        im = torch.zeros(2, 1, 1, 8)
+        im[0, :, :, 4:] = -10000.0
+        d = fku._pad_additive_f32(im, 2, 8)
+        assert torch.equal(d, im.view(2, 8))
+        im[1, :, :, 1:] = -10000.0          # invisible to a version counter: must not be served from a cache
+        assert torch.equal(fku._pad_additive_f32(im, 2, 8), im.view(2, 8))
+    # a malformed mask is rejected even when a well-formed one was converted just before
+    with pytest.raises(RuntimeError, match="pad_mask"):
+        fku._pad_additive_f32(torch.zeros(2, 1, 8, 8), 2, 8)
+
+
 @pytest.mark.parametrize("make,mods,fused", [
     (tiny_gpt2, (modeling_gpt2.GPT2Attention, modeling_gpt2.GPT2MLP),
      (modeling_gpt2.FusedGPT2Attention, modeling_gpt2.FusedGPT2MLP)),

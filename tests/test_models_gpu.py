@@ -293,12 +293,47 @@ def test_padding_mask_conversion_is_reused_and_invalidated():
     mask = torch.zeros(b, 1, 1, s, device=DEV)
     mask[1, :, :, 40:] = -10000.0
     y1 = FusedScaleMaskSoftmax.apply(x, mask, 0.5, True)
-    first = fku._pad_cache[2]
+    first = fku._pad_cache.entry[2]
     y2 = FusedScaleMaskSoftmax.apply(x, mask, 0.5, True)
-    assert fku._pad_cache[2] is first and torch.equal(y1, y2)      # same tensor, unmodified: reused
+    assert fku._pad_cache.entry[2] is first and torch.equal(y1, y2)      # same tensor, unmodified: reused
     mask[0, :, :, 10:] = -10000.0                                    # in-place change bumps the version
     y3 = FusedScaleMaskSoftmax.apply(x, mask, 0.5, True)
-    assert fku._pad_cache[2] is not first
+    assert fku._pad_cache.entry[2] is not first
     want = torch.softmax((x * 0.5 + mask).masked_fill(
         ~torch.tril(torch.ones(s, s, dtype=torch.bool, device=DEV)), float("-inf")), -1)
     assert (y3 - want).abs().max().item() <= 1e-6
+
+
+def test_padding_mask_under_inference_mode_and_interleaved_masks():
+    """A mask created under torch.inference_mode() has no version counter; the
+    conversion must not ask for one. Two masks used in turn must never see each
+    other's conversion."""
+    b, h, s = 2, 2, 64
+    tril = torch.tril(torch.ones(s, s, dtype=torch.bool, device=DEV))
+    with torch.inference_mode():
+        x = torch.randn(b, h, s, s, device=DEV)
+        m1 = torch.zeros(b, 1, 1, s, device=DEV)
+        m1[1, :, :, 40:] = -10000.0
+        m2 = torch.zeros(b, 1, 1, s, device=DEV)
+        m2[0, :, :, 7:] = -10000.0
+        for mask in (m1, m2, m1, m2):
+            y = FusedScaleMaskSoftmax.apply(x, mask, 0.5, True)
+            want = torch.softmax((x * 0.5 + mask).masked_fill(~tril, float("-inf")), -1)
+            assert (y - want).abs().max().item() <= 1e-6
+        m1[0, :, :, 3:] = -10000.0           # in place, invisible to any version counter
+        y = FusedScaleMaskSoftmax.apply(x, m1, 0.5, True)
+        want = torch.softmax((x * 0.5 + m1).masked_fill(~tril, float("-inf")), -1)
+        assert (y - want).abs().max().item() <= 1e-6
+        yw = fku.FusedScaleMaskWindowSoftmax.apply(x, m2, 0.5, 16)
+        band = tril & ~torch.tril(torch.ones(s, s, dtype=torch.bool, device=DEV), -16)
+        want = torch.softmax((x * 0.5 + m2).masked_fill(~band, float("-inf")), -1)
+        assert (yw - want).abs().max().item() <= 1e-6
+    n1 = torch.zeros(b, 1, 1, s, device=DEV)
+    n1[1, :, :, 20:] = -10000.0
+    n2 = torch.zeros(b, 1, 1, s, device=DEV)
+    n2[0, :, :, 50:] = -10000.0
+    xx = x.clone()
+    for mask in (n1, n2, n1, n2):
+        y = FusedScaleMaskSoftmax.apply(xx, mask, 0.5, True)
+        want = torch.softmax((xx * 0.5 + mask).masked_fill(~tril, float("-inf")), -1)
+        assert (y - want).abs().max().item() <= 1e-6
