@@ -273,12 +273,14 @@ def dropout_threshold(p):
     return 0xFFFF if t >= 65535.0 else int(t)
 
 
-def dropout_bits(seed, offset, n):
-    """The 16 random bits of elements 0..n-1: element i owns the low (i even)
-    or high (i odd) half of word (i mod 8) // 2 of Philox4x32-10 with
-    key = seed and counter = (offset // 4 as 64 bits, i // 8 as 64 bits)."""
+def dropout_bits(seed, offset, n, start=0):
+    """The 16 random bits of elements start..start+n-1 (start a multiple of 8):
+    element i owns the low (i even) or high (i odd) half of word (i mod 8) // 2
+    of Philox4x32-10 with key = seed and counter = (offset // 4 as 64 bits,
+    i // 8 as 64 bits)."""
+    assert start % 8 == 0
     groups = (n + 7) // 8
-    g = np.arange(groups, dtype=np.uint64)
+    g = np.arange(groups, dtype=np.uint64) + np.uint64(start // 8)
     block = np.uint64(offset // 4)
     c0 = np.full(groups, block & _LO, dtype=np.uint64).astype(np.uint32)
     c1 = np.full(groups, block >> _S32, dtype=np.uint64).astype(np.uint32)
@@ -290,9 +292,9 @@ def dropout_bits(seed, offset, n):
     return halves.reshape(-1)[:n]
 
 
-def dropout_keep_mask(seed, offset, n, p):
-    """keep[i], i in [0, n): the element's 16 bits >= floor(p * 2^16)."""
-    return dropout_bits(seed, offset, n) >= np.uint32(dropout_threshold(p))
+def dropout_keep_mask(seed, offset, n, p, start=0):
+    """keep[i], i in [start, start + n): the element's 16 bits >= floor(p * 2^16)."""
+    return dropout_bits(seed, offset, n, start) >= np.uint32(dropout_threshold(p))
 
 
 def bias_dropout_add_fwd(x, bias, residual, p, keep, dtype=np.float32):

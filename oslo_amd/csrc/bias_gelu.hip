@@ -21,7 +21,7 @@ static __device__ __align__(256) float scratch[OSLO_STATIC_WORKSPACE_BYTES / siz
 namespace oslo {
 namespace {
 
-template <typename T, int VEC, int U>
+template <typename T, int VEC, int U, bool NT>
 __global__ __launch_bounds__(kBlockThreads) void bias_gelu_fwd_kernel(
     T *out, const T *y, const T *__restrict__ bias, int64_t rows, int64_t cols,
     int col_tiles, int rows_per_block) {
@@ -31,7 +31,7 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_fwd_kernel(
   RawVec<T, VEC> raw[U];
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    raw[u] = buffer_load_raw<T, VEC, true>(yrs, ew_offset<T>(pos, u, cols));
+    raw[u] = buffer_load_raw<T, VEC, NT>(yrs, ew_offset<T>(pos, u, cols));
   float b[VEC];
   load_f32_cached<T, VEC>(b, bias + pos.c0);
   // rows past the end were read as zeros and their stores are dropped by the
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_fwd_kernel(
   }
 }
 
-template <typename T, int VEC, int U, bool WANT_DBIAS>
+template <typename T, int VEC, int U, bool WANT_DBIAS, bool NT>
 __global__ __launch_bounds__(kBlockThreads) void bias_gelu_bwd_kernel(
     T *dy, float *__restrict__ partial, const T *g, const T *y,
     const T *__restrict__ bias, int64_t rows, int64_t cols, int col_tiles,
@@ -63,8 +63,8 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_bwd_kernel(
     RawVec<T, VEC> graw[U], yraw[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      graw[u] = buffer_load_raw<T, VEC, true>(grs, ew_offset<T>(pos, u, cols));
-      yraw[u] = buffer_load_raw<T, VEC, true>(yrs, ew_offset<T>(pos, u, cols));
+      graw[u] = buffer_load_raw<T, VEC, NT>(grs, ew_offset<T>(pos, u, cols));
+      yraw[u] = buffer_load_raw<T, VEC, NT>(yrs, ew_offset<T>(pos, u, cols));
     }
     float b[VEC];
     load_f32_cached<T, VEC>(b, bias + pos.c0);
@@ -96,8 +96,12 @@ int launch_fwd(T *out, const T *y, const T *bias, int64_t rows, int64_t cols,
                hipStream_t stream) {
   const EwPlan p = plan_elementwise(rows, cols / VEC, kFwdMaxTx, kFwdUnroll);
   if (!p.ok) return fail(OSLO_E_UNSUPPORTED, "bias_gelu_fwd: tensor too large for one launch");
-  bias_gelu_fwd_kernel<T, VEC, kFwdUnroll><<<p.grid, p.block, 0, stream>>>(
-      out, y, bias, rows, cols, p.col_tiles, p.rows_per_block);
+  if (stream_loads(2 * rows * cols * (int64_t)sizeof(T)))
+    bias_gelu_fwd_kernel<T, VEC, kFwdUnroll, true><<<p.grid, p.block, 0, stream>>>(
+        out, y, bias, rows, cols, p.col_tiles, p.rows_per_block);
+  else
+    bias_gelu_fwd_kernel<T, VEC, kFwdUnroll, false><<<p.grid, p.block, 0, stream>>>(
+        out, y, bias, rows, cols, p.col_tiles, p.rows_per_block);
   return check_launch("bias_gelu_fwd");
 }
 
@@ -106,18 +110,22 @@ int launch_bwd(T *dy, T *dbias, float *ws, const T *g, const T *y,
                const T *bias, int64_t rows, int64_t cols, hipStream_t stream) {
   const EwPlan p = plan_elementwise(rows, cols / VEC, kBwdMaxTx, kGeluBwdUnroll);
   if (!p.ok) return fail(OSLO_E_UNSUPPORTED, "bias_gelu_bwd: tensor too large for one launch");
+  auto go = [&]<bool WANT, bool NT>() {
+    bias_gelu_bwd_kernel<T, VEC, kGeluBwdUnroll, WANT, NT>
+        <<<p.grid, p.block, 0, stream>>>(dy, WANT ? ws : nullptr, g, y, bias, rows,
+                                         cols, p.col_tiles, p.rows_per_block);
+  };
+  const bool nt = stream_loads(3 * rows * cols * (int64_t)sizeof(T));
   if (dbias) {
-    bias_gelu_bwd_kernel<T, VEC, kGeluBwdUnroll, true>
-        <<<p.grid, p.block, 0, stream>>>(dy, ws, g, y, bias, rows, cols,
-                                         p.col_tiles, p.rows_per_block);
+    if (nt) go.template operator()<true, true>();
+    else go.template operator()<true, false>();
     int s = check_launch("bias_gelu_bwd");
     if (s != OSLO_OK) return s;
     launch_colsum_finish<T>(dbias, ws, p.row_blocks, cols, stream);
     return check_launch("bias_gelu_bwd(dbias)");
   }
-  bias_gelu_bwd_kernel<T, VEC, kGeluBwdUnroll, false>
-      <<<p.grid, p.block, 0, stream>>>(dy, nullptr, g, y, bias, rows, cols,
-                                       p.col_tiles, p.rows_per_block);
+  if (nt) go.template operator()<false, true>();
+  else go.template operator()<false, false>();
   return check_launch("bias_gelu_bwd");
 }
 

@@ -29,6 +29,17 @@ constexpr int kBwdMaxTx = 32;  // backward kernels: narrower and taller tiles,
 constexpr int kBwdMinUnroll = 4;
 constexpr int kBwdMinRowsPerBlock = kBlockThreads / kBwdMaxTx * kBwdMinUnroll;
 
+// Cache policy of the loads. MI355X has a 256 MB memory-side cache in front of
+// HBM. Tensors far larger than it gain nothing there and are read with
+// non-temporal loads (a scaled copy of [16384,16384] bf16: 159 us against
+// 167-172 us with plain loads). Tensors that fit were usually just written by
+// the kernel before (a GEMM's output, the forward's activations) and a good
+// part of them is still in that cache: there plain loads are faster (the same
+// copy at [16384,4096]: 38.2 us against 43.1 us non-temporal).
+inline bool stream_loads(int64_t bytes_loaded) {
+  return bytes_loaded > (256ll << 20);
+}
+
 struct EwPlan {
   dim3 grid, block;
   int rows_per_block;

@@ -5,7 +5,7 @@
 
 #include <stdint.h>
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define OSLO_HD __host__ __device__ __forceinline__
 #else
 #define OSLO_HD inline

@@ -3,6 +3,8 @@ computes (dropout off), forward and backward, with and without padding, in the
 dtypes the families run in; and the operator API behaves like torch ops under
 autograd and the device generator."""
 
+import copy
+
 import numpy as np
 import pytest
 import torch
@@ -28,9 +30,13 @@ def models():
     }
 
 
-# logits are O(1); fused and unfused differ by the rounding of 16-bit
-# intermediates (the unfused path rounds after every operator)
-LOGIT_TOL = {torch.float32: 2e-4, torch.float16: 2e-2, torch.bfloat16: 1.5e-1}
+# In fp32 fused and unfused logits (O(1)) agree to 2e-4. In 16-bit the two
+# round at different places (the unfused path after every operator), so they
+# are both measured against the unfused model run in fp32 on the same weights:
+# the fused model may be no further from it than the unfused 16-bit model is
+# (1.5x on the maximum, which for these tiny models is a noisy statistic; 1.1x
+# on the mean).
+LOGIT_TOL_FP32 = 2e-4
 
 
 @pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
@@ -45,14 +51,20 @@ def test_fused_model_matches_unfused(family, dtype, padded):
         mask = torch.ones(3, 96, device=DEV)
         mask[1, 60:] = 0
         mask[2, 17:] = 0
+    keep = torch.ones(3, 96, dtype=torch.bool, device=DEV) if mask is None else mask.bool()
     with torch.no_grad():
         want = m(ids, attention_mask=mask)["logits"].float()
+        ref = None if dtype == torch.float32 else copy.deepcopy(m).float()(ids, attention_mask=mask)["logits"]
         m.fuse()
         got = m(ids, attention_mask=mask)["logits"].float()
     assert torch.isfinite(got).all()
-    keep = torch.ones(3, 96, dtype=torch.bool, device=DEV) if mask is None else mask.bool()
-    err = (got - want).abs()[keep].max().item()     # rows of padded queries are not compared
-    assert err <= LOGIT_TOL[dtype], f"{family} {dtype}: logits differ by {err}"
+    if dtype == torch.float32:
+        err = (got - want).abs()[keep].max().item()     # rows of padded queries are not compared
+        assert err <= LOGIT_TOL_FP32, f"{family} {dtype}: logits differ by {err}"
+        return
+    err_f, err_u = (got - ref).abs()[keep], (want - ref).abs()[keep]
+    assert err_f.max().item() <= 1.5 * err_u.max().item(), (family, dtype, err_f.max().item(), err_u.max().item())
+    assert err_f.mean().item() <= 1.1 * err_u.mean().item(), (family, dtype, err_f.mean().item(), err_u.mean().item())
 
 
 @pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
@@ -87,14 +99,22 @@ def test_prompt_attention_runs_as_one_kernel_at_inference(family, dtype, padded,
         want = m(ids, attention_mask=mask, use_cache=True)
         step_mask = None if mask is None else torch.cat([mask, torch.ones(3, 1, device=DEV)], dim=1)
         want_step = m(ids[:, :1], attention_mask=step_mask, past_key_values=want["past_key_values"])["logits"]
+        m32 = copy.deepcopy(m).float()
+        ref = m32(ids, attention_mask=mask, use_cache=True)
+        ref_step = m32(ids[:, :1], attention_mask=step_mask, past_key_values=ref["past_key_values"])["logits"]
         m.fuse()
         got = m(ids, attention_mask=mask, use_cache=True)
         got_step = m(ids[:, :1], attention_mask=step_mask, past_key_values=got["past_key_values"])["logits"]
     assert calls == [(3, 4, 160, 64)] * 2
     keep = torch.ones(3, 160, dtype=torch.bool, device=DEV) if mask is None else mask.bool()
-    err = (got["logits"].float() - want["logits"].float()).abs()[keep].max().item()
-    assert err <= LOGIT_TOL[dtype], f"{family} {dtype}: logits differ by {err}"
-    assert (got_step.float() - want_step.float()).abs().max().item() <= LOGIT_TOL[dtype]
+    # fused and unfused 16-bit logits against the unfused fp32 model on the same weights
+    err_f = (got["logits"].float() - ref["logits"]).abs()[keep]
+    err_u = (want["logits"].float() - ref["logits"]).abs()[keep]
+    assert err_f.max().item() <= 1.5 * err_u.max().item(), (family, dtype, err_f.max().item(), err_u.max().item())
+    assert err_f.mean().item() <= 1.1 * err_u.mean().item(), (family, dtype, err_f.mean().item(), err_u.mean().item())
+    step_f = (got_step.float() - ref_step).abs()
+    step_u = (want_step.float() - ref_step).abs()
+    assert step_f.max().item() <= 1.5 * step_u.max().item() and step_f.mean().item() <= 1.1 * step_u.mean().item()
     # with gradients recorded the three-launch path (which has a backward) is taken
     calls.clear()
     m(ids, attention_mask=mask)

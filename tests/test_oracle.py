@@ -290,6 +290,10 @@ def test_dropout_mask_statistics_and_thresholds():
     assert (orc.dropout_keep_mask(1234, 4, n, p) != keep).mean() > 0.1
     assert (orc.dropout_keep_mask(1235, 0, n, p) != keep).mean() > 0.1
     assert np.array_equal(orc.dropout_keep_mask(1234, 0, n, p), keep)
+    # a band of the mask asked for by its first element equals that band of the whole
+    assert np.array_equal(orc.dropout_keep_mask(1234, 0, 1000, p, start=4096), keep[4096:5096])
+    assert np.array_equal(orc.dropout_bits(1234, 8, 24, start=(1 << 35) + 8),
+                          orc.dropout_bits(1234, 8, (1 << 3) + 24, start=1 << 35)[8:])
 
 
 def test_bias_dropout_add_closed_forms():
