@@ -447,6 +447,56 @@ int oslo_attention_prefill_fwd(void *out, const void *q, const void *k,
                                const int64_t *strides, int dtype,
                                oslo_stream_t stream);
 
+/*
+ * oslo_attention_prefill_fwd that also stores what its backward needs:
+ * lse[b*heads + h, i] (fp32, [batch*heads, S], 16-byte aligned) = log2 of
+ * sum_s 2^(log2(e) * (scale*q.k + pad)) over the visible keys of query i.
+ * The forward a training step runs (oslo/models/gptj/modeling_gptj.py:936-951
+ * with gradients recorded).
+ */
+int oslo_attention_prefill_fwd_lse(void *out, float *lse, const void *q,
+                                   const void *k, const void *v,
+                                   const float *pad, float scale, int64_t batch,
+                                   int64_t heads, int64_t S, int64_t head_dim,
+                                   int64_t window, const int64_t *strides,
+                                   int dtype, oslo_stream_t stream);
+
+/* Bytes of fp32 workspace oslo_attention_prefill_bwd needs. */
+size_t oslo_attention_prefill_bwd_workspace_bytes(int64_t batch, int64_t heads,
+                                                  int64_t S);
+
+/*
+ * Backward of the causal prompt attention: from the gradient dout of the
+ * output, the inputs q, k, v, the forward's out and lse
+ * (oslo_attention_prefill_fwd_lse), with P[i,s] = 2^(log2(e)*(scale*q_i.k_s +
+ * pad[s]) - lse[i]) over the visible keys,
+ *   dv[s] = sum_i P[i,s] dout[i]
+ *   dS[i,s] = scale * P[i,s] * (dout[i].v[s] - sum_d dout[i,d]*out[i,d])
+ *   dq[i] = sum_s dS[i,s] k[s],   dk[s] = sum_i dS[i,s] q[i].
+ * strides[24]: batch, head and position strides, in elements, of q, k, v, out,
+ * dout, dq, dk, dv in that order (the limits of oslo_attention_prefill_fwd).
+ * P and dS are rounded to the storage type before the products that sum over
+ * them, every sum is fp32, each gradient is rounded once. No [S, S] tensor is
+ * read or written; nothing is accumulated with atomics, so the result is the
+ * same from run to run. workspace: oslo_attention_prefill_bwd_workspace_bytes
+ * bytes (16-byte aligned), contents irrelevant before and after. No output may
+ * alias an input.
+ * Replaces what autograd records for matmul(q, k^T) ->
+ * FusedScaleMaskSoftmax.apply -> matmul(probs, v) of the fused attention in a
+ * training step (oslo/models/gptj/modeling_gptj.py:936-951,
+ *  oslo/models/gpt_neo/modeling_gpt_neo.py:993-1008,
+ *  oslo/models/gpt2/modeling_gpt2.py:1435-1459): two matmul backwards around
+ * the softmax kernel's backward, all on [B, H, S, S] tensors.
+ */
+int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const void *dout,
+                               const void *q, const void *k, const void *v,
+                               const void *out, const float *lse,
+                               float *workspace, const float *pad, float scale,
+                               int64_t batch, int64_t heads, int64_t S,
+                               int64_t head_dim, int64_t window,
+                               const int64_t *strides, int dtype,
+                               oslo_stream_t stream);
+
 /* Repeated n-gram blocking (beam search) ------------------------------------ */
 
 /*

@@ -52,6 +52,10 @@ root):
   by torch.nn.functional.scaled_dot_product_attention, by the closed form for
   equal scores -- the running mean of the values -- and by attention_decode
   on the last row);
+* attention_prefill_bwd: what autograd derives for those operators (pinned by
+  torch.autograd through torch.nn.functional.scaled_dot_product_attention in
+  float64, by central differences of attention_prefill, and by the identities
+  sum_k dS = 0 per row and dV = dO for a single position);
 * build_sample_idx / build_blending_indices:
   oslo/fused_kernels/bindings/pybind_datasets.cpp:35-160 (pinned by the closed
   form "sample k starts at token k*seq_length", the share bound of the
@@ -222,6 +226,37 @@ def attention_prefill(q, k, v, scale, pad=None, dtype=np.float64):
             e = np.exp(scores - scores.max())
             out[b, i] = (e / e.sum()) @ v[b, :i + 1]
     return out
+
+
+def attention_prefill_bwd(q, k, v, dout, scale, pad=None, window=None, dtype=np.float64):
+    """Gradients of attention_prefill (with GPT-Neo's sliding window if given:
+    row i attends keys i - window < s <= i) for the upstream gradient dout:
+    q, k, v, dout [n, S, d] -> (dq, dk, dv). With P the probabilities,
+    dV = P^T dO, dP = dO V^T, dS = P o (dP - rowsum(dP o P)), dQ = scale dS K,
+    dK = scale dS^T Q: what autograd derives for the matmul, softmax, matmul
+    of oslo/models/gptj/modeling_gptj.py:151-191."""
+    q, k, v, dout = (np.asarray(t, dtype=dtype) for t in (q, k, v, dout))
+    n, S, _ = q.shape
+    if pad is not None:
+        pad = np.broadcast_to(np.asarray(pad, dtype=dtype), (n, S))
+    i = np.arange(S)
+    visible = i[None, :] <= i[:, None]
+    if window is not None and window > 0:
+        visible &= i[None, :] > i[:, None] - int(window)
+    dq, dk, dv = np.zeros_like(q), np.zeros_like(k), np.zeros_like(v)
+    for b in range(n):
+        scores = scale * (q[b] @ k[b].T)
+        if pad is not None:
+            scores = scores + pad[b][None, :]
+        scores = np.where(visible, scores, -np.inf)
+        e = np.exp(scores - scores.max(axis=1, keepdims=True))
+        p = e / e.sum(axis=1, keepdims=True)
+        dv[b] = p.T @ dout[b]
+        dp = dout[b] @ v[b].T
+        ds = p * (dp - (dp * p).sum(axis=1, keepdims=True))
+        dq[b] = scale * (ds @ k[b])
+        dk[b] = scale * (ds.T @ q[b])
+    return dq, dk, dv
 
 
 def bias_gelu_bwd(g, y, bias, dtype=np.float32):

@@ -30,6 +30,7 @@ SOURCES = [
     "linear_rows.hip",
     "attention_decode.hip",
     "attention_prefill.hip",
+    "attention_prefill_bwd.hip",
     "dataset_index.hip",
 ]
 

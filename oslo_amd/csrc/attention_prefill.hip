@@ -33,7 +33,7 @@
 // tile of keys is taken in two steps of 32, each a step of the running
 // softmax, and the next tile's global loads are in flight meanwhile.
 
-#include "common.hpp"
+#include "attention.hpp"
 
 namespace oslo {
 namespace {
@@ -43,30 +43,11 @@ constexpr int kKeysPerTile = 64;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kSlack = 8.0f; // see the kernel: how far a score may exceed the reference maximum
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-template <typename T>
-struct MatrixOp;
-template <>
-struct MatrixOp<bf16> {
-  typedef bf16 Frag __attribute__((ext_vector_type(8)));
-  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-};
-template <>
-struct MatrixOp<f16> {
-  typedef f16 Frag __attribute__((ext_vector_type(8)));
-  static __device__ __forceinline__ f32x16 run(Frag a, Frag b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  }
-};
-
 struct PrefillArgs {
   void *out;
   const void *q, *k, *v;
   const float *pad; // [batch, S] additive, or null
+  float *lse;       // [batch * heads, S] or null: log2 of the row's sum of exponentials
   int64_t q_b, q_h, q_s; // element strides: batch, head, position
   int64_t k_b, k_h, k_s;
   int64_t v_b, v_h, v_s;
@@ -79,10 +60,6 @@ struct PrefillArgs {
   int query_blocks;
   int window; // 0: every key up to the query; else the last `window` of them
 };
-
-__device__ __forceinline__ float other_half(float v) {
-  return __shfl_xor(v, 32, kWave);
-}
 
 template <typename T, int D, bool HAS_PAD, bool HAS_WINDOW>
 __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_prefill_kernel(
@@ -195,7 +172,8 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
     if constexpr (HAS_PAD) {
       if (tid < kKeysPerTile / 4)
         *reinterpret_cast<float4 *>(&pad_lds[4 * tid]) = make_float4(
-            padreg.x * kLog2e, padreg.y * kLog2e, padreg.z * kLog2e, padreg.w * kLog2e);
+            fmaxf(padreg.x * kLog2e, kMaskFloorLog2), fmaxf(padreg.y * kLog2e, kMaskFloorLog2),
+            fmaxf(padreg.z * kLog2e, kMaskFloorLog2), fmaxf(padreg.w * kLog2e, kMaskFloorLog2));
     }
 #pragma unroll
     for (int j = 0; j < kLoadsK; ++j) {
@@ -420,6 +398,8 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   l += other_half(l);
   const float inv = 1.0f / l;
   if (qrow >= S) return;
+  if (a.lse != nullptr && half == 0)
+    a.lse[(int64_t)bh * S + qrow] = m + __builtin_amdgcn_logf(l); // v_log_f32 is log2
   T *op = static_cast<T *>(a.out) + b * a.o_b + hd * a.o_h + (int64_t)qrow * a.o_s;
   typedef T Out4 __attribute__((ext_vector_type(4)));
 #pragma unroll
@@ -473,13 +453,11 @@ int launch_prefill(const PrefillArgs &a, int head_dim, hipStream_t stream) {
 } // namespace
 } // namespace oslo
 
-extern "C" int oslo_attention_prefill_fwd(void *out, const void *q, const void *k,
-                                          const void *v, const float *pad,
-                                          float scale, int64_t batch, int64_t heads,
-                                          int64_t S, int64_t head_dim,
-                                          int64_t window,
-                                          const int64_t *strides, int dtype,
-                                          oslo_stream_t stream) {
+namespace {
+int prefill_entry(void *out, float *lse, const void *q, const void *k, const void *v,
+                  const float *pad, float scale, int64_t batch, int64_t heads,
+                  int64_t S, int64_t head_dim, int64_t window,
+                  const int64_t *strides, int dtype, oslo_stream_t stream) {
   using namespace oslo;
   if (batch < 0 || heads < 0 || S < 0 || head_dim < 0 || window < 0)
     return fail(OSLO_E_BAD_ARG, "oslo_attention_prefill_fwd: negative size");
@@ -516,7 +494,7 @@ extern "C" int oslo_attention_prefill_fwd(void *out, const void *q, const void *
     return fail(OSLO_E_UNSUPPORTED,
                 "oslo_attention_prefill_fwd: with a padding mask S must be a multiple of 4 and the mask 16-byte aligned");
   PrefillArgs a;
-  a.out = out, a.q = q, a.k = k, a.v = v, a.pad = pad;
+  a.out = out, a.q = q, a.k = k, a.v = v, a.pad = pad, a.lse = lse;
   a.q_b = strides[0], a.q_h = strides[1], a.q_s = strides[2];
   a.k_b = strides[3], a.k_h = strides[4], a.k_s = strides[5];
   a.v_b = strides[6], a.v_h = strides[7], a.v_s = strides[8];
@@ -533,4 +511,29 @@ extern "C" int oslo_attention_prefill_fwd(void *out, const void *q, const void *
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == OSLO_F16) return launch_prefill<f16>(a, (int)head_dim, st);
   return launch_prefill<bf16>(a, (int)head_dim, st);
+}
+} // namespace
+
+extern "C" int oslo_attention_prefill_fwd(void *out, const void *q, const void *k,
+                                          const void *v, const float *pad,
+                                          float scale, int64_t batch, int64_t heads,
+                                          int64_t S, int64_t head_dim,
+                                          int64_t window,
+                                          const int64_t *strides, int dtype,
+                                          oslo_stream_t stream) {
+  return prefill_entry(out, nullptr, q, k, v, pad, scale, batch, heads, S, head_dim,
+                       window, strides, dtype, stream);
+}
+
+extern "C" int oslo_attention_prefill_fwd_lse(void *out, float *lse, const void *q,
+                                              const void *k, const void *v,
+                                              const float *pad, float scale,
+                                              int64_t batch, int64_t heads, int64_t S,
+                                              int64_t head_dim, int64_t window,
+                                              const int64_t *strides, int dtype,
+                                              oslo_stream_t stream) {
+  if (lse == nullptr && batch > 0 && heads > 0 && S > 0)
+    return oslo::fail(OSLO_E_BAD_ARG, "oslo_attention_prefill_fwd_lse: null lse");
+  return prefill_entry(out, lse, q, k, v, pad, scale, batch, heads, S, head_dim,
+                       window, strides, dtype, stream);
 }

@@ -1,0 +1,592 @@
+// Backward of the one-kernel causal prompt attention (attention_prefill.hip):
+// dQ, dK and dV from Q, K, V, dO, the forward's output O and the log-sum-exp
+// of every row, without the [S, S] matrices in memory. With
+//   P  = exp2(scale*log2e * Q K^T + pad*log2e - lse)      (the probabilities)
+//   dP = dO V^T,   delta[q] = sum_d dO[q,d] * O[q,d]
+//   dS = scale * P o (dP - delta)
+// the gradients are dV = P^T dO, dQ = dS K, dK = dS^T Q. It replaces, for
+// training, the backward of the three launches of the reference's fused
+// attention (oslo/models/gptj/modeling_gptj.py:936-951: matmul, softmax
+// kernel, matmul, differentiated by autograd), which keeps the probabilities
+// and their gradient as [B, H, S, S] tensors.
+//
+// One kernel template serves every gradient. A block owns 128 positions (32
+// per wave, one per lane of each half) and walks over the positions of the
+// other kind in tiles: for dQ it owns queries and walks the keys up to the
+// diagonal, for dK and dV it owns keys and walks the queries from the
+// diagonal on. Both score-like products put the own position in the lane:
+//   T1[other, own] = Other1 (A operand, LDS, rows = other) x Own1^T (B, fixed)
+//   T2[other, own] = Other2 (A operand, LDS)               x Own2^T (B, fixed)
+// (dQ: T1 = K Q^T = S^T, T2 = V dO^T = dP^T; dK/dV: T1 = Q K^T = S, T2 = dO V^T
+// = dP), so P and dS come out in the accumulator layout of
+// v_mfma_f32_32x32x16, which is also the B-operand layout of the accumulating
+// products
+//   Acc^T[d, own] += OtherT (A operand, LDS, rows = features) x X[other, own]
+// (dQ^T += K^T dS^T; dK^T += Q^T dS; dV^T += dO^T P) once the contraction
+// order is permuted the way the forward does it for V^T. Quantities indexed by
+// the own position are per-lane scalars, those indexed by the other position
+// are read per tile from LDS. Each block sums in a fixed order and no two
+// blocks write the same element: the gradients are deterministic. The price is
+// that scores are computed twice (once per owner kind), 7 matrix products per
+// visible (query, key) tile instead of 5.
+
+#include "attention.hpp"
+
+namespace oslo {
+namespace {
+
+constexpr int kOwnPerBlock = 128;
+constexpr float kLog2eB = 1.4426950408889634f;
+
+enum Role { kRoleDQ = 0, kRoleDKV = 1, kRoleDK = 2, kRoleDV = 3 };
+
+struct Strides3 {
+  int64_t b, h, s; // element strides: batch, head, position
+};
+
+struct BwdArgs {
+  const void *q, *k, *v, *dout;
+  void *dq, *dk, *dv;
+  const float *lse;   // [batch * heads, S], log2 units, from the forward
+  const float *delta; // [batch * heads, S]
+  const float *pad;   // [batch, S] additive, or null
+  Strides3 sq, sk, sv, sdo, sdq, sdk, sdv;
+  float scale, scale_log2e;
+  int S, heads, batch_heads, head_groups, own_blocks, window;
+};
+
+template <int D>
+constexpr int tile_positions() { return D == 256 ? 32 : 64; }
+
+// Bytes of dynamic LDS a role needs.
+template <typename T, int D, int ROLE>
+constexpr unsigned bwd_lds_bytes() {
+  constexpr int kTile = tile_positions<D>();
+  constexpr unsigned tile = kTile * D * sizeof(T);
+  unsigned n = tile;                                   // Other1, natural
+  if (ROLE != kRoleDV) n += tile;                      // Other2, natural
+  if (ROLE != kRoleDV) n += tile;                      // OtherT for the dS product
+  if (ROLE == kRoleDKV || ROLE == kRoleDV) n += tile;  // OtherT for the P product
+  n += 2 * kTile * sizeof(float);                      // per-position values of the tile
+  if (D == 256) n += kOwnPerBlock * D * sizeof(T);     // Own1 operands
+  return n;
+}
+
+template <typename T, int D, int ROLE, bool HAS_PAD, bool HAS_WINDOW>
+__global__ __launch_bounds__(kBlockThreads, D == 64 && ROLE != kRoleDKV ? 2 : 1) void attention_bwd_kernel(
+    const BwdArgs a) {
+  using Op = MatrixOp<T>;
+  using Frag = typename Op::Frag;
+  constexpr bool kKeysOwn = ROLE != kRoleDQ;
+  constexpr bool kNeedT2 = ROLE != kRoleDV;
+  constexpr bool kAccS = ROLE != kRoleDV;
+  constexpr bool kAccP = ROLE == kRoleDKV || ROLE == kRoleDV;
+  constexpr int kTile = tile_positions<D>();
+  constexpr int kStepsPerTile = kTile / 32;
+  constexpr int kChunks = D / 8;   // 16-byte chunks of a position
+  constexpr int kSteps = D / 16;   // contraction steps over the features
+  constexpr int kBlocksD = D / 32; // 32-row blocks of an accumulator
+  constexpr int kTChunks = kTile / 8;
+  constexpr int kLoadsN = kTile * kChunks / kBlockThreads; // per thread, natural tile
+  constexpr int kRowsPerPass = kBlockThreads / kChunks;
+  constexpr int kSwizzleN = kChunks >= 16 ? 15 : 7;
+  constexpr int kTasks = kTChunks * kChunks; // 8 x 8 transpositions per tile
+  constexpr bool kOwn1InLds = D == 256;
+
+  // Dynamic LDS: the tiles the role needs, the per-position values of a tile,
+  // and (head_dim 256) the Own1 operands, each wave its own 16 KiB.
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  constexpr int kTileElems = kTile * D;
+  constexpr int kOffO2 = kTileElems;
+  constexpr int kOffTs = kOffO2 + (kNeedT2 ? kTileElems : 0);
+  constexpr int kOffTp = kOffTs + (kAccS ? kTileElems : 0);
+  constexpr int kOffEnd = kOffTp + (kAccP ? kTileElems : 0);
+  static_assert(kOffEnd * sizeof(T) + 2 * kTile * sizeof(float) +
+                        (kOwn1InLds ? kOwnPerBlock * D * sizeof(T) : 0) ==
+                    bwd_lds_bytes<T, D, ROLE>(),
+                "LDS layout and size disagree");
+  T *const o1_lds = reinterpret_cast<T *>(lds_raw);
+  T *const o2_lds = o1_lds + kOffO2;
+  T *const ts_lds = o1_lds + kOffTs;
+  T *const tp_lds = o1_lds + kOffTp;
+  float *const row_a = reinterpret_cast<float *>(o1_lds + kOffEnd);
+  float *const row_b = row_a + kTile;
+  u32x4 *const own1_lds = reinterpret_cast<u32x4 *>(row_b + kTile);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int half = lane >> 5;
+  const int col = lane & 31;
+
+  // All blocks of a head run on one XCD (its q, k, v, dO stay in that L2); the
+  // blocks with the most tiles start first.
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  const int bh = xcd + 8 * (slot % a.head_groups);
+  const int idx = slot / a.head_groups;
+  const int own_block = kKeysOwn ? idx : a.own_blocks - 1 - idx;
+  if (bh >= a.batch_heads) return; // the whole block
+  const int b = bh / a.heads;
+  const int hd = bh - b * a.heads;
+  const int S = a.S;
+  const int own0 = own_block * kOwnPerBlock;
+  const int wave_own0 = own0 + 32 * wave;
+  const int own = wave_own0 + col;
+  const int window = HAS_WINDOW ? a.window : 0;
+
+  auto slice = [&](const void *p, const Strides3 &st) {
+    return static_cast<const T *>(p) + b * st.b + hd * st.h;
+  };
+  auto bound = [&](const T *p, const Strides3 &st) {
+    // rows at or past S fall outside the descriptor and read as zeros
+    return make_rsrc(p, (uint32_t)(((int64_t)(S - 1) * st.s + D) * sizeof(T)));
+  };
+  // Own1 / Own2: B operands of T1 / T2. Other1 / Other2: their A operands.
+  // OtherS / OtherP: what the dS / P products contract with.
+  const Strides3 &st_own1 = kKeysOwn ? a.sk : a.sq;
+  const Strides3 &st_own2 = kKeysOwn ? a.sv : a.sdo;
+  const Strides3 &st_o1 = kKeysOwn ? a.sq : a.sk;
+  const Strides3 &st_o2 = kKeysOwn ? a.sdo : a.sv;
+  const BufRsrc own1_rs = bound(slice(kKeysOwn ? a.k : a.q, st_own1), st_own1);
+  const BufRsrc own2_rs = bound(slice(kKeysOwn ? a.v : a.dout, st_own2), st_own2);
+  const BufRsrc o1_rs = bound(slice(kKeysOwn ? a.q : a.k, st_o1), st_o1);
+  const BufRsrc o2_rs = bound(slice(kKeysOwn ? a.dout : a.v, st_o2), st_o2);
+  const uint32_t own1_row = (uint32_t)st_own1.s * sizeof(T);
+  const uint32_t own2_row = (uint32_t)st_own2.s * sizeof(T);
+  const uint32_t o1_row = (uint32_t)st_o1.s * sizeof(T);
+  const uint32_t o2_row = (uint32_t)st_o2.s * sizeof(T);
+
+  // B operands of the own positions: lane (position, half) holds features
+  // 16 s + 8 half .. + 7 of its position
+  Frag own1[kOwn1InLds ? 1 : kSteps];
+  Frag own2[kNeedT2 ? kSteps : 1];
+  u32x4 *own1_mine = own1_lds + wave * kSteps * kWave + lane;
+  {
+    u32x4 tmp[kSteps];
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s)
+      tmp[s] = __builtin_amdgcn_raw_buffer_load_b128(
+          own1_rs, (uint32_t)own * own1_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0);
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+      if constexpr (kOwn1InLds) own1_mine[s * kWave] = tmp[s];
+      else own1[s] = __builtin_bit_cast(Frag, tmp[s]);
+    }
+  }
+  if constexpr (kNeedT2) {
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s)
+      own2[s] = __builtin_bit_cast(
+          Frag, __builtin_amdgcn_raw_buffer_load_b128(
+                    own2_rs, (uint32_t)own * own2_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0));
+  }
+
+  // Per-lane values of the own position: for a query its log-sum-exp and
+  // delta, for a key its padding value (log2 units).
+  const int64_t stat_row = (int64_t)bh * S;
+  float own_lse = 0.f, own_delta = 0.f, own_pad = 0.f;
+  if constexpr (!kKeysOwn) {
+    if (own < S) {
+      own_lse = a.lse[stat_row + own];
+      own_delta = a.delta[stat_row + own];
+    }
+  } else if constexpr (HAS_PAD) {
+    if (own < S) own_pad = fmaxf(a.pad[(int64_t)b * S + own] * kLog2eB, kMaskFloorLog2);
+  }
+
+  // Per-position values of a tile of the other kind travel with the tile: for
+  // keys the padding value (row_a), for queries log-sum-exp (row_a) and delta
+  // (row_b). Positions at or past S read as zeros, which is harmless: their
+  // q and dO rows (or k and v rows) are zeros too and a key past the end is
+  // behind the causal mask of every query.
+  const BufRsrc ra_rs = kKeysOwn ? make_rsrc(a.lse + stat_row, (uint32_t)S * 4u)
+                                 : make_rsrc(HAS_PAD ? a.pad + (int64_t)b * S : nullptr,
+                                             HAS_PAD ? (uint32_t)S * 4u : 0u);
+  const BufRsrc rb_rs = make_rsrc(kKeysOwn ? a.delta + stat_row : nullptr, kKeysOwn ? (uint32_t)S * 4u : 0u);
+  constexpr bool kRowA = kKeysOwn || HAS_PAD;
+
+  const int n_ch = tid % kChunks, n_r0 = tid / kChunks;
+  const bool t_task = tid < kTasks;
+  const int t_g = tid % kChunks, t_kg = tid / kChunks;
+  u32x4 n1reg[kLoadsN], n2reg[kNeedT2 ? kLoadsN : 1], tsreg[kAccS ? 8 : 1], tpreg[kAccP ? 8 : 1];
+  float4 rareg = make_float4(0.f, 0.f, 0.f, 0.f), rbreg = rareg;
+
+  auto issue_loads = [&](int pos0) {
+    if (tid < kTile / 4) {
+      // S % 4 may be non-zero only without a padding mask, and lse / delta are
+      // allocated by the caller for whole rows: the 16-byte loads stay aligned
+      // because S rows start at multiples of S floats only when S % 4 == 0;
+      // otherwise take the values one by one
+      if constexpr (kRowA) {
+        if ((S & 3) == 0) {
+          rareg = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                 ra_rs, (uint32_t)(pos0 + 4 * tid) * 4u, 0, 0));
+        } else {
+          rareg.x = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ra_rs, (uint32_t)(pos0 + 4 * tid) * 4u, 0, 0));
+          rareg.y = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ra_rs, (uint32_t)(pos0 + 4 * tid + 1) * 4u, 0, 0));
+          rareg.z = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ra_rs, (uint32_t)(pos0 + 4 * tid + 2) * 4u, 0, 0));
+          rareg.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ra_rs, (uint32_t)(pos0 + 4 * tid + 3) * 4u, 0, 0));
+        }
+      }
+      if constexpr (kKeysOwn) {
+        if ((S & 3) == 0) {
+          rbreg = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                 rb_rs, (uint32_t)(pos0 + 4 * tid) * 4u, 0, 0));
+        } else {
+          rbreg.x = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb_rs, (uint32_t)(pos0 + 4 * tid) * 4u, 0, 0));
+          rbreg.y = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb_rs, (uint32_t)(pos0 + 4 * tid + 1) * 4u, 0, 0));
+          rbreg.z = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb_rs, (uint32_t)(pos0 + 4 * tid + 2) * 4u, 0, 0));
+          rbreg.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb_rs, (uint32_t)(pos0 + 4 * tid + 3) * 4u, 0, 0));
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kLoadsN; ++j) {
+      const uint32_t row = (uint32_t)(pos0 + n_r0 + j * kRowsPerPass);
+      n1reg[j] = __builtin_amdgcn_raw_buffer_load_b128(o1_rs, row * o1_row + (uint32_t)n_ch * 16u, 0, 0);
+      if constexpr (kNeedT2)
+        n2reg[j] = __builtin_amdgcn_raw_buffer_load_b128(o2_rs, row * o2_row + (uint32_t)n_ch * 16u, 0, 0);
+    }
+    if (t_task) {
+      // a task: the 8 positions of contraction chunk t_kg (positions
+      // 16 u + 8 jj + 4 h + t for chunk 2 u + h) x 8 features
+      const int pbase = pos0 + 16 * (t_kg >> 1) + 4 * (t_kg & 1);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t row = (uint32_t)(pbase + 8 * (i >> 2) + (i & 3));
+        // the dS product contracts with Other1's tensor (K or Q), the P
+        // product with Other2's (dO)
+        if constexpr (kAccS)
+          tsreg[i] = __builtin_amdgcn_raw_buffer_load_b128(o1_rs, row * o1_row + (uint32_t)t_g * 16u, 0, 0);
+        if constexpr (kAccP)
+          tpreg[i] = __builtin_amdgcn_raw_buffer_load_b128(o2_rs, row * o2_row + (uint32_t)t_g * 16u, 0, 0);
+      }
+    }
+  };
+  auto transpose_into = [&](T *dst, const u32x4 (&src)[8]) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { // 8 x 8 transposition of 16-bit values
+      u32x4 tr;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const uint32_t lo = src[2 * w][e >> 1], hi = src[2 * w + 1][e >> 1];
+        tr[w] = (e & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+      }
+      const int d = 8 * t_g + e;
+      *reinterpret_cast<u32x4 *>(&dst[(d * kTChunks + ((t_kg + e + t_g) & (kTChunks - 1))) * 8]) = tr;
+    }
+  };
+  auto store_tile = [&]() {
+    if (tid < kTile / 4) {
+      if constexpr (kKeysOwn) {
+        *reinterpret_cast<float4 *>(&row_a[4 * tid]) = rareg;
+        *reinterpret_cast<float4 *>(&row_b[4 * tid]) = rbreg;
+      } else if constexpr (HAS_PAD) {
+        *reinterpret_cast<float4 *>(&row_a[4 * tid]) = make_float4(
+            fmaxf(rareg.x * kLog2eB, kMaskFloorLog2), fmaxf(rareg.y * kLog2eB, kMaskFloorLog2),
+            fmaxf(rareg.z * kLog2eB, kMaskFloorLog2), fmaxf(rareg.w * kLog2eB, kMaskFloorLog2));
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kLoadsN; ++j) {
+      const int row = n_r0 + j * kRowsPerPass;
+      const int at = (row * kChunks + (n_ch ^ (row & kSwizzleN))) * 8;
+      *reinterpret_cast<u32x4 *>(&o1_lds[at]) = n1reg[j];
+      if constexpr (kNeedT2) *reinterpret_cast<u32x4 *>(&o2_lds[at]) = n2reg[j];
+    }
+    if (t_task) {
+      if constexpr (kAccS) transpose_into(ts_lds, tsreg);
+      if constexpr (kAccP) transpose_into(tp_lds, tpreg);
+    }
+  };
+
+  f32x16 acc_s[kAccS ? kBlocksD : 1], acc_p[kAccP ? kBlocksD : 1];
+#pragma unroll
+  for (int i = 0; i < (kAccS ? kBlocksD : 1); ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc_s[i][r] = 0.f;
+#pragma unroll
+  for (int i = 0; i < (kAccP ? kBlocksD : 1); ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc_p[i][r] = 0.f;
+
+  // Tiles of the other kind this block walks.
+  int first_tile, tiles;
+  if constexpr (!kKeysOwn) {
+    const int last_key = (own0 + kOwnPerBlock < S ? own0 + kOwnPerBlock : S) - 1;
+    tiles = last_key / kTile + 1;
+    first_tile = HAS_WINDOW && own0 - window + 1 > 0 ? (own0 - window + 1) / kTile : 0;
+  } else {
+    first_tile = own0 / kTile;
+    int last_q = S - 1;
+    if (HAS_WINDOW && own0 + kOwnPerBlock - 1 + window - 1 < last_q) last_q = own0 + kOwnPerBlock - 1 + window - 1;
+    tiles = last_q / kTile + 1;
+  }
+
+  // One step: 32 positions of the other kind against the wave's 32 own ones.
+  auto step = [&](int pos0, int kb) {
+    const int ob = pos0 + 32 * kb;
+    bool diagonal;
+    if constexpr (!kKeysOwn) { // other = keys ob .. ob+31, own = queries
+      if (ob > wave_own0 + 31) return;                                  // every key is ahead of the wave's queries
+      if (HAS_WINDOW && ob + 31 <= wave_own0 - window) return;          // or behind their windows
+      diagonal = ob + 31 > wave_own0 || (HAS_WINDOW && ob <= wave_own0 + 31 - window);
+    } else { // other = queries ob .. ob+31, own = keys
+      if (ob + 31 < wave_own0) return;                                  // every query is before the wave's keys
+      if (HAS_WINDOW && ob >= wave_own0 + 31 + window) return;          // or past their windows
+      diagonal = ob < wave_own0 + 31 || (HAS_WINDOW && ob + 31 >= wave_own0 + window);
+    }
+
+    f32x16 t1, t2;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) t1[r] = t2[r] = 0.f;
+    const int orow = 32 * kb + col;
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+      const int at = (orow * kChunks + ((2 * s + half) ^ (orow & kSwizzleN))) * 8;
+      const Frag f1 = *reinterpret_cast<const Frag *>(&o1_lds[at]);
+      if constexpr (kOwn1InLds)
+        t1 = Op::run(f1, __builtin_bit_cast(Frag, own1_mine[s * kWave]), t1);
+      else
+        t1 = Op::run(f1, own1[s], t1);
+      if constexpr (kNeedT2) {
+        const Frag f2 = *reinterpret_cast<const Frag *>(&o2_lds[at]);
+        t2 = Op::run(f2, own2[s], t2);
+      }
+    }
+
+    // P = exp2(scale*log2e * T1 + pad - lse); dS = scale * P * (T2 - delta)
+    float p[16], ds[16];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float ra[4] = {0.f, 0.f, 0.f, 0.f}, rb[4] = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (kRowA) {
+        const float4 v4 = *reinterpret_cast<const float4 *>(&row_a[32 * kb + 8 * j + 4 * half]);
+        ra[0] = v4.x, ra[1] = v4.y, ra[2] = v4.z, ra[3] = v4.w;
+      }
+      if constexpr (kKeysOwn) {
+        const float4 v4 = *reinterpret_cast<const float4 *>(&row_b[32 * kb + 8 * j + 4 * half]);
+        rb[0] = v4.x, rb[1] = v4.y, rb[2] = v4.z, rb[3] = v4.w;
+      }
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) {
+        const int r = 4 * j + tt;
+        // keys own: pad of the lane, lse and delta of the row; queries own: the reverse
+        const float shift = kKeysOwn ? own_pad - ra[tt] : ra[tt] - own_lse;
+        p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(t1[r], a.scale_log2e, shift));
+        if constexpr (kNeedT2) ds[r] = t2[r] - (kKeysOwn ? rb[tt] : own_delta);
+      }
+    }
+    if (diagonal) {
+      asm volatile(""); // a branch of its own: only the tiles at the diagonal (and the window's edge) compare
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int other = ob + 8 * (r >> 2) + 4 * half + (r & 3);
+        const int key = kKeysOwn ? own : other, query = kKeysOwn ? other : own;
+        const bool visible = key <= query && (!HAS_WINDOW || key > query - window);
+        p[r] = visible ? p[r] : 0.f;
+      }
+    }
+    Frag pf[2], sf[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        pf[u][i] = static_cast<T>(p[8 * u + i]);
+        if constexpr (kNeedT2) sf[u][i] = static_cast<T>(a.scale * (p[8 * u + i] * ds[8 * u + i]));
+      }
+
+    // Acc^T += OtherT x X, 16 positions of the step at a time
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int i = 0; i < kBlocksD; ++i) {
+        const int d = 32 * i + col;
+        const int at = (d * kTChunks + ((4 * kb + 2 * u + half + d + (d >> 3)) & (kTChunks - 1))) * 8;
+        if constexpr (kAccS)
+          acc_s[i] = Op::run(*reinterpret_cast<const Frag *>(&ts_lds[at]), sf[u], acc_s[i]);
+        if constexpr (kAccP)
+          acc_p[i] = Op::run(*reinterpret_cast<const Frag *>(&tp_lds[at]), pf[u], acc_p[i]);
+      }
+    }
+  };
+
+  issue_loads(first_tile * kTile);
+  for (int t = first_tile; t < tiles; ++t) {
+    const int pos0 = t * kTile;
+    __syncthreads(); // the reads of the previous tile are done
+    store_tile();
+    __syncthreads();
+    if (t + 1 < tiles) issue_loads(pos0 + kTile);
+#pragma unroll
+    for (int kb = 0; kb < kStepsPerTile; ++kb) step(pos0, kb);
+  }
+
+  if (own >= S) return;
+  typedef T Out4 __attribute__((ext_vector_type(4)));
+  auto write = [&](void *base, const Strides3 &st, const f32x16 (&acc)[kBlocksD]) {
+    T *op = static_cast<T *>(base) + b * st.b + hd * st.h + (int64_t)own * st.s;
+#pragma unroll
+    for (int i = 0; i < kBlocksD; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        Out4 w;
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(acc[i][4 * j + tt]);
+        *reinterpret_cast<Out4 *>(op + 32 * i + 8 * j + 4 * half) = w;
+      }
+  };
+  if constexpr (ROLE == kRoleDQ) write(a.dq, a.sdq, acc_s);
+  if constexpr (ROLE == kRoleDKV || ROLE == kRoleDK) write(a.dk, a.sdk, acc_s);
+  if constexpr (ROLE == kRoleDKV || ROLE == kRoleDV) write(a.dv, a.sdv, acc_p);
+}
+
+// delta[bh, q] = sum_d dO[q, d] * O[q, d], fp32. D / 8 lanes share a row.
+template <typename T, int D>
+__global__ __launch_bounds__(kBlockThreads) void attention_delta_kernel(
+    float *delta, const T *out, const T *dout, Strides3 so, Strides3 sdo, int S,
+    int heads, int64_t rows) {
+  constexpr int kLanes = D / 8;
+  constexpr int kRows = kBlockThreads / kLanes;
+  int64_t row = (int64_t)blockIdx.x * kRows + threadIdx.x / kLanes;
+  const bool live = row < rows;
+  if (!live) row = rows - 1; // the lanes of a group stay together for the reduction
+  const int part = threadIdx.x % kLanes;
+  const int64_t bh = row / S;
+  const int q = (int)(row - bh * S);
+  const int64_t b = bh / heads, hd = bh - b * heads;
+  typedef T Vec8 __attribute__((ext_vector_type(8)));
+  const Vec8 o = *reinterpret_cast<const Vec8 *>(out + b * so.b + hd * so.h + (int64_t)q * so.s + 8 * part);
+  const Vec8 g = *reinterpret_cast<const Vec8 *>(dout + b * sdo.b + hd * sdo.h + (int64_t)q * sdo.s + 8 * part);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s = __builtin_fmaf(static_cast<float>(o[i]), static_cast<float>(g[i]), s);
+  s = sum_over_lanes<kLanes>(s);
+  if (live && part == 0) delta[row] = s;
+}
+
+template <typename T, int D, int ROLE>
+int launch_role(const BwdArgs &a, hipStream_t stream) {
+  const dim3 grid((unsigned)(8 * a.head_groups * a.own_blocks));
+  constexpr unsigned kLds = bwd_lds_bytes<T, D, ROLE>();
+  auto go = [&]<bool HAS_PAD, bool HAS_WINDOW>() -> int {
+    auto *kernel = attention_bwd_kernel<T, D, ROLE, HAS_PAD, HAS_WINDOW>;
+    if (kLds > 48 * 1024) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
+      if (e != hipSuccess)
+        return fail(OSLO_E_LAUNCH, "oslo_attention_prefill_bwd: %u bytes of dynamic LDS refused: %s", kLds,
+                    hipGetErrorString(e));
+    }
+    kernel<<<grid, dim3(kBlockThreads), kLds, stream>>>(a);
+    return check_launch("attention_prefill_bwd");
+  };
+  if (a.window > 0) {
+    if (a.pad != nullptr) return go.template operator()<true, true>();
+    return go.template operator()<false, true>();
+  }
+  if (a.pad != nullptr) return go.template operator()<true, false>();
+  return go.template operator()<false, false>();
+}
+
+template <typename T, int D>
+int launch_bwd_dim(const BwdArgs &a, float *delta, const void *out, const Strides3 &so,
+                   hipStream_t stream) {
+  const int64_t rows = (int64_t)a.batch_heads * a.S;
+  constexpr int kRows = kBlockThreads / (D / 8);
+  attention_delta_kernel<T, D><<<dim3((unsigned)((rows + kRows - 1) / kRows)), dim3(kBlockThreads), 0, stream>>>(
+      delta, static_cast<const T *>(out), static_cast<const T *>(a.dout), so, a.sdo, a.S, a.heads, rows);
+  int s = check_launch("attention_prefill_bwd(delta)");
+  if (s != OSLO_OK) return s;
+  s = launch_role<T, D, kRoleDQ>(a, stream);
+  if (s != OSLO_OK) return s;
+  if constexpr (D == 256) {
+    // two accumulators of 128 registers per lane do not fit beside the
+    // operands: dK and dV take a pass each
+    s = launch_role<T, D, kRoleDK>(a, stream);
+    if (s != OSLO_OK) return s;
+    return launch_role<T, D, kRoleDV>(a, stream);
+  } else {
+    return launch_role<T, D, kRoleDKV>(a, stream);
+  }
+}
+
+template <typename T>
+int launch_bwd(const BwdArgs &a, float *delta, const void *out, const Strides3 &so, int head_dim,
+               hipStream_t stream) {
+  switch (head_dim) {
+    case 64: return launch_bwd_dim<T, 64>(a, delta, out, so, stream);
+    case 128: return launch_bwd_dim<T, 128>(a, delta, out, so, stream);
+    default: return launch_bwd_dim<T, 256>(a, delta, out, so, stream);
+  }
+}
+
+} // namespace
+} // namespace oslo
+
+extern "C" size_t oslo_attention_prefill_bwd_workspace_bytes(int64_t batch, int64_t heads, int64_t S) {
+  if (batch <= 0 || heads <= 0 || S <= 0) return 0;
+  return (size_t)batch * (size_t)heads * (size_t)S * sizeof(float);
+}
+
+extern "C" int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const void *dout,
+                                          const void *q, const void *k, const void *v,
+                                          const void *out, const float *lse,
+                                          float *workspace, const float *pad, float scale,
+                                          int64_t batch, int64_t heads, int64_t S,
+                                          int64_t head_dim, int64_t window,
+                                          const int64_t *strides, int dtype,
+                                          oslo_stream_t stream) {
+  using namespace oslo;
+  const char *name = "oslo_attention_prefill_bwd";
+  if (batch < 0 || heads < 0 || S < 0 || head_dim < 0 || window < 0)
+    return fail(OSLO_E_BAD_ARG, "%s: negative size", name);
+  if (dtype != OSLO_F16 && dtype != OSLO_BF16) {
+    if (dtype == OSLO_F32) return fail(OSLO_E_UNSUPPORTED, "%s: fp16 and bf16 are taken, not fp32", name);
+    return fail(OSLO_E_BAD_ARG, "unknown dtype %d", dtype);
+  }
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+    return fail(OSLO_E_UNSUPPORTED, "%s: heads of %lld features (64, 128 or 256 are taken)", name,
+                (long long)head_dim);
+  if (!(scale > 0.0f)) return fail(OSLO_E_BAD_ARG, "%s: the scale must be positive", name);
+  if (batch == 0 || heads == 0 || S == 0) return OSLO_OK;
+  if (!dq || !dk || !dv || !dout || !q || !k || !v || !out || !lse || !workspace || !strides)
+    return fail(OSLO_E_BAD_ARG, "%s: null pointer", name);
+  if (batch * heads > (int64_t)0x7fffffff / 8 || batch * heads * S > (int64_t)0x7fffffff)
+    return fail(OSLO_E_UNSUPPORTED, "%s: too many rows for one launch", name);
+  // strides: q, k, v, out, dout, dq, dk, dv (batch, head, position each)
+  const void *ptrs[8] = {q, k, v, out, dout, dq, dk, dv};
+  for (int i = 0; i < 8; ++i) {
+    if (!aligned16(ptrs[i])) return fail(OSLO_E_UNSUPPORTED, "%s: tensors must be 16-byte aligned", name);
+    const int64_t sb = strides[3 * i], sh = strides[3 * i + 1], ss = strides[3 * i + 2];
+    if (sb < 0 || sh < 0 || ss < head_dim || sb % 8 || sh % 8 || ss % 8)
+      return fail(OSLO_E_UNSUPPORTED,
+                  "%s: strides must be multiples of 8 elements, the position stride at least head_dim", name);
+    if ((S + kOwnPerBlock) * ss * 2 > (int64_t)0x7fffffff)
+      return fail(OSLO_E_UNSUPPORTED, "%s: a head's slice exceeds 2 GiB", name);
+  }
+  if (pad != nullptr && (S % 4 != 0 || !aligned16(pad)))
+    return fail(OSLO_E_UNSUPPORTED,
+                "%s: with a padding mask S must be a multiple of 4 and the mask 16-byte aligned", name);
+  if (!aligned16(lse) || !aligned16(workspace))
+    return fail(OSLO_E_UNSUPPORTED, "%s: lse and workspace must be 16-byte aligned", name);
+  auto st = [&](int i) { return Strides3{strides[3 * i], strides[3 * i + 1], strides[3 * i + 2]}; };
+  BwdArgs a;
+  a.q = q, a.k = k, a.v = v, a.dout = dout, a.dq = dq, a.dk = dk, a.dv = dv;
+  a.lse = lse, a.delta = workspace, a.pad = pad;
+  a.sq = st(0), a.sk = st(1), a.sv = st(2), a.sdo = st(4), a.sdq = st(5), a.sdk = st(6), a.sdv = st(7);
+  a.scale = scale;
+  a.scale_log2e = scale * kLog2eB;
+  a.S = (int)S;
+  a.heads = (int)heads;
+  a.batch_heads = (int)(batch * heads);
+  a.head_groups = (a.batch_heads + 7) / 8;
+  a.own_blocks = (int)((S + kOwnPerBlock - 1) / kOwnPerBlock);
+  a.window = window >= S ? 0 : (int)window;
+  if ((int64_t)8 * a.head_groups * a.own_blocks > (int64_t)0x7fffffff)
+    return fail(OSLO_E_UNSUPPORTED, "%s: too many blocks for one launch", name);
+  hipStream_t stm = static_cast<hipStream_t>(stream);
+  if (dtype == OSLO_F16) return launch_bwd<f16>(a, workspace, out, st(3), (int)head_dim, stm);
+  return launch_bwd<bf16>(a, workspace, out, st(3), (int)head_dim, stm);
+}

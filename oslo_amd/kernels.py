@@ -579,15 +579,7 @@ def attention_decode_forward(query, key, value, pos, scale, window=0, new_key=No
 PREFILL_HEAD_DIMS = (64, 128, 256)
 
 
-def attention_prefill_forward(query, key, value, scale, pad=None, window=0):
-    """Causal attention of a whole prompt in one kernel: query, key, value
-    [B, H, S, D] fp16/bf16 views (features contiguous, any batch/head/position
-    strides that are multiples of 8 elements), ``pad`` an optional additive
-    fp32 [B, S] key mask, ``window`` > 0 a sliding window (query i sees keys
-    i - window < s <= i). Returns softmax(scale * q k^T + causal + pad) v,
-    shaped [B, H, S, D] over [B, S, H, D] memory, so that merging the heads
-    afterwards moves nothing (oslo/models/gptj/modeling_gptj.py:936-951 and
-    the ``_merge_heads`` that follows it). The [S, S] scores never reach memory."""
+def _prefill_args(query, key, value, pad):
     _device_tensor(query, "query")
     _device_tensor(key, "key", query)
     _device_tensor(value, "value", query)
@@ -598,29 +590,86 @@ def attention_prefill_forward(query, key, value, scale, pad=None, window=0):
     _require(key.dtype == query.dtype and value.dtype == query.dtype, "query, key and value differ in dtype")
     b, h, s, d = query.shape
     _require(d in PREFILL_HEAD_DIMS, f"attention_prefill: heads of {d} features (64, 128 or 256 are taken)")
-
-    def strided(t):
-        ok = t.stride(3) == 1 and all(st % 8 == 0 for st in t.stride()[:3]) and t.data_ptr() % 16 == 0 \
-            and (s == 1 or t.stride(2) >= d) and (s + 128) * t.stride(2) * 2 < 2 ** 31  # 32-bit offsets in a head
-        return t if ok else t.contiguous()
-
-    q, k, v = strided(query), strided(key), strided(value)
     if pad is not None:
         _device_tensor(pad, "pad", query)
         _require(pad.dtype == torch.float32 and tuple(pad.shape) == (b, s), "pad must be fp32 [B, S]")
         _require(s % 4 == 0, "attention_prefill: with a padding mask S must be a multiple of 4")
         pad = pad.contiguous()
-    out = torch.empty((b, s, h, d), dtype=query.dtype, device=query.device).permute(0, 2, 1, 3)
-    if out.numel() == 0:
-        return out
-    strides = (ctypes.c_int64 * 12)()
-    for i, t in enumerate((q, k, v, out)):
+    return code, pad
+
+
+def _prefill_strided(t):
+    """t as the prompt attention can read it: features contiguous, strides
+    multiples of 8 elements, 32-bit byte offsets inside a head; a copy if not."""
+    s, d = t.shape[2], t.shape[3]
+    ok = t.stride(3) == 1 and all(st % 8 == 0 for st in t.stride()[:3]) and t.data_ptr() % 16 == 0 \
+        and (s == 1 or t.stride(2) >= d) and (s + 128) * t.stride(2) * 2 < 2 ** 31
+    return t if ok else t.contiguous()
+
+
+def _stride_table(tensors):
+    strides = (ctypes.c_int64 * (3 * len(tensors)))()
+    for i, t in enumerate(tensors):
         strides[3 * i], strides[3 * i + 1], strides[3 * i + 2] = t.stride(0), t.stride(1), t.stride(2)
+    return strides
+
+
+def attention_prefill_forward(query, key, value, scale, pad=None, window=0, want_lse=False):
+    """Causal attention of a whole prompt in one kernel: query, key, value
+    [B, H, S, D] fp16/bf16 views (features contiguous, any batch/head/position
+    strides that are multiples of 8 elements), ``pad`` an optional additive
+    fp32 [B, S] key mask, ``window`` > 0 a sliding window (query i sees keys
+    i - window < s <= i). Returns softmax(scale * q k^T + causal + pad) v,
+    shaped [B, H, S, D] over [B, S, H, D] memory, so that merging the heads
+    afterwards moves nothing (oslo/models/gptj/modeling_gptj.py:936-951 and
+    the ``_merge_heads`` that follows it). The [S, S] scores never reach memory.
+    With ``want_lse`` also the fp32 [B, H, S] log2-sum-exp of every row, which
+    ``attention_prefill_backward`` takes."""
+    code, pad = _prefill_args(query, key, value, pad)
+    b, h, s, d = query.shape
+    q, k, v = _prefill_strided(query), _prefill_strided(key), _prefill_strided(value)
+    out = torch.empty((b, s, h, d), dtype=query.dtype, device=query.device).permute(0, 2, 1, 3)
+    lse = torch.empty((b, h, s), dtype=torch.float32, device=query.device) if want_lse else None
+    if out.numel() > 0:
+        strides = _stride_table((q, k, v, out))
+        with _on_device(q):
+            if want_lse:
+                _lib.check(_lib.load().oslo_attention_prefill_fwd_lse(
+                    _ptr(out), _ptr(lse), _ptr(q), _ptr(k), _ptr(v), _ptr(pad), float(scale), b, h, s, d,
+                    int(window), strides, code, _stream(q)))
+            else:
+                _lib.check(_lib.load().oslo_attention_prefill_fwd(
+                    _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(pad), float(scale), b, h, s, d, int(window), strides,
+                    code, _stream(q)))
+    return (out, lse) if want_lse else out
+
+
+def attention_prefill_backward(grad_out, query, key, value, out, lse, scale, pad=None, window=0):
+    """Gradients of ``attention_prefill_forward`` with respect to query, key and
+    value (each [B, H, S, D], dense), from the gradient of its output, its
+    inputs, its output and the log-sum-exp it returned with ``want_lse``. The
+    [S, S] probabilities are recomputed tile by tile; nothing of that size is
+    stored."""
+    code, pad = _prefill_args(query, key, value, pad)
+    _device_tensor(grad_out, "grad_out", query)
+    _require(grad_out.shape == query.shape and out.shape == query.shape, "grad_out and out must be shaped like query")
+    _require(grad_out.dtype == query.dtype and out.dtype == query.dtype, "grad_out and out must have query's dtype")
+    b, h, s, d = query.shape
+    _require(lse.dtype == torch.float32 and tuple(lse.shape) == (b, h, s) and lse.is_contiguous(),
+             "lse must be the fp32 [B, H, S] tensor of the forward")
+    q, k, v, o, g = (_prefill_strided(t) for t in (query, key, value, out, grad_out))
+    dq, dk, dv = (torch.empty((b, h, s, d), dtype=query.dtype, device=query.device) for _ in range(3))
+    if dq.numel() == 0:
+        return dq, dk, dv
+    lib = _lib.load()
+    ws = torch.empty(max(lib.oslo_attention_prefill_bwd_workspace_bytes(b, h, s) // 4, 1), dtype=torch.float32,
+                     device=query.device)
+    strides = _stride_table((q, k, v, o, g, dq, dk, dv))
     with _on_device(q):
-        _lib.check(_lib.load().oslo_attention_prefill_fwd(
-            _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(pad), float(scale), b, h, s, d, int(window), strides, code,
-            _stream(q)))
-    return out
+        _lib.check(lib.oslo_attention_prefill_bwd(
+            _ptr(dq), _ptr(dk), _ptr(dv), _ptr(g), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(ws),
+            _ptr(pad), float(scale), b, h, s, d, int(window), strides, code, _stream(q)))
+    return dq, dk, dv
 
 
 def rotary_qkv_forward(query, key, value, sin, cos, rotary_dim, offset=0):

@@ -1,0 +1,177 @@
+"""Backward of the one-kernel prompt attention, called through the C ABI,
+against the CPU oracle in float64 (small cases) and the same formulas in
+float64 on the device (large ones).
+
+Tolerance. With REL the half-ulp of the storage type (2^-8 bf16, 2^-11 fp16),
+every rounding moves a value by at most REL of its magnitude:
+  * each gradient is an fp32 sum rounded once:                REL * |ref|
+  * P and dS are rounded before the products that sum them:   REL * (P^T |dO|),
+    REL * scale * (|dS| |K|), REL * scale * (|dS|^T |Q|)
+  * delta is formed from the forward's *rounded* output, so it is off by up
+    to REL * sum_d |dO| |O| =: e_delta, which moves dS by scale * P * e_delta.
+The bar is twice the sum of these bounds (they are computed in float64 for the
+case at hand) plus 1e-4."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oslo_oracle as orc
+from oslo_amd import kernels
+from tests.util import IDS, f32, randn
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+HALVES = [torch.float16, torch.bfloat16]
+REL = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}
+
+
+def reference(q, k, v, do, scale, pad=None, window=0):
+    """float64 gradients and the error bounds described above, on the inputs' device."""
+    q, k, v, do = q.double(), k.double(), v.double(), do.double()
+    s = q.shape[2]
+    w = q @ k.transpose(-1, -2) * scale
+    if pad is not None:
+        w = w + pad.double()[:, None, None, :]
+    i = torch.arange(s, device=q.device)
+    hidden = i[None, :] > i[:, None]
+    if window:
+        hidden = hidden | (i[None, :] <= i[:, None] - window)
+    p = torch.softmax(w.masked_fill(hidden, float("-inf")), -1)
+    o = p @ v
+    dv = p.transpose(-1, -2) @ do
+    dp = do @ v.transpose(-1, -2)
+    delta = (do * o).sum(-1, keepdim=True)
+    ds = p * (dp - delta)
+    dq = scale * (ds @ k)
+    dk = scale * (ds.transpose(-1, -2) @ q)
+    e_delta = (do.abs() * o.abs()).sum(-1, keepdim=True)
+    ds_mag = ds.abs() + p * e_delta
+    bounds = {
+        "dq": dq.abs() + scale * (ds_mag @ k.abs()),
+        "dk": dk.abs() + scale * (ds_mag.transpose(-1, -2) @ q.abs()),
+        "dv": dv.abs() + p.transpose(-1, -2) @ do.abs(),
+    }
+    return o, {"dq": dq, "dk": dk, "dv": dv}, bounds
+
+
+def run(q, k, v, do, scale, pad=None, window=0):
+    out, lse = kernels.attention_prefill_forward(q, k, v, scale, pad, window, want_lse=True)
+    dq, dk, dv = kernels.attention_prefill_backward(do, q, k, v, out, lse, scale, pad, window)
+    return out, lse, {"dq": dq, "dk": dk, "dv": dv}
+
+
+def check(got, want, bounds, dtype, what):
+    for name in ("dq", "dk", "dv"):
+        assert torch.isfinite(got[name]).all(), (name, what)
+        excess = ((got[name].double() - want[name]).abs() - 2 * REL[dtype] * bounds[name]).max().item()
+        assert excess <= 1e-4, (name, excess, what)
+
+
+def padding(b, s, seed):
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.randint(max(1, s // 2), s + 1, (b,), generator=g)
+    return torch.where(torch.arange(s)[None, :] < lens[:, None], 0.0, -10000.0).float()
+
+
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+@pytest.mark.parametrize("d", [64, 128, 256])
+@pytest.mark.parametrize("s", [1, 8, 31, 64, 65, 128, 200, 332])
+def test_backward_matches_oracle(s, d, dtype):
+    b, h = 2, 3
+    q, k, v, do = (randn((b, h, s, d), dtype, seed=11 * s + i) for i in range(4))
+    scale = 1.0 / math.sqrt(d)
+    dev = [t.to(DEV) for t in (q, k, v, do)]
+    for pad in ([None, padding(b, s, s)] if s % 4 == 0 else [None]):
+        out, lse, got = run(*dev, scale, None if pad is None else pad.to(DEV))
+        flat = [f32(t).reshape(b * h, s, d) for t in (q, k, v, do)]
+        want = orc.attention_prefill_bwd(*flat, scale, None if pad is None else pad.numpy().repeat(h, axis=0))
+        _, _, bounds = reference(*dev, scale, None if pad is None else pad.to(DEV))
+        want = {n: torch.from_numpy(w.reshape(b, h, s, d)).to(DEV) for n, w in zip(("dq", "dk", "dv"), want)}
+        check(got, want, bounds, dtype, (s, d, pad is not None))
+        # the log-sum-exp the forward hands over: log2 of the sum of 2^(log2e * score) over the visible keys
+        scores = np.einsum("bhid,bhjd->bhij", f32(q).astype(np.float64), f32(k).astype(np.float64)) * scale
+        if pad is not None:
+            scores = scores + pad.numpy().astype(np.float64)[:, None, None, :]
+        scores = np.where(np.tril(np.ones((s, s), dtype=bool)), scores, -np.inf)
+        m = scores.max(-1, keepdims=True)
+        want_lse = (m[..., 0] + np.log(np.exp(scores - m).sum(-1))) * math.log2(math.e)
+        assert np.abs(f32(lse).astype(np.float64) - want_lse).max() <= 2e-3 * (1 + np.abs(want_lse).max() * 1e-3)
+
+
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+@pytest.mark.parametrize("b,h,s,d", [(2, 8, 1024, 64), (1, 5, 1000, 128), (1, 4, 2048, 256), (1, 2, 2300, 128)])
+def test_backward_long_prompts(b, h, s, d, dtype):
+    q, k, v, do = (randn((b, h, s, d), dtype, seed=s + i).to(DEV) for i in range(4))
+    pads = [None, padding(b, s, 3).to(DEV)] if s % 4 == 0 else [None]
+    for p in pads:
+        _, _, got = run(q, k, v, do, 0.1, p)
+        _, want, bounds = reference(q, k, v, do, 0.1, p)
+        check(got, want, bounds, dtype, (b, h, s, d, p is not None))
+
+
+# windows shorter than a step of 32, ragged against steps, tiles and blocks, and at least the prompt
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+@pytest.mark.parametrize("window", [1, 5, 32, 33, 64, 100, 256, 300, 700])
+def test_backward_sliding_window(window, dtype):
+    for (b, h, s, d) in ((2, 3, 520, 64), (1, 2, 360, 128), (1, 2, 700, 256)):
+        q, k, v, do = (randn((b, h, s, d), dtype, seed=window + i).to(DEV) for i in range(4))
+        pad = padding(b, s, window).to(DEV)
+        for p in (None, pad):
+            _, _, got = run(q, k, v, do, 0.1, p, window)
+            _, want, bounds = reference(q, k, v, do, 0.1, p, window)
+            check(got, want, bounds, dtype, (b, h, s, d, window, p is not None))
+    b, h, s, d = 1, 2, 96, 64
+    q, k, v, do = (randn((b, h, s, d), dtype, seed=3 * window + i) for i in range(4))
+    dev = [t.to(DEV) for t in (q, k, v, do)]
+    _, _, got = run(*dev, 0.1, None, window)
+    want = orc.attention_prefill_bwd(*[f32(t).reshape(b * h, s, d) for t in (q, k, v, do)], 0.1, None, window)
+    want = {n: torch.from_numpy(w.reshape(b, h, s, d)).to(DEV) for n, w in zip(("dq", "dk", "dv"), want)}
+    _, _, bounds = reference(*dev, 0.1, None, window)
+    check(got, want, bounds, dtype, ("oracle", window))
+
+
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+def test_backward_strided_inputs_determinism_and_closed_forms(dtype):
+    """q, k, v as slices of one packed projection and the gradient of the output
+    in merged-heads memory (how a model hands them over); two runs give the same
+    bits; with equal scores the probabilities are 1/(i+1), so dV is a weighted
+    suffix sum of dO; a single position passes dO through to dV and gives
+    (all but) no gradient to q and k."""
+    b, h, s, d = 2, 4, 384, 64
+    packed = randn((b, s, 3, h, d), dtype, seed=1).to(DEV)
+    q, k, v = (packed[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    do = randn((b, s, h, d), dtype, seed=2).to(DEV).permute(0, 2, 1, 3)
+    _, _, got = run(q, k, v, do, 0.125)
+    _, want, bounds = reference(q, k, v, do, 0.125)
+    check(got, want, bounds, dtype, "strided")
+    _, _, again = run(q, k, v, do, 0.125)
+    assert all(torch.equal(got[n], again[n]) for n in got)
+    zero = torch.zeros_like(q)
+    _, _, flat = run(zero, k, v, do, 0.125)
+    weights = 1.0 / torch.arange(1, s + 1, device=DEV, dtype=torch.float64)
+    suffix = torch.flip(torch.cumsum(torch.flip(do.double() * weights[None, None, :, None], [2]), 2), [2])
+    excess = ((flat["dv"].double() - suffix).abs() - 2 * REL[dtype] * (suffix.abs() + 8.0)).max().item()
+    assert excess <= 1e-4
+    one = [t[:, :, :1].contiguous() for t in (q, k, v, do)]
+    _, _, single = run(*one, 0.125)
+    # the one probability is exactly 1; dP and delta are the same dot product summed in two orders,
+    # so dS (and with it dq, dk) is zero up to the rounding of an fp32 sum
+    assert torch.equal(single["dv"], one[3])
+    assert single["dq"].abs().max().item() <= 1e-4 and single["dk"].abs().max().item() <= 1e-4
+
+
+def test_backward_rejects_what_it_cannot_take():
+    q = torch.zeros(1, 2, 16, 48, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError):
+        kernels.attention_prefill_forward(q, q, q, 1.0, want_lse=True)          # head size
+    q = torch.zeros(1, 2, 16, 64, dtype=torch.float32, device=DEV)
+    with pytest.raises(RuntimeError):
+        kernels.attention_prefill_forward(q, q, q, 1.0, want_lse=True)          # fp32
+    q = torch.zeros(1, 2, 16, 64, dtype=torch.bfloat16, device=DEV)
+    out, lse = kernels.attention_prefill_forward(q, q, q, 1.0, want_lse=True)
+    with pytest.raises(RuntimeError):
+        kernels.attention_prefill_backward(q, q, q, q, out, lse[:, :1], 1.0)    # lse of another shape

@@ -478,3 +478,40 @@ def test_attention_decode_against_library_and_closed_form():
     win = orc.attention_decode(np.zeros((n, d)), k, v, last, 1.0, window=3)
     assert np.allclose(win, v[:, 5:8].mean(axis=1), atol=1e-12)
     assert np.allclose(orc.attention_decode(q, k, v, 0, 1.0), v[:, 0], atol=1e-12)   # one visible key
+
+
+def test_attention_prefill_bwd_against_autograd_and_differences():
+    g = torch.Generator().manual_seed(5)
+    n, S, d, scale = 2, 13, 8, 0.3
+    q, k, v, do = (torch.randn((n, S, d), generator=g, dtype=torch.float64) for _ in range(4))
+    pad = torch.zeros(n, S, dtype=torch.float64)
+    pad[1, 9:] = -10000.0
+    i = torch.arange(S)
+    for use_pad, window in ((False, None), (True, None), (False, 4), (True, 5)):
+        qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+        keep = i[None, :] <= i[:, None]
+        if window:
+            keep = keep & (i[None, :] > i[:, None] - window)
+        mask = torch.zeros(n, S, S, dtype=torch.float64).masked_fill(~keep, float("-inf"))
+        if use_pad:
+            mask = mask + pad[:, None, :]
+        out = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, attn_mask=mask, scale=scale)
+        out.backward(do)
+        dq, dk, dv = orc.attention_prefill_bwd(q.numpy(), k.numpy(), v.numpy(), do.numpy(), scale,
+                                               pad.numpy() if use_pad else None, window)
+        for got, want in ((dq, qq.grad), (dk, kk.grad), (dv, vv.grad)):
+            assert np.abs(got - want.numpy()).max() <= 1e-12
+    # central differences of the forward restatement (no window there), one entry of each input
+    f = lambda a, b_, c: float((orc.attention_prefill(a, b_, c, scale, pad.numpy()) * do.numpy()).sum())
+    dq, dk, dv = orc.attention_prefill_bwd(q.numpy(), k.numpy(), v.numpy(), do.numpy(), scale, pad.numpy())
+    eps = 1e-6
+    for which, grad in enumerate((dq, dk, dv)):
+        for idx in ((0, 3, 2), (1, 7, 5), (1, 12, 0)):
+            args = [q.numpy().copy(), k.numpy().copy(), v.numpy().copy()]
+            args[which][idx] += eps
+            up = f(*args)
+            args[which][idx] -= 2 * eps
+            assert abs((up - f(*args)) / (2 * eps) - grad[idx]) <= 1e-7
+    # a single position: the probability is 1, dV = dO, dQ = dK = 0
+    dq1, dk1, dv1 = orc.attention_prefill_bwd(q[:, :1].numpy(), k[:, :1].numpy(), v[:, :1].numpy(), do[:, :1].numpy(), scale)
+    assert np.array_equal(dv1, do[:, :1].numpy()) and not dq1.any() and not dk1.any()
