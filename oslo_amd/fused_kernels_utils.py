@@ -543,6 +543,29 @@ class FusedDecodeAttention(object):
                                                              new_key, new_value)
 
 
+class _PrefillAttention(torch.autograd.Function):
+    """The prompt attention with its backward: the forward keeps q, k, v, its
+    output and one fp32 number per row (the log-sum-exp); the backward
+    recomputes the probabilities tile by tile on the matrix cores."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, pad, scale, window):
+        out, lse = get_custom_kernels().attention_prefill_forward(query, key, value, scale, pad, window,
+                                                                  want_lse=True)
+        ctx.save_for_backward(query, key, value, out, lse)
+        ctx.pad = pad
+        ctx.args = (float(scale), int(window))
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        query, key, value, out, lse = ctx.saved_tensors
+        scale, window = ctx.args
+        dq, dk, dv = get_custom_kernels().attention_prefill_backward(
+            grad_out, query, key, value, out, lse, scale, ctx.pad, window)
+        return dq, dk, dv, None, None, None
+
+
 class FusedPrefillAttention(object):
     """
     Kernel fusion function: causal attention over a whole prompt
@@ -555,9 +578,13 @@ class FusedPrefillAttention(object):
     query, key and value as [B, H, S, D] (views with any strides), the model's
     additive padding mask [B, 1, 1, S] or None, and the scale; it returns the
     attention output shaped [B, H, S, D] over [B, S, H, D] memory, which
-    ``FusedMergeHeads`` turns into [B, S, H*D] without a copy. Inference only
-    (no backward, no attention dropout, no probabilities to return), fp16 and
-    bf16, heads of 64, 128 or 256 features.
+    ``FusedMergeHeads`` turns into [B, S, H*D] without a copy. fp16 and bf16,
+    heads of 64, 128 or 256 features; no probabilities to return. With
+    gradients recorded the forward also keeps the log-sum-exp of every row and
+    the backward recomputes the probabilities from it, so a training step
+    stores no [B, H, S, S] tensor either. Attention dropout is not part of
+    the kernel: a module that drops attention probabilities in training keeps
+    the softmax kernel with fused dropout between its two matmuls.
     """
 
     MIN_LENGTH = 2  # one query is a decoding step (FusedDecodeAttention); from two on, one launch beats three
@@ -577,15 +604,17 @@ class FusedPrefillAttention(object):
                 s % 4 == 0 and attention_mask.is_floating_point() and attention_mask.numel() == b * s
                 and tuple(attention_mask.shape) in ((b, 1, 1, s), (b, s))):
             return False
-        return not _needs_grad(query, key)
+        return True
 
     @staticmethod
     def apply(query, key, value, attention_mask=None, scale=None, window=None):
         """``window``: GPT-Neo's local attention (query i sees keys i - window < s <= i)."""
         b, _, s, _ = query.shape
         pad = None if attention_mask is None else attention_mask.reshape(b, s).float()
-        return get_custom_kernels().attention_prefill_forward(query, key, value, 1.0 if scale is None else scale, pad,
-                                                              window or 0)
+        scale = 1.0 if scale is None else scale
+        if _needs_grad(query, key, value):
+            return _PrefillAttention.apply(query, key, value, pad, scale, window or 0)
+        return get_custom_kernels().attention_prefill_forward(query, key, value, scale, pad, window or 0)
 
 
 class FusedLinearRows(object):

@@ -115,10 +115,12 @@ def test_prompt_attention_runs_as_one_kernel_at_inference(family, dtype, padded,
     step_f = (got_step.float() - ref_step).abs()
     step_u = (want_step.float() - ref_step).abs()
     assert step_f.max().item() <= 1.5 * step_u.max().item() and step_f.mean().item() <= 1.1 * step_u.mean().item()
-    # with gradients recorded the three-launch path (which has a backward) is taken
+    # with gradients recorded (eval mode: no attention dropout) the same kernel runs, keeping what its backward needs
     calls.clear()
-    m(ids, attention_mask=mask)
-    assert calls == []
+    loss = m(ids, attention_mask=mask)["logits"].float().square().mean()
+    assert calls == [(3, 4, 160, 64)] * 2
+    loss.backward()
+    assert all(torch.isfinite(p.grad).all() for p in m.parameters() if p.grad is not None)
 
 
 @pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
@@ -357,3 +359,52 @@ def test_padding_mask_under_inference_mode_and_interleaved_masks():
         y = FusedScaleMaskSoftmax.apply(xx, mask, 0.5, True)
         want = torch.softmax((xx * 0.5 + mask).masked_fill(~tril, float("-inf")), -1)
         assert (y - want).abs().max().item() <= 1e-6
+
+
+@pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
+@pytest.mark.parametrize("padded", [False, True], ids=["nopad", "pad"])
+def test_training_through_the_one_kernel_attention_matches_unfused_gradients(family, padded, monkeypatch):
+    """No attention dropout, bf16, heads of 64: a fused model's training step
+    goes through the one-kernel attention and its backward. Loss and parameter
+    gradients are compared with the unfused model's, both against the unfused
+    model in fp32 on the same weights."""
+    big = {
+        "gpt2": lambda: GPT2LMHeadModel(GPT2Config(vocab_size=512, n_positions=256, n_embd=256, n_layer=2, n_head=4,
+                                                   resid_pdrop=0.0, embd_pdrop=0.0, attn_pdrop=0.0)),
+        "gptj": lambda: GPTJForCausalLM(GPTJConfig(vocab_size=512, n_positions=256, n_embd=256, n_layer=2, n_head=4,
+                                                   rotary_dim=16)),
+        "gpt_neo": lambda: GPTNeoForCausalLM(GPTNeoConfig(vocab_size=512, max_position_embeddings=256,
+                                                          hidden_size=256, num_layers=2, num_heads=4, window_size=32)),
+    }
+    torch.manual_seed(0)
+    m = big[family]().to(DEV, torch.bfloat16).train()
+    ids = torch.randint(0, 512, (3, 160), device=DEV)
+    mask = None
+    if padded:
+        mask = torch.ones(3, 160, device=DEV)
+        mask[1, 100:] = 0
+        mask[2, 17:] = 0
+    labels = ids if mask is None else ids.masked_fill(mask == 0, -100)
+
+    def grads(model):
+        model.zero_grad(set_to_none=True)
+        loss = model(ids, attention_mask=mask, labels=labels)["loss"]
+        loss.backward()
+        return loss.item(), {n: p.grad.float().clone() for n, p in model.named_parameters() if p.grad is not None}
+
+    ref_loss, ref = grads(copy.deepcopy(m).float())
+    un_loss, un = grads(m)
+    calls = []
+    real = fku._PrefillAttention.apply
+    monkeypatch.setattr(fku._PrefillAttention, "apply", staticmethod(lambda *a: (calls.append(1), real(*a))[1]))
+    m.fuse()
+    fu_loss, fu = grads(m)
+    assert len(calls) == 2                                    # both layers (GPT-Neo: the global and the local one)
+    assert abs(fu_loss - ref_loss) <= 1.5 * abs(un_loss - ref_loss) + 2e-3
+    assert fu.keys() == un.keys() == ref.keys()
+    num_f = sum((fu[n] - ref[n]).square().sum().item() for n in ref)
+    num_u = sum((un[n] - ref[n]).square().sum().item() for n in ref)
+    den = sum(ref[n].square().sum().item() for n in ref)
+    assert all(torch.isfinite(g).all() for g in fu.values())
+    # relative L2 error of the whole gradient: the fused model no further from fp32 than the unfused bf16 one
+    assert (num_f / den) ** 0.5 <= 1.25 * (num_u / den) ** 0.5 + 1e-3, ((num_f / den) ** 0.5, (num_u / den) ** 0.5)
