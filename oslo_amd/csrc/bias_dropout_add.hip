@@ -11,7 +11,7 @@
 namespace oslo {
 namespace {
 
-template <typename T, int VEC, int U, bool DROP, bool HAS_BIAS, bool HAS_RES, bool NT>
+template <typename T, int VEC, int U, bool DROP, bool HAS_BIAS, bool HAS_RES, int OUT>
 __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_fwd_kernel(
     T *out, const T *x, const T *__restrict__ bias, const T *residual,
     float keep_scale, uint32_t threshold, uint64_t seed, uint64_t offset,
@@ -23,12 +23,12 @@ __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_fwd_kernel(
   RawVec<T, VEC> xraw[U], rraw[HAS_RES ? U : 1];
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    xraw[u] = buffer_load_raw<T, VEC, NT>(xrs, ew_offset<T>(pos, u, cols));
+    xraw[u] = buffer_load_raw<T, VEC, true>(xrs, ew_offset<T>(pos, u, cols));
   if constexpr (HAS_RES) {
     const BufRsrc rrs = ew_rsrc<T>(residual, pos, rows_per_block, rows, cols);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      rraw[u] = buffer_load_raw<T, VEC, NT>(rrs, ew_offset<T>(pos, u, cols));
+      rraw[u] = buffer_load_raw<T, VEC, true>(rrs, ew_offset<T>(pos, u, cols));
   }
   float b[VEC];
   if constexpr (HAS_BIAS) load_f32_cached<T, VEC>(b, bias + pos.c0);
@@ -52,11 +52,11 @@ __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_fwd_kernel(
       if constexpr (HAS_RES) t += tr[u][j];
       tx[u][j] = t;
     }
-    buffer_store_f32<T, VEC, kStreamOut>(ors, ew_offset<T>(pos, u, cols), tx[u]);
+    buffer_store_f32<T, VEC, OUT>(ors, ew_offset<T>(pos, u, cols), tx[u]);
   }
 }
 
-template <typename T, int VEC, int U, bool DROP, bool WANT_DBIAS, bool NT>
+template <typename T, int VEC, int U, bool DROP, bool WANT_DBIAS, int OUT>
 __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_bwd_kernel(
     T *dx, float *__restrict__ partial, const T *g, float keep_scale,
     uint32_t threshold, uint64_t seed, uint64_t offset, int64_t rows,
@@ -72,7 +72,7 @@ __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_bwd_kernel(
     RawVec<T, VEC> graw[U];
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      graw[u] = buffer_load_raw<T, VEC, NT>(grs, ew_offset<T>(pos, u, cols));
+      graw[u] = buffer_load_raw<T, VEC, true>(grs, ew_offset<T>(pos, u, cols));
     // rows past the end were read as zeros (they add nothing to dbias) and
     // their stores are dropped by the same bound
     const BufRsrc drs = ew_rsrc<T>(dx, pos, rows_per_block, rows, cols);
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(kBlockThreads) void bias_dropout_add_bwd_kernel(
       }
       // with no dropout dx == g bit for bit; still written, dx may be a
       // different buffer
-      buffer_store_f32<T, VEC, kStreamOut>(drs, ew_offset<T>(pos, u, cols), tg[u]);
+      buffer_store_f32<T, VEC, OUT>(drs, ew_offset<T>(pos, u, cols), tg[u]);
     }
   }
   if constexpr (WANT_DBIAS)
@@ -107,15 +107,15 @@ int launch_fwd(T *out, const T *x, const T *bias, const T *res,
                hipStream_t stream) {
   const EwPlan p = plan_elementwise(rows, cols / VEC, kFwdMaxTx, kFwdUnroll);
   if (!p.ok) return fail(OSLO_E_UNSUPPORTED, "bias_dropout_add_fwd: tensor too large for one launch");
-  const bool nt = stream_loads((res ? 3 : 2) * rows * cols * (int64_t)sizeof(T));
+  const bool keep = keep_output_cached(rows * cols * (int64_t)sizeof(T));
   auto go = [&]<bool DROP, bool HB, bool HR>() {
-    if (nt)
-      bias_dropout_add_fwd_kernel<T, VEC, kFwdUnroll, DROP, HB, HR, true>
+    if (keep)
+      bias_dropout_add_fwd_kernel<T, VEC, kFwdUnroll, DROP, HB, HR, kOutKeep>
           <<<p.grid, p.block, 0, stream>>>(out, x, bias, res, a.keep_scale,
                                            a.threshold, a.seed, a.offset, rows,
                                            cols, p.col_tiles, p.rows_per_block);
     else
-      bias_dropout_add_fwd_kernel<T, VEC, kFwdUnroll, DROP, HB, HR, false>
+      bias_dropout_add_fwd_kernel<T, VEC, kFwdUnroll, DROP, HB, HR, kOutStream>
           <<<p.grid, p.block, 0, stream>>>(out, x, bias, res, a.keep_scale,
                                            a.threshold, a.seed, a.offset, rows,
                                            cols, p.col_tiles, p.rows_per_block);
@@ -139,15 +139,15 @@ int launch_bwd(T *dx, T *dbias, float *ws, const T *g, const DropArgs &a,
                int64_t rows, int64_t cols, hipStream_t stream) {
   const EwPlan p = plan_elementwise(rows, cols / VEC, kBwdMaxTx, kDropBwdUnroll);
   if (!p.ok) return fail(OSLO_E_UNSUPPORTED, "bias_dropout_add_bwd: tensor too large for one launch");
-  const bool nt = stream_loads(2 * rows * cols * (int64_t)sizeof(T));
+  const bool keep = keep_output_cached(rows * cols * (int64_t)sizeof(T));
   auto go = [&]<bool DROP, bool WANT>() {
-    if (nt)
-      bias_dropout_add_bwd_kernel<T, VEC, kDropBwdUnroll, DROP, WANT, true>
+    if (keep)
+      bias_dropout_add_bwd_kernel<T, VEC, kDropBwdUnroll, DROP, WANT, kOutKeep>
           <<<p.grid, p.block, 0, stream>>>(dx, ws, g, a.keep_scale, a.threshold,
                                            a.seed, a.offset, rows, cols,
                                            p.col_tiles, p.rows_per_block);
     else
-      bias_dropout_add_bwd_kernel<T, VEC, kDropBwdUnroll, DROP, WANT, false>
+      bias_dropout_add_bwd_kernel<T, VEC, kDropBwdUnroll, DROP, WANT, kOutStream>
           <<<p.grid, p.block, 0, stream>>>(dx, ws, g, a.keep_scale, a.threshold,
                                            a.seed, a.offset, rows, cols,
                                            p.col_tiles, p.rows_per_block);

@@ -21,7 +21,7 @@ static __device__ __align__(256) float scratch[OSLO_STATIC_WORKSPACE_BYTES / siz
 namespace oslo {
 namespace {
 
-template <typename T, int VEC, int U, bool NT>
+template <typename T, int VEC, int U, int OUT>
 __global__ __launch_bounds__(kBlockThreads) void bias_gelu_fwd_kernel(
     T *out, const T *y, const T *__restrict__ bias, int64_t rows, int64_t cols,
     int col_tiles, int rows_per_block) {
@@ -31,7 +31,7 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_fwd_kernel(
   RawVec<T, VEC> raw[U];
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    raw[u] = buffer_load_raw<T, VEC, NT>(yrs, ew_offset<T>(pos, u, cols));
+    raw[u] = buffer_load_raw<T, VEC, true>(yrs, ew_offset<T>(pos, u, cols));
   float b[VEC];
   load_f32_cached<T, VEC>(b, bias + pos.c0);
   // rows past the end were read as zeros and their stores are dropped by the
@@ -43,11 +43,11 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_fwd_kernel(
     raw_to_f32<T, VEC>(t[u], raw[u]);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) t[u][j] = gelu_fwd(t[u][j] + b[j]);
-    buffer_store_f32<T, VEC, kStreamOut>(ors, ew_offset<T>(pos, u, cols), t[u]);
+    buffer_store_f32<T, VEC, OUT>(ors, ew_offset<T>(pos, u, cols), t[u]);
   }
 }
 
-template <typename T, int VEC, int U, bool WANT_DBIAS, bool NT>
+template <typename T, int VEC, int U, bool WANT_DBIAS, int OUT>
 __global__ __launch_bounds__(kBlockThreads) void bias_gelu_bwd_kernel(
     T *dy, float *__restrict__ partial, const T *g, const T *y,
     const T *__restrict__ bias, int64_t rows, int64_t cols, int col_tiles,
@@ -63,8 +63,8 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_bwd_kernel(
     RawVec<T, VEC> graw[U], yraw[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      graw[u] = buffer_load_raw<T, VEC, NT>(grs, ew_offset<T>(pos, u, cols));
-      yraw[u] = buffer_load_raw<T, VEC, NT>(yrs, ew_offset<T>(pos, u, cols));
+      graw[u] = buffer_load_raw<T, VEC, true>(grs, ew_offset<T>(pos, u, cols));
+      yraw[u] = buffer_load_raw<T, VEC, true>(yrs, ew_offset<T>(pos, u, cols));
     }
     float b[VEC];
     load_f32_cached<T, VEC>(b, bias + pos.c0);
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(kBlockThreads) void bias_gelu_bwd_kernel(
         tg[u][j] = gelu_grad(ty_[u][j] + b[j]) * tg[u][j];
         if constexpr (WANT_DBIAS) acc[j] += tg[u][j];
       }
-      buffer_store_f32<T, VEC, kStreamOut>(drs, ew_offset<T>(pos, u, cols), tg[u]);
+      buffer_store_f32<T, VEC, OUT>(drs, ew_offset<T>(pos, u, cols), tg[u]);
     }
   }
   if constexpr (WANT_DBIAS)
@@ -96,11 +96,11 @@ int launch_fwd(T *out, const T *y, const T *bias, int64_t rows, int64_t cols,
                hipStream_t stream) {
   const EwPlan p = plan_elementwise(rows, cols / VEC, kFwdMaxTx, kFwdUnroll);
   if (!p.ok) return fail(OSLO_E_UNSUPPORTED, "bias_gelu_fwd: tensor too large for one launch");
-  if (stream_loads(2 * rows * cols * (int64_t)sizeof(T)))
-    bias_gelu_fwd_kernel<T, VEC, kFwdUnroll, true><<<p.grid, p.block, 0, stream>>>(
+  if (keep_output_cached(rows * cols * (int64_t)sizeof(T)))
+    bias_gelu_fwd_kernel<T, VEC, kFwdUnroll, kOutKeep><<<p.grid, p.block, 0, stream>>>(
         out, y, bias, rows, cols, p.col_tiles, p.rows_per_block);
   else
-    bias_gelu_fwd_kernel<T, VEC, kFwdUnroll, false><<<p.grid, p.block, 0, stream>>>(
+    bias_gelu_fwd_kernel<T, VEC, kFwdUnroll, kOutStream><<<p.grid, p.block, 0, stream>>>(
         out, y, bias, rows, cols, p.col_tiles, p.rows_per_block);
   return check_launch("bias_gelu_fwd");
 }
@@ -110,22 +110,25 @@ int launch_bwd(T *dy, T *dbias, float *ws, const T *g, const T *y,
                const T *bias, int64_t rows, int64_t cols, hipStream_t stream) {
   const EwPlan p = plan_elementwise(rows, cols / VEC, kBwdMaxTx, kGeluBwdUnroll);
   if (!p.ok) return fail(OSLO_E_UNSUPPORTED, "bias_gelu_bwd: tensor too large for one launch");
-  auto go = [&]<bool WANT, bool NT>() {
-    bias_gelu_bwd_kernel<T, VEC, kGeluBwdUnroll, WANT, NT>
-        <<<p.grid, p.block, 0, stream>>>(dy, WANT ? ws : nullptr, g, y, bias, rows,
-                                         cols, p.col_tiles, p.rows_per_block);
+  const bool keep = keep_output_cached(rows * cols * (int64_t)sizeof(T));
+  auto go = [&]<bool WANT>() {
+    if (keep)
+      bias_gelu_bwd_kernel<T, VEC, kGeluBwdUnroll, WANT, kOutKeep>
+          <<<p.grid, p.block, 0, stream>>>(dy, WANT ? ws : nullptr, g, y, bias, rows,
+                                           cols, p.col_tiles, p.rows_per_block);
+    else
+      bias_gelu_bwd_kernel<T, VEC, kGeluBwdUnroll, WANT, kOutStream>
+          <<<p.grid, p.block, 0, stream>>>(dy, WANT ? ws : nullptr, g, y, bias, rows,
+                                           cols, p.col_tiles, p.rows_per_block);
   };
-  const bool nt = stream_loads(3 * rows * cols * (int64_t)sizeof(T));
   if (dbias) {
-    if (nt) go.template operator()<true, true>();
-    else go.template operator()<true, false>();
+    go.template operator()<true>();
     int s = check_launch("bias_gelu_bwd");
     if (s != OSLO_OK) return s;
     launch_colsum_finish<T>(dbias, ws, p.row_blocks, cols, stream);
     return check_launch("bias_gelu_bwd(dbias)");
   }
-  if (nt) go.template operator()<false, true>();
-  else go.template operator()<false, false>();
+  go.template operator()<false>();
   return check_launch("bias_gelu_bwd");
 }
 

@@ -29,15 +29,23 @@ constexpr int kBwdMaxTx = 32;  // backward kernels: narrower and taller tiles,
 constexpr int kBwdMinUnroll = 4;
 constexpr int kBwdMinRowsPerBlock = kBlockThreads / kBwdMaxTx * kBwdMinUnroll;
 
-// Cache policy of the loads. MI355X has a 256 MB memory-side cache in front of
-// HBM. Tensors far larger than it gain nothing there and are read with
-// non-temporal loads (a scaled copy of [16384,16384] bf16: 159 us against
-// 167-172 us with plain loads). Tensors that fit were usually just written by
-// the kernel before (a GEMM's output, the forward's activations) and a good
-// part of them is still in that cache: there plain loads are faster (the same
-// copy at [16384,4096]: 38.2 us against 43.1 us non-temporal).
-inline bool stream_loads(int64_t bytes_loaded) {
-  return bytes_loaded > (256ll << 20);
+// Cache policy of the epilogue kernels. Loads are non-temporal. Stores are
+// written through at device scope (sc1), with the non-temporal hint only for
+// tensors beyond the 256 MB memory-side cache in front of HBM: without it a
+// smaller output stays in that cache for the kernel that consumes it next.
+// Measured on a scaled copy, bf16, as a fraction of the HBM peak; "warm" = the
+// same buffers every launch (what a consumer sees whose input was just
+// produced), "cold" = four sets of buffers in turn:
+//   [16384,4096]  nt loads + sc1 stores      warm 0.865  cold 0.775
+//                 nt loads + sc1 nt stores   warm 0.778  cold 0.779
+//                 plain loads + sc1 nt       warm 0.874  cold 0.765
+//   [16384,8192]  0.872 / 0.783,  0.787 / 0.789,  0.878 / 0.772
+// At [16384,16384] the forward kernels do not care, the backward kernels (which
+// also write their dbias partial rows) lose 2-3 % without the hint.
+constexpr int kOutKeep = 16;       // sc1
+constexpr int kOutStream = 16 | 2; // sc1 nt
+inline bool keep_output_cached(int64_t tensor_bytes) {
+  return tensor_bytes <= (256ll << 20);
 }
 
 struct EwPlan {
