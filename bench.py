@@ -435,16 +435,16 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         # its backward (the forward that stores the log-sum-exp first): 7 matrix products per visible
         # tile where the forward has 2, so 14 flops per score and feature
         lse = torch.empty((B, Hh, S), dtype=torch.float32, device=dev)
-        check(lib.oslo_attention_prefill_fwd_lse(P(o), P(lse), P(q), P(k), P(v), None, D ** -0.5, B, Hh, S, D, 0,
-                                                 strides, BF16, st))
+        check(lib.oslo_attention_prefill_fwd_lse(P(o), P(lse), P(q), P(k), P(v), None, D ** -0.5, 0.0, 0, 0,
+                                                 B, Hh, S, D, 0, strides, BF16, st))
         do = randn((B, S, Hh, D), 60, 1.0, torch.bfloat16)
         dq, dk, dv = (torch.empty((B, Hh, S, D), dtype=torch.bfloat16, device=dev) for _ in range(3))
         wsb = torch.empty(lib.oslo_attention_prefill_bwd_workspace_bytes(B, Hh, S) // 4, dtype=torch.float32, device=dev)
         dense, merged = [Hh * S * D, S * D, D], [S * Hh * D, D, Hh * D]
         bstr = (ctypes.c_int64 * 24)(*(3 * dense + 2 * merged + 3 * dense))
         t = time_launches(lambda: check(lib.oslo_attention_prefill_bwd(
-            P(dq), P(dk), P(dv), P(do), P(q), P(k), P(v), P(o), P(lse), P(wsb), None, D ** -0.5, B, Hh, S, D, 0,
-            bstr, BF16, st)), max(5, n // 4), 3)
+            P(dq), P(dk), P(dv), P(do), P(q), P(k), P(v), P(o), P(lse), P(wsb), None, D ** -0.5, 0.0, 0, 0,
+            B, Hh, S, D, 0, bstr, BF16, st)), max(5, n // 4), 3)
         bflops = 7 * flops // 2
         res.append({"kernel": f"attention_prefill_bwd bf16 [{B},{Hh},{S},{D}] causal (dq, dk, dv; "
                               f"{4 if D == 256 else 3} launches)", "bound": "mfma",

@@ -448,18 +448,29 @@ int oslo_attention_prefill_fwd(void *out, const void *q, const void *k,
                                oslo_stream_t stream);
 
 /*
- * oslo_attention_prefill_fwd that also stores what its backward needs:
- * lse[b*heads + h, i] (fp32, [batch*heads, S], 16-byte aligned) = log2 of
- * sum_s 2^(log2(e) * (scale*q.k + pad)) over the visible keys of query i.
- * The forward a training step runs (oslo/models/gptj/modeling_gptj.py:936-951
- * with gradients recorded).
+ * oslo_attention_prefill_fwd for a training step. It also stores what the
+ * backward needs: lse[b*heads + h, i] (fp32, [batch*heads, S], 16-byte
+ * aligned) = log2 of sum_s 2^(log2(e) * (scale*q.k + pad)) over the visible
+ * keys of query i. And it can apply attention dropout, p in [0, 1): the
+ * probability of (query i, key s) of head (b, h) is multiplied by keep/(1-p)
+ * before it meets v, with keep drawn exactly as
+ * oslo_softmax_causal_dropout_fwd draws it for element (b, h, i, s) of a
+ * [batch, heads, S, S] tensor (Philox4x32-10, counter (offset/4, flat
+ * index/8), 16 bits per element; one call consumes 4 units of generator
+ * offset); then S must be a multiple of 8. lse is that of the probabilities
+ * before dropout. p == 0 draws nothing.
+ * Replaces matmul(q, k^T) -> FusedScaleMaskSoftmax.apply -> attn_dropout ->
+ * matmul(probs, v) with gradients recorded
+ * (oslo/models/gptj/modeling_gptj.py:936-951).
  */
 int oslo_attention_prefill_fwd_lse(void *out, float *lse, const void *q,
                                    const void *k, const void *v,
-                                   const float *pad, float scale, int64_t batch,
-                                   int64_t heads, int64_t S, int64_t head_dim,
-                                   int64_t window, const int64_t *strides,
-                                   int dtype, oslo_stream_t stream);
+                                   const float *pad, float scale, float p,
+                                   uint64_t philox_seed, uint64_t philox_offset,
+                                   int64_t batch, int64_t heads, int64_t S,
+                                   int64_t head_dim, int64_t window,
+                                   const int64_t *strides, int dtype,
+                                   oslo_stream_t stream);
 
 /* Bytes of fp32 workspace oslo_attention_prefill_bwd needs. */
 size_t oslo_attention_prefill_bwd_workspace_bytes(int64_t batch, int64_t heads,
@@ -468,10 +479,11 @@ size_t oslo_attention_prefill_bwd_workspace_bytes(int64_t batch, int64_t heads,
 /*
  * Backward of the causal prompt attention: from the gradient dout of the
  * output, the inputs q, k, v, the forward's out and lse
- * (oslo_attention_prefill_fwd_lse), with P[i,s] = 2^(log2(e)*(scale*q_i.k_s +
- * pad[s]) - lse[i]) over the visible keys,
- *   dv[s] = sum_i P[i,s] dout[i]
- *   dS[i,s] = scale * P[i,s] * (dout[i].v[s] - sum_d dout[i,d]*out[i,d])
+ * (oslo_attention_prefill_fwd_lse) and its p, seed and offset, with
+ * P[i,s] = 2^(log2(e)*(scale*q_i.k_s + pad[s]) - lse[i]) over the visible keys
+ * and m[i,s] = keep[i,s]/(1-p) (the forward's mask, regenerated; 1 if p == 0),
+ *   dv[s] = sum_i m[i,s] P[i,s] dout[i]
+ *   dS[i,s] = scale * P[i,s] * (m[i,s] * dout[i].v[s] - sum_d dout[i,d]*out[i,d])
  *   dq[i] = sum_s dS[i,s] k[s],   dk[s] = sum_i dS[i,s] q[i].
  * strides[24]: batch, head and position strides, in elements, of q, k, v, out,
  * dout, dq, dk, dv in that order (the limits of oslo_attention_prefill_fwd).
@@ -482,8 +494,8 @@ size_t oslo_attention_prefill_bwd_workspace_bytes(int64_t batch, int64_t heads,
  * bytes (16-byte aligned), contents irrelevant before and after. No output may
  * alias an input.
  * Replaces what autograd records for matmul(q, k^T) ->
- * FusedScaleMaskSoftmax.apply -> matmul(probs, v) of the fused attention in a
- * training step (oslo/models/gptj/modeling_gptj.py:936-951,
+ * FusedScaleMaskSoftmax.apply -> attn_dropout -> matmul(probs, v) of the fused
+ * attention in a training step (oslo/models/gptj/modeling_gptj.py:936-951,
  *  oslo/models/gpt_neo/modeling_gpt_neo.py:993-1008,
  *  oslo/models/gpt2/modeling_gpt2.py:1435-1459): two matmul backwards around
  * the softmax kernel's backward, all on [B, H, S, S] tensors.
@@ -492,10 +504,11 @@ int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const void *dout,
                                const void *q, const void *k, const void *v,
                                const void *out, const float *lse,
                                float *workspace, const float *pad, float scale,
-                               int64_t batch, int64_t heads, int64_t S,
-                               int64_t head_dim, int64_t window,
-                               const int64_t *strides, int dtype,
-                               oslo_stream_t stream);
+                               float p, uint64_t philox_seed,
+                               uint64_t philox_offset, int64_t batch,
+                               int64_t heads, int64_t S, int64_t head_dim,
+                               int64_t window, const int64_t *strides,
+                               int dtype, oslo_stream_t stream);
 
 /* Repeated n-gram blocking (beam search) ------------------------------------ */
 

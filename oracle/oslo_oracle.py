@@ -210,9 +210,11 @@ def attention_decode(q, k, v, last, scale, window=0, dtype=np.float64):
     return out
 
 
-def attention_prefill(q, k, v, scale, pad=None, dtype=np.float64):
+def attention_prefill(q, k, v, scale, pad=None, dtype=np.float64, keep=None, p=0.0):
     """q, k, v [n, S, d]; pad None or additive [S] / [n, S] key mask -> [n, S, d]:
-    row i attends keys 0..i."""
+    row i attends keys 0..i. keep (bool [n, S, S]) and p: attention dropout, the
+    probabilities are multiplied by keep / (1 - p) before they meet the values
+    (self.attn_dropout, oslo/models/gptj/modeling_gptj.py:947-948)."""
     q, k, v = (np.asarray(t, dtype=dtype) for t in (q, k, v))
     n, S, _ = q.shape
     if pad is not None:
@@ -224,17 +226,22 @@ def attention_prefill(q, k, v, scale, pad=None, dtype=np.float64):
             if pad is not None:
                 scores = scores + pad[b, :i + 1]
             e = np.exp(scores - scores.max())
-            out[b, i] = (e / e.sum()) @ v[b, :i + 1]
+            probs = e / e.sum()
+            if keep is not None:
+                probs = np.where(keep[b, i, :i + 1], probs / (1.0 - p), 0.0)
+            out[b, i] = probs @ v[b, :i + 1]
     return out
 
 
-def attention_prefill_bwd(q, k, v, dout, scale, pad=None, window=None, dtype=np.float64):
+def attention_prefill_bwd(q, k, v, dout, scale, pad=None, window=None, dtype=np.float64, keep=None, p=0.0):
     """Gradients of attention_prefill (with GPT-Neo's sliding window if given:
     row i attends keys i - window < s <= i) for the upstream gradient dout:
     q, k, v, dout [n, S, d] -> (dq, dk, dv). With P the probabilities,
     dV = P^T dO, dP = dO V^T, dS = P o (dP - rowsum(dP o P)), dQ = scale dS K,
     dK = scale dS^T Q: what autograd derives for the matmul, softmax, matmul
-    of oslo/models/gptj/modeling_gptj.py:151-191."""
+    of oslo/models/gptj/modeling_gptj.py:151-191. With attention dropout (keep
+    bool [n, S, S], p) the values met m o P, m = keep / (1 - p): dV = (m o P)^T
+    dO and dP = m o (dO V^T)."""
     q, k, v, dout = (np.asarray(t, dtype=dtype) for t in (q, k, v, dout))
     n, S, _ = q.shape
     if pad is not None:
@@ -250,10 +257,11 @@ def attention_prefill_bwd(q, k, v, dout, scale, pad=None, window=None, dtype=np.
             scores = scores + pad[b][None, :]
         scores = np.where(visible, scores, -np.inf)
         e = np.exp(scores - scores.max(axis=1, keepdims=True))
-        p = e / e.sum(axis=1, keepdims=True)
-        dv[b] = p.T @ dout[b]
-        dp = dout[b] @ v[b].T
-        ds = p * (dp - (dp * p).sum(axis=1, keepdims=True))
+        prob = e / e.sum(axis=1, keepdims=True)
+        m = np.ones_like(prob) if keep is None else np.where(keep[b], 1.0 / (1.0 - p), 0.0)
+        dv[b] = (m * prob).T @ dout[b]
+        dp = m * (dout[b] @ v[b].T)
+        ds = prob * (dp - (dp * prob).sum(axis=1, keepdims=True))
         dq[b] = scale * (ds @ k[b])
         dk[b] = scale * (ds.T @ q[b])
     return dq, dk, dv

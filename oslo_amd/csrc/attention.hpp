@@ -5,6 +5,7 @@
 #pragma once
 
 #include "common.hpp"
+#include "dropout.hpp"
 
 namespace oslo {
 
@@ -38,5 +39,53 @@ __device__ __forceinline__ float other_half(float v) {
 // of a row -inf and its softmax 0/0; they are floored at a value that still
 // underflows every exponential but keeps the arithmetic finite.
 constexpr float kMaskFloorLog2 = -1e30f;
+
+// Attention dropout inside the attention kernels. The keep flag of the
+// probability of (query q, key k) of head bh is the one the softmax kernel with
+// fused dropout draws for the flat index ((bh*S + q)*S + k) of a
+// [batch, heads, S, S] tensor: Philox4x32-10, one draw per group of eight
+// consecutive keys, 16 bits per key (S must be a multiple of 8, so that a
+// group lies inside one row). A wave needs the flags of a 32 x 32 tile of
+// (query, key) pairs per step: 128 draws, two per lane. Lane (query q0 + lane %
+// 32, pair lane / 32) draws the groups of keys k0 + 16*(lane/32) .. +15, turns
+// each into a byte of keep bits and puts the two bytes into the wave's own 128
+// bytes of LDS, [query][key / 8]; every lane then reads back the bits of the
+// pairs its accumulator registers hold, whichever of query and key is the lane.
+__device__ __forceinline__ void stage_keep_bits(uint32_t *wave_bits /* 32 words */, const DropArgs &d,
+                                                int64_t bh, int S, int q0, int k0, int lane) {
+  const int qi = lane & 31, pair = lane >> 5;
+  const uint64_t group = ((uint64_t)bh * S + (uint64_t)(q0 + qi)) * (uint64_t)(S >> 3) +
+                         (uint64_t)((k0 >> 3) + 2 * pair);
+  uint32_t two = 0;
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    const Philox4 w = dropout_draw(d.seed, d.offset, group + e);
+    uint32_t byte = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      byte |= ((w.w[j] & 0xFFFFu) >= d.threshold ? 1u : 0u) << (2 * j);
+      byte |= ((w.w[j] >> 16) >= d.threshold ? 1u : 0u) << (2 * j + 1);
+    }
+    two |= byte << (8 * e);
+  }
+  // all lanes of the wave have read the previous step's bits before these stores
+  __builtin_amdgcn_wave_barrier();
+  reinterpret_cast<unsigned short *>(wave_bits)[2 * qi + pair] = (unsigned short)two;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Keep bits of accumulator register r (row 8*(r/4) + 4*half + r%4 of the tile)
+// when the lane is the query and the rows are keys: one word per lane, bit =
+// the key's index in the tile.
+__device__ __forceinline__ uint32_t keep_word_query_lane(const uint32_t *wave_bits, int col) {
+  return wave_bits[col];
+}
+// ... and when the lane is the key (column `col` of the tile) and the rows are
+// queries: four words (queries 8j + 4*half .. + 3) per j, bit = col.
+__device__ __forceinline__ u32x4 keep_words_key_lane(const uint32_t *wave_bits, int j, int half) {
+  return *reinterpret_cast<const u32x4 *>(&wave_bits[8 * j + 4 * half]);
+}
 
 } // namespace oslo

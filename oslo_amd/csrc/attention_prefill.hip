@@ -59,9 +59,10 @@ struct PrefillArgs {
   int head_groups; // ceil(batch_heads / 8)
   int query_blocks;
   int window; // 0: every key up to the query; else the last `window` of them
+  DropArgs drop; // attention dropout (the DROP variants of the kernel)
 };
 
-template <typename T, int D, bool HAS_PAD, bool HAS_WINDOW>
+template <typename T, int D, bool HAS_PAD, bool HAS_WINDOW, bool DROP>
 __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_prefill_kernel(
     const PrefillArgs a) {
   using Op = MatrixOp<T>;
@@ -83,6 +84,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   __shared__ __align__(16) T k_lds[kKeysPerTile * D];  // [key][chunk ^ (key & kSwizzleK)][8]
   __shared__ __align__(16) T vt_lds[D * kKeysPerTile]; // [d][(slot + d + d/8) & 7][8]
   __shared__ __align__(16) float pad_lds[HAS_PAD ? kKeysPerTile : 4]; // the tile's mask values, log2 units
+  __shared__ __align__(16) uint32_t keep_lds[DROP ? kWavesPerBlock : 1][32]; // a wave's keep bits of a step
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -324,6 +326,14 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
       sum += sc[r];
     }
     l += sum;
+    if constexpr (DROP) {
+      // attention dropout: the sum keeps every probability, the product with V
+      // only the kept ones (their 1/(1-p) goes into the final normalisation)
+      stage_keep_bits(keep_lds[wave], a.drop, bh, S, wave_q0, keyb, lane);
+      const uint32_t bits = keep_word_query_lane(keep_lds[wave], col) >> (4 * half);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[r] = (bits >> (8 * (r >> 2) + (r & 3))) & 1u ? sc[r] : 0.f;
+    }
 
     // P^T as B operands, in the storage type like the unfused path's cast
     Frag pf[2];
@@ -396,7 +406,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   }
 
   l += other_half(l);
-  const float inv = 1.0f / l;
+  const float inv = DROP ? a.drop.keep_scale / l : 1.0f / l;
   if (qrow >= S) return;
   if (a.lse != nullptr && half == 0)
     a.lse[(int64_t)bh * S + qrow] = m + __builtin_amdgcn_logf(l); // v_log_f32 is log2
@@ -422,7 +432,8 @@ int launch_prefill_dim(const PrefillArgs &a, hipStream_t stream) {
   // setting, not a stream operation) before every launch.
   constexpr unsigned kDynamic = D == 256 ? kQueriesPerBlock * D * sizeof(T) : 0;
   auto go = [&]<bool HAS_PAD, bool HAS_WINDOW>() -> int {
-    auto *kernel = attention_prefill_kernel<T, D, HAS_PAD, HAS_WINDOW>;
+    auto *kernel = a.drop.drop ? attention_prefill_kernel<T, D, HAS_PAD, HAS_WINDOW, true>
+                               : attention_prefill_kernel<T, D, HAS_PAD, HAS_WINDOW, false>;
     if (kDynamic > 0) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynamic);
@@ -454,7 +465,8 @@ int launch_prefill(const PrefillArgs &a, int head_dim, hipStream_t stream) {
 } // namespace oslo
 
 namespace {
-int prefill_entry(void *out, float *lse, const void *q, const void *k, const void *v,
+int prefill_entry(void *out, float *lse, const oslo::DropArgs &drop, const void *q,
+                  const void *k, const void *v,
                   const float *pad, float scale, int64_t batch, int64_t heads,
                   int64_t S, int64_t head_dim, int64_t window,
                   const int64_t *strides, int dtype, oslo_stream_t stream) {
@@ -494,7 +506,10 @@ int prefill_entry(void *out, float *lse, const void *q, const void *k, const voi
     return fail(OSLO_E_UNSUPPORTED,
                 "oslo_attention_prefill_fwd: with a padding mask S must be a multiple of 4 and the mask 16-byte aligned");
   PrefillArgs a;
-  a.out = out, a.q = q, a.k = k, a.v = v, a.pad = pad, a.lse = lse;
+  if (drop.drop && S % 8 != 0)
+    return fail(OSLO_E_UNSUPPORTED,
+                "oslo_attention_prefill_fwd_lse: with attention dropout S must be a multiple of 8");
+  a.out = out, a.q = q, a.k = k, a.v = v, a.pad = pad, a.lse = lse, a.drop = drop;
   a.q_b = strides[0], a.q_h = strides[1], a.q_s = strides[2];
   a.k_b = strides[3], a.k_h = strides[4], a.k_s = strides[5];
   a.v_b = strides[6], a.v_h = strides[7], a.v_s = strides[8];
@@ -521,19 +536,26 @@ extern "C" int oslo_attention_prefill_fwd(void *out, const void *q, const void *
                                           int64_t window,
                                           const int64_t *strides, int dtype,
                                           oslo_stream_t stream) {
-  return prefill_entry(out, nullptr, q, k, v, pad, scale, batch, heads, S, head_dim,
+  oslo::DropArgs none{};
+  return prefill_entry(out, nullptr, none, q, k, v, pad, scale, batch, heads, S, head_dim,
                        window, strides, dtype, stream);
 }
 
 extern "C" int oslo_attention_prefill_fwd_lse(void *out, float *lse, const void *q,
                                               const void *k, const void *v,
-                                              const float *pad, float scale,
-                                              int64_t batch, int64_t heads, int64_t S,
+                                              const float *pad, float scale, float p,
+                                              uint64_t philox_seed,
+                                              uint64_t philox_offset, int64_t batch,
+                                              int64_t heads, int64_t S,
                                               int64_t head_dim, int64_t window,
                                               const int64_t *strides, int dtype,
                                               oslo_stream_t stream) {
+  oslo::DropArgs drop;
+  const int s = oslo::make_drop_args("oslo_attention_prefill_fwd_lse", p, philox_seed,
+                                     philox_offset, &drop);
+  if (s != OSLO_OK) return s;
   if (lse == nullptr && batch > 0 && heads > 0 && S > 0)
     return oslo::fail(OSLO_E_BAD_ARG, "oslo_attention_prefill_fwd_lse: null lse");
-  return prefill_entry(out, lse, q, k, v, pad, scale, batch, heads, S, head_dim,
+  return prefill_entry(out, lse, drop, q, k, v, pad, scale, batch, heads, S, head_dim,
                        window, strides, dtype, stream);
 }

@@ -53,6 +53,7 @@ struct BwdArgs {
   Strides3 sq, sk, sv, sdo, sdq, sdk, sdv;
   float scale, scale_log2e;
   int S, heads, batch_heads, head_groups, own_blocks, window;
+  DropArgs drop; // attention dropout of the forward (the DROP variants)
 };
 
 template <int D>
@@ -72,7 +73,7 @@ constexpr unsigned bwd_lds_bytes() {
   return n;
 }
 
-template <typename T, int D, int ROLE, bool HAS_PAD, bool HAS_WINDOW>
+template <typename T, int D, int ROLE, bool HAS_PAD, bool HAS_WINDOW, bool DROP>
 __global__ __launch_bounds__(kBlockThreads, D == 64 && ROLE != kRoleDKV ? 2 : 1) void attention_bwd_kernel(
     const BwdArgs a) {
   using Op = MatrixOp<T>;
@@ -112,6 +113,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 64 && ROLE != kRoleDKV ? 2 : 1)
   float *const row_a = reinterpret_cast<float *>(o1_lds + kOffEnd);
   float *const row_b = row_a + kTile;
   u32x4 *const own1_lds = reinterpret_cast<u32x4 *>(row_b + kTile);
+  __shared__ __align__(16) uint32_t keep_lds[DROP ? kWavesPerBlock : 1][32]; // a wave's keep bits of a step
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -357,7 +359,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 64 && ROLE != kRoleDKV ? 2 : 1)
     }
 
     // P = exp2(scale*log2e * T1 + pad - lse); dS = scale * P * (T2 - delta)
-    float p[16], ds[16];
+    float p[16], dl[16]; // the probabilities; delta of each register's query
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       float ra[4] = {0.f, 0.f, 0.f, 0.f}, rb[4] = {0.f, 0.f, 0.f, 0.f};
@@ -375,7 +377,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 64 && ROLE != kRoleDKV ? 2 : 1)
         // keys own: pad of the lane, lse and delta of the row; queries own: the reverse
         const float shift = kKeysOwn ? own_pad - ra[tt] : ra[tt] - own_lse;
         p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(t1[r], a.scale_log2e, shift));
-        if constexpr (kNeedT2) ds[r] = t2[r] - (kKeysOwn ? rb[tt] : own_delta);
+        dl[r] = kKeysOwn ? rb[tt] : own_delta;
       }
     }
     if (diagonal) {
@@ -388,13 +390,37 @@ __global__ __launch_bounds__(kBlockThreads, D == 64 && ROLE != kRoleDKV ? 2 : 1)
         p[r] = visible ? p[r] : 0.f;
       }
     }
+    // With attention dropout the forward multiplied V with keep * P / (1-p): the
+    // P product takes the kept probabilities (1/(1-p) goes onto dV at the end),
+    // and the gradient of the dropped-out probabilities is keep * dP / (1-p).
+    float pk[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) pk[r] = p[r];
+    if constexpr (DROP) {
+      stage_keep_bits(keep_lds[wave], a.drop, bh, S, kKeysOwn ? ob : wave_own0, kKeysOwn ? wave_own0 : ob, lane);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        u32x4 words;
+        uint32_t bits = 0;
+        if constexpr (kKeysOwn) words = keep_words_key_lane(keep_lds[wave], j, half);
+        else bits = keep_word_query_lane(keep_lds[wave], col) >> (8 * j + 4 * half);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+          const int r = 4 * j + tt;
+          const bool keep = kKeysOwn ? ((words[tt] >> col) & 1u) != 0 : ((bits >> tt) & 1u) != 0;
+          pk[r] = keep ? p[r] : 0.f;
+          if constexpr (kNeedT2) t2[r] = keep ? t2[r] * a.drop.keep_scale : 0.f;
+        }
+      }
+    }
     Frag pf[2], sf[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        pf[u][i] = static_cast<T>(p[8 * u + i]);
-        if constexpr (kNeedT2) sf[u][i] = static_cast<T>(a.scale * (p[8 * u + i] * ds[8 * u + i]));
+        pf[u][i] = static_cast<T>(pk[8 * u + i]);
+        if constexpr (kNeedT2)
+          sf[u][i] = static_cast<T>(a.scale * (p[8 * u + i] * (t2[8 * u + i] - dl[8 * u + i])));
       }
 
     // Acc^T += OtherT x X, 16 positions of the step at a time
@@ -425,7 +451,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 64 && ROLE != kRoleDKV ? 2 : 1)
 
   if (own >= S) return;
   typedef T Out4 __attribute__((ext_vector_type(4)));
-  auto write = [&](void *base, const Strides3 &st, const f32x16 (&acc)[kBlocksD]) {
+  auto write = [&](void *base, const Strides3 &st, const f32x16 (&acc)[kBlocksD], float factor) {
     T *op = static_cast<T *>(base) + b * st.b + hd * st.h + (int64_t)own * st.s;
 #pragma unroll
     for (int i = 0; i < kBlocksD; ++i)
@@ -433,13 +459,13 @@ __global__ __launch_bounds__(kBlockThreads, D == 64 && ROLE != kRoleDKV ? 2 : 1)
       for (int j = 0; j < 4; ++j) {
         Out4 w;
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(acc[i][4 * j + tt]);
+        for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(acc[i][4 * j + tt] * factor);
         *reinterpret_cast<Out4 *>(op + 32 * i + 8 * j + 4 * half) = w;
       }
   };
-  if constexpr (ROLE == kRoleDQ) write(a.dq, a.sdq, acc_s);
-  if constexpr (ROLE == kRoleDKV || ROLE == kRoleDK) write(a.dk, a.sdk, acc_s);
-  if constexpr (ROLE == kRoleDKV || ROLE == kRoleDV) write(a.dv, a.sdv, acc_p);
+  if constexpr (ROLE == kRoleDQ) write(a.dq, a.sdq, acc_s, 1.0f);
+  if constexpr (ROLE == kRoleDKV || ROLE == kRoleDK) write(a.dk, a.sdk, acc_s, 1.0f);
+  if constexpr (ROLE == kRoleDKV || ROLE == kRoleDV) write(a.dv, a.sdv, acc_p, DROP ? a.drop.keep_scale : 1.0f);
 }
 
 // delta[bh, q] = sum_d dO[q, d] * O[q, d], fp32. D / 8 lanes share a row.
@@ -471,7 +497,8 @@ int launch_role(const BwdArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)(8 * a.head_groups * a.own_blocks));
   constexpr unsigned kLds = bwd_lds_bytes<T, D, ROLE>();
   auto go = [&]<bool HAS_PAD, bool HAS_WINDOW>() -> int {
-    auto *kernel = attention_bwd_kernel<T, D, ROLE, HAS_PAD, HAS_WINDOW>;
+    auto *kernel = a.drop.drop ? attention_bwd_kernel<T, D, ROLE, HAS_PAD, HAS_WINDOW, true>
+                               : attention_bwd_kernel<T, D, ROLE, HAS_PAD, HAS_WINDOW, false>;
     if (kLds > 48 * 1024) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
@@ -534,6 +561,8 @@ extern "C" int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const vo
                                           const void *q, const void *k, const void *v,
                                           const void *out, const float *lse,
                                           float *workspace, const float *pad, float scale,
+                                          float p, uint64_t philox_seed,
+                                          uint64_t philox_offset,
                                           int64_t batch, int64_t heads, int64_t S,
                                           int64_t head_dim, int64_t window,
                                           const int64_t *strides, int dtype,
@@ -550,7 +579,12 @@ extern "C" int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const vo
     return fail(OSLO_E_UNSUPPORTED, "%s: heads of %lld features (64, 128 or 256 are taken)", name,
                 (long long)head_dim);
   if (!(scale > 0.0f)) return fail(OSLO_E_BAD_ARG, "%s: the scale must be positive", name);
+  DropArgs drop;
+  const int ds = make_drop_args(name, p, philox_seed, philox_offset, &drop);
+  if (ds != OSLO_OK) return ds;
   if (batch == 0 || heads == 0 || S == 0) return OSLO_OK;
+  if (drop.drop && S % 8 != 0)
+    return fail(OSLO_E_UNSUPPORTED, "%s: with attention dropout S must be a multiple of 8", name);
   if (!dq || !dk || !dv || !dout || !q || !k || !v || !out || !lse || !workspace || !strides)
     return fail(OSLO_E_BAD_ARG, "%s: null pointer", name);
   if (batch * heads > (int64_t)0x7fffffff / 8 || batch * heads * S > (int64_t)0x7fffffff)
@@ -574,7 +608,7 @@ extern "C" int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const vo
   auto st = [&](int i) { return Strides3{strides[3 * i], strides[3 * i + 1], strides[3 * i + 2]}; };
   BwdArgs a;
   a.q = q, a.k = k, a.v = v, a.dout = dout, a.dq = dq, a.dk = dk, a.dv = dv;
-  a.lse = lse, a.delta = workspace, a.pad = pad;
+  a.lse = lse, a.delta = workspace, a.pad = pad, a.drop = drop;
   a.sq = st(0), a.sk = st(1), a.sv = st(2), a.sdo = st(4), a.sdq = st(5), a.sdk = st(6), a.sdv = st(7);
   a.scale = scale;
   a.scale_log2e = scale * kLog2eB;

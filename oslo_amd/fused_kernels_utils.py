@@ -546,31 +546,33 @@ class FusedDecodeAttention(object):
 class _PrefillAttention(torch.autograd.Function):
     """The prompt attention with its backward: the forward keeps q, k, v, its
     output and one fp32 number per row (the log-sum-exp); the backward
-    recomputes the probabilities tile by tile on the matrix cores."""
+    recomputes the probabilities (and the dropout mask, from the same Philox
+    seed and offset) tile by tile on the matrix cores."""
 
     @staticmethod
-    def forward(ctx, query, key, value, pad, scale, window):
+    def forward(ctx, query, key, value, pad, scale, window, p):
+        seed, offset = _next_philox(query.device) if p > 0.0 else (0, 0)
         out, lse = get_custom_kernels().attention_prefill_forward(query, key, value, scale, pad, window,
-                                                                  want_lse=True)
+                                                                  want_lse=True, p=p, seed=seed, offset=offset)
         ctx.save_for_backward(query, key, value, out, lse)
         ctx.pad = pad
-        ctx.args = (float(scale), int(window))
+        ctx.args = (float(scale), int(window), float(p), seed, offset)
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         query, key, value, out, lse = ctx.saved_tensors
-        scale, window = ctx.args
+        scale, window, p, seed, offset = ctx.args
         dq, dk, dv = get_custom_kernels().attention_prefill_backward(
-            grad_out, query, key, value, out, lse, scale, ctx.pad, window)
-        return dq, dk, dv, None, None, None
+            grad_out, query, key, value, out, lse, scale, ctx.pad, window, p, seed, offset)
+        return dq, dk, dv, None, None, None, None
 
 
 class FusedPrefillAttention(object):
     """
     Kernel fusion function: causal attention over a whole prompt
 
-    Before fusion: Matmul (Q * K^T) -> (Scale + Mask + Softmax) -> Matmul (Score * V)
+    Before fusion: Matmul (Q * K^T) -> (Scale + Mask + Softmax) -> Dropout -> Matmul (Score * V)
     After fusion: one kernel on the matrix cores; the [S, S] scores stay on chip
 
     Not in the reference, whose fused attention keeps both matmuls around the
@@ -582,9 +584,10 @@ class FusedPrefillAttention(object):
     heads of 64, 128 or 256 features; no probabilities to return. With
     gradients recorded the forward also keeps the log-sum-exp of every row and
     the backward recomputes the probabilities from it, so a training step
-    stores no [B, H, S, S] tensor either. Attention dropout is not part of
-    the kernel: a module that drops attention probabilities in training keeps
-    the softmax kernel with fused dropout between its two matmuls.
+    stores no [B, H, S, S] tensor either. ``dropout_p`` > 0 (training) drops
+    attention probabilities inside the kernel, with the keep mask the softmax
+    kernel with fused dropout would draw from the device generator (S must be
+    a multiple of 8 then).
     """
 
     MIN_LENGTH = 2  # one query is a decoding step (FusedDecodeAttention); from two on, one launch beats three
@@ -595,9 +598,9 @@ class FusedPrefillAttention(object):
             return False
         if query.dtype not in (torch.half, torch.bfloat16) or key.dtype != query.dtype:
             return False
-        if training and dropout_p > 0.0:
-            return False
         b, _, s, d = query.shape
+        if training and dropout_p > 0.0 and (s % 8 != 0 or not dropout_p < 1.0):
+            return False
         if d not in (64, 128, 256) or s < FusedPrefillAttention.MIN_LENGTH or s * d * query.element_size() >= 2 ** 30:
             return False
         if attention_mask is not None and not (
@@ -607,13 +610,14 @@ class FusedPrefillAttention(object):
         return True
 
     @staticmethod
-    def apply(query, key, value, attention_mask=None, scale=None, window=None):
-        """``window``: GPT-Neo's local attention (query i sees keys i - window < s <= i)."""
+    def apply(query, key, value, attention_mask=None, scale=None, window=None, dropout_p=0.0):
+        """``window``: GPT-Neo's local attention (query i sees keys i - window < s <= i).
+        ``dropout_p``: attention dropout, 0 outside training."""
         b, _, s, _ = query.shape
         pad = None if attention_mask is None else attention_mask.reshape(b, s).float()
         scale = 1.0 if scale is None else scale
-        if _needs_grad(query, key, value):
-            return _PrefillAttention.apply(query, key, value, pad, scale, window or 0)
+        if dropout_p > 0.0 or _needs_grad(query, key, value):
+            return _PrefillAttention.apply(query, key, value, pad, scale, window or 0, float(dropout_p))
         return get_custom_kernels().attention_prefill_forward(query, key, value, scale, pad, window or 0)
 
 

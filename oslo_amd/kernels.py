@@ -614,7 +614,8 @@ def _stride_table(tensors):
     return strides
 
 
-def attention_prefill_forward(query, key, value, scale, pad=None, window=0, want_lse=False):
+def attention_prefill_forward(query, key, value, scale, pad=None, window=0, want_lse=False, p=0.0, seed=0,
+                              offset=0):
     """Causal attention of a whole prompt in one kernel: query, key, value
     [B, H, S, D] fp16/bf16 views (features contiguous, any batch/head/position
     strides that are multiples of 8 elements), ``pad`` an optional additive
@@ -624,9 +625,12 @@ def attention_prefill_forward(query, key, value, scale, pad=None, window=0, want
     afterwards moves nothing (oslo/models/gptj/modeling_gptj.py:936-951 and
     the ``_merge_heads`` that follows it). The [S, S] scores never reach memory.
     With ``want_lse`` also the fp32 [B, H, S] log2-sum-exp of every row, which
-    ``attention_prefill_backward`` takes."""
+    ``attention_prefill_backward`` takes; then ``p`` > 0 applies attention
+    dropout inside the kernel (keep mask of Philox ``seed`` / ``offset`` as the
+    softmax kernel with fused dropout draws it; S a multiple of 8)."""
     code, pad = _prefill_args(query, key, value, pad)
     b, h, s, d = query.shape
+    _require(p == 0.0 or want_lse, "attention dropout belongs to the training forward (want_lse)")
     q, k, v = _prefill_strided(query), _prefill_strided(key), _prefill_strided(value)
     out = torch.empty((b, s, h, d), dtype=query.dtype, device=query.device).permute(0, 2, 1, 3)
     lse = torch.empty((b, h, s), dtype=torch.float32, device=query.device) if want_lse else None
@@ -635,8 +639,8 @@ def attention_prefill_forward(query, key, value, scale, pad=None, window=0, want
         with _on_device(q):
             if want_lse:
                 _lib.check(_lib.load().oslo_attention_prefill_fwd_lse(
-                    _ptr(out), _ptr(lse), _ptr(q), _ptr(k), _ptr(v), _ptr(pad), float(scale), b, h, s, d,
-                    int(window), strides, code, _stream(q)))
+                    _ptr(out), _ptr(lse), _ptr(q), _ptr(k), _ptr(v), _ptr(pad), float(scale), float(p), int(seed),
+                    int(offset), b, h, s, d, int(window), strides, code, _stream(q)))
             else:
                 _lib.check(_lib.load().oslo_attention_prefill_fwd(
                     _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(pad), float(scale), b, h, s, d, int(window), strides,
@@ -644,12 +648,14 @@ def attention_prefill_forward(query, key, value, scale, pad=None, window=0, want
     return (out, lse) if want_lse else out
 
 
-def attention_prefill_backward(grad_out, query, key, value, out, lse, scale, pad=None, window=0):
+def attention_prefill_backward(grad_out, query, key, value, out, lse, scale, pad=None, window=0, p=0.0, seed=0,
+                               offset=0):
     """Gradients of ``attention_prefill_forward`` with respect to query, key and
     value (each [B, H, S, D], dense), from the gradient of its output, its
-    inputs, its output and the log-sum-exp it returned with ``want_lse``. The
-    [S, S] probabilities are recomputed tile by tile; nothing of that size is
-    stored."""
+    inputs, its output and the log-sum-exp it returned with ``want_lse`` (and
+    its ``p``, ``seed``, ``offset`` if it dropped attention probabilities). The
+    [S, S] probabilities and their keep mask are recomputed tile by tile;
+    nothing of that size is stored."""
     code, pad = _prefill_args(query, key, value, pad)
     _device_tensor(grad_out, "grad_out", query)
     _require(grad_out.shape == query.shape and out.shape == query.shape, "grad_out and out must be shaped like query")
@@ -668,7 +674,8 @@ def attention_prefill_backward(grad_out, query, key, value, out, lse, scale, pad
     with _on_device(q):
         _lib.check(lib.oslo_attention_prefill_bwd(
             _ptr(dq), _ptr(dk), _ptr(dv), _ptr(g), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(ws),
-            _ptr(pad), float(scale), b, h, s, d, int(window), strides, code, _stream(q)))
+            _ptr(pad), float(scale), float(p), int(seed), int(offset), b, h, s, d, int(window), strides, code,
+            _stream(q)))
     return dq, dk, dv
 
 

@@ -201,9 +201,10 @@ class FusedGPT2Attention(GPT2Attention):
                                              self._attention_scale(value), None, *fresh)
             w = None
         elif prompt:
-            # a whole prompt at inference: one kernel, the scores stay on chip
-            out, w = FusedPrefillAttention.apply(query, key, value, attention_mask,
-                                                 self._attention_scale(value)), None
+            # a whole prompt: one kernel, the scores stay on chip (in training too: it has a backward
+            # and drops attention probabilities itself)
+            out, w = FusedPrefillAttention.apply(query, key, value, attention_mask, self._attention_scale(value),
+                                                 None, self.attn_dropout.p if self.training else 0.0), None
         elif fused:
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)
         else:

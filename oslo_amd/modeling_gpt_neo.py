@@ -179,9 +179,11 @@ class FusedGPTNeoSelfAttention(GPTNeoSelfAttention):
                                              None, self._window(), *fresh)
             w = None
         elif prompt:
-            # a whole prompt at inference: one kernel, the scores stay on chip (a local
+            # a whole prompt: one kernel, the scores stay on chip (in training too: it has a backward
+            # and drops attention probabilities itself) (a local
             # layer's window included)
-            out, w = FusedPrefillAttention.apply(query, key, value, attention_mask, None, self._window()), None
+            out, w = FusedPrefillAttention.apply(query, key, value, attention_mask, None, self._window(),
+                                                 self.attn_dropout.p if self.training else 0.0), None
         elif fused and static:
             out, w = FusedGPTNeoSelfAttention._fused_attn(self, query, key, value, attention_mask, head_mask, False)
         elif fused:

@@ -229,8 +229,10 @@ class FusedGPTJAttention(GPTJAttention):
                                              1.0 / self.scale_attn, None, *fresh)
             w = None
         elif prompt:
-            # a whole prompt at inference: one kernel, the scores stay on chip
-            out, w = FusedPrefillAttention.apply(query, key, value, attention_mask, 1.0 / self.scale_attn), None
+            # a whole prompt: one kernel, the scores stay on chip (in training too: it has a backward
+            # and drops attention probabilities itself)
+            out, w = FusedPrefillAttention.apply(query, key, value, attention_mask, 1.0 / self.scale_attn, None,
+                                                 self.attn_dropout.p if self.training else 0.0), None
         elif fused:
             out, w = self._fused_attn(query, key, value, attention_mask, head_mask, causal)
         else:

@@ -29,7 +29,7 @@ HALVES = [torch.float16, torch.bfloat16]
 REL = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}
 
 
-def reference(q, k, v, do, scale, pad=None, window=0):
+def reference(q, k, v, do, scale, pad=None, window=0, keep=None, p_drop=0.0):
     """float64 gradients and the error bounds described above, on the inputs' device."""
     q, k, v, do = q.double(), k.double(), v.double(), do.double()
     s = q.shape[2]
@@ -41,9 +41,10 @@ def reference(q, k, v, do, scale, pad=None, window=0):
     if window:
         hidden = hidden | (i[None, :] <= i[:, None] - window)
     p = torch.softmax(w.masked_fill(hidden, float("-inf")), -1)
-    o = p @ v
-    dv = p.transpose(-1, -2) @ do
-    dp = do @ v.transpose(-1, -2)
+    m = torch.ones_like(p) if keep is None else keep.double() / (1.0 - p_drop)   # the dropout factor on P
+    o = (m * p) @ v
+    dv = (m * p).transpose(-1, -2) @ do
+    dp = m * (do @ v.transpose(-1, -2))
     delta = (do * o).sum(-1, keepdim=True)
     ds = p * (dp - delta)
     dq = scale * (ds @ k)
@@ -53,7 +54,7 @@ def reference(q, k, v, do, scale, pad=None, window=0):
     bounds = {
         "dq": dq.abs() + scale * (ds_mag @ k.abs()),
         "dk": dk.abs() + scale * (ds_mag.transpose(-1, -2) @ q.abs()),
-        "dv": dv.abs() + p.transpose(-1, -2) @ do.abs(),
+        "dv": dv.abs() + (m * p).transpose(-1, -2) @ do.abs(),
     }
     return o, {"dq": dq, "dk": dk, "dv": dv}, bounds
 
@@ -162,6 +163,78 @@ def test_backward_strided_inputs_determinism_and_closed_forms(dtype):
     # so dS (and with it dq, dk) is zero up to the rounding of an fp32 sum
     assert torch.equal(single["dv"], one[3])
     assert single["dq"].abs().max().item() <= 1e-4 and single["dk"].abs().max().item() <= 1e-4
+
+
+def keep_mask(b, h, s, p, seed, offset):
+    """The mask of the softmax kernel with fused dropout: flat index over [B, H, S, S]."""
+    return torch.from_numpy(orc.dropout_keep_mask(seed, offset, b * h * s * s, p).reshape(b, h, s, s))
+
+
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+@pytest.mark.parametrize("d", [64, 128, 256])
+@pytest.mark.parametrize("s", [8, 64, 200, 328])
+def test_attention_dropout_forward_and_backward(s, d, dtype):
+    """Attention dropout inside the kernels: the forward equals the oracle's
+    with the keep mask the softmax kernel with fused dropout draws for the same
+    seed and offset, the log-sum-exp is that of the undropped probabilities,
+    the backward regenerates the same mask."""
+    b, h, p, seed, offset = 2, 3, 0.25, 1234, 8
+    scale = 1.0 / math.sqrt(d)
+    q, k, v, do = (randn((b, h, s, d), dtype, seed=13 * s + i) for i in range(4))
+    dev = [t.to(DEV) for t in (q, k, v, do)]
+    keep = keep_mask(b, h, s, p, seed, offset)
+    for pad, window in ((None, 0), (padding(b, s, s), 0), (None, 40)):
+        padd = None if pad is None else pad.to(DEV)
+        out, lse = kernels.attention_prefill_forward(*dev[:3], scale, padd, window, want_lse=True, p=p, seed=seed,
+                                                     offset=offset)
+        plain, lse0 = kernels.attention_prefill_forward(*dev[:3], scale, padd, window, want_lse=True)
+        assert torch.equal(lse, lse0)
+        o_ref, want, bounds = reference(*dev, scale, padd, window, keep.to(DEV), p)
+        vmax = 4.0 / (1 - p)
+        excess = ((out.double() - o_ref).abs() - REL[dtype] * (o_ref.abs() + vmax)).max().item()
+        assert excess <= 1e-4, (excess, s, d, "forward")
+        dq, dk, dv = kernels.attention_prefill_backward(dev[3], *dev[:3], out, lse, scale, padd, window, p, seed, offset)
+        check({"dq": dq, "dk": dk, "dv": dv}, want, bounds, dtype, (s, d, pad is not None, window))
+        if pad is None and window == 0 and s <= 64:
+            flat = [f32(t).reshape(b * h, s, d) for t in (q, k, v, do)]
+            kf = keep.numpy().reshape(b * h, s, s)
+            o_orc = orc.attention_prefill(*flat[:3], scale, keep=kf, p=p).reshape(b, h, s, d)
+            assert np.abs(o_orc - o_ref.cpu().numpy()).max() <= 1e-9
+            g_orc = orc.attention_prefill_bwd(*flat, scale, keep=kf, p=p)
+            for n, g in zip(("dq", "dk", "dv"), g_orc):
+                assert np.abs(g.reshape(b, h, s, d) - want[n].cpu().numpy()).max() <= 1e-9
+    # another offset is another mask; the same one repeats bit for bit
+    again = kernels.attention_prefill_forward(*dev[:3], scale, None, 0, want_lse=True, p=p, seed=seed, offset=offset)[0]
+    other = kernels.attention_prefill_forward(*dev[:3], scale, None, 0, want_lse=True, p=p, seed=seed, offset=offset + 4)[0]
+    first = kernels.attention_prefill_forward(*dev[:3], scale, None, 0, want_lse=True, p=p, seed=seed, offset=offset)[0]
+    assert torch.equal(again, first) and not torch.equal(again, other)
+
+
+def test_attention_dropout_long_prompt_and_operator():
+    """At [2,4,1024,128]: against the float64 formulas with the regenerated mask;
+    and through FusedPrefillAttention.apply, which takes seed and offset from the
+    device generator and advances it like the softmax kernel with dropout."""
+    from oslo_amd import FusedPrefillAttention
+    dtype, b, h, s, d, p = torch.bfloat16, 2, 4, 1024, 128, 0.1
+    q, k, v, do = (randn((b, h, s, d), dtype, seed=40 + i).to(DEV) for i in range(4))
+    torch.manual_seed(77)
+    gen = torch.cuda.default_generators[0]
+    seed, off0 = gen.initial_seed(), gen.get_offset()
+    qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+    out = FusedPrefillAttention.apply(qq, kk, vv, None, 0.1, None, p)
+    assert gen.get_offset() == off0 + 4
+    out.backward(do)
+    keep = keep_mask(b, h, s, p, seed, off0).to(DEV)
+    o_ref, want, bounds = reference(q, k, v, do, 0.1, None, 0, keep, p)
+    assert ((out.detach().double() - o_ref).abs() - REL[dtype] * (o_ref.abs() + 4.0 / (1 - p))).max().item() <= 1e-4
+    check({"dq": qq.grad, "dk": kk.grad, "dv": vv.grad}, want, bounds, dtype, "operator")
+    # the fraction of (query, key) pairs dropped, read off a forward with v = identity-like columns:
+    # with q = 0 the probabilities of row i are 1/(i+1), so out[i] = sum_s keep/(1-p)/(i+1) * v[s]
+    ones = torch.ones_like(v)
+    frac = kernels.attention_prefill_forward(torch.zeros_like(q), k, ones, 1.0, None, 0, want_lse=True, p=p,
+                                             seed=seed, offset=off0)[0][..., 0].double()
+    want_frac = (keep.double().tril().sum(-1) / (1 - p)) / torch.arange(1, s + 1, device=DEV)
+    assert (frac - want_frac).abs().max().item() <= 2.0 ** -7 * 2
 
 
 def test_backward_rejects_what_it_cannot_take():

@@ -189,14 +189,14 @@ def test_prefill_operator_gate_and_errors():
     mask = padding(1, 256, 1).to(DEV).view(1, 1, 1, 256).half()
     assert FusedPrefillAttention.is_available(q, q)
     assert FusedPrefillAttention.is_available(q, q, mask)
-    assert not FusedPrefillAttention.is_available(q, q, training=True, dropout_p=0.1)
+    assert FusedPrefillAttention.is_available(q, q, training=True, dropout_p=0.1)       # dropout inside the kernel
+    assert not FusedPrefillAttention.is_available(q[:, :, :250], q[:, :, :250], training=True, dropout_p=0.1)  # S % 8
     assert not FusedPrefillAttention.is_available(q.float(), q.float())
     assert FusedPrefillAttention.is_available(q[:, :, :5], q[:, :, :5])            # short prompts too
     assert not FusedPrefillAttention.is_available(q[:, :, :1], q[:, :, :1])        # one query: a decoding step
     assert not FusedPrefillAttention.is_available(q[:, :, :128], q)                # a cache longer than the prompt
     assert not FusedPrefillAttention.is_available(q[..., :32], q[..., :32])        # head size
-    assert not FusedPrefillAttention.is_available(q.requires_grad_(), q)
-    q = q.detach()
+    assert FusedPrefillAttention.is_available(q.clone().requires_grad_(), q)             # it has a backward
     out = FusedPrefillAttention.apply(q, q, q, mask, 0.125)
     check(out, device_reference(q, q, q, 0.125, mask.view(1, 256).float()), torch.float16, "operator")
     with pytest.raises(RuntimeError):

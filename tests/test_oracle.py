@@ -515,3 +515,22 @@ def test_attention_prefill_bwd_against_autograd_and_differences():
     # a single position: the probability is 1, dV = dO, dQ = dK = 0
     dq1, dk1, dv1 = orc.attention_prefill_bwd(q[:, :1].numpy(), k[:, :1].numpy(), v[:, :1].numpy(), do[:, :1].numpy(), scale)
     assert np.array_equal(dv1, do[:, :1].numpy()) and not dq1.any() and not dk1.any()
+
+
+def test_attention_prefill_dropout_against_autograd():
+    """The probabilities times keep / (1 - p): forward and gradients against
+    torch operators in float64 with the same mask."""
+    g = torch.Generator().manual_seed(6)
+    n, S, d, scale, p = 2, 11, 4, 0.4, 0.25
+    q, k, v, do = (torch.randn((n, S, d), generator=g, dtype=torch.float64) for _ in range(4))
+    keep = torch.rand((n, S, S), generator=g) >= p
+    qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+    i = torch.arange(S)
+    w = (qq @ kk.transpose(-1, -2) * scale).masked_fill(i[None, :] > i[:, None], float("-inf"))
+    out = (torch.softmax(w, -1) * keep / (1 - p)) @ vv
+    out.backward(do)
+    got = orc.attention_prefill(q.numpy(), k.numpy(), v.numpy(), scale, keep=keep.numpy(), p=p)
+    assert np.abs(got - out.detach().numpy()).max() <= 1e-12
+    grads = orc.attention_prefill_bwd(q.numpy(), k.numpy(), v.numpy(), do.numpy(), scale, keep=keep.numpy(), p=p)
+    for a, b in zip(grads, (qq.grad, kk.grad, vv.grad)):
+        assert np.abs(a - b.numpy()).max() <= 1e-12
