@@ -241,7 +241,9 @@ __global__ __launch_bounds__(kMergeThreads) void attention_decode_merge_kernel(
       sum = __builtin_fmaf(w, base[s * stride + 1], sum);
     }
     sum = wave_allreduce(sum, OpAdd());
-    const float inv = 1.0f / sum;
+    // no visible key at all (a position below 0 read from device memory): every
+    // weight stays 0 and the output is zeros, never an unwritten accumulator
+    const float inv = sum > 0.f ? 1.0f / sum : 0.f;
     for (int s = threadIdx.x; s < splits; s += kWave) weight[s] *= inv;
   }
   __syncthreads();
