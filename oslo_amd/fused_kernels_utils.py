@@ -531,6 +531,8 @@ class FusedDecodeAttention(object):
         head_bytes = query.size(3) * query.element_size()
         if head_bytes not in (128, 256, 512, 1024) or key.size(2) * head_bytes >= 2 ** 31:
             return False
+        if key.size(2) > 2048 * (32 if head_bytes == 1024 else 64):  # the merge kernel takes 2048 splits of 32 / 64 keys
+            return False
         return not _needs_grad(query, key)
 
     @staticmethod
@@ -640,20 +642,26 @@ class FusedLinearRows(object):
     """
 
     @staticmethod
-    def is_available(x, weight, bias=None, conv1d=False):
-        if not (isinstance(x, torch.Tensor) and x.is_cuda and weight.is_cuda) or x.dim() < 1 or weight.dim() != 2:
+    def is_available(x, weight, bias=None, conv1d=False, rows_of=None):
+        """``rows_of``: a tensor whose leading dimensions give the rows when ``x``
+        itself does not exist yet (the second projection of a feed-forward
+        module is asked about before the first has run); ``x`` may then be None."""
+        ref = x if x is not None else rows_of
+        if not (isinstance(ref, torch.Tensor) and ref.is_cuda and weight.is_cuda) or ref.dim() < 1 or weight.dim() != 2:
             return False
         n, k = (weight.shape[1], weight.shape[0]) if conv1d else weight.shape
-        if k == 0 or x.shape[-1] != k or x.dtype != weight.dtype:
+        if k == 0 or ref.dtype != weight.dtype or (x is not None and x.shape[-1] != k):
             return False
-        if x.dtype not in (torch.half, torch.bfloat16, torch.float32) or not weight.is_contiguous():
+        if ref.dtype not in (torch.half, torch.bfloat16, torch.float32) or not weight.is_contiguous():
             return False
-        rows = x.numel() // k
-        es = x.element_size()
+        rows = ref.numel() // ref.shape[-1] if ref.shape[-1] else 0
+        es = ref.element_size()
         if not 0 < rows <= kernels.LINEAR_ROWS_MAX or (k * es) % 16 or n * k * es >= 2 ** 31:
             return False
         if conv1d and (n * es) % 16:
             return False
+        if x is None:
+            return not _needs_grad(rows_of, weight, bias)
         return not _needs_grad(x, weight, bias)
 
     @staticmethod

@@ -251,7 +251,8 @@ class FusedGPTNeoMLP(GPTNeoMLP):
 
     def forward(self, x, residual=None):
         """``residual``: added to the output (the residual connection of the block)."""
-        if FusedLinearRows.is_available(x, self.c_fc.weight, self.c_fc.bias):
+        if FusedLinearRows.is_available(x, self.c_fc.weight, self.c_fc.bias) and \
+                FusedLinearRows.is_available(None, self.c_proj.weight, self.c_proj.bias, rows_of=x):
             # a decoding step: each projection is one pass over its weight with
             # the bias (and the activation, and the residual) applied to the fp32 sums
             x = FusedLinearRows.apply(x, self.c_fc.weight, self.c_fc.bias, self.config.activation_function)

@@ -270,7 +270,8 @@ class FusedGPTJMLP(GPTJMLP):
 
     def forward(self, x, residual=None):
         """``residual``: added to the output (the residual connection of the block)."""
-        if FusedLinearRows.is_available(x, self.fc_in.weight, self.fc_in.bias):
+        if FusedLinearRows.is_available(x, self.fc_in.weight, self.fc_in.bias) and \
+                FusedLinearRows.is_available(None, self.fc_out.weight, self.fc_out.bias, rows_of=x):
             # a decoding step: each projection is one pass over its weight with
             # the bias (and the activation, and the residual) applied to the fp32 sums
             x = FusedLinearRows.apply(x, self.fc_in.weight, self.fc_in.bias, self.config.activation_function)

@@ -408,3 +408,21 @@ def test_training_through_the_one_kernel_attention_matches_unfused_gradients(fam
     assert all(torch.isfinite(g).all() for g in fu.values())
     # relative L2 error of the whole gradient: the fused model no further from fp32 than the unfused bf16 one
     assert (num_f / den) ** 0.5 <= 1.25 * (num_u / den) ** 0.5 + 1e-3, ((num_f / den) ** 0.5, (num_u / den) ** 0.5)
+
+
+def test_decoding_step_falls_back_when_only_the_second_projection_fits_no_kernel():
+    """A feed-forward width whose rows are not a multiple of 16 bytes: the first
+    projection ([n_inner, n_embd] rows of n_embd) would take the few-row
+    kernel, the second ([n_embd, n_inner] rows of n_inner) cannot. The fused
+    module must take the matmul path for both instead of raising."""
+    torch.manual_seed(0)
+    m = GPTJForCausalLM(GPTJConfig(vocab_size=256, n_positions=64, n_embd=128, n_layer=2, n_head=4, rotary_dim=16,
+                                   n_inner=132)).to(DEV, torch.float16).eval()
+    ids = torch.randint(0, 256, (2, 9), device=DEV)
+    with torch.no_grad():
+        want = m(ids, use_cache=True)
+        want_step = m(ids[:, :1], past_key_values=want["past_key_values"])["logits"].float()
+        m.fuse()
+        got = m(ids, use_cache=True)
+        got_step = m(ids[:, :1], past_key_values=got["past_key_values"])["logits"].float()
+    assert (got_step - want_step).abs().max().item() <= 2e-2
