@@ -568,6 +568,52 @@ int oslo_build_blending_indices(int32_t *dataset_index,
                                 const double *weights, int32_t num_datasets,
                                 int64_t size);
 
+/*
+ * Samples of consecutive sentences for a BERT-style dataset. docs: int64
+ * [docs_len], document d is the sentences docs[d] .. docs[d+1]-1; sizes: int32
+ * [sizes_len], tokens per sentence; host memory. Every epoch walks the
+ * documents in order; a document with fewer than min_num_sent sentences, or
+ * (if it has at least two) with a sentence of more than 512 tokens, is skipped;
+ * sentences are added to a sample until its length reaches the target and at
+ * least min_num_sent sentences are in it and more than one is left in the
+ * document, or until the document ends. The target is max_seq_length, except
+ * that with short_seq_prob > 0 one draw in round(1/short_seq_prob) of
+ * mt19937(seed) gives a short one, 2 + draw mod (max_seq_length - 1). An epoch
+ * is not started once max_num_samples rows exist. The rows of all epochs are
+ * shuffled with mt19937_64(seed + 1), from the last row down.
+ * With maps == NULL the call returns the number of rows; otherwise maps must
+ * hold exactly that many rows of 3 indices (first sentence, one past the last,
+ * target length), uint32 (index_bytes 4) or uint64 (8; needed beyond 2^32
+ * sentences), and the same number is returned. A negative return value is an
+ * oslo_status.
+ * Replaces build_mapping
+ * (oslo/fused_kernels/bindings/pybind_datasets.cpp:163-372), which allocates
+ * the array itself and does not check docs against sizes.
+ */
+int64_t oslo_build_mapping(void *maps, int64_t rows, int index_bytes,
+                           const int64_t *docs, int64_t docs_len,
+                           const int32_t *sizes, int64_t sizes_len,
+                           int32_t num_epochs, uint64_t max_num_samples,
+                           int32_t max_seq_length, double short_seq_prob,
+                           int32_t seed, int32_t min_num_sent);
+
+/*
+ * Blocks of consecutive sentences for a retrieval dataset: as above with the
+ * target max_seq_length - titles_sizes[d] (int32 [docs_len - 1], the tokens of
+ * document d's title), at least two sentences per block and behind a block that
+ * ends early (one with use_one_sent_blocks), no random lengths. Rows of 4
+ * indices: first sentence, one past the last, the document, and the block's
+ * serial number within its epoch.
+ * Replaces build_blocks_mapping
+ * (oslo/fused_kernels/bindings/pybind_datasets.cpp:374-574).
+ */
+int64_t oslo_build_blocks_mapping(void *maps, int64_t rows, int index_bytes,
+                                  const int64_t *docs, int64_t docs_len,
+                                  const int32_t *sizes, int64_t sizes_len,
+                                  const int32_t *titles_sizes, int32_t num_epochs,
+                                  uint64_t max_num_samples, int32_t max_seq_length,
+                                  int32_t seed, int use_one_sent_blocks);
+
 #ifdef __cplusplus
 }
 #endif

@@ -60,7 +60,14 @@ root):
   oslo/fused_kernels/bindings/pybind_datasets.cpp:35-160 (pinned by the closed
   form "sample k starts at token k*seq_length", the share bound of the
   blending, and, where oracle/_ref holds a build of it, the reference's own
-  module).
+  module);
+* build_mapping / build_blocks_mapping and the two Mersenne Twisters they draw
+  from: oslo/fused_kernels/bindings/pybind_datasets.cpp:163-574 (the
+  generators pinned by the C++ standard's 10000th-output values; the cutting
+  by a cumulative-sum formulation of "the shortest run of sentences that
+  reaches the target" for fixed targets and by the invariants every row must
+  satisfy for random ones; the whole, where oracle/_ref holds a build of it, by
+  the reference's own module).
 
 Parity unpinned: none of the functions above. The reference itself holds no
 golden vectors for this path.
@@ -449,3 +456,130 @@ def build_blending_indices(weights, num_datasets, size):
         dataset_sample_index[i] = drawn[best]
         drawn[best] += 1
     return dataset_index, dataset_sample_index
+
+
+class MersenneTwister:
+    """std::mt19937 (w=32) and std::mt19937_64 (w=64) as the C++ standard
+    defines them ([rand.predef]: the 10000th output of a default-constructed
+    engine, seed 5489, is 4123659995 and 9981545732273789042 respectively);
+    the reference draws sample lengths from the first and shuffles with the
+    second (oslo/fused_kernels/bindings/pybind_datasets.cpp:218, :346)."""
+
+    PARAMS = {
+        32: dict(n=624, m=397, r=31, a=0x9908B0DF, u=11, d=0xFFFFFFFF, s=7, b=0x9D2C5680, t=15, c=0xEFC60000, l=18,
+                 f=1812433253),
+        64: dict(n=312, m=156, r=31, a=0xB5026F5AA96619E9, u=29, d=0x5555555555555555, s=17, b=0x71D67FFFEDA60000,
+                 t=37, c=0xFFF7EEE000000000, l=43, f=6364136223846793005),
+    }
+
+    def __init__(self, seed, w=32):
+        self.w, self.p = w, self.PARAMS[w]
+        self.full = (1 << w) - 1
+        state = [seed & self.full]
+        for i in range(1, self.p["n"]):
+            prev = state[-1]
+            state.append((self.p["f"] * (prev ^ (prev >> (w - 2))) + i) & self.full)
+        self.state, self.at = state, self.p["n"]
+
+    def _twist(self):
+        p, x = self.p, self.state
+        upper = (self.full >> p["r"]) << p["r"]
+        lower = self.full ^ upper
+        for i in range(p["n"]):
+            y = (x[i] & upper) | (x[(i + 1) % p["n"]] & lower)
+            x[i] = x[(i + p["m"]) % p["n"]] ^ (y >> 1) ^ (p["a"] if y & 1 else 0)
+        self.at = 0
+
+    def __call__(self):
+        p = self.p
+        if self.at == p["n"]:
+            self._twist()
+        y = self.state[self.at]
+        self.at += 1
+        y ^= (y >> p["u"]) & p["d"]
+        y ^= (y << p["s"]) & p["b"]
+        y ^= (y << p["t"]) & p["c"]
+        y ^= y >> p["l"]
+        return y & self.full
+
+
+LONG_SENTENCE_LEN = 512  # oslo/fused_kernels/bindings/pybind_datasets.cpp:32
+
+
+def _shuffle_rows(rows, seed):
+    """oslo/fused_kernels/bindings/pybind_datasets.cpp:346-355 (and :543-553)."""
+    gen = MersenneTwister(seed + 1, 64)
+    for i in range(len(rows) - 1, 0, -1):
+        j = gen() % (i + 1)
+        rows[i], rows[j] = rows[j], rows[i]
+    return rows
+
+
+def build_mapping(docs, sizes, num_epochs, max_num_samples, max_seq_length, short_seq_prob, seed, min_num_sent):
+    """oslo/fused_kernels/bindings/pybind_datasets.cpp:163-372, the second of
+    its two passes (the first only counts). Returns uint32 [num_samples, 3]
+    (uint64 beyond 2^32 sentences, :384-412)."""
+    # C's round(): halves away from zero (:205-208)
+    ratio = int(np.floor(1.0 / short_seq_prob + 0.5)) if short_seq_prob > 0 else 0
+    gen = MersenneTwister(seed, 32)
+
+    def target_len():                                       # :163-176
+        if ratio == 0:
+            return max_seq_length
+        draw = gen()
+        if draw % ratio == 0:
+            return 2 + draw % (max_seq_length - 1)
+        return max_seq_length
+
+    rows = []
+    for _ in range(num_epochs):
+        if len(rows) >= max_num_samples:
+            break
+        for doc in range(len(docs) - 1):
+            first, last = int(docs[doc]), int(docs[doc + 1])
+            start, remain = first, last - first
+            long_sentence = remain > 1 and any(int(sizes[s]) > LONG_SENTENCE_LEN for s in range(first, last))
+            if remain >= min_num_sent and not long_sentence:
+                seq_len, num_sent, target = 0, 0, target_len()
+                for s in range(first, last):
+                    seq_len += int(sizes[s])
+                    num_sent += 1
+                    remain -= 1
+                    if (seq_len >= target and remain > 1 and num_sent >= min_num_sent) or remain == 0:
+                        rows.append((start, s + 1, target))
+                        start = s + 1
+                        target = target_len()
+                        seq_len, num_sent = 0, 0
+    dtype = np.uint64 if len(sizes) > np.iinfo(np.uint32).max else np.uint32
+    return np.array(_shuffle_rows(rows, seed), dtype=dtype).reshape(-1, 3)
+
+
+def build_blocks_mapping(docs, sizes, titles_sizes, num_epochs, max_num_samples, max_seq_length, seed,
+                         use_one_sent_blocks):
+    """oslo/fused_kernels/bindings/pybind_datasets.cpp:374-574. Returns uint32
+    [num_blocks, 4]: first sentence, one past the last, document, block id."""
+    min_num_sent = 1 if use_one_sent_blocks else 2
+    rows = []
+    for _ in range(num_epochs):
+        block_id = 0
+        if len(rows) >= max_num_samples:
+            break
+        for doc in range(len(docs) - 1):
+            first, last = int(docs[doc]), int(docs[doc + 1])
+            target = max_seq_length - int(titles_sizes[doc])
+            start, remain = first, last - first
+            long_sentence = remain >= min_num_sent and any(
+                int(sizes[s]) > LONG_SENTENCE_LEN for s in range(first, last))
+            if remain >= min_num_sent and not long_sentence:
+                seq_len, num_sent = 0, 0
+                for s in range(first, last):
+                    seq_len += int(sizes[s])
+                    num_sent += 1
+                    remain -= 1
+                    if (seq_len >= target and remain >= min_num_sent and num_sent >= min_num_sent) or remain == 0:
+                        rows.append((start, s + 1, doc, block_id))
+                        block_id += 1
+                        start = s + 1
+                        seq_len, num_sent = 0, 0
+    dtype = np.uint64 if len(sizes) > np.iinfo(np.uint32).max else np.uint32
+    return np.array(_shuffle_rows(rows, seed), dtype=dtype).reshape(-1, 4)

@@ -75,6 +75,11 @@ PROTOTYPES = {
     "oslo_build_sample_idx": (
         _c.c_int, [_P, _I64, _P, _I64, _P, _I64, _c.c_int32, _c.c_int32, _I64]),
     "oslo_build_blending_indices": (_c.c_int, [_P, _P, _P, _c.c_int32, _I64]),
+    "oslo_build_mapping": (
+        _I64, [_P, _I64, _c.c_int, _P, _I64, _P, _I64, _c.c_int32, _U64, _c.c_int32, _c.c_double, _c.c_int32,
+               _c.c_int32]),
+    "oslo_build_blocks_mapping": (
+        _I64, [_P, _I64, _c.c_int, _P, _I64, _P, _I64, _P, _c.c_int32, _U64, _c.c_int32, _c.c_int32, _c.c_int]),
 }
 
 ABI_VERSION = 1

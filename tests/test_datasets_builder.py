@@ -1,7 +1,8 @@
 """Index builders of the data pipeline (host code in liboslo_amd.so): against
 the oracle, against what the definitions fix (sample k starts at token
 k*seq_length of the document stream; blending keeps every dataset within one
-sample of its share), and against the reference's own C++ module where
+sample of its share; a span is the shortest run of sentences that reaches its
+target), and against the reference's own C++ module where
 oracle/_ref holds a build of it."""
 
 import importlib.util
@@ -115,6 +116,155 @@ def test_build_blending_indices_argument_errors():
         b.build_blending_indices(np.zeros(2, dtype=np.int32), np.zeros(3, dtype=np.int64), [1.0], 1, 3)
     with pytest.raises(RuntimeError, match="weights"):
         b.build_blending_indices(np.zeros(3, dtype=np.int32), np.zeros(3, dtype=np.int64), [1.0], 2, 3)
+
+
+def sentence_corpus(seed, num_docs, max_sents, max_tokens, long_every=0):
+    """docs (int64 [num_docs + 1]) and sizes (int32 per sentence); some documents
+    are empty or have one sentence; every `long_every`-th holds a sentence of
+    more than 512 tokens."""
+    rng = np.random.default_rng(seed)
+    counts = rng.integers(0, max_sents + 1, num_docs)
+    docs = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    sizes = rng.integers(1, max_tokens + 1, int(docs[-1])).astype(np.int32)
+    if long_every:
+        for d in range(0, num_docs, long_every):
+            if counts[d]:
+                sizes[docs[d] + rng.integers(0, counts[d])] = 513 + d
+    return docs, sizes
+
+
+def test_mersenne_twisters_of_the_oracle():
+    """[rand.predef] of the C++ standard: the 10000th output of the default
+    engines."""
+    for width, want in ((32, 4123659995), (64, 9981545732273789042)):
+        gen = orc.MersenneTwister(5489, width)
+        for _ in range(9999):
+            gen()
+        assert gen() == want
+
+
+def greedy_spans(docs, sizes, target_of, min_num_sent, min_behind, long_from):
+    """The cutting said another way, for a fixed target per document: a span
+    ends at the first sentence where the running token count (from the span's
+    start) reaches the target, never before min_num_sent sentences are in it,
+    and only while at least min_behind sentences would be left; what is left
+    when that fails goes into the document's last span."""
+    out = []
+    for d in range(len(docs) - 1):
+        first, last = int(docs[d]), int(docs[d + 1])
+        n = last - first
+        if n < min_num_sent or (n >= long_from and (sizes[first:last] > 512).any()):
+            continue
+        csum = np.concatenate([[0], np.cumsum(sizes[first:last].astype(np.int64))])
+        start = 0
+        while start < n:
+            reach = int(np.searchsorted(csum, csum[start] + target_of(d), side="left"))  # csum[reach] >= ...
+            end = max(reach, start + max(min_num_sent, 1))
+            if end > n - min_behind:
+                end = n
+            out.append((first + start, first + end, d))
+            start = end
+    return out
+
+
+MAPPING_CASES = [  # seed, num_docs, max_sents, max_tokens, epochs, max_seq_length, short_seq_prob, min_num_sent, long_every
+    (1, 20, 6, 40, 1, 64, 0.0, 2, 0),
+    (2, 200, 12, 100, 3, 128, 0.1, 2, 7),
+    (3, 50, 30, 20, 2, 16, 0.4, 1, 0),      # 1/0.4 = 2.5 rounds to 3, not to 2
+    (4, 100, 8, 200, 2, 512, 1.0, 3, 5),    # every sample short
+    (5, 1, 1, 10, 1, 8, 0.0, 2, 0),         # nothing to cut
+    (6, 300, 5, 300, 4, 256, 0.05, 2, 3),
+]
+
+
+@pytest.mark.parametrize("case", MAPPING_CASES)
+def test_build_mapping(case):
+    seed, num_docs, max_sents, max_tokens, epochs, max_len, prob, min_sent, long_every = case
+    docs, sizes = sentence_corpus(seed, num_docs, max_sents, max_tokens, long_every)
+    args = (docs, sizes, epochs, 10**9, max_len, prob, 1234 + seed, min_sent)
+    got = get_datasets_builder().build_mapping(*args)
+    want = orc.build_mapping(*args)
+    assert got.dtype == np.uint32 and got.shape == want.shape and got.shape[1] == 3
+    assert np.array_equal(got, want)
+    # every row: a run of sentences inside one document, target in [2, max_len];
+    # per epoch the rows tile each document they come from
+    rows = got[np.lexsort((got[:, 1], got[:, 0]))].astype(np.int64)
+    assert ((rows[:, 2] >= 2) & (rows[:, 2] <= max_len)).all()
+    doc_of = np.searchsorted(docs, rows[:, 0], side="right") - 1
+    assert (rows[:, 1] > rows[:, 0]).all() and (rows[:, 1] <= docs[doc_of + 1]).all()
+    covered = np.zeros(len(sizes), dtype=np.int64)
+    for a, b, _ in rows:
+        covered[a:b] += 1
+    assert set(np.unique(covered)) <= {0, epochs}
+    if prob == 0.0:
+        spans = greedy_spans(docs, sizes, lambda d: max_len, min_sent, 2, 2)
+        want_rows = sorted((a, b, max_len) for a, b, _ in spans) * 1
+        assert sorted(map(tuple, rows.tolist())) == sorted(want_rows * epochs)
+    ref = reference_module()
+    if ref is not None:
+        assert np.array_equal(got, ref.build_mapping(*args))
+
+
+def test_build_mapping_stops_starting_epochs_at_max_num_samples():
+    docs, sizes = sentence_corpus(11, 40, 6, 50)
+    b = get_datasets_builder()
+    one = b.build_mapping(docs, sizes, 1, 10**9, 64, 0.0, 7, 2)
+    many = b.build_mapping(docs, sizes, 5, len(one) + 1, 64, 0.0, 7, 2)   # a second epoch starts, a third does not
+    assert len(many) == 2 * len(one)
+    assert np.array_equal(many, orc.build_mapping(docs, sizes, 5, len(one) + 1, 64, 0.0, 7, 2))
+    ref = reference_module()
+    if ref is not None:
+        assert np.array_equal(many, ref.build_mapping(docs, sizes, 5, len(one) + 1, 64, 0.0, 7, 2))
+
+
+BLOCK_CASES = [  # seed, num_docs, max_sents, max_tokens, epochs, max_seq_length, one_sent_blocks, long_every
+    (1, 20, 6, 40, 1, 64, False, 0),
+    (2, 200, 12, 100, 3, 128, True, 7),
+    (3, 50, 30, 20, 2, 48, False, 0),
+    (4, 100, 8, 200, 2, 288, True, 5),
+    (5, 1, 1, 10, 1, 40, False, 0),
+]
+
+
+@pytest.mark.parametrize("case", BLOCK_CASES)
+def test_build_blocks_mapping(case):
+    seed, num_docs, max_sents, max_tokens, epochs, max_len, one_sent, long_every = case
+    docs, sizes = sentence_corpus(seed, num_docs, max_sents, max_tokens, long_every)
+    titles = np.random.default_rng(seed).integers(1, 32, num_docs).astype(np.int32)
+    args = (docs, sizes, titles, epochs, 10**9, max_len, 99 + seed, one_sent)
+    got = get_datasets_builder().build_blocks_mapping(*args)
+    want = orc.build_blocks_mapping(*args)
+    assert got.dtype == np.uint32 and got.shape == want.shape and got.shape[1] == 4
+    assert np.array_equal(got, want)
+    least = 1 if one_sent else 2
+    spans = greedy_spans(docs, sizes, lambda d: max_len - int(titles[d]), least, least, least)
+    rows = sorted(map(tuple, got[:, :3].astype(np.int64).tolist()))
+    assert rows == sorted(spans * epochs)
+    # block ids: 0 .. blocks-per-epoch - 1 in document order, every epoch again
+    per_epoch = len(spans)
+    if per_epoch:
+        order = np.lexsort((got[:, 0], got[:, 3]))
+        assert np.array_equal(got[order, 3], np.repeat(np.arange(per_epoch), epochs))
+        first_epoch = got[order][::epochs]
+        assert np.array_equal(first_epoch[:, 0], np.array(sorted(a for a, _, _ in spans)))
+    ref = reference_module()
+    if ref is not None:
+        assert np.array_equal(got, ref.build_blocks_mapping(*args))
+
+
+def test_span_builders_reject_bad_input():
+    b = get_datasets_builder()
+    docs, sizes = sentence_corpus(3, 10, 4, 20)
+    with pytest.raises(RuntimeError, match="ascending"):
+        b.build_mapping(docs[::-1].copy(), sizes, 1, 100, 64, 0.0, 1, 2)
+    with pytest.raises(RuntimeError, match="ascending"):
+        b.build_mapping(docs + 1, sizes, 1, 100, 64, 0.0, 1, 2)        # runs past the last sentence
+    with pytest.raises(RuntimeError, match="seed"):
+        b.build_mapping(docs, sizes, 1, 100, 64, 0.0, 0, 2)
+    with pytest.raises(RuntimeError, match="short_seq_prob"):
+        b.build_mapping(docs, sizes, 1, 100, 64, 1.5, 1, 2)
+    with pytest.raises(RuntimeError, match="titles_sizes"):
+        b.build_blocks_mapping(docs, sizes, np.zeros(3, dtype=np.int32), 1, 100, 64, 1, False)
 
 
 def test_reference_build_is_used_when_present():
