@@ -34,6 +34,39 @@ __device__ __forceinline__ float other_half(float v) {
   return __shfl_xor(v, 32, kWave);
 }
 
+// Maximum and sum of the values lanes l and l ^ 32 hold, in both lanes, on the
+// vector ALU (no LDS queue involved): v_permlane32_swap exchanges the upper
+// half of its first register with the lower half of its second; given two
+// copies of a value it leaves the lower half's value in every lane of the
+// first and the upper half's in every lane of the second. (Written out, with
+// idle cycles either side for the instruction's register hazards: through the
+// builtin the two results came back as one register.)
+__device__ __forceinline__ void halves_split(float v, float &lower, float &upper) {
+  lower = v, upper = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lower), "+v"(upper));
+}
+__device__ __forceinline__ float halves_max(float v) {
+  float lo, hi;
+  halves_split(v, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float halves_sum(float v) {
+  float lo, hi;
+  halves_split(v, lo, hi);
+  return lo + hi;
+}
+
+// Calls f with four pointers the compiler may take to address distinct memory
+// (the two buffers a tile reads and the two it writes while it is computed):
+// without that it keeps every LDS read behind every LDS write that precedes it
+// in the source.
+template <typename T, typename F>
+__device__ __forceinline__ void with_distinct_buffers(const T *__restrict__ read_a, T *__restrict__ write_a,
+                                                      const T *__restrict__ read_b, T *__restrict__ write_b,
+                                                      F &&f) {
+  f(read_a, write_a, read_b, write_b);
+}
+
 // Additive mask values travel in log2 units. Masks of -inf or of the most
 // negative finite number (as some callers build them) would make every score
 // of a row -inf and its softmax 0/0; they are floored at a value that still

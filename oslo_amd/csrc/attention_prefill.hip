@@ -12,26 +12,27 @@
 // HBM: 4 * S^2/2 * head_dim flops per head against 4 * S * head_dim elements.
 //
 // One block of four waves takes 128 queries of one head, 32 per wave, and walks
-// the keys in tiles of 64. Everything is computed transposed, so that a query
+// the keys in tiles of 32. Everything is computed transposed, so that a query
 // is a lane and not a register index:
 //   S^T[key, q] = K_tile (A operand, rows = keys, from LDS) x Q^T (B operand,
 //                 held in registers for the whole kernel),
 //   O^T[d, q]  += V_tile^T (A operand, rows = features, from LDS) x P^T (B).
 // In the accumulator layout of v_mfma_f32_32x32x16 a lane holds one column
-// (lane % 32 = the query) and 16 rows, so the running maximum, the sum and
-// the rescaling of O are per-lane scalars: the softmax needs one exchange
-// between the two halves of the wave per step and no LDS. The 16 rows of a
-// lane are keys 8j + 4h + t (j, t = 0..3; h = lane / 32), and a B operand
-// wants, per half, 8 consecutive contraction slots: the probabilities are used
-// where they are, and the contraction order is permuted instead -- V^T is
-// written to LDS with key 8j + 4h + t of each group of 16 (j = 0, 1 there) at
-// slot 8h + 4j + t.
-// V arrives as [key][feature]; each thread transposes an 8 x 8 block in
-// registers and writes 128-bit rows of V^T. Both LDS tiles are swizzled by
-// 16-byte chunk so that the 128-bit reads of a wave (the LDS serves 16 lanes
-// at a time: 16 rows at one chunk) and the writes spread over the banks. A
-// tile of keys is taken in two steps of 32, each a step of the running
-// softmax, and the next tile's global loads are in flight meanwhile.
+// (lane % 32 = the query) and 16 rows, so the reference maximum, the sum and
+// the rescaling of O are per-lane scalars: the softmax needs no LDS. The 16
+// rows of a lane are keys 8j + 4h + t (j, t = 0..3; h = lane / 32), and a B
+// operand wants, per half, 8 consecutive contraction slots: the probabilities
+// are used where they are, and the contraction order of V^T is permuted to
+// match.
+// K and V tiles go from global memory straight into LDS (three buffers each),
+// stored as they are in memory; the transposition of V happens in the LDS
+// read (ds_read_b64_tr_b16). What limits the kernel is not the matrix core
+// alone but what a wave can issue: with one wave per SIMD (head_dim 256: O^T
+// and Q^T take 192 of a lane's registers) a matrix product keeps the wave from
+// issuing for most of its 32 cycles, and every other instruction costs four
+// more. So a tile is one straight run of code, ordered by hand: the products
+// of S^T with the next tiles' loads between them, then the products of
+// O^T of the previous tile with the softmax of this one between them.
 
 #include "attention.hpp"
 
@@ -39,9 +40,17 @@ namespace oslo {
 namespace {
 
 constexpr int kQueriesPerBlock = 128;
-constexpr int kKeysPerTile = 64;
+constexpr int kKeysPerTile = 32;
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kSlack = 8.0f; // see the kernel: how far a score may exceed the reference maximum
+// See the kernel: how far a score may exceed the reference maximum (log2
+// units). A general tile raises the maximum of a query when a score exceeds it
+// by more than kRaise; the scheduled tiles do not look at the scores but at a
+// lane's sum of 16 exponentials: none of them exceeds the sum, and a sum above
+// 2^kSlack means a score more than kSlack - 4 = kRaise above the maximum, so
+// that doing such a tile again the general way does raise it.
+constexpr float kSlack = 8.0f;
+constexpr float kRaise = 4.0f;
+constexpr float kSumLimit = 256.0f; // 2^kSlack
 
 struct PrefillArgs {
   void *out;
@@ -62,8 +71,26 @@ struct PrefillArgs {
   DropArgs drop; // attention dropout (the DROP variants of the kernel)
 };
 
+// Tiles of K and of V go from global memory straight into LDS (buffer loads
+// with the LDS as destination: a wave's instruction puts its 64 x 16 bytes at
+// consecutive addresses), three buffers each: the one being read, the one that
+// has landed and the one in flight. Both are stored as they are in memory,
+// [key][feature], 16-byte chunks permuted within a key's row so that the lanes
+// the LDS serves together hit different banks: K is read 16 bytes per lane by
+// 16 lanes with consecutive keys (chunk ^ key), V through the transposing read,
+// 8 bytes per lane by 4 keys x 4 chunk halves (chunk ^ 2 (key % 4)). The
+// permutation is applied on the global side: a lane fetches the chunk that
+// belongs at its LDS slot.
+constexpr int kBuffers = 3;
+constexpr int kPadSlots = kBlockThreads; // mask values of a tile: the first 32 count, every thread writes one
+template <typename T, int D>
+constexpr unsigned prefill_lds_bytes() {
+  return 2u * kBuffers * kKeysPerTile * D * sizeof(T) + 2u * kPadSlots * sizeof(float) +
+         kWavesPerBlock * 32u * sizeof(uint32_t);
+}
+
 template <typename T, int D, bool HAS_PAD, bool HAS_WINDOW, bool DROP>
-__global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_prefill_kernel(
+__global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) void attention_prefill_kernel(
     const PrefillArgs a) {
   using Op = MatrixOp<T>;
   using Frag = typename Op::Frag;
@@ -71,26 +98,22 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   constexpr int kSteps = D / 16;   // contraction steps of Q K^T
   constexpr int kBlocksD = D / 32; // 32-row blocks of O^T
   constexpr int kLoadsK = kKeysPerTile * kChunks / kBlockThreads; // per thread and tile
-  constexpr int kSwizzleK = kChunks >= 16 ? 15 : 7;                // rows over which K's chunks rotate
-  // At head_dim 256 the 64 registers of Q^T are what pushes a wave past its
-  // 256 vector registers: the compiler then parks half of Q^T in the
-  // accumulator file, moves it back before every product and has one buffer
-  // left for the K operand, so that every product waits for its own LDS read.
-  // There Q^T lives in (dynamic) LDS instead, in operand order, each wave its
-  // own 16 KiB, and both operands of S^T = K Q^T are read from LDS.
-  constexpr bool kQInLds = D == 256;
-  constexpr bool kTwoLoops = D == 256; // see `step` below
-  extern __shared__ __align__(16) unsigned char dynamic_lds[];
-  __shared__ __align__(16) T k_lds[kKeysPerTile * D];  // [key][chunk ^ (key & kSwizzleK)][8]
-  __shared__ __align__(16) T vt_lds[D * kKeysPerTile]; // [d][(slot + d + d/8) & 7][8]
-  __shared__ __align__(16) float pad_lds[HAS_PAD ? kKeysPerTile : 4]; // the tile's mask values, log2 units
-  __shared__ __align__(16) uint32_t keep_lds[DROP ? kWavesPerBlock : 1][32]; // a wave's keep bits of a step
+  constexpr int kRowsPerPass = kBlockThreads / kChunks;
+  constexpr int kTile = kKeysPerTile * D;      // elements of a K or V buffer
+  constexpr int kRowBytes = D * (int)sizeof(T);
+  constexpr int kKeyShift = D == 64 ? 1 : 0;   // rows of 128 bytes: two keys share a set of banks
+  constexpr int kSwizzleK = kChunks >= 16 ? 15 : 7;
+  extern __shared__ __align__(1024) unsigned char lds_raw[];
+  T *const k_lds = reinterpret_cast<T *>(lds_raw); // [3][key][chunk ^ swizzle(key)][8]
+  T *const vt_lds = k_lds + kBuffers * kTile;      // [3][key][chunk ^ 2 (key % 4)][8]
+  float *const pad_lds = reinterpret_cast<float *>(vt_lds + kBuffers * kTile); // [2][key], log2 units
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int half = lane >> 5;
   const int col = lane & 31;
+  uint32_t *const keep_lds = reinterpret_cast<uint32_t *>(pad_lds + 2 * kPadSlots) + 32 * wave;
 
   // All query blocks of a head run on one XCD (blocks go round-robin over
   // the 8 XCDs), so its keys and values are read from HBM into one L2; the
@@ -110,91 +133,151 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   const T *vp = static_cast<const T *>(a.v) + b * a.v_b + hd * a.v_h;
   // rows at or past S fall outside the descriptors and read as zeros
   const BufRsrc qrs = make_rsrc(qp, (uint32_t)(((int64_t)(S - 1) * a.q_s + D) * sizeof(T)));
-  const BufRsrc krs = make_rsrc(kp, (uint32_t)(((int64_t)(S - 1) * a.k_s + D) * sizeof(T)));
-  const BufRsrc vrs = make_rsrc(vp, (uint32_t)(((int64_t)(S - 1) * a.v_s + D) * sizeof(T)));
   const uint32_t q_row = (uint32_t)a.q_s * sizeof(T);
   const uint32_t k_row = (uint32_t)a.k_s * sizeof(T);
   const uint32_t v_row = (uint32_t)a.v_s * sizeof(T);
 
-  // Q^T as B operands: lane (query, half) holds features 16 s + 8 half .. + 7
+  // Q^T as B operands, in registers for the whole kernel: lane (query, half)
+  // holds features 16 s + 8 half .. + 7
   const int wave_q0 = q0 + 32 * wave;
   const int qrow = wave_q0 + col;
-  Frag qf[kQInLds ? 1 : kSteps];
-  u32x4 *q_lds = reinterpret_cast<u32x4 *>(dynamic_lds) + wave * kSteps * kWave + lane;
-  if constexpr (kQInLds) {
-    u32x4 tmp[kSteps];
+  Frag qf[kSteps];
 #pragma unroll
-    for (int s = 0; s < kSteps; ++s)
-      tmp[s] = __builtin_amdgcn_raw_buffer_load_b128(
-          qrs, (uint32_t)qrow * q_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0);
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s) q_lds[s * kWave] = tmp[s];
-  } else {
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s)
-      qf[s] = __builtin_bit_cast(
-          Frag, __builtin_amdgcn_raw_buffer_load_b128(
-                    qrs, (uint32_t)qrow * q_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0));
-  }
+  for (int s = 0; s < kSteps; ++s)
+    qf[s] = __builtin_bit_cast(
+        Frag, __builtin_amdgcn_raw_buffer_load_b128(
+                  qrs, (uint32_t)qrow * q_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0));
 
   const float *padr = HAS_PAD ? a.pad + (int64_t)b * S : nullptr;
-  const int behind = HAS_WINDOW ? qrow - a.window : -1; // the last key behind the query's window
+  const int window = HAS_WINDOW ? a.window : 0;
+  const int behind = HAS_WINDOW ? qrow - window : -1; // the last key behind the query's window
 
-  // A tile travels global -> registers -> LDS; the loads of the next tile are
-  // in flight while this one is computed.
-  // K: thread takes chunk tid % kChunks of rows tid / kChunks + j * (256 / kChunks).
-  // V: a task is 8 keys (one contraction chunk 2u + h of the tile) x 8 features.
-  const int k_ch = tid % kChunks, k_r0 = tid / kChunks;
-  const bool v_task = tid < D;
-  const int v_g = tid % kChunks, v_kg = tid / kChunks;
-  u32x4 kreg[kLoadsK], vreg[8];
-  // the padding mask of a tile travels with it: 16 lanes take four keys each
-  // (keys at or past S read as 0; they only meet queries they are masked for)
-  const BufRsrc prs = make_rsrc(padr, HAS_PAD ? (uint32_t)S * (uint32_t)sizeof(float) : 0u);
-  float4 padreg = make_float4(0.f, 0.f, 0.f, 0.f);
-  auto issue_loads = [&](int key0) {
-    if constexpr (HAS_PAD) {
-      if (tid < kKeysPerTile / 4)
-        padreg = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                prs, (uint32_t)(key0 + 4 * tid) * (uint32_t)sizeof(float), 0, 0));
+  const int last_key = (q0 + kQueriesPerBlock < S ? q0 + kQueriesPerBlock : S) - 1;
+  const int tiles = last_key / kKeysPerTile + 1;
+  // with a sliding window the block starts at the tile of its first query's
+  // first visible key
+  const int first_tile = HAS_WINDOW && q0 - window + 1 > 0 ? (q0 - window + 1) / kKeysPerTile : 0;
+  // Tiles [plain_begin, plain_end) are visible in full to every query of the
+  // block: no comparison, no wave sits one out. The block's first tile is not
+  // among them (its queries have no reference maximum yet).
+  const int plain_end = q0 / kKeysPerTile;
+  int plain_begin = !HAS_WINDOW ? 0
+                    : q0 + kQueriesPerBlock - window > 0
+                        ? (q0 + kQueriesPerBlock - window + kKeysPerTile - 1) / kKeysPerTile
+                        : 0;
+  if (plain_begin < first_tile + 1) plain_begin = first_tile + 1;
+
+  // A tile travels global -> LDS without passing through registers. While tile
+  // t is computed (S^T of tile t, then O^T += V^T P^T of tile t - 1 under the
+  // softmax of tile t) the loads of K of tile t + 2 and of V of tile t + 1 are
+  // issued, into the buffers that tile t - 1 (K) and tile t - 2 (V) have left;
+  // they are waited for a whole tile later, before the barrier that opens tile
+  // t + 2. The staging is cut into items (one load each), so that a tile's
+  // straight-line code can place them one by one.
+  // Load j of wave w fills the 64 slots of 16 bytes from (4 j + w) * 64 on: slot
+  // sigma is (row = sigma / kChunks, chunk position = sigma % kChunks) and holds
+  // the chunk whose index is the position with the row's permutation undone.
+  uint32_t k_off[kLoadsK], v_off[kLoadsK];
+#pragma unroll
+  for (int j = 0; j < kLoadsK; ++j) {
+    const int sigma = (4 * j + wave) * kWave + lane;
+    const int row = sigma / kChunks, at = sigma % kChunks;
+    k_off[j] = (uint32_t)row * k_row + (uint32_t)(at ^ ((row >> kKeyShift) & kSwizzleK)) * 16u;
+    v_off[j] = (uint32_t)row * v_row + (uint32_t)(at ^ (2 * (row & 3))) * 16u;
+  }
+  // the padding mask of a tile travels with its keys, through a register: one
+  // value per thread of the first 32 (the others read outside the descriptor,
+  // zeros, and write words nobody reads: no branch)
+  float padreg = 0.f;
+  // A tile is loaded through a descriptor of its own (base = the tile's first
+  // key, size = what is left of the head's slice from there, nothing for tiles
+  // past the block's last one: rows at or past S and whole tiles that are not
+  // needed read as zeros without a memory access). The descriptors of the next
+  // tiles to load are kept as scalars and stepped from tile to tile; the vector
+  // offsets of a thread's loads are the same for every tile.
+  struct TileSource {
+    uint64_t base;  // the tile's first key
+    uint32_t left;  // bytes from there to the end of the head's slice
+    uint32_t step;  // bytes from a tile to the next
+    int tile;       // its index
+    __device__ __forceinline__ void start(const void *p, uint32_t bytes, uint32_t row_bytes, int t) {
+      step = kKeysPerTile * row_bytes;
+      tile = t;
+      const uint32_t skip = (uint32_t)(t < 0 ? 0 : t) * step;
+      base = reinterpret_cast<uint64_t>(p) + skip;
+      left = skip < bytes ? bytes - skip : 0u;
     }
-#pragma unroll
-    for (int j = 0; j < kLoadsK; ++j)
-      kreg[j] = __builtin_amdgcn_raw_buffer_load_b128(
-          krs, (uint32_t)(key0 + k_r0 + j * (kBlockThreads / kChunks)) * k_row + (uint32_t)k_ch * 16u, 0, 0);
-    if (v_task) {
-      const int kbase = key0 + 16 * (v_kg >> 1) + 4 * (v_kg & 1);
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        vreg[i] = __builtin_amdgcn_raw_buffer_load_b128(
-            vrs, (uint32_t)(kbase + 8 * (i >> 2) + (i & 3)) * v_row + (uint32_t)v_g * 16u, 0, 0);
+    __device__ __forceinline__ void advance() {
+      base += step;
+      left = left > step ? left - step : 0u;
+      ++tile;
+    }
+    // raw 32-bit buffer descriptor (word 3 = 0x00020000, as make_rsrc builds it)
+    __device__ __forceinline__ u32x4 descriptor(int tiles) const {
+      u32x4 d; // (read as scalars: the hand-written load takes the descriptor in scalar registers)
+      d[0] = __builtin_amdgcn_readfirstlane((uint32_t)base);
+      d[1] = __builtin_amdgcn_readfirstlane((uint32_t)(base >> 32) & 0xffffu);
+      d[2] = __builtin_amdgcn_readfirstlane(tile >= 0 && tile < tiles ? left : 0u);
+      d[3] = 0x00020000u;
+      return d;
     }
   };
-  auto store_tile = [&]() {
+  TileSource k_src, v_src, pad_src; // the next tiles to load: K of tile t + 2, V of tile t + 1, mask of tile t + 2
+  k_src.start(kp, (uint32_t)(((int64_t)(S - 1) * a.k_s + D) * sizeof(T)), k_row, first_tile);
+  v_src.start(vp, (uint32_t)(((int64_t)(S - 1) * a.v_s + D) * sizeof(T)), v_row, first_tile);
+  if constexpr (HAS_PAD) pad_src.start(padr, (uint32_t)S * (uint32_t)sizeof(float), (uint32_t)sizeof(float), first_tile);
+  // (lanes past the tile's 32 mask values read outside every descriptor)
+  const uint32_t pad_off = tid < kKeysPerTile ? (uint32_t)tid * (uint32_t)sizeof(float) : 0x80000000u;
+  constexpr int kItems = 2 * kLoadsK + (HAS_PAD ? 2 : 0);
+  constexpr int kLoadsPerTile = 2 * kLoadsK + (HAS_PAD ? 1 : 0); // what a tile leaves in flight
+  // The load itself is written out: the compiler, told of a load into LDS,
+  // waits for every such load before the next LDS read of any buffer; these
+  // are waited for by count, a tile later (wait_loads).
+  auto load_to_lds = [&](const u32x4 &desc, const T *dst, uint32_t offset) __attribute__((always_inline)) {
+    const uint32_t at = __builtin_amdgcn_readfirstlane((uint32_t)reinterpret_cast<uintptr_t>(dst)); // LDS addresses are the low 32 bits
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");
+  };
+  // the three buffers of K and of V, as element offsets, in the order (tile t,
+  // t + 1, t + 2) and (t - 1, t, t + 1); rotated from tile to tile
+  int k_at[3] = {0, kTile, 2 * kTile}, v_at[3] = {2 * kTile, 0, kTile};
+  int t = first_tile;
+  auto next_tile = [&]() __attribute__((always_inline)) {
+    ++t;
+    const int k0 = k_at[0], v0 = v_at[0];
+    k_at[0] = k_at[1], k_at[1] = k_at[2], k_at[2] = k0;
+    v_at[0] = v_at[1], v_at[1] = v_at[2], v_at[2] = v0;
+  };
+  auto k_buffer = [&](int d) __attribute__((always_inline)) { return k_lds + k_at[d]; };      // of tile t + d, d = 0 .. 2
+  auto v_buffer = [&](int d) __attribute__((always_inline)) { return vt_lds + v_at[d + 1]; }; // of tile t + d, d = -1 .. 1
+  // item `it` of the staging of a tile: the loads of K of tile t + 2 into kw,
+  // then those of V of tile t + 1 into vw, then the mask values
+  auto stage_item = [&](int it, T *kw, T *vw) __attribute__((always_inline)) {
+    if (it < kLoadsK) {
+      load_to_lds(k_src.descriptor(tiles), kw + (4 * it + wave) * (kWave * 8), k_off[it]);
+      if (it == kLoadsK - 1) k_src.advance();
+      return;
+    }
+    it -= kLoadsK;
+    if (it < kLoadsK) {
+      load_to_lds(v_src.descriptor(tiles), vw + (4 * it + wave) * (kWave * 8), v_off[it]);
+      if (it == kLoadsK - 1) v_src.advance();
+      return;
+    }
+    it -= kLoadsK;
     if constexpr (HAS_PAD) {
-      if (tid < kKeysPerTile / 4)
-        *reinterpret_cast<float4 *>(&pad_lds[4 * tid]) = make_float4(
-            fmaxf(padreg.x * kLog2e, kMaskFloorLog2), fmaxf(padreg.y * kLog2e, kMaskFloorLog2),
-            fmaxf(padreg.z * kLog2e, kMaskFloorLog2), fmaxf(padreg.w * kLog2e, kMaskFloorLog2));
-    }
-#pragma unroll
-    for (int j = 0; j < kLoadsK; ++j) {
-      const int row = k_r0 + j * (kBlockThreads / kChunks);
-      *reinterpret_cast<u32x4 *>(&k_lds[(row * kChunks + (k_ch ^ (row & kSwizzleK))) * 8]) = kreg[j];
-    }
-    if (v_task) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) { // 8 x 8 transposition of 16-bit values
-        u32x4 tr;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const uint32_t lo = vreg[2 * w][e >> 1], hi = vreg[2 * w + 1][e >> 1];
-          tr[w] = (e & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
-        }
-        const int d = 8 * v_g + e;
-        *reinterpret_cast<u32x4 *>(&vt_lds[(d * 8 + ((v_kg + e + v_g) & 7)) * 8]) = tr;
+      if (it == 0) { // the values loaded a tile ago belong to tile t + 1
+        pad_lds[((t + 1) & 1) * kPadSlots + tid] = fmaxf(padreg * kLog2e, kMaskFloorLog2);
+      } else {
+        padreg = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                               make_rsrc(reinterpret_cast<const void *>(pad_src.base), pad_src.descriptor(tiles)[2]), pad_off, 0, 0));
+        pad_src.advance();
       }
     }
+  };
+  // what the loads issued before the current tile's have to be waited for with
+  // (the tile's own stay in flight): vmcnt <= N, nothing else
+  auto wait_loads = []<int N>() __attribute__((always_inline)) {
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
   };
 
   f32x16 o[kBlocksD];
@@ -202,210 +285,353 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
   for (int i = 0; i < kBlocksD; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
-  float m = -INFINITY; // running maximum of the query's scores, log2 units
+  float m = -INFINITY; // reference maximum of the query's scores, log2 units
   float l = 0.f;       // this lane's share of the running sum
+  Frag pf[2];          // P^T of the last tile computed, not yet multiplied with V
+  bool pending = false; // wave-uniform: pf holds such a tile (the one before the current)
 
-  const int last_key = (q0 + kQueriesPerBlock < S ? q0 + kQueriesPerBlock : S) - 1;
-  const int tiles = last_key / kKeysPerTile + 1;
-  // with a sliding window the block starts at the tile of its first query's
-  // first visible key
-  const int window = HAS_WINDOW ? a.window : 0;
-  const int first_tile = HAS_WINDOW && q0 - window + 1 > 0 ? (q0 - window + 1) / kKeysPerTile : 0;
-  // One step of 32 keys of the tile in LDS. RESCALE: O may be rescaled to a
-  // higher reference maximum. The loop over the tiles runs the variant without
-  // it and falls back, for a single step, when a query that has already
-  // accumulated something needs a higher reference: with the multiplications
-  // of O in the same loop, the compiler copies all of O's accumulators to
-  // vector registers in every tile (it places the copies that the rare
-  // multiplication needs ahead of the branch), 128 moves and 128 registers at
-  // head_dim 256. Returns false if nothing was done for that reason.
-  auto step = [&]<bool RESCALE>(int key0, int kb) -> bool {
-    const int keyb = key0 + 32 * kb;
+  // K operand s of the tile at kb: lane (key, half) takes chunk 2 s + half of
+  // its key's row, wherever the permutation has put it
+  const uint32_t k_lane = (uint32_t)col * kRowBytes + (uint32_t)((half ^ ((col >> kKeyShift) & kSwizzleK)) << 4);
+  auto read_k = [&](const T *kb, int s) __attribute__((always_inline)) {
+    return *reinterpret_cast<const Frag *>(reinterpret_cast<const char *>(kb) + (k_lane ^ (uint32_t)(s << 5)));
+  };
+  // Operand n of O^T += V^T P^T (the first 16 keys into every block of O^T,
+  // then the other 16), through the transposing LDS read: of 16 lanes, lane j
+  // points at 8 bytes (4 features) of one key; lane i gets back, of the four
+  // words that lanes i/4 + 4k point at, element i % 4 each. With lane j at key
+  // j / 4 and feature block j % 4, lane i holds feature i of the four keys:
+  // what a lane of the product's A operand needs (its own feature, contraction
+  // in its registers). Two reads make an operand: slots 0..3 are keys 16u + 4h +
+  // 0..3, slots 4..7 keys 16u + 8 + 4h + 0..3, h the lane's half of the wave:
+  // where the accumulator layout leaves the probabilities (rows 8j' + 4h + t of
+  // S^T), so that P^T is used where it is.
+  typedef short Short4 __attribute__((ext_vector_type(4)));
+  typedef short Short8 __attribute__((ext_vector_type(8)));
+  uint32_t v_lane[2]; // for even and odd blocks of 32 features
+  {
+    const int j = lane & 15, group = lane >> 4; // group: bit 0 = second 16 features of the block, bit 1 = half
+    const int key = 4 * (group >> 1) + (j >> 2);
+    const int x = (2 * (group & 1) + ((j & 3) >> 1)) ^ (2 * (j >> 2) & 3); // chunk within the block of four chunks
+    const int flip = (j >> 2) >> 1; // the permutation's bit 2 swaps neighbouring blocks
+    const uint32_t base = (uint32_t)key * kRowBytes + (uint32_t)x * 16u + (uint32_t)(j & 1) * 8u;
+    v_lane[0] = base + 64u * (uint32_t)flip;
+    v_lane[1] = base + 64u * (uint32_t)(1 ^ flip);
+  }
+  auto read_v = [&](const T *vb, int n) __attribute__((always_inline)) {
+    const int u = n / kBlocksD, i = n % kBlocksD;
+    const char *at = reinterpret_cast<const char *>(vb) + v_lane[i & 1] + 64 * (i & ~1) + 16 * u * kRowBytes;
+    const Short4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) Short4 *)(at));
+    const Short4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) Short4 *)(at + 8 * kRowBytes));
+    return __builtin_bit_cast(Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+  // scale and padding mask (without a mask the scores stay raw: the scale,
+  // positive, commutes with the maximum and goes into the exponent's
+  // multiply-add)
+  auto add_pad = [&](f32x16 &sc, int t) __attribute__((always_inline)) {
+    if constexpr (HAS_PAD) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float4 p4 = *reinterpret_cast<const float4 *>(&pad_lds[(t & 1) * kPadSlots + 8 * j + 4 * half]);
+        sc[4 * j + 0] = __builtin_fmaf(sc[4 * j + 0], a.scale_log2e, p4.x);
+        sc[4 * j + 1] = __builtin_fmaf(sc[4 * j + 1], a.scale_log2e, p4.y);
+        sc[4 * j + 2] = __builtin_fmaf(sc[4 * j + 2], a.scale_log2e, p4.z);
+        sc[4 * j + 3] = __builtin_fmaf(sc[4 * j + 3], a.scale_log2e, p4.w);
+      }
+    }
+  };
+  auto tile_max = [&](const f32x16 &sc) __attribute__((always_inline)) -> float {
+    float mt = sc[0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mt = fmaxf(mt, sc[r]);
+    if constexpr (!HAS_PAD) mt *= a.scale_log2e;
+    return halves_max(mt);
+  };
+  auto exponential = [&](float x, float shift) __attribute__((always_inline)) {
+    if constexpr (HAS_PAD)
+      return __builtin_amdgcn_exp2f(x - shift);
+    else
+      return __builtin_amdgcn_exp2f(__builtin_fmaf(x, a.scale_log2e, -shift));
+  };
+  // attention dropout: the sum keeps every probability, the product with V
+  // only the kept ones (their 1/(1-p) goes into the final normalisation);
+  // then P^T in the storage type, like the unfused path's cast
+  auto finish_probabilities = [&](f32x16 &sc, int keyb, Frag (&p)[2]) __attribute__((always_inline)) {
+    if constexpr (DROP) {
+      stage_keep_bits(keep_lds, a.drop, bh, S, wave_q0, keyb, lane);
+      const uint32_t bits = keep_word_query_lane(keep_lds, col) >> (4 * half);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[r] = (bits >> (8 * (r >> 2) + (r & 3))) & 1u ? sc[r] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) p[u][i] = static_cast<T>(sc[8 * u + i]);
+  };
+
+  // The reference maximum m only follows the scores when they exceed it by
+  // more than kSlack (log2 units): exponentials up to 2^kSlack are as exact
+  // as those up to 1 in fp32, fp16 and bf16, and the softmax does not depend
+  // on the shift. Rescaling O costs as much as the softmax of a tile, and with
+  // an exact running maximum some query of a wave raises it in most tiles;
+  // with the slack it happens in the first tiles only.
+
+  // Any tile, in plain order: the first of a block, those the causal or window
+  // boundary crosses (some waves sit them out), and those of the plain range
+  // in which a query's reference maximum has to rise. `with_previous`: stage
+  // the next tile and multiply the pending P^T of the previous one first. Only
+  // the RESCALE variant can raise the reference maximum of a query that has
+  // already accumulated something; the other returns false when that is
+  // needed, having done no more than the staging and the pending product. With
+  // the multiplications of O in the code that every tile runs through, the
+  // compiler copies all of O's accumulators to vector registers in every tile
+  // (it places the copies that the rare multiplication needs ahead of the
+  // branch).
+  auto general_tile = [&]<bool RESCALE>(int t, bool with_previous) __attribute__((always_inline)) -> bool {
+    if (with_previous) {
+#pragma unroll
+      for (int it = 0; it < kItems; ++it) stage_item(it, k_buffer(2), v_buffer(1));
+      if (pending) {
+        const T *vb = v_buffer(-1);
+#pragma unroll
+        for (int n = 0; n < 2 * kBlocksD; ++n) o[n % kBlocksD] = Op::run(read_v(vb, n), pf[n / kBlocksD], o[n % kBlocksD]);
+      }
+      pending = false;
+    }
+    const int keyb = t * kKeysPerTile;
     if (keyb > wave_q0 + 31) return true; // every key is ahead of the wave's queries
     if (HAS_WINDOW && keyb + 31 <= wave_q0 - window) return true; // or behind their windows
-
-    // S^T = K Q^T
     f32x16 sc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) sc[r] = 0.f;
-    const int key = 32 * kb + col;
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
-      const Frag kf = *reinterpret_cast<const Frag *>(
-          &k_lds[(key * kChunks + ((2 * s + half) ^ (key & kSwizzleK))) * 8]);
-      if constexpr (kQInLds)
-        sc = Op::run(kf, __builtin_bit_cast(Frag, q_lds[s * kWave]), sc);
-      else
-        sc = Op::run(kf, qf[s], sc);
-    }
-    // The LDS reads run kAhead steps ahead of the products that use them (left
-    // alone, the scheduler keeps one operand buffer and every product waits
-    // out its own read). 0x100: LDS reads, 0x008: matrix products.
     {
-      constexpr int kReads = kQInLds ? 2 : 1; // per step
-      constexpr int kAhead = kSteps < 3 ? kSteps : 3;
-      __builtin_amdgcn_sched_group_barrier(0x100, kReads * kAhead, 0);
+      const T *kb = k_buffer(0);
 #pragma unroll
-      for (int s = 0; s < kSteps - kAhead; ++s) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+      for (int s = 0; s < kSteps; ++s) sc = Op::run(read_k(kb, s), qf[s], sc);
     }
-
-    // Causal and padding mask, maximum. Without a padding mask the scores
-    // stay raw: the scale (positive) commutes with the maximum and goes
-    // into the exponent's multiply-add.
-    const bool diagonal = keyb + 31 > wave_q0 || (HAS_WINDOW && keyb <= wave_q0 + 31 - window);
-    float mt = -INFINITY;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float pv[4] = {0.f, 0.f, 0.f, 0.f};
-      if constexpr (HAS_PAD) {
-        const float4 p4 = *reinterpret_cast<const float4 *>(&pad_lds[32 * kb + 8 * j + 4 * half]);
-        pv[0] = p4.x, pv[1] = p4.y, pv[2] = p4.z, pv[3] = p4.w;
-      }
-#pragma unroll
-      for (int tt = 0; tt < 4; ++tt) {
-        float x = sc[4 * j + tt];
-        if constexpr (HAS_PAD) x = __builtin_fmaf(x, a.scale_log2e, pv[tt]);
-        sc[4 * j + tt] = x;
-      }
-    }
-    if (diagonal) {
-      // a branch of its own (the empty asm keeps it one): the comparisons
-      // run in the last tiles of a block only
-      asm volatile("");
+    add_pad(sc, t);
+    if (keyb + 31 > wave_q0 || (HAS_WINDOW && keyb <= wave_q0 + 31 - window)) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int kr = keyb + 8 * (r >> 2) + 4 * half + (r & 3);
         sc[r] = kr <= qrow && (!HAS_WINDOW || kr > behind) ? sc[r] : -INFINITY;
       }
     }
+    const float mt = tile_max(sc);
+    // Without a window key 0 is visible to every query and m is finite after
+    // the first tile; with one, a query may see nothing in the first tiles of
+    // its wave: m stays -inf, nothing is rescaled, and the exponentials (of
+    // -inf) are taken against 0.
+    const bool raise = mt > m + kRaise; // true at the first visible key (m = -inf)
+    if (__any(raise && m != -INFINITY)) { // wave-uniform
+      if constexpr (!RESCALE) return false;
+      const float m_new = raise ? mt : m;
+      const float alpha = raise ? __builtin_amdgcn_exp2f(m - m_new) : 1.0f; // 0 where m was -inf (nothing accumulated)
+      l *= alpha;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sc[r]);
-    if constexpr (!HAS_PAD) mt *= a.scale_log2e;
-    mt = fmaxf(mt, other_half(mt));
-    // The reference maximum m only follows the scores when they exceed it by
-    // more than kSlack (log2 units): exponentials up to 2^kSlack are as exact
-    // as those up to 1 in fp32, fp16 and bf16, and the softmax does not
-    // depend on the shift. Rescaling O costs as much as the softmax of a
-    // step, and with an exact running maximum some query of a wave raises it
-    // in most steps; with the slack it happens in the first steps only.
-    // Without a window key 0 is visible to every query and m is finite
-    // after the first step; with one, a query may see nothing in the first
-    // steps of its wave: m stays -inf, nothing is rescaled, and the
-    // exponentials (of -inf) are taken against 0.
-    const bool raise = mt > m + kSlack; // true at the first visible key (m = -inf)
-    if constexpr (RESCALE) {
-      if (__any(raise)) { // wave-uniform
-        const float m_new = raise ? mt : m;
-        const float alpha = !HAS_WINDOW || raise ? __builtin_amdgcn_exp2f(m - m_new) : 1.0f;
-        m = m_new;
-        l *= alpha;
+      for (int i = 0; i < kBlocksD; ++i)
 #pragma unroll
-        for (int i = 0; i < kBlocksD; ++i)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
-      }
+        for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
+      m = m_new;
     } else {
-      // a query that has accumulated nothing yet (m = -inf) takes its
-      // reference maximum without rescaling anything; any other raise is
-      // left to the caller's slow path, before this step has changed anything
-      if (__any(raise && m != -INFINITY)) return false;
       m = raise ? mt : m;
     }
-    float sum = 0.f;
     const float shift = HAS_WINDOW && m == -INFINITY ? 0.f : m;
+    float sum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      if constexpr (HAS_PAD)
-        sc[r] = __builtin_amdgcn_exp2f(sc[r] - shift);
-      else
-        sc[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[r], a.scale_log2e, -shift));
+      sc[r] = exponential(sc[r], shift);
       sum += sc[r];
     }
     l += sum;
-    if constexpr (DROP) {
-      // attention dropout: the sum keeps every probability, the product with V
-      // only the kept ones (their 1/(1-p) goes into the final normalisation)
-      stage_keep_bits(keep_lds[wave], a.drop, bh, S, wave_q0, keyb, lane);
-      const uint32_t bits = keep_word_query_lane(keep_lds[wave], col) >> (4 * half);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sc[r] = (bits >> (8 * (r >> 2) + (r & 3))) & 1u ? sc[r] : 0.f;
-    }
-
-    // P^T as B operands, in the storage type like the unfused path's cast
-    Frag pf[2];
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int i = 0; i < 8; ++i) pf[u][i] = static_cast<T>(sc[8 * u + i]);
-
-    // O^T += V^T P^T, the first 16 keys into every block of O^T, then the
-    // other 16: the products of the first half only need the first half of
-    // the exponentials
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-#pragma unroll
-      for (int i = 0; i < kBlocksD; ++i) {
-        const int d = 32 * i + col;
-        const Frag vf = *reinterpret_cast<const Frag *>(
-            &vt_lds[(d * 8 + ((4 * kb + 2 * u + half + d + (d >> 3)) & 7)) * 8]);
-        o[i] = Op::run(vf, pf[u], o[i]);
-      }
-    }
-    {
-      constexpr int kProducts = 2 * kBlocksD;
-      constexpr int kAhead = kProducts < 3 ? kProducts : 3;
-      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 1);
-#pragma unroll
-      for (int n = 0; n < kProducts - kAhead; ++n) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 1);
-    }
+    finish_probabilities(sc, keyb, pf);
+    pending = true;
     return true;
   };
-
-  issue_loads(first_tile * kKeysPerTile);
-  int t = first_tile;
-  if constexpr (!kTwoLoops) {
-    for (; t < tiles; ++t) {
-      const int key0 = t * kKeysPerTile;
-      __syncthreads(); // the reads of the previous tile are done
-      store_tile();
-      __syncthreads();
-      if (t + 1 < tiles) issue_loads(key0 + kKeysPerTile);
-      step.template operator()<true>(key0, 0);
-      step.template operator()<true>(key0, 1);
-    }
-  }
-  while (kTwoLoops && t < tiles) {
-    int redo = -1; // the step of tile t that needs the rescaling variant
-    for (; t < tiles; ++t) {
-      const int key0 = t * kKeysPerTile;
-      __syncthreads(); // the reads of the previous tile are done
-      store_tile();
-      __syncthreads();
-      if (t + 1 < tiles) issue_loads(key0 + kKeysPerTile);
-      if (!step.template operator()<false>(key0, 0)) {
-        redo = 0;
-        break;
+  // Tiles [t, end) the general way. The tiles run in an inner loop that
+  // contains no multiplication of O; a tile in which some reference maximum
+  // has to rise leaves that loop, is done with the rescaling variant, and the
+  // loop is entered again.
+  auto general_range = [&](int end) __attribute__((always_inline)) {
+    while (t < end) {
+      bool rescale = false;
+      for (; t < end; next_tile()) {
+        wait_loads.template operator()<kLoadsPerTile>();
+        __syncthreads(); // tile t's K and tile t - 1's V are in LDS; the buffers written next have been read
+        if (!general_tile.template operator()<false>(t, true)) {
+          rescale = true;
+          break;
+        }
       }
-      if (!step.template operator()<false>(key0, 1)) {
-        redo = 1;
-        break;
-      }
+      if (!rescale) break;
+      general_tile.template operator()<true>(t, false);
+      next_tile();
     }
-    if (redo < 0) break;
-#pragma unroll 1
-    for (int kb = redo; kb < 2; ++kb) step.template operator()<true>(t * kKeysPerTile, kb);
-    ++t;
+  };
+
+  // prologue: K of the first two tiles and V of the first on their way, all
+  // issued before any is waited for (the sources then stand at tile t + 2 and
+  // t + 1, where a tile's staging expects them)
+  {
+#pragma unroll
+    for (int it = 0; it < kLoadsK; ++it) stage_item(it, k_buffer(0), nullptr);
+    if constexpr (HAS_PAD) {
+      stage_item(kItems - 1, nullptr, nullptr);
+      pad_lds[(first_tile & 1) * kPadSlots + tid] = fmaxf(padreg * kLog2e, kMaskFloorLog2);
+    }
+#pragma unroll
+    for (int it = 0; it < 2 * kLoadsK; ++it) stage_item(it, k_buffer(1), v_buffer(0));
+    if constexpr (HAS_PAD) stage_item(kItems - 1, nullptr, nullptr);
   }
 
-  l += other_half(l);
+  // A tile as one straight run of code, its order fixed by hand (the fences
+  // keep the compiler's scheduler from moving anything across them). First the
+  // matrix products of S^T (tile t), whose K operands are read from LDS kRing
+  // products ahead, with a share of the staging in each product's shadow; then
+  // those of O^T (tile t - 1), with a slice of the softmax of tile t in each
+  // one's shadow. A wave issues in order, so whatever it issues between two
+  // products beyond the seven vector-ALU slots one product lasts leaves the
+  // matrix core idle. The run assumes that no reference maximum rises; the
+  // caller looks at the tile's maximum `mt` afterwards and, if one has to,
+  // throws the tile's probabilities away and does the tile again the general
+  // way. MASKED: the causal boundary crosses the tile. FIRST: the block's first
+  // tile: nothing is pending, and the tile's maximum becomes the reference.
+  auto scheduled_tile = [&]<bool MASKED, bool FIRST>(int t, float &mt, float &sum, Frag (&pn)[2])
+                            __attribute__((always_inline)) {
+    with_distinct_buffers(k_buffer(0), k_buffer(2), v_buffer(-1), v_buffer(1),
+                          [&](const T *kr, T *kw, const T *vr, T *vw) __attribute__((always_inline)) {
+      constexpr int kRing = 4;
+      constexpr int kProducts = 2 * kBlocksD;
+      constexpr int kPerStep = (kItems + kSteps - 1) / kSteps;
+      Frag ring[kRing];
+#pragma unroll
+      for (int s = 0; s < kRing; ++s) ring[s] = read_k(kr, s);
+      __builtin_amdgcn_sched_barrier(0);
+      f32x16 sc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) {
+        sc = Op::run(ring[s % kRing], qf[s], sc);
+        const int next = s + kRing;
+        if (next < kSteps)
+          ring[s % kRing] = read_k(kr, next);
+        else if (!FIRST && next - kSteps < kProducts)
+          ring[s % kRing] = read_v(vr, next - kSteps);
+#pragma unroll
+        for (int it = s * kPerStep; it < (s + 1) * kPerStep && it < kItems; ++it) stage_item(it, kw, vw);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // softmax slices, spread over the products: the exponentials (an
+      // exponential is added to the sum one slice later: the adder would wait
+      // for it), the conversion last. Only the first tile takes the maximum;
+      // elsewhere the caller looks at the sum (an exponential above 2^kSlack
+      // shows there) to see whether a reference maximum has to rise.
+      sum = 0.f;
+      auto slice_of = [](int r) __attribute__((always_inline)) { return FIRST ? 1 + r * (kProducts - 1) / 16 : r * kProducts / 16; };
+#pragma unroll
+      for (int n = 0; n < kProducts; ++n) {
+        if constexpr (!FIRST) {
+          const int at = (kSteps + n) % kRing;
+          o[n % kBlocksD] = Op::run(ring[at], pf[n / kBlocksD], o[n % kBlocksD]);
+          if (n + kRing < kProducts) ring[at] = read_v(vr, n + kRing);
+        }
+        if (n == 0) {
+          add_pad(sc, t);
+          if constexpr (MASKED) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int kr_ = t * kKeysPerTile + 8 * (r >> 2) + 4 * half + (r & 3);
+              sc[r] = kr_ <= qrow ? sc[r] : -INFINITY;
+            }
+          }
+          if constexpr (FIRST) {
+            mt = tile_max(sc);
+            m = mt;
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          if (slice_of(r) == n) {
+            sc[r] = exponential(sc[r], m);
+            // (an empty statement that "changes" a value keeps its computation
+            // in this slice: the results are only used behind the branch that
+            // follows the tile)
+            asm volatile("" : "+v"(sc[r]));
+          }
+          if (slice_of(r) == n - 1) sum += sc[r];
+        }
+        if (n == kProducts - 1) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (slice_of(r) == n) sum += sc[r];
+          finish_probabilities(sc, t * kKeysPerTile, pn);
+          u32x4 p0 = __builtin_bit_cast(u32x4, pn[0]), p1 = __builtin_bit_cast(u32x4, pn[1]);
+          asm volatile("" : "+v"(p0), "+v"(p1), "+v"(sum));
+          pn[0] = __builtin_bit_cast(Frag, p0), pn[1] = __builtin_bit_cast(Frag, p1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    });
+  };
+
+  if constexpr (HAS_WINDOW) {
+    general_range(plain_begin < tiles ? plain_begin : tiles);
+  } else {
+    // the block's first tile (the causal boundary crosses it in the first block)
+    wait_loads.template operator()<0>();
+    __syncthreads();
+    float mt, sum;
+    scheduled_tile.template operator()<true, true>(t, mt, sum, pf);
+    l = sum;
+    pending = true;
+    next_tile();
+  }
+
+  // Tiles every query of the block sees in full, then (without a window) those
+  // the causal boundary crosses, each kind in a loop of its own (one loop with
+  // a branch per kind has the compiler shuffle the accumulators where the
+  // branches meet, in every tile). A wave whose queries all lie before a tile
+  // still computes it, every score masked: it adds zeros, and it would wait at
+  // the tile's barrier anyway.
+  auto scheduled_range = [&]<bool MASKED>(int end) __attribute__((always_inline)) {
+    while (t < end && pending) {
+      bool rescale = false;
+      for (; t < end; next_tile()) {
+        wait_loads.template operator()<kLoadsPerTile>();
+        __syncthreads(); // tile t's K (and tile t - 1's V) are in LDS; the buffers written next have been read
+        float mt, sum;
+        Frag pn[2];
+        scheduled_tile.template operator()<MASKED, false>(t, mt, sum, pn);
+        if (__any(!(sum <= kSumLimit))) {
+          rescale = true;
+          pending = false;
+          break;
+        }
+        l += sum;
+        pf[0] = pn[0], pf[1] = pn[1];
+      }
+      if (!rescale) break;
+      general_tile.template operator()<true>(t, false);
+      pending = true; // (a wave the tile lies ahead of has multiplied nothing: zeros follow)
+      next_tile();
+    }
+  };
+  scheduled_range.template operator()<false>(plain_end);
+  if constexpr (!HAS_WINDOW) scheduled_range.template operator()<true>(tiles);
+  if constexpr (HAS_WINDOW) general_range(tiles);
+
+  wait_loads.template operator()<0>(); // (nothing may still be on its way into LDS when the block ends)
+  __syncthreads(); // V of the last tile is in LDS
+  if (pending) {
+    const T *vb = v_buffer(-1);
+#pragma unroll
+    for (int n = 0; n < 2 * kBlocksD; ++n) o[n % kBlocksD] = Op::run(read_v(vb, n), pf[n / kBlocksD], o[n % kBlocksD]);
+  }
+
+  l = halves_sum(l);
   const float inv = DROP ? a.drop.keep_scale / l : 1.0f / l;
   if (qrow >= S) return;
   if (a.lse != nullptr && half == 0)
@@ -426,15 +652,14 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : 2) void attention_pre
 template <typename T, int D>
 int launch_prefill_dim(const PrefillArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)(8 * a.head_groups * a.query_blocks));
-  // head_dim 256 keeps Q^T in dynamic LDS: 128 queries x 256 features. Static
-  // and dynamic LDS together exceed the 64 KiB a kernel gets unasked, so the
-  // limit is raised for the kernel (on the current device; a host-side
-  // setting, not a stream operation) before every launch.
-  constexpr unsigned kDynamic = D == 256 ? kQueriesPerBlock * D * sizeof(T) : 0;
+  // All LDS of the kernel is dynamic. At head_dim 256 it exceeds the 64 KiB a
+  // kernel gets unasked, so the limit is raised for the kernel (on the current
+  // device; a host-side setting, not a stream operation) before every launch.
+  constexpr unsigned kDynamic = prefill_lds_bytes<T, D>();
   auto go = [&]<bool HAS_PAD, bool HAS_WINDOW>() -> int {
     auto *kernel = a.drop.drop ? attention_prefill_kernel<T, D, HAS_PAD, HAS_WINDOW, true>
                                : attention_prefill_kernel<T, D, HAS_PAD, HAS_WINDOW, false>;
-    if (kDynamic > 0) {
+    if (kDynamic > 64u * 1024u) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynamic);
       if (e != hipSuccess)
