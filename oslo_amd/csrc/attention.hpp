@@ -72,6 +72,7 @@ __device__ __forceinline__ void with_distinct_buffers(const T *__restrict__ read
 // of a row -inf and its softmax 0/0; they are floored at a value that still
 // underflows every exponential but keeps the arithmetic finite.
 constexpr float kMaskFloorLog2 = -1e30f;
+constexpr float kMaskFloor = -1e30f; // the same for mask values kept in natural units
 
 // Attention dropout inside the attention kernels. The keep flag of the
 // probability of (query q, key k) of head bh is the one the softmax kernel with

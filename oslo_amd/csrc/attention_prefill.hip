@@ -61,7 +61,7 @@ struct PrefillArgs {
   int64_t k_b, k_h, k_s;
   int64_t v_b, v_h, v_s;
   int64_t o_b, o_h, o_s;
-  float scale_log2e;
+  float scale, scale_log2e;
   int S;
   int heads;
   int batch_heads;
@@ -82,10 +82,10 @@ struct PrefillArgs {
 // permutation is applied on the global side: a lane fetches the chunk that
 // belongs at its LDS slot.
 constexpr int kBuffers = 3;
-constexpr int kPadSlots = kBlockThreads; // mask values of a tile: the first 32 count, every thread writes one
+constexpr int kPadSlots = kBlockThreads; // mask values of a tile: the first 32 count, every wave loads 64
 template <typename T, int D>
 constexpr unsigned prefill_lds_bytes() {
-  return 2u * kBuffers * kKeysPerTile * D * sizeof(T) + 2u * kPadSlots * sizeof(float) +
+  return 2u * kBuffers * kKeysPerTile * D * sizeof(T) + kBuffers * kPadSlots * sizeof(float) +
          kWavesPerBlock * 32u * sizeof(uint32_t);
 }
 
@@ -106,14 +106,14 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   extern __shared__ __align__(1024) unsigned char lds_raw[];
   T *const k_lds = reinterpret_cast<T *>(lds_raw); // [3][key][chunk ^ swizzle(key)][8]
   T *const vt_lds = k_lds + kBuffers * kTile;      // [3][key][chunk ^ 2 (key % 4)][8]
-  float *const pad_lds = reinterpret_cast<float *>(vt_lds + kBuffers * kTile); // [2][key], log2 units
+  float *const pad_lds = reinterpret_cast<float *>(vt_lds + kBuffers * kTile); // [3][key], as loaded
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int half = lane >> 5;
   const int col = lane & 31;
-  uint32_t *const keep_lds = reinterpret_cast<uint32_t *>(pad_lds + 2 * kPadSlots) + 32 * wave;
+  uint32_t *const keep_lds = reinterpret_cast<uint32_t *>(pad_lds + kBuffers * kPadSlots) + 32 * wave;
 
   // All query blocks of a head run on one XCD (blocks go round-robin over
   // the 8 XCDs), so its keys and values are read from HBM into one L2; the
@@ -185,10 +185,10 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     k_off[j] = (uint32_t)row * k_row + (uint32_t)(at ^ ((row >> kKeyShift) & kSwizzleK)) * 16u;
     v_off[j] = (uint32_t)row * v_row + (uint32_t)(at ^ (2 * (row & 3))) * 16u;
   }
-  // the padding mask of a tile travels with its keys, through a register: one
-  // value per thread of the first 32 (the others read outside the descriptor,
-  // zeros, and write words nobody reads: no branch)
-  float padreg = 0.f;
+  // The padding mask of a tile travels with its keys, the same way: every
+  // wave loads 64 values into a quarter of its own of the tile's slots; the
+  // first 32 of the first wave's are the tile's (lanes past them, and the
+  // other waves, read outside the descriptor: zeros, and no branch).
   // A tile is loaded through a descriptor of its own (base = the tile's first
   // key, size = what is left of the head's slice from there, nothing for tiles
   // past the block's last one: rows at or past S and whole tiles that are not
@@ -228,7 +228,8 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   if constexpr (HAS_PAD) pad_src.start(padr, (uint32_t)S * (uint32_t)sizeof(float), (uint32_t)sizeof(float), first_tile);
   // (lanes past the tile's 32 mask values read outside every descriptor)
   const uint32_t pad_off = tid < kKeysPerTile ? (uint32_t)tid * (uint32_t)sizeof(float) : 0x80000000u;
-  constexpr int kItems = 2 * kLoadsK + (HAS_PAD ? 2 : 0);
+  int pad_at[3] = {0, kPadSlots, 2 * kPadSlots}; // the mask slots of tiles t, t + 1, t + 2
+  constexpr int kItems = 2 * kLoadsK + (HAS_PAD ? 1 : 0);
   constexpr int kLoadsPerTile = 2 * kLoadsK + (HAS_PAD ? 1 : 0); // what a tile leaves in flight
   // The load itself is written out: the compiler, told of a load into LDS,
   // waits for every such load before the next LDS read of any buffer; these
@@ -246,6 +247,10 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     const int k0 = k_at[0], v0 = v_at[0];
     k_at[0] = k_at[1], k_at[1] = k_at[2], k_at[2] = k0;
     v_at[0] = v_at[1], v_at[1] = v_at[2], v_at[2] = v0;
+    if constexpr (HAS_PAD) {
+      const int p0 = pad_at[0];
+      pad_at[0] = pad_at[1], pad_at[1] = pad_at[2], pad_at[2] = p0;
+    }
   };
   auto k_buffer = [&](int d) __attribute__((always_inline)) { return k_lds + k_at[d]; };      // of tile t + d, d = 0 .. 2
   auto v_buffer = [&](int d) __attribute__((always_inline)) { return vt_lds + v_at[d + 1]; }; // of tile t + d, d = -1 .. 1
@@ -265,13 +270,10 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     }
     it -= kLoadsK;
     if constexpr (HAS_PAD) {
-      if (it == 0) { // the values loaded a tile ago belong to tile t + 1
-        pad_lds[((t + 1) & 1) * kPadSlots + tid] = fmaxf(padreg * kLog2e, kMaskFloorLog2);
-      } else {
-        padreg = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                               make_rsrc(reinterpret_cast<const void *>(pad_src.base), pad_src.descriptor(tiles)[2]), pad_off, 0, 0));
-        pad_src.advance();
-      }
+      const uint32_t at = __builtin_amdgcn_readfirstlane(
+          (uint32_t)reinterpret_cast<uintptr_t>(pad_lds + pad_at[2] + wave * kWave));
+      asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(at), "v"(pad_off), "s"(pad_src.descriptor(tiles)) : "m0");
+      pad_src.advance();
     }
   };
   // what the loads issued before the current tile's have to be waited for with
@@ -330,30 +332,29 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   // scale and padding mask (without a mask the scores stay raw: the scale,
   // positive, commutes with the maximum and goes into the exponent's
   // multiply-add)
-  auto add_pad = [&](f32x16 &sc, int t) __attribute__((always_inline)) {
+  auto add_pad = [&](f32x16 &sc) __attribute__((always_inline)) {
     if constexpr (HAS_PAD) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float4 p4 = *reinterpret_cast<const float4 *>(&pad_lds[(t & 1) * kPadSlots + 8 * j + 4 * half]);
-        sc[4 * j + 0] = __builtin_fmaf(sc[4 * j + 0], a.scale_log2e, p4.x);
-        sc[4 * j + 1] = __builtin_fmaf(sc[4 * j + 1], a.scale_log2e, p4.y);
-        sc[4 * j + 2] = __builtin_fmaf(sc[4 * j + 2], a.scale_log2e, p4.z);
-        sc[4 * j + 3] = __builtin_fmaf(sc[4 * j + 3], a.scale_log2e, p4.w);
+        const float4 p4 = *reinterpret_cast<const float4 *>(&pad_lds[pad_at[0] + 8 * j + 4 * half]);
+        sc[4 * j + 0] = __builtin_fmaf(sc[4 * j + 0], a.scale, fmaxf(p4.x, kMaskFloor));
+        sc[4 * j + 1] = __builtin_fmaf(sc[4 * j + 1], a.scale, fmaxf(p4.y, kMaskFloor));
+        sc[4 * j + 2] = __builtin_fmaf(sc[4 * j + 2], a.scale, fmaxf(p4.z, kMaskFloor));
+        sc[4 * j + 3] = __builtin_fmaf(sc[4 * j + 3], a.scale, fmaxf(p4.w, kMaskFloor));
       }
     }
   };
+  // what turns a score as add_pad leaves it into log2 units
+  const float to_log2 = HAS_PAD ? kLog2e : a.scale_log2e;
   auto tile_max = [&](const f32x16 &sc) __attribute__((always_inline)) -> float {
     float mt = sc[0];
 #pragma unroll
     for (int r = 1; r < 16; ++r) mt = fmaxf(mt, sc[r]);
-    if constexpr (!HAS_PAD) mt *= a.scale_log2e;
+    mt *= to_log2;
     return halves_max(mt);
   };
   auto exponential = [&](float x, float shift) __attribute__((always_inline)) {
-    if constexpr (HAS_PAD)
-      return __builtin_amdgcn_exp2f(x - shift);
-    else
-      return __builtin_amdgcn_exp2f(__builtin_fmaf(x, a.scale_log2e, -shift));
+    return __builtin_amdgcn_exp2f(__builtin_fmaf(x, to_log2, -shift));
   };
   // attention dropout: the sum keeps every probability, the product with V
   // only the kept ones (their 1/(1-p) goes into the final normalisation);
@@ -411,7 +412,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
 #pragma unroll
       for (int s = 0; s < kSteps; ++s) sc = Op::run(read_k(kb, s), qf[s], sc);
     }
-    add_pad(sc, t);
+    add_pad(sc);
     if (keyb + 31 > wave_q0 || (HAS_WINDOW && keyb <= wave_q0 + 31 - window)) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -477,13 +478,16 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   {
 #pragma unroll
     for (int it = 0; it < kLoadsK; ++it) stage_item(it, k_buffer(0), nullptr);
-    if constexpr (HAS_PAD) {
+    if constexpr (HAS_PAD) { // the mask values of the first tile, then (as the staging of a tile expects) of the second
+      const int p2 = pad_at[2];
+      pad_at[2] = pad_at[0];
       stage_item(kItems - 1, nullptr, nullptr);
-      pad_lds[(first_tile & 1) * kPadSlots + tid] = fmaxf(padreg * kLog2e, kMaskFloorLog2);
+      pad_at[2] = pad_at[1];
+      stage_item(kItems - 1, nullptr, nullptr);
+      pad_at[2] = p2;
     }
 #pragma unroll
     for (int it = 0; it < 2 * kLoadsK; ++it) stage_item(it, k_buffer(1), v_buffer(0));
-    if constexpr (HAS_PAD) stage_item(kItems - 1, nullptr, nullptr);
   }
 
   // A tile as one straight run of code, its order fixed by hand (the fences
@@ -539,7 +543,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
           if (n + kRing < kProducts) ring[at] = read_v(vr, n + kRing);
         }
         if (n == 0) {
-          add_pad(sc, t);
+          add_pad(sc);
           if constexpr (MASKED) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -739,6 +743,7 @@ int prefill_entry(void *out, float *lse, const oslo::DropArgs &drop, const void 
   a.k_b = strides[3], a.k_h = strides[4], a.k_s = strides[5];
   a.v_b = strides[6], a.v_h = strides[7], a.v_s = strides[8];
   a.o_b = strides[9], a.o_h = strides[10], a.o_s = strides[11];
+  a.scale = scale;
   a.scale_log2e = scale * kLog2e;
   a.S = (int)S;
   a.heads = (int)heads;
