@@ -40,37 +40,39 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 # profiles/bench_kernels_hbm_traffic.md and, for the two kernels of the step,
 # profiles/causal_softmax_fp16_8x16x2048x2048_hbm_traffic.md.
 MEASURED_TRAFFIC = {
-    "linear_rows fc_in + bias + gelu bf16 1 x [16384,4096]": 134699008,
-    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135285043,
-    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134601011,
-    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136612249,
+    "linear_rows fc_in + bias + gelu bf16 1 x [16384,4096]": 134699021,
+    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135284954,
+    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134601023,
+    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136610240,
     "linear_rows attention projection bf16 1 x [4096,4096]": 33740800,
     "linear_rows attention projection bf16 8 x [4096,4096]": 34370560,
-    "attention_decode bf16 1 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 17573888,
-    "attention_decode bf16 8 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 136477696,
-    "causal_fwd fp16 [8,16,2048,2048]": 1627472076,
-    "causal_bwd fp16 [8,16,2048,2048]": 2181120204,
-    "causal_fwd bf16 [8,16,2048,2048]": 1627459788,
-    "causal_bwd bf16 [8,16,2048,2048] (in place)": 2181120204,
-    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635900211,
-    "causal_dropout_bwd p=0.1 bf16 [8,16,2048,2048] (in place)": 2214719488,
-    "causal_fwd fp32 [8,16,2048,2048]": 3238067404,
-    "causal_bwd fp32 [8,16,2048,2048] (in place)": 4328580915,
-    "causal_fwd bf16 [1,16,8192,8192]": 3229695795,
-    "masked_fwd bf16 [16,16,1024,1024] key mask": 1082271948,
-    "masked_bwd bf16 [16,16,1024,1024]": 1610650624,
-    "bias_gelu_fwd bf16 [16384,16384]": 1073874739,
-    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677932953,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610759168,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141059379,
-    "bias_gelu_fwd bf16 [16384,4096]": 268489523,
-    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419568230,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402726297,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285347840,
-    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807980441,
-    "causal_fwd bf16 [8,16,2048,2048] with padding mask": 1628022988,
-    "causal_window_fwd window 256 bf16 [8,16,2048,2048]": 1230656716,
-    "causal_window_bwd window 256 bf16 [8,16,2048,2048] (in place)": 1387504640,
+    "attention_decode bf16 1 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 17573906,
+    "attention_decode bf16 8 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 136477702,
+    "causal_fwd fp16 [8,16,2048,2048]": 1627471925,
+    "causal_bwd fp16 [8,16,2048,2048]": 2181120040,
+    "causal_fwd bf16 [8,16,2048,2048]": 1627459651,
+    "causal_bwd bf16 [8,16,2048,2048] (in place)": 2181120131,
+    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635900235,
+    "causal_dropout_bwd p=0.1 bf16 [8,16,2048,2048] (in place)": 2214719510,
+    "causal_fwd fp32 [8,16,2048,2048]": 3238067312,
+    "causal_bwd fp32 [8,16,2048,2048] (in place)": 4328580380,
+    "causal_fwd bf16 [1,16,8192,8192]": 3229695244,
+    "masked_fwd bf16 [16,16,1024,1024] key mask": 1082271787,
+    "masked_bwd bf16 [16,16,1024,1024]": 1610650634,
+    "bias_gelu_fwd bf16 [16384,16384]": 1073876432,
+    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677947891,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610759196,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141067825,
+    "bias_gelu_fwd bf16 [16384,4096]": 268493619,
+    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419584301,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402709923,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285361377,
+    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 808012571,
+    "causal_fwd bf16 [8,16,2048,2048] with padding mask": 1628022937,
+    "causal_window_fwd window 256 bf16 [8,16,2048,2048]": 1230656579,
+    "causal_window_bwd window 256 bf16 [8,16,2048,2048] (in place)": 1387504728,
+    "causal_fwd bf16 [4,16,4096,4096]": 3238084608,
+    "causal_bwd bf16 [4,16,4096,4096] (in place)": 4328603740,
 }
 
 
