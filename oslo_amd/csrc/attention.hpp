@@ -67,6 +67,60 @@ __device__ __forceinline__ void with_distinct_buffers(const T *__restrict__ read
   f(read_a, write_a, read_b, write_b);
 }
 
+// Loads from global memory straight into LDS, for kernels that stream tiles
+// of [position][feature] rows. A tile is loaded through a descriptor of its
+// own (base = the tile's first row, size = what is left of the head's slice
+// from there, nothing for tiles outside [0, end): rows past the slice and
+// whole tiles that are not needed read as zeros without a memory access),
+// kept as scalars and stepped from tile to tile.
+struct TileStream {
+  uint64_t base; // the tile's first row
+  uint32_t left; // bytes from there to the end of the slice
+  uint32_t step; // bytes from a tile to the next
+  int tile, end;
+  __device__ __forceinline__ void start(const void *p, uint32_t bytes, uint32_t row_bytes, int rows_per_tile, int t,
+                                        int tiles_end) {
+    step = (uint32_t)rows_per_tile * row_bytes;
+    tile = t;
+    end = tiles_end;
+    const uint32_t skip = (uint32_t)(t < 0 ? 0 : t) * step;
+    base = reinterpret_cast<uint64_t>(p) + skip;
+    left = skip < bytes ? bytes - skip : 0u;
+  }
+  __device__ __forceinline__ void advance() {
+    base += step;
+    left = left > step ? left - step : 0u;
+    ++tile;
+  }
+  // raw 32-bit buffer descriptor (word 3 = 0x00020000, as make_rsrc builds it),
+  // read as scalars: the hand-written loads take it in scalar registers
+  __device__ __forceinline__ u32x4 descriptor() const {
+    u32x4 d;
+    d[0] = __builtin_amdgcn_readfirstlane((uint32_t)base);
+    d[1] = __builtin_amdgcn_readfirstlane((uint32_t)(base >> 32) & 0xffffu);
+    d[2] = __builtin_amdgcn_readfirstlane(tile >= 0 && tile < end ? left : 0u);
+    d[3] = 0x00020000u;
+    return d;
+  }
+};
+// The loads themselves are written out: the compiler, told of a load into LDS
+// (the builtin), waits for every such load before the next LDS read of any
+// buffer. These are waited for by count (wait_vm). A wave's instruction puts
+// its 64 x 16 (or 64 x 4) bytes at consecutive LDS addresses from `dst` on.
+__device__ __forceinline__ void lds_load_b128(const u32x4 &desc, const void *dst, uint32_t offset) {
+  const uint32_t at = __builtin_amdgcn_readfirstlane((uint32_t)reinterpret_cast<uintptr_t>(dst));
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");
+}
+__device__ __forceinline__ void lds_load_b32(const u32x4 &desc, const void *dst, uint32_t offset) {
+  const uint32_t at = __builtin_amdgcn_readfirstlane((uint32_t)reinterpret_cast<uintptr_t>(dst));
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");
+}
+// vmcnt <= N, nothing else: all but the N most recent loads have arrived
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
 // Additive mask values travel in log2 units. Masks of -inf or of the most
 // negative finite number (as some callers build them) would make every score
 // of a row -inf and its softmax 0/0; they are floored at a value that still

@@ -468,6 +468,398 @@ __global__ __launch_bounds__(kBlockThreads, D == 64 && ROLE != kRoleDKV ? 2 : 1)
   if constexpr (ROLE == kRoleDKV || ROLE == kRoleDV) write(a.dv, a.sdv, acc_p, DROP ? a.drop.keep_scale : 1.0f);
 }
 
+// ---------------------------------------------------------------------------
+// The same gradients for the plain case (no padding mask, no window, no
+// dropout), the way the forward is built: tiles of 32 positions of the other
+// kind loaded straight into LDS (four buffers per tensor), stored as they are
+// in memory, read as A operands of the score-like products 16 bytes per lane
+// and as A operands of the accumulating product through the transposing read
+// (no transposed copy, no staging through registers); a tile's code ordered by
+// hand: the products of T1, those of T2, then the accumulating products of the
+// previous tile with this tile's probabilities and score gradients worked out
+// between them. One permutation of a row's 16-byte chunks serves both reads
+// (f(row) below). dK and dV take a pass each at every head size.
+// ---------------------------------------------------------------------------
+
+constexpr int kSchedTile = 32;
+constexpr int kSchedBuffers = 4;
+
+template <typename T, int D, int ROLE>
+constexpr unsigned sched_lds_bytes() {
+  return 2u * kSchedBuffers * kSchedTile * D * sizeof(T) + kSchedBuffers * 2u * 256u * sizeof(float);
+}
+
+template <typename T, int D, int ROLE>
+__global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) void attention_bwd_scheduled_kernel(
+    const BwdArgs a) {
+  static_assert(ROLE == kRoleDQ || ROLE == kRoleDK || ROLE == kRoleDV, "one gradient per pass");
+  using Op = MatrixOp<T>;
+  using Frag = typename Op::Frag;
+  constexpr bool kKeysOwn = ROLE != kRoleDQ;
+  constexpr bool kNeedT2 = ROLE != kRoleDV;
+  constexpr int kChunks = D / 8;   // 16-byte chunks of a position
+  constexpr int kSteps = D / 16;   // contraction steps over the features
+  constexpr int kBlocksD = D / 32; // 32-row blocks of the accumulator
+  constexpr int kLoadsN = kSchedTile * kChunks / kBlockThreads; // loads per thread and tile of a tensor
+  constexpr int kTile = kSchedTile * D; // elements
+  constexpr int kRowBytes = D * (int)sizeof(T);
+  constexpr int kSwizzle = kChunks >= 16 ? 15 : 7;
+  constexpr int kRowSlots = 256; // floats of a tile's per-position values: the first 32 count
+
+  extern __shared__ __align__(1024) unsigned char lds_raw[];
+  T *const o1_lds = reinterpret_cast<T *>(lds_raw);            // [4][position][chunk ^ f(position)][8]
+  T *const o2_lds = o1_lds + kSchedBuffers * kTile;            // the same for the second tensor
+  float *const rows_lds = reinterpret_cast<float *>(o2_lds + kSchedBuffers * kTile); // [4][lse, delta][256]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int half = lane >> 5;
+  const int col = lane & 31;
+
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  const int bh = xcd + 8 * (slot % a.head_groups);
+  const int idx = slot / a.head_groups;
+  const int own_block = kKeysOwn ? idx : a.own_blocks - 1 - idx;
+  if (bh >= a.batch_heads) return; // the whole block
+  const int b = bh / a.heads;
+  const int hd = bh - b * a.heads;
+  const int S = a.S;
+  const int own0 = own_block * kOwnPerBlock;
+  const int wave_own0 = own0 + 32 * wave;
+  const int own = wave_own0 + col;
+
+  auto slice = [&](const void *p, const Strides3 &st) __attribute__((always_inline)) {
+    return static_cast<const T *>(p) + b * st.b + hd * st.h;
+  };
+  auto slice_bytes = [&](const Strides3 &st) __attribute__((always_inline)) {
+    return (uint32_t)(((int64_t)(S - 1) * st.s + D) * sizeof(T));
+  };
+  const Strides3 &st_own1 = kKeysOwn ? a.sk : a.sq;
+  const Strides3 &st_own2 = kKeysOwn ? a.sv : a.sdo;
+  const Strides3 &st_o1 = kKeysOwn ? a.sq : a.sk;
+  const Strides3 &st_o2 = kKeysOwn ? a.sdo : a.sv;
+  const T *own1_p = slice(kKeysOwn ? a.k : a.q, st_own1);
+  const T *own2_p = slice(kKeysOwn ? a.v : a.dout, st_own2);
+  const T *o1_p = slice(kKeysOwn ? a.q : a.k, st_o1);
+  const T *o2_p = slice(kKeysOwn ? a.dout : a.v, st_o2);
+  const uint32_t o1_row = (uint32_t)st_o1.s * sizeof(T);
+  const uint32_t o2_row = (uint32_t)st_o2.s * sizeof(T);
+
+  // B operands of the own positions, in registers for the whole kernel
+  Frag own1[kSteps], own2[kNeedT2 ? kSteps : 1];
+  {
+    const BufRsrc rs1 = make_rsrc(own1_p, slice_bytes(st_own1));
+    const uint32_t row1 = (uint32_t)st_own1.s * sizeof(T);
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s)
+      own1[s] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(
+                                             rs1, (uint32_t)own * row1 + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0));
+    if constexpr (kNeedT2) {
+      const BufRsrc rs2 = make_rsrc(own2_p, slice_bytes(st_own2));
+      const uint32_t row2 = (uint32_t)st_own2.s * sizeof(T);
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s)
+        own2[s] = __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(
+                                               rs2, (uint32_t)own * row2 + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0));
+    }
+  }
+  const int64_t stat_row = (int64_t)bh * S;
+  float own_lse = 0.f, own_delta = 0.f;
+  if constexpr (!kKeysOwn) {
+    if (own < S) {
+      own_lse = a.lse[stat_row + own];
+      own_delta = a.delta[stat_row + own];
+    }
+  }
+
+  // Tiles of the other kind this block walks; those the causal boundary
+  // crosses: for queries the last four, for keys the first four.
+  int first_tile, tiles, boundary_from, boundary_to;
+  if constexpr (!kKeysOwn) {
+    const int last_key = (own0 + kOwnPerBlock < S ? own0 + kOwnPerBlock : S) - 1;
+    tiles = last_key / kSchedTile + 1;
+    first_tile = 0;
+    boundary_from = own0 / kSchedTile, boundary_to = tiles;
+  } else {
+    first_tile = own0 / kSchedTile;
+    tiles = (S - 1) / kSchedTile + 1;
+    boundary_from = first_tile, boundary_to = first_tile + kOwnPerBlock / kSchedTile;
+  }
+
+  // The permutation of a row's chunks: chunk c of row r lies at c ^ f(r). The
+  // 16 lanes that read 16 consecutive rows at one chunk (natural operands) must
+  // get 16 values of f, the 16 lanes of a transposing read (rows 4c .. 4c + 3,
+  // two chunks, both halves of each) four values that differ above bit 0: f
+  // puts the row's two low bits at bits 1 and 2, bit 2 at bit 0, bit 3 stays.
+  auto f_of = [](int r) __attribute__((always_inline)) { return (((r & 3) << 1) | ((r >> 2) & 1) | (r & 8)) & kSwizzle; };
+  uint32_t o1_off[kLoadsN], o2_off[kLoadsN];
+#pragma unroll
+  for (int j = 0; j < kLoadsN; ++j) {
+    const int sigma = (4 * j + wave) * kWave + lane;
+    const int row = sigma / kChunks, at = sigma % kChunks;
+    o1_off[j] = (uint32_t)row * o1_row + (uint32_t)(at ^ f_of(row)) * 16u;
+    o2_off[j] = (uint32_t)row * o2_row + (uint32_t)(at ^ f_of(row)) * 16u;
+  }
+  const uint32_t row_off = tid < kSchedTile ? (uint32_t)tid * 4u : 0x80000000u;
+  TileStream o1_src, o2_src, lse_src, delta_src; // the next tile to load (tile t + 2 while tile t is computed)
+  o1_src.start(o1_p, slice_bytes(st_o1), o1_row, kSchedTile, first_tile, tiles);
+  o2_src.start(o2_p, slice_bytes(st_o2), o2_row, kSchedTile, first_tile, tiles);
+  if constexpr (kKeysOwn) {
+    lse_src.start(a.lse + stat_row, (uint32_t)S * 4u, 4u, kSchedTile, first_tile, tiles);
+    delta_src.start(a.delta + stat_row, (uint32_t)S * 4u, 4u, kSchedTile, first_tile, tiles);
+  }
+  constexpr int kItems = 2 * kLoadsN + (kKeysOwn ? 2 : 0);
+  constexpr int kLoadsPerTile = kItems;
+  int t = first_tile;
+  // buffer of tile t + d
+  auto buffer_of = [&](int d) __attribute__((always_inline)) { return (t + d) & (kSchedBuffers - 1); };
+  // item `it` of the staging of tile t: the loads of tile t + 2
+  auto stage_item = [&](int it) __attribute__((always_inline)) {
+    const int buf = buffer_of(2);
+    if (it < kLoadsN) {
+      lds_load_b128(o1_src.descriptor(), o1_lds + buf * kTile + (4 * it + wave) * (kWave * 8), o1_off[it]);
+      if (it == kLoadsN - 1) o1_src.advance();
+      return;
+    }
+    it -= kLoadsN;
+    if (it < kLoadsN) {
+      lds_load_b128(o2_src.descriptor(), o2_lds + buf * kTile + (4 * it + wave) * (kWave * 8), o2_off[it]);
+      if (it == kLoadsN - 1) o2_src.advance();
+      return;
+    }
+    it -= kLoadsN;
+    if constexpr (kKeysOwn) {
+      // every wave loads 64 values into a quarter of its own; the first 32 of the first wave's count
+      float *dst = rows_lds + (buf * 2 + it) * kRowSlots + wave * kWave;
+      if (it == 0) {
+        lds_load_b32(lse_src.descriptor(), dst, row_off);
+        lse_src.advance();
+      } else {
+        lds_load_b32(delta_src.descriptor(), dst, row_off);
+        delta_src.advance();
+      }
+    }
+  };
+
+  // natural operand s of the tile in `base`: lane (row, half) takes chunk 2 s + half of its row
+  const uint32_t nat_lane = (uint32_t)col * kRowBytes + (uint32_t)((half ^ f_of(col)) << 4);
+  auto read_natural = [&](const T *base, int s) __attribute__((always_inline)) {
+    return *reinterpret_cast<const Frag *>(reinterpret_cast<const char *>(base) + (nat_lane ^ (uint32_t)(s << 5)));
+  };
+  // Transposed operand n (16 positions u into block i of 32 features): of 16
+  // lanes, lane j points at 8 bytes (4 features) of position j / 4; lane i gets
+  // back feature i of the four positions. Two reads make an operand: slots 0..3
+  // are positions 16u + 4h + 0..3, slots 4..7 positions 16u + 8 + 4h + 0..3 (h
+  // the lane's half of the wave): the rows the accumulator layout gives a lane.
+  typedef short Short4 __attribute__((ext_vector_type(4)));
+  uint32_t tr_lane[2]; // for even and odd blocks of 32 features
+  {
+    const int j = lane & 15, group = lane >> 4;
+    const int kq = j >> 2, fb = j & 3, hh = group >> 1, fg = group & 1;
+    // f of the lane's rows 16u + 8jj + 4hh + kq is 2 kq | hh | 8 jj; the part below bit 3:
+    const int flow = ((kq << 1) | hh) & kSwizzle;
+    const int x = (2 * fg + (fb >> 1)) ^ (flow & 3);
+    const int flip = flow >> 2; // its bit 2 swaps neighbouring blocks of four chunks
+    const uint32_t base = (uint32_t)(4 * hh + kq) * kRowBytes + (uint32_t)x * 16u + (uint32_t)(fb & 1) * 8u;
+    tr_lane[0] = base + 64u * (uint32_t)flip;
+    tr_lane[1] = base + 64u * (uint32_t)(1 ^ flip);
+  }
+  auto read_transposed = [&](const T *base, int n) __attribute__((always_inline)) {
+    const int u = n / kBlocksD, i = n % kBlocksD;
+    Short4 part[2];
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+      // rows with bit 3 set (jj = 1) have bit 3 of f set: blocks two apart swap (head sizes of 16 chunks and more)
+      const int ii = kSwizzle >= 8 ? i ^ (2 * jj) : i;
+      const char *at = reinterpret_cast<const char *>(base) + tr_lane[ii & 1] + 64 * (ii & ~1) +
+                       (16 * u + 8 * jj) * kRowBytes;
+      part[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) Short4 *)(at));
+    }
+    return __builtin_bit_cast(Frag, __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+
+  f32x16 acc[kBlocksD];
+#pragma unroll
+  for (int i = 0; i < kBlocksD; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+  Frag xf[2]; // what the accumulating product takes of the last tile computed: P or P o (dP - delta)
+
+  // which tensor the accumulating product reads transposed: K (dQ), Q (dK), dO (dV)
+  auto transposed_tile = [&](int d) __attribute__((always_inline)) {
+    return (ROLE == kRoleDV ? o2_lds : o1_lds) + buffer_of(d) * kTile;
+  };
+  // slice `n` of `slices` of a tile's elementwise work: P = exp2(scale*log2e *
+  // T1 - lse), X = P (dV) or P (T2 - delta) (the scale goes onto the result)
+  auto elementwise = [&]<bool MASKED>(f32x16 &t1, const f32x16 &t2, int n, int slices, Frag (&x)[2])
+                         __attribute__((always_inline)) {
+    const float *rows = rows_lds + buffer_of(0) * 2 * kRowSlots;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      if (r * slices / 16 != n) continue;
+      const int rr = 8 * (r >> 2) + 4 * half + (r & 3); // the register's row of the tile
+      float lse_r = own_lse, delta_r = own_delta;
+      if constexpr (kKeysOwn) {
+        lse_r = rows[rr];
+        if constexpr (kNeedT2) delta_r = rows[kRowSlots + rr];
+      }
+      float p = __builtin_amdgcn_exp2f(__builtin_fmaf(t1[r], a.scale_log2e, -lse_r));
+      if constexpr (MASKED) {
+        const int other = t * kSchedTile + rr;
+        const bool visible = kKeysOwn ? own <= other : other <= own;
+        p = visible ? p : 0.f;
+      }
+      if constexpr (kNeedT2) p *= t2[r] - delta_r;
+      t1[r] = p;
+      asm volatile("" : "+v"(t1[r])); // (keeps the computation in its slice)
+    }
+    if (n == slices - 1) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[u][i] = static_cast<T>(t1[8 * u + i]);
+    }
+  };
+
+  // prologue: the first two tiles on their way
+#pragma unroll
+  for (int rep = 0; rep < 2; ++rep) {
+    t = first_tile - 2 + rep; // (an item loads tile t + 2)
+#pragma unroll
+    for (int it = 0; it < kItems; ++it) stage_item(it);
+  }
+  t = first_tile;
+
+  // the block's first tile: nothing to accumulate yet; plain order
+  {
+    wait_vm<kLoadsPerTile>();
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < kItems; ++it) stage_item(it);
+    f32x16 t1, t2;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) t1[r] = t2[r] = 0.f;
+    const T *b1 = o1_lds + buffer_of(0) * kTile, *b2 = o2_lds + buffer_of(0) * kTile;
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) t1 = Op::run(read_natural(b1, s), own1[s], t1);
+    if constexpr (kNeedT2) {
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) t2 = Op::run(read_natural(b2, s), own2[s], t2);
+    }
+    elementwise.template operator()<true>(t1, t2, 0, 1, xf);
+    ++t;
+  }
+
+  // A tile as one straight run of code between fences: the products of T1 with
+  // the next tiles' loads between them, those of T2, then the accumulating
+  // products of the previous tile with this tile's elementwise work between
+  // them. Operands are read from LDS kRing products ahead.
+  auto scheduled_tile = [&]<bool MASKED>() __attribute__((always_inline)) {
+    constexpr int kRing = 4;
+    constexpr int kProducts = 2 * kBlocksD;
+    constexpr int kOperands = kSteps + (kNeedT2 ? kSteps : 0) + kProducts;
+    constexpr int kPerStep = (kItems + kSteps - 1) / kSteps;
+    const T *b1 = o1_lds + buffer_of(0) * kTile, *b2 = o2_lds + buffer_of(0) * kTile;
+    const T *bt = transposed_tile(-1);
+    Frag ring[kRing];
+    auto read_operand = [&](int p) __attribute__((always_inline)) {
+      if (p < kSteps) ring[p % kRing] = read_natural(b1, p);
+      else if (kNeedT2 && p < 2 * kSteps) ring[p % kRing] = read_natural(b2, p - kSteps);
+      else ring[p % kRing] = read_transposed(bt, p - (kNeedT2 ? 2 : 1) * kSteps);
+    };
+#pragma unroll
+    for (int p = 0; p < kRing; ++p) read_operand(p);
+    __builtin_amdgcn_sched_barrier(0);
+    f32x16 t1, t2;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) t1[r] = t2[r] = 0.f;
+    int p = 0;
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s, ++p) {
+      t1 = Op::run(ring[p % kRing], own1[s], t1);
+      if (p + kRing < kOperands) read_operand(p + kRing);
+#pragma unroll
+      for (int it = s * kPerStep; it < (s + 1) * kPerStep && it < kItems; ++it) stage_item(it);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (kNeedT2) {
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s, ++p) {
+        t2 = Op::run(ring[p % kRing], own2[s], t2);
+        if (p + kRing < kOperands) read_operand(p + kRing);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    Frag xn[2];
+#pragma unroll
+    for (int n = 0; n < kProducts; ++n, ++p) {
+      acc[n % kBlocksD] = Op::run(ring[p % kRing], xf[n / kBlocksD], acc[n % kBlocksD]);
+      if (p + kRing < kOperands) read_operand(p + kRing);
+      elementwise.template operator()<MASKED>(t1, t2, n, kProducts, xn);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    xf[0] = xn[0], xf[1] = xn[1];
+  };
+  // each kind of tile in a loop of its own
+  auto run_tiles = [&]<bool MASKED>(int end) __attribute__((always_inline)) {
+    for (; t < end; ++t) {
+      wait_vm<kLoadsPerTile>();
+      __syncthreads(); // tile t is in LDS; the buffer written next (tile t - 2's) has been read
+      scheduled_tile.template operator()<MASKED>();
+    }
+  };
+  if constexpr (!kKeysOwn) {
+    run_tiles.template operator()<false>(boundary_from < tiles ? boundary_from : tiles);
+    run_tiles.template operator()<true>(tiles);
+  } else {
+    run_tiles.template operator()<true>(boundary_to < tiles ? boundary_to : tiles);
+    run_tiles.template operator()<false>(tiles);
+  }
+  // the last tile's accumulating products
+  wait_vm<0>(); // (nothing may still be on its way into LDS when the block ends)
+  __syncthreads();
+  {
+    const T *bt = transposed_tile(-1);
+#pragma unroll
+    for (int n = 0; n < 2 * kBlocksD; ++n)
+      acc[n % kBlocksD] = Op::run(read_transposed(bt, n), xf[n / kBlocksD], acc[n % kBlocksD]);
+  }
+
+  if (own >= S) return;
+  typedef T Out4 __attribute__((ext_vector_type(4)));
+  const Strides3 &st_out = ROLE == kRoleDQ ? a.sdq : ROLE == kRoleDK ? a.sdk : a.sdv;
+  void *out_base = ROLE == kRoleDQ ? a.dq : ROLE == kRoleDK ? a.dk : a.dv;
+  const float factor = kNeedT2 ? a.scale : 1.0f;
+  T *op = static_cast<T *>(out_base) + b * st_out.b + hd * st_out.h + (int64_t)own * st_out.s;
+#pragma unroll
+  for (int i = 0; i < kBlocksD; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      Out4 w;
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(acc[i][4 * j + tt] * factor);
+      *reinterpret_cast<Out4 *>(op + 32 * i + 8 * j + 4 * half) = w;
+    }
+}
+
+template <typename T, int D, int ROLE>
+int launch_scheduled_role(const BwdArgs &a, hipStream_t stream) {
+  const dim3 grid((unsigned)(8 * a.head_groups * a.own_blocks));
+  constexpr unsigned kLds = sched_lds_bytes<T, D, ROLE>();
+  auto *kernel = attention_bwd_scheduled_kernel<T, D, ROLE>;
+  if (kLds > 64u * 1024u) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
+    if (e != hipSuccess)
+      return fail(OSLO_E_LAUNCH, "oslo_attention_prefill_bwd: %u bytes of dynamic LDS refused: %s", kLds,
+                  hipGetErrorString(e));
+  }
+  kernel<<<grid, dim3(kBlockThreads), kLds, stream>>>(a);
+  return check_launch("attention_prefill_bwd");
+}
+
 // delta[bh, q] = sum_d dO[q, d] * O[q, d], fp32. D / 8 lanes share a row.
 template <typename T, int D>
 __global__ __launch_bounds__(kBlockThreads) void attention_delta_kernel(
@@ -526,6 +918,14 @@ int launch_bwd_dim(const BwdArgs &a, float *delta, const void *out, const Stride
       delta, static_cast<const T *>(out), static_cast<const T *>(a.dout), so, a.sdo, a.S, a.heads, rows);
   int s = check_launch("attention_prefill_bwd(delta)");
   if (s != OSLO_OK) return s;
+  if (a.pad == nullptr && a.window == 0 && !a.drop.drop) {
+    // the plain case: the hand-ordered kernel, a pass per gradient
+    s = launch_scheduled_role<T, D, kRoleDQ>(a, stream);
+    if (s != OSLO_OK) return s;
+    s = launch_scheduled_role<T, D, kRoleDK>(a, stream);
+    if (s != OSLO_OK) return s;
+    return launch_scheduled_role<T, D, kRoleDV>(a, stream);
+  }
   s = launch_role<T, D, kRoleDQ>(a, stream);
   if (s != OSLO_OK) return s;
   if constexpr (D == 256) {
