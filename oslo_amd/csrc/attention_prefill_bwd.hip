@@ -469,8 +469,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 64 && ROLE != kRoleDKV ? 2 : 1)
 }
 
 // ---------------------------------------------------------------------------
-// The same gradients for the plain case (no padding mask, no window, no
-// dropout), the way the forward is built: tiles of 32 positions of the other
+// The same gradients without a sliding window, the way the forward is built: tiles of 32 positions of the other
 // kind loaded straight into LDS (four buffers per tensor), stored as they are
 // in memory, read as A operands of the score-like products 16 bytes per lane
 // and as A operands of the accumulating product through the transposing read
@@ -486,10 +485,11 @@ constexpr int kSchedBuffers = 4;
 
 template <typename T, int D, int ROLE>
 constexpr unsigned sched_lds_bytes() {
-  return 2u * kSchedBuffers * kSchedTile * D * sizeof(T) + kSchedBuffers * 2u * 256u * sizeof(float);
+  return 2u * kSchedBuffers * kSchedTile * D * sizeof(T) + kSchedBuffers * 2u * 256u * sizeof(float) +
+         kWavesPerBlock * 32u * sizeof(uint32_t);
 }
 
-template <typename T, int D, int ROLE>
+template <typename T, int D, int ROLE, bool HAS_PAD, bool DROP>
 __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) void attention_bwd_scheduled_kernel(
     const BwdArgs a) {
   static_assert(ROLE == kRoleDQ || ROLE == kRoleDK || ROLE == kRoleDV, "one gradient per pass");
@@ -509,13 +509,16 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   extern __shared__ __align__(1024) unsigned char lds_raw[];
   T *const o1_lds = reinterpret_cast<T *>(lds_raw);            // [4][position][chunk ^ f(position)][8]
   T *const o2_lds = o1_lds + kSchedBuffers * kTile;            // the same for the second tensor
-  float *const rows_lds = reinterpret_cast<float *>(o2_lds + kSchedBuffers * kTile); // [4][lse, delta][256]
+  // per-position values of a tile: queries: log-sum-exp and delta; keys: the padding mask's value
+  float *const rows_lds = reinterpret_cast<float *>(o2_lds + kSchedBuffers * kTile); // [4][2][256]
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int half = lane >> 5;
   const int col = lane & 31;
+  uint32_t *const keep_lds =
+      reinterpret_cast<uint32_t *>(rows_lds + kSchedBuffers * 2 * kRowSlots) + 32 * wave; // a wave's keep bits of a tile
 
   const int xcd = blockIdx.x & 7;
   const int slot = blockIdx.x >> 3;
@@ -566,12 +569,14 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     }
   }
   const int64_t stat_row = (int64_t)bh * S;
-  float own_lse = 0.f, own_delta = 0.f;
+  float own_lse = 0.f, own_delta = 0.f, own_pad = 0.f; // (the padding value in log2 units)
   if constexpr (!kKeysOwn) {
     if (own < S) {
       own_lse = a.lse[stat_row + own];
       own_delta = a.delta[stat_row + own];
     }
+  } else if constexpr (HAS_PAD) {
+    if (own < S) own_pad = fmaxf(a.pad[(int64_t)b * S + own] * kLog2eB, kMaskFloorLog2);
   }
 
   // Tiles of the other kind this block walks; those the causal boundary
@@ -609,8 +614,11 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   if constexpr (kKeysOwn) {
     lse_src.start(a.lse + stat_row, (uint32_t)S * 4u, 4u, kSchedTile, first_tile, tiles);
     delta_src.start(a.delta + stat_row, (uint32_t)S * 4u, 4u, kSchedTile, first_tile, tiles);
+  } else if constexpr (HAS_PAD) { // the keys' mask values take the first of the two rows
+    lse_src.start(a.pad + (int64_t)b * S, (uint32_t)S * 4u, 4u, kSchedTile, first_tile, tiles);
   }
-  constexpr int kItems = 2 * kLoadsN + (kKeysOwn ? 2 : 0);
+  constexpr int kRowItems = kKeysOwn ? 2 : HAS_PAD ? 1 : 0;
+  constexpr int kItems = 2 * kLoadsN + kRowItems;
   constexpr int kLoadsPerTile = kItems;
   int t = first_tile;
   // buffer of tile t + d
@@ -630,7 +638,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
       return;
     }
     it -= kLoadsN;
-    if constexpr (kKeysOwn) {
+    if constexpr (kRowItems > 0) {
       // every wave loads 64 values into a quarter of its own; the first 32 of the first wave's count
       float *dst = rows_lds + (buf * 2 + it) * kRowSlots + wave * kWave;
       if (it == 0) {
@@ -692,26 +700,55 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     return (ROLE == kRoleDV ? o2_lds : o1_lds) + buffer_of(d) * kTile;
   };
   // slice `n` of `slices` of a tile's elementwise work: P = exp2(scale*log2e *
-  // T1 - lse), X = P (dV) or P (T2 - delta) (the scale goes onto the result)
+  // T1 + pad*log2e - lse), X = P (dV) or P (T2 - delta) (the scale goes onto
+  // the result). With attention dropout the forward multiplied V with
+  // keep * P / (1-p): the P product takes the kept probabilities (1/(1-p) goes
+  // onto dV at the end), and the gradient of the dropped-out probabilities is
+  // keep * dP / (1-p). The keep bits of the tile are drawn in the first slice.
+  u32x4 keep_words[4];
+  uint32_t keep_bits = 0;
   auto elementwise = [&]<bool MASKED>(f32x16 &t1, const f32x16 &t2, int n, int slices, Frag (&x)[2])
                          __attribute__((always_inline)) {
     const float *rows = rows_lds + buffer_of(0) * 2 * kRowSlots;
+    if constexpr (DROP) {
+      if (n == 0) {
+        const int other0 = t * kSchedTile;
+        stage_keep_bits(keep_lds, a.drop, bh, S, kKeysOwn ? other0 : wave_own0, kKeysOwn ? wave_own0 : other0, lane);
+        if constexpr (kKeysOwn) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) keep_words[j] = keep_words_key_lane(keep_lds, j, half);
+        } else {
+          keep_bits = keep_word_query_lane(keep_lds, col) >> (4 * half);
+        }
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       if (r * slices / 16 != n) continue;
       const int rr = 8 * (r >> 2) + 4 * half + (r & 3); // the register's row of the tile
-      float lse_r = own_lse, delta_r = own_delta;
+      float shift, delta_r = own_delta;
       if constexpr (kKeysOwn) {
-        lse_r = rows[rr];
+        shift = own_pad - rows[rr];
         if constexpr (kNeedT2) delta_r = rows[kRowSlots + rr];
+      } else if constexpr (HAS_PAD) {
+        shift = __builtin_fmaf(fmaxf(rows[rr], kMaskFloor), kLog2eB, -own_lse);
+      } else {
+        shift = -own_lse;
       }
-      float p = __builtin_amdgcn_exp2f(__builtin_fmaf(t1[r], a.scale_log2e, -lse_r));
+      float p = __builtin_amdgcn_exp2f(__builtin_fmaf(t1[r], a.scale_log2e, shift));
       if constexpr (MASKED) {
         const int other = t * kSchedTile + rr;
         const bool visible = kKeysOwn ? own <= other : other <= own;
         p = visible ? p : 0.f;
       }
-      if constexpr (kNeedT2) p *= t2[r] - delta_r;
+      float grad = t2[r];
+      if constexpr (DROP) {
+        const bool keep = kKeysOwn ? ((keep_words[r >> 2][r & 3] >> col) & 1u) != 0
+                                   : ((keep_bits >> (8 * (r >> 2) + (r & 3))) & 1u) != 0;
+        grad = keep ? grad * a.drop.keep_scale : 0.f;
+        if constexpr (!kNeedT2) p = keep ? p : 0.f;
+      }
+      if constexpr (kNeedT2) p *= grad - delta_r;
       t1[r] = p;
       asm volatile("" : "+v"(t1[r])); // (keeps the computation in its slice)
     }
@@ -831,7 +868,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   typedef T Out4 __attribute__((ext_vector_type(4)));
   const Strides3 &st_out = ROLE == kRoleDQ ? a.sdq : ROLE == kRoleDK ? a.sdk : a.sdv;
   void *out_base = ROLE == kRoleDQ ? a.dq : ROLE == kRoleDK ? a.dk : a.dv;
-  const float factor = kNeedT2 ? a.scale : 1.0f;
+  const float factor = kNeedT2 ? a.scale : DROP ? a.drop.keep_scale : 1.0f;
   T *op = static_cast<T *>(out_base) + b * st_out.b + hd * st_out.h + (int64_t)own * st_out.s;
 #pragma unroll
   for (int i = 0; i < kBlocksD; ++i)
@@ -848,16 +885,24 @@ template <typename T, int D, int ROLE>
 int launch_scheduled_role(const BwdArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)(8 * a.head_groups * a.own_blocks));
   constexpr unsigned kLds = sched_lds_bytes<T, D, ROLE>();
-  auto *kernel = attention_bwd_scheduled_kernel<T, D, ROLE>;
-  if (kLds > 64u * 1024u) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
-    if (e != hipSuccess)
-      return fail(OSLO_E_LAUNCH, "oslo_attention_prefill_bwd: %u bytes of dynamic LDS refused: %s", kLds,
-                  hipGetErrorString(e));
+  auto go = [&]<bool HAS_PAD, bool DROP>() -> int {
+    auto *kernel = attention_bwd_scheduled_kernel<T, D, ROLE, HAS_PAD, DROP>;
+    if (kLds > 64u * 1024u) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
+      if (e != hipSuccess)
+        return fail(OSLO_E_LAUNCH, "oslo_attention_prefill_bwd: %u bytes of dynamic LDS refused: %s", kLds,
+                    hipGetErrorString(e));
+    }
+    kernel<<<grid, dim3(kBlockThreads), kLds, stream>>>(a);
+    return check_launch("attention_prefill_bwd");
+  };
+  if (a.pad != nullptr) {
+    if (a.drop.drop) return go.template operator()<true, true>();
+    return go.template operator()<true, false>();
   }
-  kernel<<<grid, dim3(kBlockThreads), kLds, stream>>>(a);
-  return check_launch("attention_prefill_bwd");
+  if (a.drop.drop) return go.template operator()<false, true>();
+  return go.template operator()<false, false>();
 }
 
 // delta[bh, q] = sum_d dO[q, d] * O[q, d], fp32. D / 8 lanes share a row.
@@ -918,8 +963,8 @@ int launch_bwd_dim(const BwdArgs &a, float *delta, const void *out, const Stride
       delta, static_cast<const T *>(out), static_cast<const T *>(a.dout), so, a.sdo, a.S, a.heads, rows);
   int s = check_launch("attention_prefill_bwd(delta)");
   if (s != OSLO_OK) return s;
-  if (a.pad == nullptr && a.window == 0 && !a.drop.drop) {
-    // the plain case: the hand-ordered kernel, a pass per gradient
+  if (a.window == 0) {
+    // no sliding window: the hand-ordered kernel, a pass per gradient
     s = launch_scheduled_role<T, D, kRoleDQ>(a, stream);
     if (s != OSLO_OK) return s;
     s = launch_scheduled_role<T, D, kRoleDK>(a, stream);
