@@ -437,8 +437,10 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         if S != 2048:  # the long prompt: forward only
             del q, k, v, o
             continue
-        # its backward (the forward that stores the log-sum-exp first): 7 matrix products per visible
-        # tile where the forward has 2, so 14 flops per score and feature
+        # its backward (the forward that stores the log-sum-exp first): counted as 7 matrix products per
+        # visible tile where the forward has 2 (14 flops per score and feature): the five of the
+        # mathematics and the scores once more for the second owner kind; the kernels run 8 (dK and
+        # dV take a pass each)
         lse = torch.empty((B, Hh, S), dtype=torch.float32, device=dev)
         check(lib.oslo_attention_prefill_fwd_lse(P(o), P(lse), P(q), P(k), P(v), None, D ** -0.5, 0.0, 0, 0,
                                                  B, Hh, S, D, 0, strides, BF16, st))
@@ -451,8 +453,8 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
             P(dq), P(dk), P(dv), P(do), P(q), P(k), P(v), P(o), P(lse), P(wsb), None, D ** -0.5, 0.0, 0, 0,
             B, Hh, S, D, 0, bstr, BF16, st)), max(5, n // 4), 3)
         bflops = 7 * flops // 2
-        res.append({"kernel": f"attention_prefill_bwd bf16 [{B},{Hh},{S},{D}] causal (dq, dk, dv; "
-                              f"{4 if D == 256 else 3} launches)", "bound": "mfma",
+        res.append({"kernel": f"attention_prefill_bwd bf16 [{B},{Hh},{S},{D}] causal (dq, dk, dv; 4 launches)",
+                    "bound": "mfma",
                     "achieved": round(bflops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(bflops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "us": round(t * 1e6, 1),
                     "algorithmic_flops": bflops, "traffic": None})
