@@ -51,6 +51,9 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kSlack = 8.0f;
 constexpr float kRaise = 4.0f;
 constexpr float kSumLimit = 256.0f; // 2^kSlack
+// The reference of a query that has not seen a key yet (sliding windows): any
+// finite score lies more than kRaise above it, and 2^(score - floor) is +inf.
+constexpr float kReferenceFloor = -3.0e38f;
 
 struct PrefillArgs {
   void *out;
@@ -287,7 +290,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   for (int i = 0; i < kBlocksD; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
-  float m = -INFINITY; // reference maximum of the query's scores, log2 units
+  float m = 0.f; // reference maximum of the query's scores, log2 units (the block's first tile sets it)
   float l = 0.f;       // this lane's share of the running sum
   Frag pf[2];          // P^T of the last tile computed, not yet multiplied with V
   bool pending = false; // wave-uniform: pf holds such a tile (the one before the current)
@@ -421,15 +424,13 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
       }
     }
     const float mt = tile_max(sc);
-    // Without a window key 0 is visible to every query and m is finite after
-    // the first tile; with one, a query may see nothing in the first tiles of
-    // its wave: m stays -inf, nothing is rescaled, and the exponentials (of
-    // -inf) are taken against 0.
-    const bool raise = mt > m + kRaise; // true at the first visible key (m = -inf)
-    if (__any(raise && m != -INFINITY)) { // wave-uniform
+    // (m is finite from the block's first tile on: with a window, the floor
+    // that tile leaves for a query that has seen no key yet)
+    const bool raise = mt > m + kRaise;
+    if (__any(raise)) { // wave-uniform
       if constexpr (!RESCALE) return false;
       const float m_new = raise ? mt : m;
-      const float alpha = raise ? __builtin_amdgcn_exp2f(m - m_new) : 1.0f; // 0 where m was -inf (nothing accumulated)
+      const float alpha = raise ? __builtin_amdgcn_exp2f(m - m_new) : 1.0f; // 0 above the floor (nothing accumulated)
       l *= alpha;
 #pragma unroll
       for (int i = 0; i < kBlocksD; ++i)
@@ -439,11 +440,10 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     } else {
       m = raise ? mt : m;
     }
-    const float shift = HAS_WINDOW && m == -INFINITY ? 0.f : m;
     float sum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      sc[r] = exponential(sc[r], shift);
+      sc[r] = exponential(sc[r], m);
       sum += sc[r];
     }
     l += sum;
@@ -451,27 +451,6 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     pending = true;
     return true;
   };
-  // Tiles [t, end) the general way. The tiles run in an inner loop that
-  // contains no multiplication of O; a tile in which some reference maximum
-  // has to rise leaves that loop, is done with the rescaling variant, and the
-  // loop is entered again.
-  auto general_range = [&](int end) __attribute__((always_inline)) {
-    while (t < end) {
-      bool rescale = false;
-      for (; t < end; next_tile()) {
-        wait_loads.template operator()<kLoadsPerTile>();
-        __syncthreads(); // tile t's K and tile t - 1's V are in LDS; the buffers written next have been read
-        if (!general_tile.template operator()<false>(t, true)) {
-          rescale = true;
-          break;
-        }
-      }
-      if (!rescale) break;
-      general_tile.template operator()<true>(t, false);
-      next_tile();
-    }
-  };
-
   // prologue: K of the first two tiles and V of the first on their way, all
   // issued before any is waited for (the sources then stand at tile t + 2 and
   // t + 1, where a tile's staging expects them)
@@ -548,12 +527,16 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
               const int kr_ = t * kKeysPerTile + 8 * (r >> 2) + 4 * half + (r & 3);
-              sc[r] = kr_ <= qrow ? sc[r] : -INFINITY;
+              sc[r] = kr_ <= qrow && (!HAS_WINDOW || kr_ > behind) ? sc[r] : -INFINITY;
             }
           }
           if constexpr (FIRST) {
             mt = tile_max(sc);
-            m = mt;
+            // With a window a query may see nothing in the first tiles of its
+            // wave: its reference then is a floor so far down that the first
+            // visible score overflows the tile's sum, which has the tile done
+            // again the general way, where the reference rises to that score.
+            m = HAS_WINDOW ? fmaxf(mt, kReferenceFloor) : mt;
           }
         }
 #pragma unroll
@@ -581,10 +564,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     });
   };
 
-  if constexpr (HAS_WINDOW) {
-    general_range(plain_begin < tiles ? plain_begin : tiles);
-  } else {
-    // the block's first tile (the causal boundary crosses it in the first block)
+  { // the block's first tile (the causal boundary, or the window's edge, may cross it)
     wait_loads.template operator()<0>();
     __syncthreads();
     float mt, sum;
@@ -594,8 +574,9 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     next_tile();
   }
 
-  // Tiles every query of the block sees in full, then (without a window) those
-  // the causal boundary crosses, each kind in a loop of its own (one loop with
+  // The tiles the edge of some query's window crosses, those every query of the
+  // block sees in full, then those the causal boundary crosses, each kind in a
+  // loop of its own (one loop with
   // a branch per kind has the compiler shuffle the accumulators where the
   // branches meet, in every tile). A wave whose queries all lie before a tile
   // still computes it, every score masked: it adds zeros, and it would wait at
@@ -623,9 +604,9 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
       next_tile();
     }
   };
+  if constexpr (HAS_WINDOW) scheduled_range.template operator()<true>(plain_begin < tiles ? plain_begin : tiles);
   scheduled_range.template operator()<false>(plain_end);
-  if constexpr (!HAS_WINDOW) scheduled_range.template operator()<true>(tiles);
-  if constexpr (HAS_WINDOW) general_range(tiles);
+  scheduled_range.template operator()<true>(tiles);
 
   wait_loads.template operator()<0>(); // (nothing may still be on its way into LDS when the block ends)
   __syncthreads(); // V of the last tile is in LDS
