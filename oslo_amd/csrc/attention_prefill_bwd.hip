@@ -27,8 +27,18 @@
 // the own position are per-lane scalars, those indexed by the other position
 // are read per tile from LDS. Each block sums in a fixed order and no two
 // blocks write the same element: the gradients are deterministic. The price is
-// that scores are computed twice (once per owner kind), 7 matrix products per
-// visible (query, key) tile instead of 5.
+// that scores are computed once per gradient: dQ takes three matrix products
+// per visible (query, key) tile, dK three, dV two, 8 instead of 5.
+//
+// The kernel is built the way the forward is: tiles of 32 positions of the
+// other kind loaded straight into LDS (four buffers per tensor), stored as they
+// are in memory, read as A operands of the score-like products 16 bytes per
+// lane and as A operands of the accumulating product through the transposing
+// read (no transposed copy, no staging through registers); a tile's code is
+// ordered by hand: the products of T1, those of T2, then the accumulating
+// products of the previous tile with this tile's probabilities and score
+// gradients worked out between them. One permutation of a row's 16-byte chunks
+// serves both reads (f(row) below).
 
 #include "attention.hpp"
 
@@ -38,7 +48,7 @@ namespace {
 constexpr int kOwnPerBlock = 128;
 constexpr float kLog2eB = 1.4426950408889634f;
 
-enum Role { kRoleDQ = 0, kRoleDKV = 1, kRoleDK = 2, kRoleDV = 3 };
+enum Role { kRoleDQ = 0, kRoleDK = 1, kRoleDV = 2 };
 
 struct Strides3 {
   int64_t b, h, s; // element strides: batch, head, position
@@ -56,430 +66,6 @@ struct BwdArgs {
   DropArgs drop; // attention dropout of the forward (the DROP variants)
 };
 
-template <int D>
-constexpr int tile_positions() { return D == 256 ? 32 : 64; }
-
-// Bytes of dynamic LDS a role needs.
-template <typename T, int D, int ROLE>
-constexpr unsigned bwd_lds_bytes() {
-  constexpr int kTile = tile_positions<D>();
-  constexpr unsigned tile = kTile * D * sizeof(T);
-  unsigned n = tile;                                   // Other1, natural
-  if (ROLE != kRoleDV) n += tile;                      // Other2, natural
-  if (ROLE != kRoleDV) n += tile;                      // OtherT for the dS product
-  if (ROLE == kRoleDKV || ROLE == kRoleDV) n += tile;  // OtherT for the P product
-  n += 2 * kTile * sizeof(float);                      // per-position values of the tile
-  if (D == 256) n += kOwnPerBlock * D * sizeof(T);     // Own1 operands
-  return n;
-}
-
-template <typename T, int D, int ROLE, bool HAS_PAD, bool HAS_WINDOW, bool DROP>
-__global__ __launch_bounds__(kBlockThreads, D == 64 && ROLE != kRoleDKV ? 2 : 1) void attention_bwd_kernel(
-    const BwdArgs a) {
-  using Op = MatrixOp<T>;
-  using Frag = typename Op::Frag;
-  constexpr bool kKeysOwn = ROLE != kRoleDQ;
-  constexpr bool kNeedT2 = ROLE != kRoleDV;
-  constexpr bool kAccS = ROLE != kRoleDV;
-  constexpr bool kAccP = ROLE == kRoleDKV || ROLE == kRoleDV;
-  constexpr int kTile = tile_positions<D>();
-  constexpr int kStepsPerTile = kTile / 32;
-  constexpr int kChunks = D / 8;   // 16-byte chunks of a position
-  constexpr int kSteps = D / 16;   // contraction steps over the features
-  constexpr int kBlocksD = D / 32; // 32-row blocks of an accumulator
-  constexpr int kTChunks = kTile / 8;
-  constexpr int kLoadsN = kTile * kChunks / kBlockThreads; // per thread, natural tile
-  constexpr int kRowsPerPass = kBlockThreads / kChunks;
-  constexpr int kSwizzleN = kChunks >= 16 ? 15 : 7;
-  constexpr int kTasks = kTChunks * kChunks; // 8 x 8 transpositions per tile
-  constexpr bool kOwn1InLds = D == 256;
-
-  // Dynamic LDS: the tiles the role needs, the per-position values of a tile,
-  // and (head_dim 256) the Own1 operands, each wave its own 16 KiB.
-  extern __shared__ __align__(16) unsigned char lds_raw[];
-  constexpr int kTileElems = kTile * D;
-  constexpr int kOffO2 = kTileElems;
-  constexpr int kOffTs = kOffO2 + (kNeedT2 ? kTileElems : 0);
-  constexpr int kOffTp = kOffTs + (kAccS ? kTileElems : 0);
-  constexpr int kOffEnd = kOffTp + (kAccP ? kTileElems : 0);
-  static_assert(kOffEnd * sizeof(T) + 2 * kTile * sizeof(float) +
-                        (kOwn1InLds ? kOwnPerBlock * D * sizeof(T) : 0) ==
-                    bwd_lds_bytes<T, D, ROLE>(),
-                "LDS layout and size disagree");
-  T *const o1_lds = reinterpret_cast<T *>(lds_raw);
-  T *const o2_lds = o1_lds + kOffO2;
-  T *const ts_lds = o1_lds + kOffTs;
-  T *const tp_lds = o1_lds + kOffTp;
-  float *const row_a = reinterpret_cast<float *>(o1_lds + kOffEnd);
-  float *const row_b = row_a + kTile;
-  u32x4 *const own1_lds = reinterpret_cast<u32x4 *>(row_b + kTile);
-  __shared__ __align__(16) uint32_t keep_lds[DROP ? kWavesPerBlock : 1][32]; // a wave's keep bits of a step
-
-  const int tid = threadIdx.x;
-  const int lane = tid & (kWave - 1);
-  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int half = lane >> 5;
-  const int col = lane & 31;
-
-  // All blocks of a head run on one XCD (its q, k, v, dO stay in that L2); the
-  // blocks with the most tiles start first.
-  const int xcd = blockIdx.x & 7;
-  const int slot = blockIdx.x >> 3;
-  const int bh = xcd + 8 * (slot % a.head_groups);
-  const int idx = slot / a.head_groups;
-  const int own_block = kKeysOwn ? idx : a.own_blocks - 1 - idx;
-  if (bh >= a.batch_heads) return; // the whole block
-  const int b = bh / a.heads;
-  const int hd = bh - b * a.heads;
-  const int S = a.S;
-  const int own0 = own_block * kOwnPerBlock;
-  const int wave_own0 = own0 + 32 * wave;
-  const int own = wave_own0 + col;
-  const int window = HAS_WINDOW ? a.window : 0;
-
-  auto slice = [&](const void *p, const Strides3 &st) {
-    return static_cast<const T *>(p) + b * st.b + hd * st.h;
-  };
-  auto bound = [&](const T *p, const Strides3 &st) {
-    // rows at or past S fall outside the descriptor and read as zeros
-    return make_rsrc(p, (uint32_t)(((int64_t)(S - 1) * st.s + D) * sizeof(T)));
-  };
-  // Own1 / Own2: B operands of T1 / T2. Other1 / Other2: their A operands.
-  // OtherS / OtherP: what the dS / P products contract with.
-  const Strides3 &st_own1 = kKeysOwn ? a.sk : a.sq;
-  const Strides3 &st_own2 = kKeysOwn ? a.sv : a.sdo;
-  const Strides3 &st_o1 = kKeysOwn ? a.sq : a.sk;
-  const Strides3 &st_o2 = kKeysOwn ? a.sdo : a.sv;
-  const BufRsrc own1_rs = bound(slice(kKeysOwn ? a.k : a.q, st_own1), st_own1);
-  const BufRsrc own2_rs = bound(slice(kKeysOwn ? a.v : a.dout, st_own2), st_own2);
-  const BufRsrc o1_rs = bound(slice(kKeysOwn ? a.q : a.k, st_o1), st_o1);
-  const BufRsrc o2_rs = bound(slice(kKeysOwn ? a.dout : a.v, st_o2), st_o2);
-  const uint32_t own1_row = (uint32_t)st_own1.s * sizeof(T);
-  const uint32_t own2_row = (uint32_t)st_own2.s * sizeof(T);
-  const uint32_t o1_row = (uint32_t)st_o1.s * sizeof(T);
-  const uint32_t o2_row = (uint32_t)st_o2.s * sizeof(T);
-
-  // B operands of the own positions: lane (position, half) holds features
-  // 16 s + 8 half .. + 7 of its position
-  Frag own1[kOwn1InLds ? 1 : kSteps];
-  Frag own2[kNeedT2 ? kSteps : 1];
-  u32x4 *own1_mine = own1_lds + wave * kSteps * kWave + lane;
-  {
-    u32x4 tmp[kSteps];
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s)
-      tmp[s] = __builtin_amdgcn_raw_buffer_load_b128(
-          own1_rs, (uint32_t)own * own1_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0);
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
-      if constexpr (kOwn1InLds) own1_mine[s * kWave] = tmp[s];
-      else own1[s] = __builtin_bit_cast(Frag, tmp[s]);
-    }
-  }
-  if constexpr (kNeedT2) {
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s)
-      own2[s] = __builtin_bit_cast(
-          Frag, __builtin_amdgcn_raw_buffer_load_b128(
-                    own2_rs, (uint32_t)own * own2_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0));
-  }
-
-  // Per-lane values of the own position: for a query its log-sum-exp and
-  // delta, for a key its padding value (log2 units).
-  const int64_t stat_row = (int64_t)bh * S;
-  float own_lse = 0.f, own_delta = 0.f, own_pad = 0.f;
-  if constexpr (!kKeysOwn) {
-    if (own < S) {
-      own_lse = a.lse[stat_row + own];
-      own_delta = a.delta[stat_row + own];
-    }
-  } else if constexpr (HAS_PAD) {
-    if (own < S) own_pad = fmaxf(a.pad[(int64_t)b * S + own] * kLog2eB, kMaskFloorLog2);
-  }
-
-  // Per-position values of a tile of the other kind travel with the tile: for
-  // keys the padding value (row_a), for queries log-sum-exp (row_a) and delta
-  // (row_b). Positions at or past S read as zeros, which is harmless: their
-  // q and dO rows (or k and v rows) are zeros too and a key past the end is
-  // behind the causal mask of every query.
-  const BufRsrc ra_rs = kKeysOwn ? make_rsrc(a.lse + stat_row, (uint32_t)S * 4u)
-                                 : make_rsrc(HAS_PAD ? a.pad + (int64_t)b * S : nullptr,
-                                             HAS_PAD ? (uint32_t)S * 4u : 0u);
-  const BufRsrc rb_rs = make_rsrc(kKeysOwn ? a.delta + stat_row : nullptr, kKeysOwn ? (uint32_t)S * 4u : 0u);
-  constexpr bool kRowA = kKeysOwn || HAS_PAD;
-
-  const int n_ch = tid % kChunks, n_r0 = tid / kChunks;
-  const bool t_task = tid < kTasks;
-  const int t_g = tid % kChunks, t_kg = tid / kChunks;
-  u32x4 n1reg[kLoadsN], n2reg[kNeedT2 ? kLoadsN : 1], tsreg[kAccS ? 8 : 1], tpreg[kAccP ? 8 : 1];
-  float4 rareg = make_float4(0.f, 0.f, 0.f, 0.f), rbreg = rareg;
-
-  auto issue_loads = [&](int pos0) {
-    if (tid < kTile / 4) {
-      // S % 4 may be non-zero only without a padding mask, and lse / delta are
-      // allocated by the caller for whole rows: the 16-byte loads stay aligned
-      // because S rows start at multiples of S floats only when S % 4 == 0;
-      // otherwise take the values one by one
-      if constexpr (kRowA) {
-        if ((S & 3) == 0) {
-          rareg = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                 ra_rs, (uint32_t)(pos0 + 4 * tid) * 4u, 0, 0));
-        } else {
-          rareg.x = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ra_rs, (uint32_t)(pos0 + 4 * tid) * 4u, 0, 0));
-          rareg.y = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ra_rs, (uint32_t)(pos0 + 4 * tid + 1) * 4u, 0, 0));
-          rareg.z = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ra_rs, (uint32_t)(pos0 + 4 * tid + 2) * 4u, 0, 0));
-          rareg.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ra_rs, (uint32_t)(pos0 + 4 * tid + 3) * 4u, 0, 0));
-        }
-      }
-      if constexpr (kKeysOwn) {
-        if ((S & 3) == 0) {
-          rbreg = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                 rb_rs, (uint32_t)(pos0 + 4 * tid) * 4u, 0, 0));
-        } else {
-          rbreg.x = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb_rs, (uint32_t)(pos0 + 4 * tid) * 4u, 0, 0));
-          rbreg.y = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb_rs, (uint32_t)(pos0 + 4 * tid + 1) * 4u, 0, 0));
-          rbreg.z = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb_rs, (uint32_t)(pos0 + 4 * tid + 2) * 4u, 0, 0));
-          rbreg.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb_rs, (uint32_t)(pos0 + 4 * tid + 3) * 4u, 0, 0));
-        }
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < kLoadsN; ++j) {
-      const uint32_t row = (uint32_t)(pos0 + n_r0 + j * kRowsPerPass);
-      n1reg[j] = __builtin_amdgcn_raw_buffer_load_b128(o1_rs, row * o1_row + (uint32_t)n_ch * 16u, 0, 0);
-      if constexpr (kNeedT2)
-        n2reg[j] = __builtin_amdgcn_raw_buffer_load_b128(o2_rs, row * o2_row + (uint32_t)n_ch * 16u, 0, 0);
-    }
-    if (t_task) {
-      // a task: the 8 positions of contraction chunk t_kg (positions
-      // 16 u + 8 jj + 4 h + t for chunk 2 u + h) x 8 features
-      const int pbase = pos0 + 16 * (t_kg >> 1) + 4 * (t_kg & 1);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const uint32_t row = (uint32_t)(pbase + 8 * (i >> 2) + (i & 3));
-        // the dS product contracts with Other1's tensor (K or Q), the P
-        // product with Other2's (dO)
-        if constexpr (kAccS)
-          tsreg[i] = __builtin_amdgcn_raw_buffer_load_b128(o1_rs, row * o1_row + (uint32_t)t_g * 16u, 0, 0);
-        if constexpr (kAccP)
-          tpreg[i] = __builtin_amdgcn_raw_buffer_load_b128(o2_rs, row * o2_row + (uint32_t)t_g * 16u, 0, 0);
-      }
-    }
-  };
-  auto transpose_into = [&](T *dst, const u32x4 (&src)[8]) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) { // 8 x 8 transposition of 16-bit values
-      u32x4 tr;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const uint32_t lo = src[2 * w][e >> 1], hi = src[2 * w + 1][e >> 1];
-        tr[w] = (e & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
-      }
-      const int d = 8 * t_g + e;
-      *reinterpret_cast<u32x4 *>(&dst[(d * kTChunks + ((t_kg + e + t_g) & (kTChunks - 1))) * 8]) = tr;
-    }
-  };
-  auto store_tile = [&]() {
-    if (tid < kTile / 4) {
-      if constexpr (kKeysOwn) {
-        *reinterpret_cast<float4 *>(&row_a[4 * tid]) = rareg;
-        *reinterpret_cast<float4 *>(&row_b[4 * tid]) = rbreg;
-      } else if constexpr (HAS_PAD) {
-        *reinterpret_cast<float4 *>(&row_a[4 * tid]) = make_float4(
-            fmaxf(rareg.x * kLog2eB, kMaskFloorLog2), fmaxf(rareg.y * kLog2eB, kMaskFloorLog2),
-            fmaxf(rareg.z * kLog2eB, kMaskFloorLog2), fmaxf(rareg.w * kLog2eB, kMaskFloorLog2));
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < kLoadsN; ++j) {
-      const int row = n_r0 + j * kRowsPerPass;
-      const int at = (row * kChunks + (n_ch ^ (row & kSwizzleN))) * 8;
-      *reinterpret_cast<u32x4 *>(&o1_lds[at]) = n1reg[j];
-      if constexpr (kNeedT2) *reinterpret_cast<u32x4 *>(&o2_lds[at]) = n2reg[j];
-    }
-    if (t_task) {
-      if constexpr (kAccS) transpose_into(ts_lds, tsreg);
-      if constexpr (kAccP) transpose_into(tp_lds, tpreg);
-    }
-  };
-
-  f32x16 acc_s[kAccS ? kBlocksD : 1], acc_p[kAccP ? kBlocksD : 1];
-#pragma unroll
-  for (int i = 0; i < (kAccS ? kBlocksD : 1); ++i)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc_s[i][r] = 0.f;
-#pragma unroll
-  for (int i = 0; i < (kAccP ? kBlocksD : 1); ++i)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc_p[i][r] = 0.f;
-
-  // Tiles of the other kind this block walks.
-  int first_tile, tiles;
-  if constexpr (!kKeysOwn) {
-    const int last_key = (own0 + kOwnPerBlock < S ? own0 + kOwnPerBlock : S) - 1;
-    tiles = last_key / kTile + 1;
-    first_tile = HAS_WINDOW && own0 - window + 1 > 0 ? (own0 - window + 1) / kTile : 0;
-  } else {
-    first_tile = own0 / kTile;
-    int last_q = S - 1;
-    if (HAS_WINDOW && own0 + kOwnPerBlock - 1 + window - 1 < last_q) last_q = own0 + kOwnPerBlock - 1 + window - 1;
-    tiles = last_q / kTile + 1;
-  }
-
-  // One step: 32 positions of the other kind against the wave's 32 own ones.
-  auto step = [&](int pos0, int kb) {
-    const int ob = pos0 + 32 * kb;
-    bool diagonal;
-    if constexpr (!kKeysOwn) { // other = keys ob .. ob+31, own = queries
-      if (ob > wave_own0 + 31) return;                                  // every key is ahead of the wave's queries
-      if (HAS_WINDOW && ob + 31 <= wave_own0 - window) return;          // or behind their windows
-      diagonal = ob + 31 > wave_own0 || (HAS_WINDOW && ob <= wave_own0 + 31 - window);
-    } else { // other = queries ob .. ob+31, own = keys
-      if (ob + 31 < wave_own0) return;                                  // every query is before the wave's keys
-      if (HAS_WINDOW && ob >= wave_own0 + 31 + window) return;          // or past their windows
-      diagonal = ob < wave_own0 + 31 || (HAS_WINDOW && ob + 31 >= wave_own0 + window);
-    }
-
-    f32x16 t1, t2;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) t1[r] = t2[r] = 0.f;
-    const int orow = 32 * kb + col;
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
-      const int at = (orow * kChunks + ((2 * s + half) ^ (orow & kSwizzleN))) * 8;
-      const Frag f1 = *reinterpret_cast<const Frag *>(&o1_lds[at]);
-      if constexpr (kOwn1InLds)
-        t1 = Op::run(f1, __builtin_bit_cast(Frag, own1_mine[s * kWave]), t1);
-      else
-        t1 = Op::run(f1, own1[s], t1);
-      if constexpr (kNeedT2) {
-        const Frag f2 = *reinterpret_cast<const Frag *>(&o2_lds[at]);
-        t2 = Op::run(f2, own2[s], t2);
-      }
-    }
-
-    // P = exp2(scale*log2e * T1 + pad - lse); dS = scale * P * (T2 - delta)
-    float p[16], dl[16]; // the probabilities; delta of each register's query
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float ra[4] = {0.f, 0.f, 0.f, 0.f}, rb[4] = {0.f, 0.f, 0.f, 0.f};
-      if constexpr (kRowA) {
-        const float4 v4 = *reinterpret_cast<const float4 *>(&row_a[32 * kb + 8 * j + 4 * half]);
-        ra[0] = v4.x, ra[1] = v4.y, ra[2] = v4.z, ra[3] = v4.w;
-      }
-      if constexpr (kKeysOwn) {
-        const float4 v4 = *reinterpret_cast<const float4 *>(&row_b[32 * kb + 8 * j + 4 * half]);
-        rb[0] = v4.x, rb[1] = v4.y, rb[2] = v4.z, rb[3] = v4.w;
-      }
-#pragma unroll
-      for (int tt = 0; tt < 4; ++tt) {
-        const int r = 4 * j + tt;
-        // keys own: pad of the lane, lse and delta of the row; queries own: the reverse
-        const float shift = kKeysOwn ? own_pad - ra[tt] : ra[tt] - own_lse;
-        p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(t1[r], a.scale_log2e, shift));
-        dl[r] = kKeysOwn ? rb[tt] : own_delta;
-      }
-    }
-    if (diagonal) {
-      asm volatile(""); // a branch of its own: only the tiles at the diagonal (and the window's edge) compare
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int other = ob + 8 * (r >> 2) + 4 * half + (r & 3);
-        const int key = kKeysOwn ? own : other, query = kKeysOwn ? other : own;
-        const bool visible = key <= query && (!HAS_WINDOW || key > query - window);
-        p[r] = visible ? p[r] : 0.f;
-      }
-    }
-    // With attention dropout the forward multiplied V with keep * P / (1-p): the
-    // P product takes the kept probabilities (1/(1-p) goes onto dV at the end),
-    // and the gradient of the dropped-out probabilities is keep * dP / (1-p).
-    float pk[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) pk[r] = p[r];
-    if constexpr (DROP) {
-      stage_keep_bits(keep_lds[wave], a.drop, bh, S, kKeysOwn ? ob : wave_own0, kKeysOwn ? wave_own0 : ob, lane);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        u32x4 words;
-        uint32_t bits = 0;
-        if constexpr (kKeysOwn) words = keep_words_key_lane(keep_lds[wave], j, half);
-        else bits = keep_word_query_lane(keep_lds[wave], col) >> (8 * j + 4 * half);
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-          const int r = 4 * j + tt;
-          const bool keep = kKeysOwn ? ((words[tt] >> col) & 1u) != 0 : ((bits >> tt) & 1u) != 0;
-          pk[r] = keep ? p[r] : 0.f;
-          if constexpr (kNeedT2) t2[r] = keep ? t2[r] * a.drop.keep_scale : 0.f;
-        }
-      }
-    }
-    Frag pf[2], sf[2];
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        pf[u][i] = static_cast<T>(pk[8 * u + i]);
-        if constexpr (kNeedT2)
-          sf[u][i] = static_cast<T>(a.scale * (p[8 * u + i] * (t2[8 * u + i] - dl[8 * u + i])));
-      }
-
-    // Acc^T += OtherT x X, 16 positions of the step at a time
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-#pragma unroll
-      for (int i = 0; i < kBlocksD; ++i) {
-        const int d = 32 * i + col;
-        const int at = (d * kTChunks + ((4 * kb + 2 * u + half + d + (d >> 3)) & (kTChunks - 1))) * 8;
-        if constexpr (kAccS)
-          acc_s[i] = Op::run(*reinterpret_cast<const Frag *>(&ts_lds[at]), sf[u], acc_s[i]);
-        if constexpr (kAccP)
-          acc_p[i] = Op::run(*reinterpret_cast<const Frag *>(&tp_lds[at]), pf[u], acc_p[i]);
-      }
-    }
-  };
-
-  issue_loads(first_tile * kTile);
-  for (int t = first_tile; t < tiles; ++t) {
-    const int pos0 = t * kTile;
-    __syncthreads(); // the reads of the previous tile are done
-    store_tile();
-    __syncthreads();
-    if (t + 1 < tiles) issue_loads(pos0 + kTile);
-#pragma unroll
-    for (int kb = 0; kb < kStepsPerTile; ++kb) step(pos0, kb);
-  }
-
-  if (own >= S) return;
-  typedef T Out4 __attribute__((ext_vector_type(4)));
-  auto write = [&](void *base, const Strides3 &st, const f32x16 (&acc)[kBlocksD], float factor) {
-    T *op = static_cast<T *>(base) + b * st.b + hd * st.h + (int64_t)own * st.s;
-#pragma unroll
-    for (int i = 0; i < kBlocksD; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        Out4 w;
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(acc[i][4 * j + tt] * factor);
-        *reinterpret_cast<Out4 *>(op + 32 * i + 8 * j + 4 * half) = w;
-      }
-  };
-  if constexpr (ROLE == kRoleDQ) write(a.dq, a.sdq, acc_s, 1.0f);
-  if constexpr (ROLE == kRoleDKV || ROLE == kRoleDK) write(a.dk, a.sdk, acc_s, 1.0f);
-  if constexpr (ROLE == kRoleDKV || ROLE == kRoleDV) write(a.dv, a.sdv, acc_p, DROP ? a.drop.keep_scale : 1.0f);
-}
-
-// ---------------------------------------------------------------------------
-// The same gradients without a sliding window, the way the forward is built: tiles of 32 positions of the other
-// kind loaded straight into LDS (four buffers per tensor), stored as they are
-// in memory, read as A operands of the score-like products 16 bytes per lane
-// and as A operands of the accumulating product through the transposing read
-// (no transposed copy, no staging through registers); a tile's code ordered by
-// hand: the products of T1, those of T2, then the accumulating products of the
-// previous tile with this tile's probabilities and score gradients worked out
-// between them. One permutation of a row's 16-byte chunks serves both reads
-// (f(row) below). dK and dV take a pass each at every head size.
-// ---------------------------------------------------------------------------
-
 constexpr int kSchedTile = 32;
 constexpr int kSchedBuffers = 4;
 
@@ -489,8 +75,8 @@ constexpr unsigned sched_lds_bytes() {
          kWavesPerBlock * 32u * sizeof(uint32_t);
 }
 
-template <typename T, int D, int ROLE, bool HAS_PAD, bool DROP>
-__global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) void attention_bwd_scheduled_kernel(
+template <typename T, int D, int ROLE, bool HAS_PAD, bool HAS_WINDOW, bool DROP>
+__global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) void attention_bwd_kernel(
     const BwdArgs a) {
   static_assert(ROLE == kRoleDQ || ROLE == kRoleDK || ROLE == kRoleDV, "one gradient per pass");
   using Op = MatrixOp<T>;
@@ -579,19 +165,34 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     if (own < S) own_pad = fmaxf(a.pad[(int64_t)b * S + own] * kLog2eB, kMaskFloorLog2);
   }
 
-  // Tiles of the other kind this block walks; those the causal boundary
-  // crosses: for queries the last four, for keys the first four.
-  int first_tile, tiles, boundary_from, boundary_to;
+  // Tiles [first_tile, tiles) of the other kind this block walks. Those before
+  // masked_until and those from plain_until on may hold pairs that are not
+  // visible; the tiles between them are visible in full to every own position.
+  // Own queries: the causal boundary crosses the last four tiles, the edges of
+  // the queries' windows the first ones. Own keys: the boundary crosses the
+  // first four; a window ends the walk at the last query that sees the block's
+  // last key, and its edge crosses the tiles from the first query that no
+  // longer sees the block's first key on.
+  const int window = HAS_WINDOW ? a.window : 0;
+  int first_tile, tiles, masked_until, plain_until;
   if constexpr (!kKeysOwn) {
     const int last_key = (own0 + kOwnPerBlock < S ? own0 + kOwnPerBlock : S) - 1;
     tiles = last_key / kSchedTile + 1;
-    first_tile = 0;
-    boundary_from = own0 / kSchedTile, boundary_to = tiles;
+    first_tile = HAS_WINDOW && own0 - window + 1 > 0 ? (own0 - window + 1) / kSchedTile : 0;
+    masked_until = HAS_WINDOW && own0 + kOwnPerBlock - window > 0
+                       ? (own0 + kOwnPerBlock - window + kSchedTile - 1) / kSchedTile
+                       : 0;
+    plain_until = own0 / kSchedTile;
   } else {
     first_tile = own0 / kSchedTile;
-    tiles = (S - 1) / kSchedTile + 1;
-    boundary_from = first_tile, boundary_to = first_tile + kOwnPerBlock / kSchedTile;
+    int last_query = S - 1;
+    if (HAS_WINDOW && own0 + kOwnPerBlock - 1 + window - 1 < last_query) last_query = own0 + kOwnPerBlock - 1 + window - 1;
+    tiles = last_query / kSchedTile + 1;
+    masked_until = first_tile + kOwnPerBlock / kSchedTile;
+    plain_until = HAS_WINDOW ? (own0 + window) / kSchedTile : tiles;
   }
+  if (masked_until > tiles) masked_until = tiles;
+  if (plain_until > tiles) plain_until = tiles;
 
   // The permutation of a row's chunks: chunk c of row r lies at c ^ f(r). The
   // 16 lanes that read 16 consecutive rows at one chunk (natural operands) must
@@ -738,7 +339,8 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
       float p = __builtin_amdgcn_exp2f(__builtin_fmaf(t1[r], a.scale_log2e, shift));
       if constexpr (MASKED) {
         const int other = t * kSchedTile + rr;
-        const bool visible = kKeysOwn ? own <= other : other <= own;
+        const bool visible = kKeysOwn ? own <= other && (!HAS_WINDOW || other - window < own)
+                                      : other <= own && (!HAS_WINDOW || other > own - window);
         p = visible ? p : 0.f;
       }
       float grad = t2[r];
@@ -847,13 +449,9 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
       scheduled_tile.template operator()<MASKED>();
     }
   };
-  if constexpr (!kKeysOwn) {
-    run_tiles.template operator()<false>(boundary_from < tiles ? boundary_from : tiles);
-    run_tiles.template operator()<true>(tiles);
-  } else {
-    run_tiles.template operator()<true>(boundary_to < tiles ? boundary_to : tiles);
-    run_tiles.template operator()<false>(tiles);
-  }
+  if constexpr (kKeysOwn || HAS_WINDOW) run_tiles.template operator()<true>(masked_until);
+  run_tiles.template operator()<false>(plain_until);
+  if constexpr (!kKeysOwn || HAS_WINDOW) run_tiles.template operator()<true>(tiles);
   // the last tile's accumulating products
   wait_vm<0>(); // (nothing may still be on its way into LDS when the block ends)
   __syncthreads();
@@ -882,11 +480,12 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
 }
 
 template <typename T, int D, int ROLE>
-int launch_scheduled_role(const BwdArgs &a, hipStream_t stream) {
+int launch_role(const BwdArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)(8 * a.head_groups * a.own_blocks));
   constexpr unsigned kLds = sched_lds_bytes<T, D, ROLE>();
   auto go = [&]<bool HAS_PAD, bool DROP>() -> int {
-    auto *kernel = attention_bwd_scheduled_kernel<T, D, ROLE, HAS_PAD, DROP>;
+    auto *kernel = a.window > 0 ? attention_bwd_kernel<T, D, ROLE, HAS_PAD, true, DROP>
+                                : attention_bwd_kernel<T, D, ROLE, HAS_PAD, false, DROP>;
     if (kLds > 64u * 1024u) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
@@ -929,31 +528,6 @@ __global__ __launch_bounds__(kBlockThreads) void attention_delta_kernel(
   if (live && part == 0) delta[row] = s;
 }
 
-template <typename T, int D, int ROLE>
-int launch_role(const BwdArgs &a, hipStream_t stream) {
-  const dim3 grid((unsigned)(8 * a.head_groups * a.own_blocks));
-  constexpr unsigned kLds = bwd_lds_bytes<T, D, ROLE>();
-  auto go = [&]<bool HAS_PAD, bool HAS_WINDOW>() -> int {
-    auto *kernel = a.drop.drop ? attention_bwd_kernel<T, D, ROLE, HAS_PAD, HAS_WINDOW, true>
-                               : attention_bwd_kernel<T, D, ROLE, HAS_PAD, HAS_WINDOW, false>;
-    if (kLds > 48 * 1024) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
-      if (e != hipSuccess)
-        return fail(OSLO_E_LAUNCH, "oslo_attention_prefill_bwd: %u bytes of dynamic LDS refused: %s", kLds,
-                    hipGetErrorString(e));
-    }
-    kernel<<<grid, dim3(kBlockThreads), kLds, stream>>>(a);
-    return check_launch("attention_prefill_bwd");
-  };
-  if (a.window > 0) {
-    if (a.pad != nullptr) return go.template operator()<true, true>();
-    return go.template operator()<false, true>();
-  }
-  if (a.pad != nullptr) return go.template operator()<true, false>();
-  return go.template operator()<false, false>();
-}
-
 template <typename T, int D>
 int launch_bwd_dim(const BwdArgs &a, float *delta, const void *out, const Strides3 &so,
                    hipStream_t stream) {
@@ -963,25 +537,12 @@ int launch_bwd_dim(const BwdArgs &a, float *delta, const void *out, const Stride
       delta, static_cast<const T *>(out), static_cast<const T *>(a.dout), so, a.sdo, a.S, a.heads, rows);
   int s = check_launch("attention_prefill_bwd(delta)");
   if (s != OSLO_OK) return s;
-  if (a.window == 0) {
-    // no sliding window: the hand-ordered kernel, a pass per gradient
-    s = launch_scheduled_role<T, D, kRoleDQ>(a, stream);
-    if (s != OSLO_OK) return s;
-    s = launch_scheduled_role<T, D, kRoleDK>(a, stream);
-    if (s != OSLO_OK) return s;
-    return launch_scheduled_role<T, D, kRoleDV>(a, stream);
-  }
+  // a pass per gradient
   s = launch_role<T, D, kRoleDQ>(a, stream);
   if (s != OSLO_OK) return s;
-  if constexpr (D == 256) {
-    // two accumulators of 128 registers per lane do not fit beside the
-    // operands: dK and dV take a pass each
-    s = launch_role<T, D, kRoleDK>(a, stream);
-    if (s != OSLO_OK) return s;
-    return launch_role<T, D, kRoleDV>(a, stream);
-  } else {
-    return launch_role<T, D, kRoleDKV>(a, stream);
-  }
+  s = launch_role<T, D, kRoleDK>(a, stream);
+  if (s != OSLO_OK) return s;
+  return launch_role<T, D, kRoleDV>(a, stream);
 }
 
 template <typename T>
