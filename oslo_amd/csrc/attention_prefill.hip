@@ -134,22 +134,16 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   const T *qp = static_cast<const T *>(a.q) + b * a.q_b + hd * a.q_h;
   const T *kp = static_cast<const T *>(a.k) + b * a.k_b + hd * a.k_h;
   const T *vp = static_cast<const T *>(a.v) + b * a.v_b + hd * a.v_h;
-  // rows at or past S fall outside the descriptors and read as zeros
-  const BufRsrc qrs = make_rsrc(qp, (uint32_t)(((int64_t)(S - 1) * a.q_s + D) * sizeof(T)));
+  // (rows at or past S fall outside the descriptors and read as zeros)
   const uint32_t q_row = (uint32_t)a.q_s * sizeof(T);
   const uint32_t k_row = (uint32_t)a.k_s * sizeof(T);
   const uint32_t v_row = (uint32_t)a.v_s * sizeof(T);
 
   // Q^T as B operands, in registers for the whole kernel: lane (query, half)
-  // holds features 16 s + 8 half .. + 7
+  // holds features 16 s + 8 half .. + 7 (loaded in the prologue, by way of LDS)
   const int wave_q0 = q0 + 32 * wave;
   const int qrow = wave_q0 + col;
   Frag qf[kSteps];
-#pragma unroll
-  for (int s = 0; s < kSteps; ++s)
-    qf[s] = __builtin_bit_cast(
-        Frag, __builtin_amdgcn_raw_buffer_load_b128(
-                  qrs, (uint32_t)qrow * q_row + (uint32_t)(16 * s + 8 * half) * sizeof(T), 0, 0));
 
   const float *padr = HAS_PAD ? a.pad + (int64_t)b * S : nullptr;
   const int window = HAS_WINDOW ? a.window : 0;
@@ -454,7 +448,26 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   // prologue: K of the first two tiles and V of the first on their way, all
   // issued before any is waited for (the sources then stand at tile t + 2 and
   // t + 1, where a tile's staging expects them)
+  // The block's queries come first. A lane's operands of Q^T are 16 bytes from
+  // each chunk pair of its own row: loaded straight from memory, every lane of
+  // a load touches a cache line of its own. The 128 rows go into LDS the way
+  // four tiles of K do, whole rows at a time (into the third buffer of K and
+  // the three of V, which lie one behind the other and are not in use yet),
+  // and each wave reads its tile from there like a tile of K. V of the first
+  // tile is loaded once every wave has its operands.
   {
+    TileStream q_src;
+    q_src.start(qp, (uint32_t)(((int64_t)(S - 1) * a.q_s + D) * sizeof(T)), q_row, kQueriesPerBlock, qb, a.query_blocks);
+    const u32x4 qd = q_src.descriptor();
+#pragma unroll
+    for (int j = 0; j < kQueriesPerBlock / kKeysPerTile; ++j)
+#pragma unroll
+      for (int it = 0; it < kLoadsK; ++it) {
+        const int sigma = (4 * it + wave) * kWave + lane;
+        const int row = sigma / kChunks, at = sigma % kChunks;
+        load_to_lds(qd, k_lds + (2 + j) * kTile + (4 * it + wave) * (kWave * 8),
+                    (uint32_t)(kKeysPerTile * j + row) * q_row + (uint32_t)(at ^ ((row >> kKeyShift) & kSwizzleK)) * 16u);
+      }
 #pragma unroll
     for (int it = 0; it < kLoadsK; ++it) stage_item(it, k_buffer(0), nullptr);
     if constexpr (HAS_PAD) { // the mask values of the first tile, then (as the staging of a tile expects) of the second
@@ -466,7 +479,14 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
       pad_at[2] = p2;
     }
 #pragma unroll
-    for (int it = 0; it < 2 * kLoadsK; ++it) stage_item(it, k_buffer(1), v_buffer(0));
+    for (int it = 0; it < kLoadsK; ++it) stage_item(it, k_buffer(1), nullptr);
+    wait_loads.template operator()<0>();
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) qf[s] = read_k(k_lds + (2 + wave) * kTile, s);
+    __syncthreads(); // (also: K of the first tile is in LDS)
+#pragma unroll
+    for (int it = kLoadsK; it < 2 * kLoadsK; ++it) stage_item(it, nullptr, v_buffer(0));
   }
 
   // A tile as one straight run of code, its order fixed by hand (the fences
@@ -565,8 +585,6 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   };
 
   { // the block's first tile (the causal boundary, or the window's edge, may cross it)
-    wait_loads.template operator()<0>();
-    __syncthreads();
     float mt, sum;
     scheduled_tile.template operator()<true, true>(t, mt, sum, pf);
     l = sum;
@@ -618,10 +636,15 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
 
   l = halves_sum(l);
   const float inv = DROP ? a.drop.keep_scale / l : 1.0f / l;
-  if (qrow >= S) return;
-  if (a.lse != nullptr && half == 0)
+  if (a.lse != nullptr && half == 0 && qrow < S)
     a.lse[(int64_t)bh * S + qrow] = m + __builtin_amdgcn_logf(l); // v_log_f32 is log2
-  T *op = static_cast<T *>(a.out) + b * a.o_b + hd * a.o_h + (int64_t)qrow * a.o_s;
+  // O^T leaves through LDS: a lane holds 4 features of its query at a time, and
+  // the queries' rows lie far apart in memory; the wave puts its 32 x D tile
+  // into LDS (once every wave is done with K and V), rows padded by 16 bytes,
+  // and stores whole rows, 16 bytes a lane.
+  __syncthreads();
+  constexpr int kOutRow = kRowBytes + 16;
+  char *const stage = reinterpret_cast<char *>(k_lds) + wave * (32 * kOutRow);
   typedef T Out4 __attribute__((ext_vector_type(4)));
 #pragma unroll
   for (int i = 0; i < kBlocksD; ++i)
@@ -630,8 +653,20 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
       Out4 w;
 #pragma unroll
       for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(o[i][4 * j + tt] * inv);
-      *reinterpret_cast<Out4 *>(op + 32 * i + 8 * j + 4 * half) = w;
+      *reinterpret_cast<Out4 *>(stage + col * kOutRow + (32 * i + 8 * j + 4 * half) * (int)sizeof(T)) = w;
     }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  T *const out_head = static_cast<T *>(a.out) + b * a.o_b + hd * a.o_h;
+  constexpr int kRowsPerStore = kWave / kChunks;
+#pragma unroll
+  for (int k = 0; k < 32 / kRowsPerStore; ++k) {
+    const int row = kRowsPerStore * k + lane / kChunks, piece = lane % kChunks;
+    const u32x4 w = *reinterpret_cast<const u32x4 *>(stage + row * kOutRow + piece * 16);
+    if (wave_q0 + row < S)
+      *reinterpret_cast<u32x4 *>(out_head + (int64_t)(wave_q0 + row) * a.o_s + 8 * piece) = w;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -1146,9 +1181,10 @@ int launch_prefill_dim(const PrefillArgs &a, hipStream_t stream) {
     };
     if (a.pad != nullptr) return pair.template operator()<true>();
     return pair.template operator()<false>();
+  } else {
+    if (a.pad != nullptr) return go.template operator()<true, false>();
+    return go.template operator()<false, false>();
   }
-  if (a.pad != nullptr) return go.template operator()<true, false>();
-  return go.template operator()<false, false>();
 }
 
 template <typename T>
