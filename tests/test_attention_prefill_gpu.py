@@ -145,6 +145,28 @@ def test_prefill_scores_that_keep_rising(d, dtype):
         check(out, device_reference(q, k, v, 16.0), dtype, ("slope", d))
 
 
+@pytest.mark.parametrize("dtype", HALVES, ids=IDS.get)
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_prefill_isolated_large_scores(d, dtype):
+    """A few queries score far above their running maximum at a few scattered
+    keys, the others never: the reference maximum has to rise for single lanes
+    of single waves in the middle of a block (where the tiles otherwise run
+    without looking at the maxima), with and without a padding mask."""
+    b, h, s = 2, 3, 900
+    q, k, v = (randn((b, h, s, d), dtype, seed=7 * d + i) for i in range(3))
+    q, k = q * 0.5, k * 0.5
+    rows = torch.arange(s)[torch.arange(s) % 37 == 5]
+    q[:, :, rows] += 3.0
+    for j, key in enumerate((70, 200, 333, 515, 640, 801)):
+        k[:, (j % h):, key] += 1.0 + j  # q.k rises by 3 (1 + j) d, times the scale
+    q, k, v = q.to(DEV), k.to(DEV), v.to(DEV)
+    pad = padding(b, s, d).to(DEV)
+    for p in (None, pad):
+        out = kernels.attention_prefill_forward(q, k, v, d ** -0.5, p)
+        assert torch.isfinite(out).all()
+        check(out, device_reference(q, k, v, d ** -0.5, p), dtype, ("isolated", d, p is not None), vmax=5.0)
+
+
 def test_prefill_full_size_properties():
     """The GPT-J shape of the benchmark, [8, 16, 2048, 256] bf16, where the oracle
     would take hours: the first row is the first value exactly, equal scores
