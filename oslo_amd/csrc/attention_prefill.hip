@@ -669,478 +669,6 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   }
 }
 
-// ---------------------------------------------------------------------------
-// head_dim 256 without a sliding window: two waves per 32 queries, 8 waves a
-// block. With one wave per query the kernel above holds 128 accumulators of
-// O^T and 64 registers of Q^T per lane, which leaves one wave per SIMD: the
-// matrix core idles whenever that wave issues anything else. Here the two
-// waves of a pair split a step of 64 keys between them for S^T and the
-// softmax (32 keys each, all 256 features of Q^T), hand each other their P^T
-// through LDS, and split the features of O^T for the second product (128 rows
-// each over all 64 keys): the same matrix products and LDS reads in total, 64
-// accumulators per lane, two waves per SIMD.
-//   step t, every wave:   barrier (K of step t, V of step t - 1 and the
-//   partner's P^T of step t - 1 are in LDS) - the partner's P^T into registers
-//   and a word into LDS that says so - the products of S^T with the loads of
-//   the next step (K) and of this one (V) between them - the products of O^T of
-//   step t - 1 with the softmax of step t between them - P^T of step t into
-//   LDS, once the partner's word says that it has taken the one before, and
-//   the wave's flag.
-// One barrier per step: the waves of a SIMD drift apart between barriers (the
-// older one is served first), so that one is at its products of S^T, which
-// are all it issues then, while the other does its softmax.
-// Both waves of a pair keep the same reference maximum per query: it only
-// moves in a general step (the first of a block, and whenever some wave of the
-// block flags a lane sum above kSumLimit: then the whole block does that step
-// again the general way, since barriers are the block's), where the waves
-// exchange their maxima through LDS.
-// ---------------------------------------------------------------------------
-constexpr int kPairThreads = 512;
-constexpr int kPairWaves = kPairThreads / kWave;
-constexpr int kPairKeys = 64;              // keys per step: 32 per wave of a pair
-constexpr int kPairPadSlots = kPairThreads; // mask values of a step: the first 64 count, every wave loads 64
-
-template <typename T>
-constexpr unsigned pair_lds_bytes() {
-  return 2u * 2u * kPairKeys * 256u * sizeof(T)     // K and V, two buffers each
-         + kPairWaves * 2u * kWave * 16u             // a wave's P^T of a step, for its partner
-         + kPairWaves * 32u * sizeof(float)          // a wave's maxima or sums, for its partner
-         + 2u * kPairPadSlots * sizeof(float)        // mask values of two steps
-         + kPairWaves * 32u * sizeof(uint32_t)       // keep bits of a wave's tile
-         + 32u * sizeof(uint32_t);                   // the waves' flags (two sets) and acknowledgements
-}
-
-template <typename T, bool HAS_PAD, bool DROP>
-__global__ __launch_bounds__(kPairThreads, 1) void attention_prefill_pair_kernel(const PrefillArgs a) {
-  using Op = MatrixOp<T>;
-  using Frag = typename Op::Frag;
-  constexpr int D = 256;
-  constexpr int kChunks = D / 8;
-  constexpr int kSteps = D / 16;    // contraction steps of Q K^T
-  constexpr int kBlocksSide = D / 64; // 32-row blocks of a wave's half of O^T
-  constexpr int kProducts = 4 * kBlocksSide; // of O^T per step: four groups of 16 keys into every block
-  constexpr int kLoads = kPairKeys * kChunks / kPairThreads; // per thread, step and tensor
-  constexpr int kTile = kPairKeys * D;
-  constexpr int kRowBytes = D * (int)sizeof(T);
-  static_assert(kProducts == 16 && kSteps == 16, "one score register per product of O^T");
-  extern __shared__ __align__(1024) unsigned char lds_raw[];
-  T *const k_lds = reinterpret_cast<T *>(lds_raw); // [2][key][chunk ^ key % 16][8]
-  T *const v_lds = k_lds + 2 * kTile;              // [2][key][chunk ^ 2 (key % 4)][8]
-  u32x4 *const p_lds = reinterpret_cast<u32x4 *>(v_lds + 2 * kTile); // [wave][2][lane]
-  float *const stat_lds = reinterpret_cast<float *>(p_lds + kPairWaves * 2 * kWave); // [wave][query]
-  float *const pad_lds = stat_lds + kPairWaves * 32;                                 // [2][slot]
-  uint32_t *const keep_all = reinterpret_cast<uint32_t *>(pad_lds + 2 * kPairPadSlots);
-  uint32_t *const flag_lds = keep_all + kPairWaves * 32;
-  uint32_t *const ack_lds = flag_lds + 16; // (the flags of even and of odd steps are sets of their own) per wave: the last step whose P^T the wave has taken from its partner
-
-  const int tid = threadIdx.x;
-  const int lane = tid & (kWave - 1);
-  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int half = lane >> 5;
-  const int col = lane & 31;
-  const int pair = wave & 3;    // which 32 queries of the block
-  const int side = wave >> 2;   // which 32 keys of a step, which 128 features of O^T
-  const int partner = wave ^ 4;
-  uint32_t *const keep_lds = keep_all + 32 * wave;
-
-  const int xcd = blockIdx.x & 7;
-  const int slot = blockIdx.x >> 3;
-  const int bh = xcd + 8 * (slot % a.head_groups);
-  const int qb = a.query_blocks - 1 - slot / a.head_groups;
-  if (bh >= a.batch_heads) return; // the whole block
-  const int b = bh / a.heads;
-  const int hd = bh - b * a.heads;
-  const int S = a.S;
-  const int q0 = qb * kQueriesPerBlock;
-
-  const T *qp = static_cast<const T *>(a.q) + b * a.q_b + hd * a.q_h;
-  const T *kp = static_cast<const T *>(a.k) + b * a.k_b + hd * a.k_h;
-  const T *vp = static_cast<const T *>(a.v) + b * a.v_b + hd * a.v_h;
-  const uint32_t q_row = (uint32_t)a.q_s * sizeof(T);
-  const uint32_t k_row = (uint32_t)a.k_s * sizeof(T);
-  const uint32_t v_row = (uint32_t)a.v_s * sizeof(T);
-
-  const int wave_q0 = q0 + 32 * pair;
-  const int qrow = wave_q0 + col;
-  Frag qf[kSteps]; // Q^T as B operands, in registers for the whole kernel (loaded below, by way of LDS)
-
-  const int last_key = (q0 + kQueriesPerBlock < S ? q0 + kQueriesPerBlock : S) - 1;
-  const int steps = last_key / kPairKeys + 1;
-  const int plain_end = q0 / kPairKeys; // the steps before it are visible in full to every query of the block
-
-  // Load j of wave w fills the 64 slots of 16 bytes from (8 j + w) * 64 on
-  // (slot = row * 32 + chunk position), with the rows' permutations applied on
-  // the global side.
-  // (Load j lies 16 rows below load 0, whose permutation it shares. The
-  // offsets of loads 1.. and the addresses of the LDS reads are worked out
-  // where they are used, from values the compiler cannot see through: kept
-  // across the loop they would cost more registers than the wave has.)
-  uint32_t k_off, v_off;
-  {
-    const int sigma = wave * kWave + lane;
-    const int row = sigma / kChunks, at = sigma % kChunks;
-    k_off = (uint32_t)row * k_row + (uint32_t)(at ^ (row & 15)) * 16u;
-    v_off = (uint32_t)row * v_row + (uint32_t)(at ^ (2 * (row & 3))) * 16u;
-  }
-  constexpr int kRowsPerLoad = kPairThreads / kChunks;
-  const uint32_t pad_off = tid < kPairKeys ? (uint32_t)tid * (uint32_t)sizeof(float) : 0x80000000u;
-  TileStream k_src, v_src, pad_src; // the next to load: K of step t + 1, V of step t, mask values of step t + 1
-  k_src.start(kp, (uint32_t)(((int64_t)(S - 1) * a.k_s + D) * sizeof(T)), k_row, kPairKeys, 0, steps);
-  v_src.start(vp, (uint32_t)(((int64_t)(S - 1) * a.v_s + D) * sizeof(T)), v_row, kPairKeys, 0, steps);
-  if constexpr (HAS_PAD)
-    pad_src.start(a.pad + (int64_t)b * S, (uint32_t)S * (uint32_t)sizeof(float), (uint32_t)sizeof(float), kPairKeys, 0, steps);
-  auto k_buffer = [&](int step) __attribute__((always_inline)) { return k_lds + (step & 1) * kTile; };
-  auto v_buffer = [&](int step) __attribute__((always_inline)) { return v_lds + (step & 1) * kTile; };
-  auto pad_buffer = [&](int step) __attribute__((always_inline)) { return pad_lds + (step & 1) * kPairPadSlots; };
-  constexpr int kItems = 2 * kLoads + (HAS_PAD ? 1 : 0);
-  // item `it` of the staging of step `step`: K of step + 1, V of step, mask values of step + 1
-  auto stage_item = [&](int it, int step) __attribute__((always_inline)) {
-    if (it < kLoads) {
-      lds_load_b128(k_src.descriptor(), k_buffer(step + 1) + (kPairWaves * it + wave) * (kWave * 8),
-                    k_off + (uint32_t)(kRowsPerLoad * it) * k_row);
-      if (it == kLoads - 1) k_src.advance();
-      return;
-    }
-    it -= kLoads;
-    if (it < kLoads) {
-      lds_load_b128(v_src.descriptor(), v_buffer(step) + (kPairWaves * it + wave) * (kWave * 8),
-                    v_off + (uint32_t)(kRowsPerLoad * it) * v_row);
-      if (it == kLoads - 1) v_src.advance();
-      return;
-    }
-    if constexpr (HAS_PAD) {
-      lds_load_b32(pad_src.descriptor(), pad_buffer(step + 1) + wave * kWave, pad_off);
-      pad_src.advance();
-    }
-  };
-
-  f32x16 o[kBlocksSide];
-#pragma unroll
-  for (int i = 0; i < kBlocksSide; ++i)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
-  float m = kReferenceFloor; // reference maximum of the query's scores, log2 units: the same in both waves of a pair
-  float l = 0.f;             // this lane's share of the running sum
-  Frag pf[2];                // the wave's own P^T of the last step computed
-
-  // K operand s: lane (key, half) takes chunk 2 s + half of its key's row
-  // (bit 8 of the lane's offset is clear: steps 8.. are 256 bytes above steps 0..7)
-  uint32_t k_lane = (uint32_t)(32 * side + col) * kRowBytes + (uint32_t)((half ^ (col & 15)) << 4);
-  auto read_k = [&](const T *kb, int s) __attribute__((always_inline)) {
-    return *reinterpret_cast<const Frag *>(reinterpret_cast<const char *>(kb) + (k_lane ^ (uint32_t)((s & 7) << 5)) +
-                                           256 * (s >> 3));
-  };
-  auto hide_invariants = [&]() __attribute__((always_inline)) { asm volatile("" : "+v"(k_lane), "+v"(k_off), "+v"(v_off)); };
-  // Operand n of O^T += V^T P^T through the transposing read (see the kernel
-  // above): group n / 4 of 16 keys into block n % 4 of the wave's features. The
-  // wave's own 32 keys come first (groups 0 and 1), then the partner's.
-  typedef short Short4 __attribute__((ext_vector_type(4)));
-  uint32_t v_lane[2][2]; // [own keys, the partner's][even, odd blocks of 32 features]
-  {
-    const int j = lane & 15, group = lane >> 4;
-    const int key = 4 * (group >> 1) + (j >> 2);
-    const int x = (2 * (group & 1) + ((j & 3) >> 1)) ^ (2 * (j >> 2) & 3);
-    const int flip = (j >> 2) >> 1;
-    const uint32_t base = (uint32_t)key * kRowBytes + (uint32_t)x * 16u + (uint32_t)(j & 1) * 8u + 256u * (uint32_t)side;
-#pragma unroll
-    for (int w = 0; w < 2; ++w) {
-      const uint32_t keys = (uint32_t)(32 * (w == 0 ? side : 1 - side)) * kRowBytes;
-      v_lane[w][0] = base + keys + 64u * (uint32_t)flip;
-      v_lane[w][1] = base + keys + 64u * (uint32_t)(1 ^ flip);
-    }
-  }
-  auto read_v = [&](const T *vb, int n) __attribute__((always_inline)) {
-    const int u = n / kBlocksSide, i = n % kBlocksSide;
-    const char *at = reinterpret_cast<const char *>(vb) + v_lane[u >> 1][i & 1] + 64 * (i & ~1) + 16 * (u & 1) * kRowBytes;
-    const Short4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) Short4 *)(at));
-    const Short4 hi =
-        __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) Short4 *)(at + 8 * kRowBytes));
-    return __builtin_bit_cast(Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-  };
-  auto add_pad = [&](f32x16 &sc, int step) __attribute__((always_inline)) {
-    if constexpr (HAS_PAD) {
-      const float *pad = pad_buffer(step) + 32 * side;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float4 p4 = *reinterpret_cast<const float4 *>(&pad[8 * j + 4 * half]);
-        sc[4 * j + 0] = __builtin_fmaf(sc[4 * j + 0], a.scale, fmaxf(p4.x, kMaskFloor));
-        sc[4 * j + 1] = __builtin_fmaf(sc[4 * j + 1], a.scale, fmaxf(p4.y, kMaskFloor));
-        sc[4 * j + 2] = __builtin_fmaf(sc[4 * j + 2], a.scale, fmaxf(p4.z, kMaskFloor));
-        sc[4 * j + 3] = __builtin_fmaf(sc[4 * j + 3], a.scale, fmaxf(p4.w, kMaskFloor));
-      }
-    }
-  };
-  const float to_log2 = HAS_PAD ? kLog2e : a.scale_log2e;
-  auto causal = [&](f32x16 &sc, int keyb) __attribute__((always_inline)) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int kr = keyb + 8 * (r >> 2) + 4 * half + (r & 3);
-      sc[r] = kr <= qrow ? sc[r] : -INFINITY;
-    }
-  };
-  auto exponential = [&](float x) __attribute__((always_inline)) {
-    return __builtin_amdgcn_exp2f(__builtin_fmaf(x, to_log2, -m));
-  };
-  auto finish_probabilities = [&](f32x16 &sc, int keyb, Frag (&p)[2]) __attribute__((always_inline)) {
-    if constexpr (DROP) {
-      stage_keep_bits(keep_lds, a.drop, bh, S, wave_q0, keyb, lane);
-      const uint32_t bits = keep_word_query_lane(keep_lds, col) >> (4 * half);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sc[r] = (bits >> (8 * (r >> 2) + (r & 3))) & 1u ? sc[r] : 0.f;
-    }
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int i = 0; i < 8; ++i) p[u][i] = static_cast<T>(sc[8 * u + i]);
-  };
-  // the wave's P^T and flag, for the partner and the block
-  auto publish = [&](const Frag (&p)[2], int step, bool flag) __attribute__((always_inline)) {
-#pragma unroll
-    for (int u = 0; u < 2; ++u) p_lds[(wave * 2 + u) * kWave + lane] = __builtin_bit_cast(u32x4, p[u]);
-    if (lane == 0) flag_lds[8 * (step & 1) + wave] = flag ? 1u : 0u;
-  };
-  auto partners = [&](Frag (&p)[2]) __attribute__((always_inline)) {
-#pragma unroll
-    for (int u = 0; u < 2; ++u) p[u] = __builtin_bit_cast(Frag, p_lds[(partner * 2 + u) * kWave + lane]);
-  };
-  auto any_flag = [&](int step) __attribute__((always_inline)) -> bool {
-    const u32x4 f0 = *reinterpret_cast<const u32x4 *>(flag_lds + 8 * (step & 1));
-    const u32x4 f1 = *reinterpret_cast<const u32x4 *>(flag_lds + 8 * (step & 1) + 4);
-    return __builtin_amdgcn_readfirstlane(f0[0] | f0[1] | f0[2] | f0[3] | f1[0] | f1[1] | f1[2] | f1[3]) != 0u;
-  };
-
-  // A step in plain order, with the pair's maxima exchanged: the block's first
-  // step (`stage`: the next step's loads are issued here), and a step that has
-  // to be done again because some reference maximum has to rise (every wave of
-  // the block does it again: the step contains a barrier). K of the step must
-  // be in LDS; O^T is not touched except for its rescaling.
-  auto general_step = [&](int t, bool stage) __attribute__((always_inline)) {
-    if (stage) {
-#pragma unroll
-      for (int it = 0; it < kItems; ++it) stage_item(it, t);
-    }
-    const int keyb = t * kPairKeys + 32 * side;
-    f32x16 sc;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
-    {
-      const T *kb = k_buffer(t);
-#pragma unroll
-      for (int s = 0; s < kSteps; ++s) sc = Op::run(read_k(kb, s), qf[s], sc);
-    }
-    add_pad(sc, t);
-    if (keyb + 31 > wave_q0) causal(sc, keyb);
-    float mt = sc[0];
-#pragma unroll
-    for (int r = 1; r < 16; ++r) mt = fmaxf(mt, sc[r]);
-    mt = halves_max(mt * to_log2);
-    if (half == 0) stat_lds[32 * wave + col] = mt;
-    __syncthreads();
-    mt = fmaxf(mt, stat_lds[32 * partner + col]);
-    const bool raise = mt > m + kRaise;
-    if (__any(raise)) { // wave-uniform
-      const float m_new = raise ? mt : m;
-      const float alpha = raise ? __builtin_amdgcn_exp2f(m - m_new) : 1.0f; // 0 above the floor (nothing accumulated)
-      l *= alpha;
-#pragma unroll
-      for (int i = 0; i < kBlocksSide; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
-      m = m_new;
-    }
-    float sum = 0.f;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      sc[r] = exponential(sc[r]);
-      sum += sc[r];
-    }
-    l += sum;
-    finish_probabilities(sc, keyb, pf);
-    publish(pf, t, false);
-  };
-
-  // The products of O^T of step t - 1 (V in `vr`, the partner's P^T in `pp`),
-  // with `between(n)` after product n.
-  auto accumulate = [&](const T *vr, Frag (&ring)[4], int first, const Frag (&pp)[2], auto &&between)
-                        __attribute__((always_inline)) {
-#pragma unroll
-    for (int n = 0; n < kProducts; ++n) {
-      const int at = (first + n) % 4;
-      const int u = n / kBlocksSide;
-      o[n % kBlocksSide] = Op::run(ring[at], u < 2 ? pf[u] : pp[u - 2], o[n % kBlocksSide]);
-      if (n + 4 < kProducts) ring[at] = read_v(vr, n + 4);
-      between(n);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-  // A step as two straight runs of code, ordered by hand (see the kernel
-  // above), under the assumption that no reference maximum rises: the caller
-  // looks at the flags after the next barrier.
-  auto scheduled_step = [&]<bool MASKED>(int t, float &sum) __attribute__((always_inline)) {
-    hide_invariants();
-    const T *kr = k_buffer(t), *vr = v_buffer(t - 1);
-    Frag pp[2];
-    partners(pp);
-    // (the LDS serves a wave's accesses in order: when this lands, the reads above have been served)
-    if (lane == 0) *reinterpret_cast<volatile uint32_t *>(&ack_lds[wave]) = (uint32_t)t;
-    Frag ring[4];
-#pragma unroll
-    for (int s = 0; s < 4; ++s) ring[s] = read_k(kr, s);
-    __builtin_amdgcn_sched_barrier(0);
-    f32x16 sc;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
-      sc = Op::run(ring[s % 4], qf[s], sc);
-      const int next = s + 4;
-      if (next < kSteps)
-        ring[s % 4] = read_k(kr, next);
-      else
-        ring[s % 4] = read_v(vr, next - kSteps);
-      // a load every other product (all waves issue theirs at the same time: a
-      // burst of loads holds up the waves that issue it)
-      if (s % 2 == 1) stage_item((s % 4 == 1 ? 0 : kLoads) + s / 4, t);
-      if (HAS_PAD && s == kSteps - 2) stage_item(2 * kLoads, t);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    sum = 0.f;
-    Frag pn[2];
-    const int keyb = t * kPairKeys + 32 * side;
-    accumulate(vr, ring, kSteps, pp, [&](int n) __attribute__((always_inline)) {
-      if (n == 0) {
-        add_pad(sc, t);
-        if constexpr (MASKED) causal(sc, keyb);
-      }
-      sc[n] = exponential(sc[n]);
-      asm volatile("" : "+v"(sc[n])); // (keeps the computation in its slice)
-      if (n > 0) sum += sc[n - 1];
-      if (n == kProducts - 1) {
-        sum += sc[n];
-        finish_probabilities(sc, keyb, pn);
-      }
-    });
-    // The partner has taken this wave's P^T of step t - 1 (it does so at the
-    // start of its step t, which it has entered: the wait ends; bounded all the
-    // same, so that a wave cannot wait for ever).
-    for (int spin = 0; spin < (1 << 20); ++spin) {
-      if (__builtin_amdgcn_readfirstlane(*reinterpret_cast<volatile uint32_t *>(&ack_lds[partner])) >= (uint32_t)t) break;
-      __builtin_amdgcn_s_sleep(1);
-    }
-    publish(pn, t, __any(!(sum <= kSumLimit)));
-    pf[0] = pn[0], pf[1] = pn[1];
-  };
-
-  // prologue: the block's queries, then K and the mask values of the first
-  // step. A lane's operands of Q^T are 16 bytes from each of 16 chunks of its
-  // own row: loaded straight from memory, every lane of a load touches a cache
-  // line of its own. The rows go into LDS (where V will go) the way a tile of
-  // K does, whole rows at a time, and are read from there like K.
-  if (lane == 0) ack_lds[wave] = 0u;
-  {
-    TileStream q_src;
-    q_src.start(qp, (uint32_t)(((int64_t)(S - 1) * a.q_s + D) * sizeof(T)), q_row, kQueriesPerBlock, qb, a.query_blocks);
-    const u32x4 qd = q_src.descriptor();
-    const int sigma = wave * kWave + lane;
-    const int row = sigma / kChunks, at = sigma % kChunks;
-    const uint32_t q_off = (uint32_t)row * q_row + (uint32_t)(at ^ (row & 15)) * 16u;
-#pragma unroll
-    for (int j = 0; j < kQueriesPerBlock * kChunks / kPairThreads; ++j)
-      lds_load_b128(qd, v_lds + (kPairWaves * j + wave) * (kWave * 8), q_off + (uint32_t)(kRowsPerLoad * j) * q_row);
-  }
-#pragma unroll
-  for (int it = 0; it < kLoads; ++it) stage_item(it, -1);
-  if constexpr (HAS_PAD) stage_item(2 * kLoads, -1);
-  wait_vm<0>();
-  __syncthreads();
-  {
-    const uint32_t q_lane = (uint32_t)(32 * pair + col) * kRowBytes + (uint32_t)((half ^ (col & 15)) << 4);
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s)
-      qf[s] = *reinterpret_cast<const Frag *>(reinterpret_cast<const char *>(v_lds) + (q_lane ^ (uint32_t)((s & 7) << 5)) +
-                                              256 * (s >> 3));
-  }
-  __syncthreads(); // every wave has its operands: the first step's loads of V may overwrite the rows
-  general_step(0, true);
-  int t = 1;
-  wait_vm<0>();
-  __syncthreads(); // barrier A of step 1
-
-  // Each kind of step in a loop of its own. Between steps: barrier A of step t
-  // has been passed and no flag is up. The inner loops contain no rescaling of
-  // O^T, and are left only at their end (a way out between the top and the
-  // products has the compiler keep two copies of O^T and move one onto the
-  // other in every step): a step whose flags come up is done again outside.
-  auto run_steps = [&]<bool MASKED>(int end) __attribute__((always_inline)) {
-    while (t < end) {
-      bool again;
-      do {
-        float sum;
-        scheduled_step.template operator()<MASKED>(t, sum);
-        ++t;
-        wait_vm<0>();
-        __syncthreads(); // barrier A of step t
-        again = any_flag(t - 1);
-        l += again ? 0.f : sum;
-      } while (!again && t < end);
-      if (!again) break;
-      general_step(t - 1, false);
-      wait_vm<0>();
-      __syncthreads(); // barrier A of step t once more: P^T of step t - 1 as redone, the flags down
-    }
-  };
-  run_steps.template operator()<false>(plain_end);
-  run_steps.template operator()<true>(steps);
-
-  // V of the last step and every P^T of it are in LDS
-  {
-    const T *vr = v_buffer(t - 1);
-    Frag pp[2], ring[4];
-    partners(pp);
-#pragma unroll
-    for (int n = 0; n < 4; ++n) ring[n] = read_v(vr, n);
-    accumulate(vr, ring, 0, pp, [](int) __attribute__((always_inline)) {});
-  }
-
-  l = halves_sum(l);
-  if (half == 0) stat_lds[32 * wave + col] = l;
-  __syncthreads();
-  l += stat_lds[32 * partner + col];
-  const float inv = DROP ? a.drop.keep_scale / l : 1.0f / l;
-  // O^T leaves through LDS: a lane holds 4 features of its query at a time, and
-  // the queries' rows lie far apart in memory; the wave puts its 32 x 128 tile
-  // into LDS (its own part of what K and V occupied: every wave is past the
-  // barrier above), rows padded to 272 bytes, and stores whole rows, 16 bytes a
-  // lane.
-  constexpr int kOutRow = 272;
-  char *const stage = reinterpret_cast<char *>(k_lds) + wave * (32 * kOutRow);
-  typedef T Out4 __attribute__((ext_vector_type(4)));
-#pragma unroll
-  for (int i = 0; i < kBlocksSide; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      Out4 w;
-#pragma unroll
-      for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(o[i][4 * j + tt] * inv);
-      *reinterpret_cast<Out4 *>(stage + col * kOutRow + (32 * i + 8 * j + 4 * half) * (int)sizeof(T)) = w;
-    }
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  T *const out_head = static_cast<T *>(a.out) + b * a.o_b + hd * a.o_h + 128 * side;
-#pragma unroll
-  for (int k = 0; k < 8; ++k) {
-    const int row = 4 * k + (lane >> 4), piece = lane & 15;
-    const u32x4 w = *reinterpret_cast<const u32x4 *>(stage + row * kOutRow + piece * 16);
-    if (wave_q0 + row < S)
-      *reinterpret_cast<u32x4 *>(out_head + (int64_t)(wave_q0 + row) * a.o_s + 8 * piece) = w;
-  }
-  if (a.lse != nullptr && lane < 32 && side == 0 && qrow < S)
-    a.lse[(int64_t)bh * S + qrow] = m + __builtin_amdgcn_logf(l); // v_log_f32 is log2
-}
-
 template <typename T, int D>
 int launch_prefill_dim(const PrefillArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)(8 * a.head_groups * a.query_blocks));
@@ -1165,26 +693,8 @@ int launch_prefill_dim(const PrefillArgs &a, hipStream_t stream) {
     if (a.pad != nullptr) return go.template operator()<true, true>();
     return go.template operator()<false, true>();
   }
-  if constexpr (D == 256) {
-    // two waves per query
-    constexpr unsigned kPairLds = pair_lds_bytes<T>();
-    auto pair = [&]<bool HAS_PAD>() -> int {
-      auto *kernel = a.drop.drop ? attention_prefill_pair_kernel<T, HAS_PAD, true>
-                                 : attention_prefill_pair_kernel<T, HAS_PAD, false>;
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPairLds);
-      if (e != hipSuccess)
-        return fail(OSLO_E_LAUNCH, "oslo_attention_prefill_fwd: %u bytes of dynamic LDS refused: %s", kPairLds,
-                    hipGetErrorString(e));
-      kernel<<<grid, dim3(kPairThreads), kPairLds, stream>>>(a);
-      return check_launch("attention_prefill_fwd");
-    };
-    if (a.pad != nullptr) return pair.template operator()<true>();
-    return pair.template operator()<false>();
-  } else {
-    if (a.pad != nullptr) return go.template operator()<true, false>();
-    return go.template operator()<false, false>();
-  }
+  if (a.pad != nullptr) return go.template operator()<true, false>();
+  return go.template operator()<false, false>();
 }
 
 template <typename T>
