@@ -41,38 +41,38 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 # profiles/causal_softmax_fp16_8x16x2048x2048_hbm_traffic.md.
 MEASURED_TRAFFIC = {
     "linear_rows fc_in + bias + gelu bf16 1 x [16384,4096]": 134699021,
-    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135284954,
-    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134601023,
-    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136610240,
+    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135284942,
+    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134601247,
+    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136612927,
     "linear_rows attention projection bf16 1 x [4096,4096]": 33740800,
     "linear_rows attention projection bf16 8 x [4096,4096]": 34370560,
     "attention_decode bf16 1 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 17573906,
-    "attention_decode bf16 8 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 136477702,
+    "attention_decode bf16 8 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 136477701,
     "causal_fwd fp16 [8,16,2048,2048]": 1627471925,
-    "causal_bwd fp16 [8,16,2048,2048]": 2181120040,
-    "causal_fwd bf16 [8,16,2048,2048]": 1627459651,
-    "causal_bwd bf16 [8,16,2048,2048] (in place)": 2181120131,
-    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635900235,
-    "causal_dropout_bwd p=0.1 bf16 [8,16,2048,2048] (in place)": 2214719510,
-    "causal_fwd fp32 [8,16,2048,2048]": 3238067312,
-    "causal_bwd fp32 [8,16,2048,2048] (in place)": 4328580380,
+    "causal_bwd fp16 [8,16,2048,2048]": 2181120053,
+    "causal_fwd bf16 [8,16,2048,2048]": 1627459639,
+    "causal_bwd bf16 [8,16,2048,2048] (in place)": 2181120139,
+    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635900348,
+    "causal_dropout_bwd p=0.1 bf16 [8,16,2048,2048] (in place)": 2214719508,
+    "causal_fwd fp32 [8,16,2048,2048]": 3238067302,
+    "causal_bwd fp32 [8,16,2048,2048] (in place)": 4328580382,
     "causal_fwd bf16 [1,16,8192,8192]": 3229695244,
-    "masked_fwd bf16 [16,16,1024,1024] key mask": 1082271787,
+    "masked_fwd bf16 [16,16,1024,1024] key mask": 1082271844,
     "masked_bwd bf16 [16,16,1024,1024]": 1610650634,
-    "bias_gelu_fwd bf16 [16384,16384]": 1073876432,
-    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677947891,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610759196,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141067825,
-    "bias_gelu_fwd bf16 [16384,4096]": 268493619,
-    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419584301,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402709923,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285361377,
-    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 808012571,
-    "causal_fwd bf16 [8,16,2048,2048] with padding mask": 1628022937,
-    "causal_window_fwd window 256 bf16 [8,16,2048,2048]": 1230656579,
-    "causal_window_bwd window 256 bf16 [8,16,2048,2048] (in place)": 1387504728,
+    "bias_gelu_fwd bf16 [16384,16384]": 1073876275,
+    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677948342,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610759110,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141068378,
+    "bias_gelu_fwd bf16 [16384,4096]": 268493596,
+    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419584344,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402710034,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285361627,
+    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807991062,
+    "causal_fwd bf16 [8,16,2048,2048] with padding mask": 1628022939,
+    "causal_window_fwd window 256 bf16 [8,16,2048,2048]": 1230656581,
+    "causal_window_bwd window 256 bf16 [8,16,2048,2048] (in place)": 1387504717,
     "causal_fwd bf16 [4,16,4096,4096]": 3238084608,
-    "causal_bwd bf16 [4,16,4096,4096] (in place)": 4328603740,
+    "causal_bwd bf16 [4,16,4096,4096] (in place)": 4328603734,
 }
 
 
@@ -458,6 +458,28 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
                     "achieved": round(bflops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(bflops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "us": round(t * 1e6, 1),
                     "algorithmic_flops": bflops, "traffic": None})
+        if D == 256:
+            # The same launches on zero operands: the same instructions in the same order (no branch of
+            # these kernels looks at the data), without the switching activity of the matrix cores'
+            # inputs. The gap to the rows above is the clock the chip sustains under that activity, not
+            # something the kernels' code decides.
+            for x in (q, k, v, do):
+                x.zero_()
+            t = time_launches(lambda: check(lib.oslo_attention_prefill_fwd(
+                P(o), P(q), P(k), P(v), None, D ** -0.5, B, Hh, S, D, 0, strides, BF16, st)), max(5, n // 2), 3)
+            res.append({"kernel": f"attention_prefill bf16 [{B},{Hh},{S},{D}] causal, zero operands (same instruction stream)",
+                        "bound": "mfma", "achieved": round(flops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
+                        "unit": "TFLOP/s", "frac": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                        "us": round(t * 1e6, 1), "algorithmic_flops": flops, "traffic": None})
+            check(lib.oslo_attention_prefill_fwd_lse(P(o), P(lse), P(q), P(k), P(v), None, D ** -0.5, 0.0, 0, 0,
+                                                     B, Hh, S, D, 0, strides, BF16, st))
+            t = time_launches(lambda: check(lib.oslo_attention_prefill_bwd(
+                P(dq), P(dk), P(dv), P(do), P(q), P(k), P(v), P(o), P(lse), P(wsb), None, D ** -0.5, 0.0, 0, 0,
+                B, Hh, S, D, 0, bstr, BF16, st)), max(5, n // 4), 3)
+            res.append({"kernel": f"attention_prefill_bwd bf16 [{B},{Hh},{S},{D}] causal, zero operands (same instruction stream)",
+                        "bound": "mfma", "achieved": round(bflops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
+                        "unit": "TFLOP/s", "frac": round(bflops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                        "us": round(t * 1e6, 1), "algorithmic_flops": bflops, "traffic": None})
         del q, k, v, o, do, dq, dk, dv, lse, wsb
     return res
 
