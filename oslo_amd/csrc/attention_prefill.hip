@@ -1,8 +1,8 @@
 // Causal attention over a whole prompt in one kernel (no [S, S] matrix in
 // memory):
 //   out[q, :] = sum_{k <= q} softmax_k(scale * Q[q, :] . K[k, :] + pad[k]) * V[k, :]
-// for every (batch, head), 16-bit inputs, fp32 accumulation. It replaces, for
-// inference, the three launches of the fused attention -- batched matmul
+// for every (batch, head), 16-bit inputs, fp32 accumulation. It replaces the
+// three launches of the fused attention -- batched matmul
 // Q K^T, the fused scale + mask + softmax, batched matmul P V
 // (oslo/models/gptj/modeling_gptj.py:936-951,
 // oslo/models/gpt_neo/modeling_gpt_neo.py:993-1008,
@@ -47,7 +47,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 // by more than kRaise; the scheduled tiles do not look at the scores but at a
 // lane's sum of 16 exponentials: none of them exceeds the sum, and a sum above
 // 2^kSlack means a score more than kSlack - 4 = kRaise above the maximum, so
-// that doing such a tile again the general way does raise it.
+// that doing such a tile again in plain order (redo_tile) does raise it.
 constexpr float kSlack = 8.0f;
 constexpr float kRaise = 4.0f;
 constexpr float kSumLimit = 256.0f; // 2^kSlack
@@ -287,7 +287,6 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   float m = 0.f; // reference maximum of the query's scores, log2 units (the block's first tile sets it)
   float l = 0.f;       // this lane's share of the running sum
   Frag pf[2];          // P^T of the last tile computed, not yet multiplied with V
-  bool pending = false; // wave-uniform: pf holds such a tile (the one before the current)
 
   // K operand s of the tile at kb: lane (key, half) takes chunk 2 s + half of
   // its key's row, wherever the permutation has put it
@@ -376,31 +375,16 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   // an exact running maximum some query of a wave raises it in most tiles;
   // with the slack it happens in the first tiles only.
 
-  // Any tile, in plain order: the first of a block, those the causal or window
-  // boundary crosses (some waves sit them out), and those of the plain range
-  // in which a query's reference maximum has to rise. `with_previous`: stage
-  // the next tile and multiply the pending P^T of the previous one first. Only
-  // the RESCALE variant can raise the reference maximum of a query that has
-  // already accumulated something; the other returns false when that is
-  // needed, having done no more than the staging and the pending product. With
-  // the multiplications of O in the code that every tile runs through, the
+  // A tile in plain order, with the rescaling of O that the scheduled tiles
+  // leave out: a scheduled tile whose sum shows that some reference maximum
+  // has to rise is done again here (its staging and the products of the tile
+  // before it are done). It is kept out of the loops of the scheduled tiles:
+  // with the multiplications of O in code that every tile runs through, the
   // compiler copies all of O's accumulators to vector registers in every tile
   // (it places the copies that the rare multiplication needs ahead of the
   // branch).
-  auto general_tile = [&]<bool RESCALE>(int t, bool with_previous) __attribute__((always_inline)) -> bool {
-    if (with_previous) {
-#pragma unroll
-      for (int it = 0; it < kItems; ++it) stage_item(it, k_buffer(2), v_buffer(1));
-      if (pending) {
-        const T *vb = v_buffer(-1);
-#pragma unroll
-        for (int n = 0; n < 2 * kBlocksD; ++n) o[n % kBlocksD] = Op::run(read_v(vb, n), pf[n / kBlocksD], o[n % kBlocksD]);
-      }
-      pending = false;
-    }
+  auto redo_tile = [&](int t) __attribute__((always_inline)) {
     const int keyb = t * kKeysPerTile;
-    if (keyb > wave_q0 + 31) return true; // every key is ahead of the wave's queries
-    if (HAS_WINDOW && keyb + 31 <= wave_q0 - window) return true; // or behind their windows
     f32x16 sc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) sc[r] = 0.f;
@@ -421,19 +405,14 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     // (m is finite from the block's first tile on: with a window, the floor
     // that tile leaves for a query that has seen no key yet)
     const bool raise = mt > m + kRaise;
-    if (__any(raise)) { // wave-uniform
-      if constexpr (!RESCALE) return false;
-      const float m_new = raise ? mt : m;
-      const float alpha = raise ? __builtin_amdgcn_exp2f(m - m_new) : 1.0f; // 0 above the floor (nothing accumulated)
-      l *= alpha;
+    const float m_new = raise ? mt : m;
+    const float alpha = raise ? __builtin_amdgcn_exp2f(m - m_new) : 1.0f; // 0 above the floor (nothing accumulated)
+    l *= alpha;
 #pragma unroll
-      for (int i = 0; i < kBlocksD; ++i)
+    for (int i = 0; i < kBlocksD; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
-      m = m_new;
-    } else {
-      m = raise ? mt : m;
-    }
+      for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
+    m = m_new;
     float sum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -442,8 +421,6 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     }
     l += sum;
     finish_probabilities(sc, keyb, pf);
-    pending = true;
-    return true;
   };
   // prologue: K of the first two tiles and V of the first on their way, all
   // issued before any is waited for (the sources then stand at tile t + 2 and
@@ -555,7 +532,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
             // With a window a query may see nothing in the first tiles of its
             // wave: its reference then is a floor so far down that the first
             // visible score overflows the tile's sum, which has the tile done
-            // again the general way, where the reference rises to that score.
+            // again in plain order, where the reference rises to that score.
             m = HAS_WINDOW ? fmaxf(mt, kReferenceFloor) : mt;
           }
         }
@@ -588,7 +565,6 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     float mt, sum;
     scheduled_tile.template operator()<true, true>(t, mt, sum, pf);
     l = sum;
-    pending = true;
     next_tile();
   }
 
@@ -600,7 +576,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   // still computes it, every score masked: it adds zeros, and it would wait at
   // the tile's barrier anyway.
   auto scheduled_range = [&]<bool MASKED>(int end) __attribute__((always_inline)) {
-    while (t < end && pending) {
+    while (t < end) {
       bool rescale = false;
       for (; t < end; next_tile()) {
         wait_loads.template operator()<kLoadsPerTile>();
@@ -610,15 +586,13 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
         scheduled_tile.template operator()<MASKED, false>(t, mt, sum, pn);
         if (__any(!(sum <= kSumLimit))) {
           rescale = true;
-          pending = false;
           break;
         }
         l += sum;
         pf[0] = pn[0], pf[1] = pn[1];
       }
       if (!rescale) break;
-      general_tile.template operator()<true>(t, false);
-      pending = true; // (a wave the tile lies ahead of has multiplied nothing: zeros follow)
+      redo_tile(t);
       next_tile();
     }
   };
@@ -628,7 +602,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
 
   wait_loads.template operator()<0>(); // (nothing may still be on its way into LDS when the block ends)
   __syncthreads(); // V of the last tile is in LDS
-  if (pending) {
+  {
     const T *vb = v_buffer(-1);
 #pragma unroll
     for (int n = 0; n < 2 * kBlocksD; ++n) o[n % kBlocksD] = Op::run(read_v(vb, n), pf[n / kBlocksD], o[n % kBlocksD]);
