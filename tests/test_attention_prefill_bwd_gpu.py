@@ -165,6 +165,33 @@ def test_backward_strided_inputs_determinism_and_closed_forms(dtype):
     assert single["dq"].abs().max().item() <= 1e-4 and single["dk"].abs().max().item() <= 1e-4
 
 
+def test_backward_full_size_properties():
+    """The GPT-J shape of the benchmark, [8, 16, 2048, 256] bf16, where the oracle
+    would take days: heads taken one at a time against the float64 formulas on
+    the device; the same call twice gives the same bits; no gradient comes
+    back for dO = 0; and the gradients are linear in dO (doubling it doubles
+    them exactly: a power of two)."""
+    dtype = torch.bfloat16
+    b, h, s, d = 8, 16, 2048, 256
+    g = torch.Generator(device=DEV).manual_seed(3)
+    q, k, v, do = (torch.randn((b, h, s, d), generator=g, device=DEV).to(dtype) for _ in range(4))
+    scale = d ** -0.5
+    out, lse, got = run(q, k, v, do, scale)
+    for bb, hh in ((0, 0), (3, 7), (7, 15)):
+        one = [t[bb:bb + 1, hh:hh + 1] for t in (q, k, v, do)]
+        _, want, bounds = reference(*one, scale)
+        check({n: t[bb:bb + 1, hh:hh + 1] for n, t in got.items()}, want, bounds, dtype, ("full size", bb, hh))
+    again = kernels.attention_prefill_backward(do, q, k, v, out, lse, scale)
+    for t, n in zip(again, ("dq", "dk", "dv")):
+        assert torch.equal(t, got[n]), n
+    twice = kernels.attention_prefill_backward(do * 2, q, k, v, out, lse, scale)
+    for t, n in zip(twice, ("dq", "dk", "dv")):
+        assert torch.equal(t, got[n] * 2), n
+    none = kernels.attention_prefill_backward(torch.zeros_like(do), q, k, v, out, lse, scale)
+    for t in none:
+        assert not t.any()
+
+
 def keep_mask(b, h, s, p, seed, offset):
     """The mask of the softmax kernel with fused dropout: flat index over [B, H, S, S]."""
     return torch.from_numpy(orc.dropout_keep_mask(seed, offset, b * h * s * s, p).reshape(b, h, s, s))
