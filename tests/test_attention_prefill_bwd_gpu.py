@@ -237,6 +237,36 @@ def test_attention_dropout_forward_and_backward(s, d, dtype):
     assert torch.equal(again, first) and not torch.equal(again, other)
 
 
+def test_random_combinations_forward_and_backward():
+    """Forty draws of (type, head size, length, scale, window, padding mask,
+    dropout) that the tests above only take one or two at a time, forward and
+    backward against the float64 formulas on the device."""
+    import random
+
+    rng = random.Random(5)
+    for case in range(40):
+        dt = rng.choice(HALVES)
+        d = rng.choice([64, 128, 256])
+        s = rng.choice([1, 2, 31, 32, 33, 64, 100, 128, 129, 200, 256, 300, 384, 500, 640, 777, 1024])
+        b, h = rng.randint(1, 2), rng.randint(1, 3)
+        scale = rng.choice([1.0 / math.sqrt(d), 0.1, 0.3])
+        window = rng.choice([0, 0, 1, 3, 31, 32, 33, 64, 100, 128, 129, 200, 300, 511])
+        pad = padding(b, s, case).to(DEV) if rng.random() < 0.4 and s % 4 == 0 else None
+        p = rng.choice([0.0, 0.0, 0.1, 0.5]) if s % 8 == 0 else 0.0
+        g = torch.Generator(device=DEV).manual_seed(case)
+        q, k, v, do = (torch.randn((b, h, s, d), generator=g, device=DEV).to(dt) for _ in range(4))
+        seed, offset = 99 + case, 4 * case
+        keep = keep_mask(b, h, s, p, seed, offset).to(DEV) if p > 0 else None
+        what = (case, dt, b, h, s, d, scale, window, pad is not None, p)
+        out, lse = kernels.attention_prefill_forward(q, k, v, scale, pad, window, want_lse=True, p=p, seed=seed,
+                                                     offset=offset)
+        dq, dk, dv = kernels.attention_prefill_backward(do, q, k, v, out, lse, scale, pad, window, p, seed, offset)
+        o_ref, want, bounds = reference(q, k, v, do, scale, pad, window, keep, p)
+        excess = ((out.double() - o_ref).abs() - REL[dt] * (o_ref.abs() + 5.0 / (1 - p))).max().item()
+        assert torch.isfinite(out).all() and excess <= 1e-4, (excess, what)
+        check({"dq": dq, "dk": dk, "dv": dv}, want, bounds, dt, what)
+
+
 def test_attention_dropout_long_prompt_and_operator():
     """At [2,4,1024,128]: against the float64 formulas with the regenerated mask;
     and through FusedPrefillAttention.apply, which takes seed and offset from the
