@@ -84,6 +84,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gptj", action="store_true", help="skip the GPT-J-6B-shaped forward comparison")
     ap.add_argument("--only", default="", help="run only the named kernel of the table (for profiling)")
+    ap.add_argument("--zero-operands", action="store_true",
+                    help="with --only attention_prefill: q, k, v of zeros (clock and power readings)")
     return ap.parse_args()
 
 
@@ -496,6 +498,9 @@ def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
         import ctypes
         B, Hh, S, D = 8, 16, 2048, 256  # the GPT-J shape of the kernel table
         q, k, v = (torch.randn(B, Hh, S, D, device=dev).to(torch.bfloat16) for _ in range(3))
+        if args.zero_operands:  # the same instruction stream without the switching activity of its inputs
+            for x in (q, k, v):
+                x.zero_()
         o = torch.empty((B, S, Hh, D), dtype=torch.bfloat16, device=dev)
         strides = (ctypes.c_int64 * 12)(*(3 * [Hh * S * D, S * D, D] + [S * Hh * D, D, Hh * D]))
         fn = lambda: check(lib.oslo_attention_prefill_fwd(
