@@ -308,9 +308,22 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   // keep * dP / (1-p). The keep bits of the tile are drawn in the first slice.
   u32x4 keep_words[4];
   uint32_t keep_bits = 0;
+  // The tile's per-position values of register r (row 8 (r / 4) + 4 half + r % 4
+  // of the tile) are read kAhead registers before they are used: read where
+  // they are used, every slice of the elementwise work would wait for the LDS.
+  // (Not at head_dim 64, where the registers for it are not there.)
+  constexpr bool kRowValues = kKeysOwn || HAS_PAD;
+  constexpr int kAhead = D >= 128 ? 4 : 0;
+  float row_a[16], row_b[16];
+  auto read_row_values = [&](int r) __attribute__((always_inline)) {
+    if constexpr (kRowValues) {
+      const float *rows = rows_lds + buffer_of(0) * 2 * kRowSlots + 8 * (r >> 2) + 4 * half + (r & 3);
+      row_a[r] = rows[0];
+      if constexpr (kKeysOwn && kNeedT2) row_b[r] = rows[kRowSlots];
+    }
+  };
   auto elementwise = [&]<bool MASKED>(f32x16 &t1, const f32x16 &t2, int n, int slices, Frag (&x)[2])
                          __attribute__((always_inline)) {
-    const float *rows = rows_lds + buffer_of(0) * 2 * kRowSlots;
     if constexpr (DROP) {
       if (n == 0) {
         const int other0 = t * kSchedTile;
@@ -327,12 +340,13 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     for (int r = 0; r < 16; ++r) {
       if (r * slices / 16 != n) continue;
       const int rr = 8 * (r >> 2) + 4 * half + (r & 3); // the register's row of the tile
+      if (r + kAhead < 16) read_row_values(r + kAhead);
       float shift, delta_r = own_delta;
       if constexpr (kKeysOwn) {
-        shift = own_pad - rows[rr];
-        if constexpr (kNeedT2) delta_r = rows[kRowSlots + rr];
+        shift = own_pad - row_a[r];
+        if constexpr (kNeedT2) delta_r = row_b[r];
       } else if constexpr (HAS_PAD) {
-        shift = __builtin_fmaf(fmaxf(rows[rr], kMaskFloor), kLog2eB, -own_lse);
+        shift = __builtin_fmaf(fmaxf(row_a[r], kMaskFloor), kLog2eB, -own_lse);
       } else {
         shift = -own_lse;
       }
@@ -387,6 +401,8 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
 #pragma unroll
       for (int s = 0; s < kSteps; ++s) t2 = Op::run(read_natural(b2, s), own2[s], t2);
     }
+#pragma unroll
+    for (int r = 0; r < kAhead; ++r) read_row_values(r);
     elementwise.template operator()<true>(t1, t2, 0, 1, xf);
     ++t;
   }
@@ -432,6 +448,9 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
       }
     }
     Frag xn[2];
+#pragma unroll
+    for (int r = 0; r < kAhead; ++r) read_row_values(r);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int n = 0; n < kProducts; ++n, ++p) {
       acc[n % kBlocksD] = Op::run(ring[p % kRing], xf[n / kBlocksD], acc[n % kBlocksD]);
