@@ -41,38 +41,38 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 # profiles/causal_softmax_fp16_8x16x2048x2048_hbm_traffic.md.
 MEASURED_TRAFFIC = {
     "linear_rows fc_in + bias + gelu bf16 1 x [16384,4096]": 134699021,
-    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135284942,
-    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134601247,
-    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136612927,
+    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135284935,
+    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134601375,
+    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136610080,
     "linear_rows attention projection bf16 1 x [4096,4096]": 33740800,
     "linear_rows attention projection bf16 8 x [4096,4096]": 34370560,
-    "attention_decode bf16 1 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 17573906,
-    "attention_decode bf16 8 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 136477701,
-    "causal_fwd fp16 [8,16,2048,2048]": 1627471925,
-    "causal_bwd fp16 [8,16,2048,2048]": 2181120053,
-    "causal_fwd bf16 [8,16,2048,2048]": 1627459639,
-    "causal_bwd bf16 [8,16,2048,2048] (in place)": 2181120139,
-    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635900348,
+    "attention_decode bf16 1 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 17573904,
+    "attention_decode bf16 8 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 136477708,
+    "causal_fwd fp16 [8,16,2048,2048]": 1627471921,
+    "causal_bwd fp16 [8,16,2048,2048]": 2181120049,
+    "causal_fwd bf16 [8,16,2048,2048]": 1627459649,
+    "causal_bwd bf16 [8,16,2048,2048] (in place)": 2181120131,
+    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635900143,
     "causal_dropout_bwd p=0.1 bf16 [8,16,2048,2048] (in place)": 2214719508,
-    "causal_fwd fp32 [8,16,2048,2048]": 3238067302,
-    "causal_bwd fp32 [8,16,2048,2048] (in place)": 4328580382,
-    "causal_fwd bf16 [1,16,8192,8192]": 3229695244,
-    "masked_fwd bf16 [16,16,1024,1024] key mask": 1082271844,
+    "causal_fwd fp32 [8,16,2048,2048]": 3238067310,
+    "causal_bwd fp32 [8,16,2048,2048] (in place)": 4328580380,
+    "causal_fwd bf16 [1,16,8192,8192]": 3229695246,
+    "masked_fwd bf16 [16,16,1024,1024] key mask": 1082175281,
     "masked_bwd bf16 [16,16,1024,1024]": 1610650634,
-    "bias_gelu_fwd bf16 [16384,16384]": 1073876275,
-    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677948342,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610759110,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141068378,
-    "bias_gelu_fwd bf16 [16384,4096]": 268493596,
-    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419584344,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402710034,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285361627,
-    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807991062,
-    "causal_fwd bf16 [8,16,2048,2048] with padding mask": 1628022939,
-    "causal_window_fwd window 256 bf16 [8,16,2048,2048]": 1230656581,
-    "causal_window_bwd window 256 bf16 [8,16,2048,2048] (in place)": 1387504717,
+    "bias_gelu_fwd bf16 [16384,16384]": 1073876258,
+    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677948211,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610759309,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141068691,
+    "bias_gelu_fwd bf16 [16384,4096]": 268493592,
+    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419584569,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402709938,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285361651,
+    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807983113,
+    "causal_fwd bf16 [8,16,2048,2048] with padding mask": 1628022937,
+    "causal_window_fwd window 256 bf16 [8,16,2048,2048]": 1230656579,
+    "causal_window_bwd window 256 bf16 [8,16,2048,2048] (in place)": 1387504736,
     "causal_fwd bf16 [4,16,4096,4096]": 3238084608,
-    "causal_bwd bf16 [4,16,4096,4096] (in place)": 4328603734,
+    "causal_bwd bf16 [4,16,4096,4096] (in place)": 4328603740,
 }
 
 
