@@ -214,11 +214,11 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   o2_src.start(o2_p, slice_bytes(st_o2), o2_row, kSchedTile, first_tile, tiles);
   if constexpr (kKeysOwn) {
     lse_src.start(a.lse + stat_row, (uint32_t)S * 4u, 4u, kSchedTile, first_tile, tiles);
-    delta_src.start(a.delta + stat_row, (uint32_t)S * 4u, 4u, kSchedTile, first_tile, tiles);
+    if constexpr (kNeedT2) delta_src.start(a.delta + stat_row, (uint32_t)S * 4u, 4u, kSchedTile, first_tile, tiles);
   } else if constexpr (HAS_PAD) { // the keys' mask values take the first of the two rows
     lse_src.start(a.pad + (int64_t)b * S, (uint32_t)S * 4u, 4u, kSchedTile, first_tile, tiles);
   }
-  constexpr int kRowItems = kKeysOwn ? 2 : HAS_PAD ? 1 : 0;
+  constexpr int kRowItems = kKeysOwn ? (kNeedT2 ? 2 : 1) : HAS_PAD ? 1 : 0; // (the dV pass needs no delta)
   constexpr int kItems = 2 * kLoadsN + kRowItems;
   constexpr int kLoadsPerTile = kItems;
   int t = first_tile;
