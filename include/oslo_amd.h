@@ -242,6 +242,9 @@ int oslo_bias_gelu_bwd(void *dy, void *dbias, float *workspace, const void *g,
  * has yet): make one call, of any size, before a graph capture begins. All
  * calls on a GPU share the one buffer: calls that may overlap there (different
  * streams, different threads) race; order them or use oslo_bias_gelu_bwd.
+ * The buffer used is the one of the calling thread's current device, which
+ * must be the device that holds the tensors (and owns the stream): a call whose
+ * tensors are on another device fails with OSLO_E_BAD_ARG.
  */
 #define OSLO_STATIC_WORKSPACE_BYTES (32u << 20)
 int oslo_bias_gelu_bwd_static(void *dy, void *dbias, const void *g,

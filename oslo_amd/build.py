@@ -52,9 +52,20 @@ FLAGS = [
 ]
 
 
+# The two prompt-attention sources name M0 as clobbered by their hand-written
+# loads into LDS (they set it themselves inside the asm statement). M0 is a
+# reserved register to the compiler, which says so once per instantiation of
+# every such statement, thousands of lines per build; silenced for these two
+# files only, so that -Wall stays readable for everything else.
+EXTRA_FLAGS = {
+    "attention_prefill.hip": ["-Wno-inline-asm"],
+    "attention_prefill_bwd.hip": ["-Wno-inline-asm"],
+}
+
+
 def _compile(src):
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC, *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass warns that it does not know the target feature; drop that
     err = "\n".join(

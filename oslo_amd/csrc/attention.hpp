@@ -107,13 +107,21 @@ struct TileStream {
 // (the builtin), waits for every such load before the next LDS read of any
 // buffer. These are waited for by count (wait_vm). A wave's instruction puts
 // its 64 x 16 (or 64 x 4) bytes at consecutive LDS addresses from `dst` on.
+// The LDS address travels in M0, written inside the same asm statement: on
+// this family a scalar write of M0 needs one wait state before a load into LDS
+// reads it, which the compiler inserts for its own code and not inside inline
+// asm, hence the s_nop. Nothing else in the attention kernels uses M0 (LDS
+// reads and writes, lane reads and the matrix products do not; there is no
+// indirect register indexing, message or interpolation instruction), and every
+// statement that needs it sets it itself, so no value of M0 has to survive
+// from one statement to the next, whatever the compiler makes of the clobber.
 __device__ __forceinline__ void lds_load_b128(const u32x4 &desc, const void *dst, uint32_t offset) {
   const uint32_t at = __builtin_amdgcn_readfirstlane((uint32_t)reinterpret_cast<uintptr_t>(dst));
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");
 }
 __device__ __forceinline__ void lds_load_b32(const u32x4 &desc, const void *dst, uint32_t offset) {
   const uint32_t at = __builtin_amdgcn_readfirstlane((uint32_t)reinterpret_cast<uintptr_t>(dst));
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");
 }
 // vmcnt <= N, nothing else: all but the N most recent loads have arrived
 template <int N>
@@ -121,12 +129,21 @@ __device__ __forceinline__ void wait_vm() {
   __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-// Additive mask values travel in log2 units. Masks of -inf or of the most
-// negative finite number (as some callers build them) would make every score
-// of a row -inf and its softmax 0/0; they are floored at a value that still
-// underflows every exponential but keeps the arithmetic finite.
-constexpr float kMaskFloorLog2 = -1e30f;
-constexpr float kMaskFloor = -1e30f; // the same for mask values kept in natural units
+// Additive mask values below kMaskFloor act as kMaskFloor, in the forward and in
+// every pass of the backward (one constant, applied to the value in natural
+// units before anything else). Callers build masks of -10000, of -inf or of the
+// most negative finite number; the last two would make every score of a row
+// -inf (0/0 in the softmax), and any value of magnitude above about 2^31 breaks
+// the kernels' arithmetic even on rows that see valid keys: a row's reference
+// maximum is the rounded product score * log2(e), an exponent is the exact
+// fma(score, log2(e), -maximum), and their difference is the product's rounding
+// error, up to half an ulp of the maximum: 6e22 at 1e30, whose exp2 is inf (and
+// inf * 0 = NaN at the next rescaling). At -2^22 that error is at most 0.25, a
+// masked key's probability still underflows to exactly 0 beside any score a
+// 16-bit model produces (|scaled score| far below 4e6), and a row whose every
+// visible key is masked comes out finite (close to the softmax of the scores
+// alone, like a -10000 mask).
+constexpr float kMaskFloor = -4194304.0f; // -2^22
 
 // Attention dropout inside the attention kernels. The keep flag of the
 // probability of (query q, key k) of head bh is the one the softmax kernel with

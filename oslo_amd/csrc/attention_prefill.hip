@@ -233,7 +233,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   // are waited for by count, a tile later (wait_loads).
   auto load_to_lds = [&](const u32x4 &desc, const T *dst, uint32_t offset) __attribute__((always_inline)) {
     const uint32_t at = __builtin_amdgcn_readfirstlane((uint32_t)reinterpret_cast<uintptr_t>(dst)); // LDS addresses are the low 32 bits
-    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");
   };
   // the three buffers of K and of V, as element offsets, in the order (tile t,
   // t + 1, t + 2) and (t - 1, t, t + 1); rotated from tile to tile
@@ -269,7 +269,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     if constexpr (HAS_PAD) {
       const uint32_t at = __builtin_amdgcn_readfirstlane(
           (uint32_t)reinterpret_cast<uintptr_t>(pad_lds + pad_at[2] + wave * kWave));
-      asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(at), "v"(pad_off), "s"(pad_src.descriptor(tiles)) : "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(at), "v"(pad_off), "s"(pad_src.descriptor(tiles)) : "m0");
       pad_src.advance();
     }
   };
@@ -305,7 +305,6 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   // where the accumulator layout leaves the probabilities (rows 8j' + 4h + t of
   // S^T), so that P^T is used where it is.
   typedef short Short4 __attribute__((ext_vector_type(4)));
-  typedef short Short8 __attribute__((ext_vector_type(8)));
   uint32_t v_lane[2]; // for even and odd blocks of 32 features
   {
     const int j = lane & 15, group = lane >> 4; // group: bit 0 = second 16 features of the block, bit 1 = half
@@ -648,17 +647,14 @@ int launch_prefill_dim(const PrefillArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)(8 * a.head_groups * a.query_blocks));
   // All LDS of the kernel is dynamic. At head_dim 256 it exceeds the 64 KiB a
   // kernel gets unasked, so the limit is raised for the kernel (on the current
-  // device; a host-side setting, not a stream operation) before every launch.
+  // device; a host-side setting, not a stream operation), once.
   constexpr unsigned kDynamic = prefill_lds_bytes<T, D>();
   auto go = [&]<bool HAS_PAD, bool HAS_WINDOW>() -> int {
     auto *kernel = a.drop.drop ? attention_prefill_kernel<T, D, HAS_PAD, HAS_WINDOW, true>
                                : attention_prefill_kernel<T, D, HAS_PAD, HAS_WINDOW, false>;
     if (kDynamic > 64u * 1024u) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynamic);
-      if (e != hipSuccess)
-        return fail(OSLO_E_LAUNCH, "oslo_attention_prefill_fwd: %u bytes of dynamic LDS refused: %s",
-                    kDynamic, hipGetErrorString(e));
+      const int s = raise_lds_limit(reinterpret_cast<const void *>(kernel), kDynamic, "oslo_attention_prefill_fwd");
+      if (s != OSLO_OK) return s;
     }
     kernel<<<grid, dim3(kBlockThreads), kDynamic, stream>>>(a);
     return check_launch("attention_prefill_fwd");

@@ -162,7 +162,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
       own_delta = a.delta[stat_row + own];
     }
   } else if constexpr (HAS_PAD) {
-    if (own < S) own_pad = fmaxf(a.pad[(int64_t)b * S + own] * kLog2eB, kMaskFloorLog2);
+    if (own < S) own_pad = fmaxf(a.pad[(int64_t)b * S + own], kMaskFloor) * kLog2eB;
   }
 
   // Tiles [first_tile, tiles) of the other kind this block walks. Those before
@@ -506,11 +506,8 @@ int launch_role(const BwdArgs &a, hipStream_t stream) {
     auto *kernel = a.window > 0 ? attention_bwd_kernel<T, D, ROLE, HAS_PAD, true, DROP>
                                 : attention_bwd_kernel<T, D, ROLE, HAS_PAD, false, DROP>;
     if (kLds > 64u * 1024u) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
-      if (e != hipSuccess)
-        return fail(OSLO_E_LAUNCH, "oslo_attention_prefill_bwd: %u bytes of dynamic LDS refused: %s", kLds,
-                    hipGetErrorString(e));
+      const int s = raise_lds_limit(reinterpret_cast<const void *>(kernel), kLds, "oslo_attention_prefill_bwd");
+      if (s != OSLO_OK) return s;
     }
     kernel<<<grid, dim3(kBlockThreads), kLds, stream>>>(a);
     return check_launch("attention_prefill_bwd");

@@ -137,13 +137,26 @@ constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 float *g_scratch_ptr[kMaxDevices];
 
-int static_scratch(float **out) {
+// `tensor`: one of the call's device tensors. Every GPU has a copy of the array
+// at an address of its own, and the one looked up is the current device's: a
+// call whose tensors live on another device is refused rather than handed a
+// scratch address of the wrong GPU.
+int static_scratch(float **out, const void *tensor) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess)
     return fail(OSLO_E_LAUNCH, "bias_gelu_bwd_static: hipGetDevice: %s", hipGetErrorString(e));
   if (dev < 0 || dev >= kMaxDevices)
     return fail(OSLO_E_UNSUPPORTED, "bias_gelu_bwd_static: device %d, at most %d are tracked", dev, kMaxDevices);
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, tensor) == hipSuccess) {
+    if (attr.type == hipMemoryTypeDevice && attr.device != dev)
+      return fail(OSLO_E_BAD_ARG,
+                  "bias_gelu_bwd_static: the tensors are on device %d, the current device is %d "
+                  "(make the tensors' device current for the call)", attr.device, dev);
+  } else {
+    (void)hipGetLastError(); // a pointer the runtime does not know: the kernels will say
+  }
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (!g_scratch_ptr[dev]) {
     float *p = nullptr;
@@ -230,7 +243,7 @@ extern "C" int oslo_bias_gelu_bwd_static(void *dy, void *dbias, const void *g,
                 (long long)rows, (long long)cols, need, (size_t)OSLO_STATIC_WORKSPACE_BYTES);
   float *ws = nullptr;
   if (dbias) {
-    const int s = static_scratch(&ws);
+    const int s = static_scratch(&ws, dy);
     if (s != OSLO_OK) return s;
   }
   // Every partial row the finishing sum reads is written by this call's first

@@ -230,6 +230,10 @@ __device__ __forceinline__ float sum_over_lanes(float v) {
 // ---------------------------------------------------------------------------
 int fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int check_launch(const char *what);
+// Lets `kernel` ask for `bytes` of dynamic LDS (more than the 64 KiB a kernel
+// gets unasked) on the current device. A host-side setting of the kernel, made
+// once per kernel and device and remembered, not per launch.
+int raise_lds_limit(const void *kernel, unsigned bytes, const char *what);
 
 inline bool aligned16(const void *p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;

@@ -4,6 +4,10 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+#include <utility>
+#include <vector>
+
 #include "elementwise.hpp"
 #include "softmax.hpp"
 
@@ -24,6 +28,22 @@ int check_launch(const char *what) {
   const hipError_t e = hipGetLastError();
   if (e == hipSuccess) return OSLO_OK;
   return fail(OSLO_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+int raise_lds_limit(const void *kernel, unsigned bytes, const char *what) {
+  static std::mutex mutex;
+  static std::vector<std::pair<const void *, int>> done; // (kernel, device)
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(OSLO_E_LAUNCH, "%s: hipGetDevice: %s", what, hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(mutex);
+  for (const auto &entry : done)
+    if (entry.first == kernel && entry.second == dev) return OSLO_OK;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess)
+    return fail(OSLO_E_LAUNCH, "%s: %u bytes of dynamic LDS refused: %s", what, bytes, hipGetErrorString(e));
+  done.emplace_back(kernel, dev);
+  return OSLO_OK;
 }
 
 } // namespace oslo

@@ -25,6 +25,7 @@ import threading
 import weakref
 
 import torch
+from torch.autograd.function import once_differentiable
 
 from . import _lib, kernels
 
@@ -78,6 +79,7 @@ class ScaledUpperTriangMaskedSoftmaxFunction(torch.autograd.Function):
         return softmax_results
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, output_grads):
         softmax_results, scale_t = ctx.saved_tensors
         input_grads = get_custom_kernels().scaled_upper_triang_masked_softmax_backward(
@@ -100,6 +102,7 @@ class ScaledMaskedSoftmaxFunction(torch.autograd.Function):
         return softmax_results
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, output_grads):
         softmax_results, scale_t = ctx.saved_tensors
         input_grads = get_custom_kernels().scaled_masked_softmax_backward(
@@ -120,6 +123,7 @@ class _CausalSoftmaxWithPad(torch.autograd.Function):
         return y
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, output_grads):
         (y,) = ctx.saved_tensors
         b, h, s, _ = y.shape
@@ -141,6 +145,7 @@ class _KeyMaskedSoftmax(torch.autograd.Function):
         return y
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, output_grads):
         (y,) = ctx.saved_tensors
         dx = get_custom_kernels().scaled_masked_softmax_backward(output_grads, y, ctx.scale)
@@ -159,6 +164,7 @@ class _CausalWindowSoftmax(torch.autograd.Function):
         return y
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, output_grads):
         (y,) = ctx.saved_tensors
         scale, window = ctx.args
@@ -184,6 +190,7 @@ class _CausalSoftmaxDropout(torch.autograd.Function):
         return yd
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, output_grads):
         inputs, stats = ctx.saved_tensors
         scale, p, seed, offset = ctx.args
@@ -354,6 +361,7 @@ class _RotaryQKV(torch.autograd.Function):
         return get_custom_kernels().rotary_qkv_forward(query, key, value, sin, cos, rotary_dim, offset)
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, grad_query, grad_key, grad_value):
         sin, cos = ctx.saved_tensors
         rotary_dim, offset = ctx.args
@@ -403,6 +411,7 @@ class _MergeHeads(torch.autograd.Function):
         return get_custom_kernels().rotary_qkv_backward(None, None, x, None, None, 0)[2]
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, grad):
         return get_custom_kernels().rotary_qkv_forward(None, None, grad, None, None, 0)[2]
 
@@ -431,6 +440,7 @@ class _SplitHeadsPacked(torch.autograd.Function):
         return get_custom_kernels().split_heads_packed_forward(qkv, heads)
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, grad_query, grad_key, grad_value):
         return get_custom_kernels().split_heads_packed_backward(grad_query, grad_key, grad_value), None
 
@@ -471,6 +481,7 @@ class FusedBiasGeLU(torch.autograd.Function):
         return get_custom_kernels().bias_gelu_forward(input, bias)
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, grad_output):
         input, bias = ctx.saved_tensors
         want_dbias = ctx.needs_input_grad[1]
@@ -549,7 +560,10 @@ class _PrefillAttention(torch.autograd.Function):
     """The prompt attention with its backward: the forward keeps q, k, v, its
     output and one fp32 number per row (the log-sum-exp); the backward
     recomputes the probabilities (and the dropout mask, from the same Philox
-    seed and offset) tile by tile on the matrix cores."""
+    seed and offset) tile by tile on the matrix cores. The backward is a raw
+    kernel call: it cannot be differentiated again (a second-order request
+    raises), and it always computes all three gradients, whichever of them the
+    caller asked for."""
 
     @staticmethod
     def forward(ctx, query, key, value, pad, scale, window, p):
@@ -562,6 +576,7 @@ class _PrefillAttention(torch.autograd.Function):
         return out
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, grad_out):
         query, key, value, out, lse = ctx.saved_tensors
         scale, window, p, seed, offset = ctx.args
@@ -733,6 +748,7 @@ class _BiasDropoutAdd(torch.autograd.Function):
         return get_custom_kernels().bias_dropout_add_forward(x, bias, residual, p, seed, offset)
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, grad_output):
         want_dbias = ctx.needs_input_grad[1]
         dx = dbias = None

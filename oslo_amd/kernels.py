@@ -658,6 +658,8 @@ def attention_prefill_backward(grad_out, query, key, value, out, lse, scale, pad
     nothing of that size is stored."""
     code, pad = _prefill_args(query, key, value, pad)
     _device_tensor(grad_out, "grad_out", query)
+    _device_tensor(out, "out", query)
+    _device_tensor(lse, "lse", query)
     _require(grad_out.shape == query.shape and out.shape == query.shape, "grad_out and out must be shaped like query")
     _require(grad_out.dtype == query.dtype and out.dtype == query.dtype, "grad_out and out must have query's dtype")
     b, h, s, d = query.shape
