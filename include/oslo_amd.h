@@ -65,6 +65,16 @@ const char *oslo_last_error(void);
 /* Scale + causal mask + softmax ------------------------------------------ */
 
 /*
+ * Size limits of every softmax entry point (causal, windowed, key-mask, with
+ * or without dropout): a row of at most oslo_softmax_max_cols() keys, and at
+ * most 2^31 - 1 rows per call (batch * heads * S, or B * H * Sq); beyond either
+ * the call returns OSLO_E_UNSUPPORTED and launches nothing. Elements are
+ * indexed with 64 bits: tensors of 2^31 elements and more are single calls
+ * (the reference launches any number of attention batches,
+ * oslo/fused_kernels/fused_triang_softmax.cu:44-60).
+ */
+
+/*
  * y[b,h,r,k] = softmax over k<=r of ( scale*x[b,h,r,k] + pad_add[b,k] ),
  * y[b,h,r,k] = 0 for k>r. x, y: [batch, heads, S, S]; y may alias x.
  * pad_add: NULL or fp32 [batch, S], added after scaling (the order of the

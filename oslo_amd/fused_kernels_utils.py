@@ -280,6 +280,8 @@ class FusedScaleMaskSoftmax(object):
             return False
         if bsz <= 0 or np <= 0 or sq <= 0:
             return False
+        if bsz * np * sq > _MAX_ROWS:  # the entry points' limit is on rows; elements are indexed with 64 bits
+            return False
         # the reference also tests divisibility by get_batch_per_block here; no
         # kernel of this library needs it
         if use_triang_mask:
@@ -288,6 +290,7 @@ class FusedScaleMaskSoftmax(object):
 
 
 _softmax_max_cols = None
+_MAX_ROWS = 2 ** 31 - 1
 
 
 def _max_cols():
@@ -821,12 +824,30 @@ class NGramRepeatBlockFunction(torch.autograd.Function):
         raise NotImplementedError
 
 
+def _banned_tokens_on_host(ngram_size, input_ids):
+    """Per hypothesis, the tokens that would complete an n-gram already in it:
+    those that followed an earlier occurrence of its last ngram_size - 1 tokens
+    (what ``_calc_banned_ngram_tokens`` gives the reference's host branch,
+    oslo/fused_kernels_utils.py:506-512)."""
+    cur_len = input_ids.shape[-1]
+    if cur_len + 1 < ngram_size:
+        return [[] for _ in range(input_ids.shape[0])]
+    banned = []
+    for row in input_ids.tolist():
+        last = row[cur_len + 1 - ngram_size:]
+        banned.append([row[i + ngram_size - 1] for i in range(cur_len - ngram_size + 1)
+                       if row[i:i + ngram_size - 1] == last])
+    return banned
+
+
 class FusedNoRepeatNGramLogitsProcessor(object):
     """Logits processor that bans every token that would repeat an n-gram
     (oslo/fused_kernels_utils.py:482-521). Callable as
-    ``processor(input_ids, scores)`` like a HuggingFace LogitsProcessor. The
-    reference computes the bans on the host for CPU tensors; here only device
-    tensors are accepted."""
+    ``processor(input_ids, scores)`` like a HuggingFace LogitsProcessor.
+    Device tensors go to the kernel and nowhere else (a missing library raises).
+    Host tensors are the reference's other branch (:505-517), which is host
+    code there too: the bans are worked out in Python and written into
+    ``scores`` in place."""
 
     def __init__(self, ngram_size: int, batch_size: int, beam_size: int):
         if not isinstance(ngram_size, int) or ngram_size <= 0:
@@ -838,11 +859,15 @@ class FusedNoRepeatNGramLogitsProcessor(object):
         self.beam_size = beam_size
 
     def __call__(self, input_ids, scores):
-        if not (input_ids.is_cuda and scores.is_cuda):
+        if input_ids.is_cuda != scores.is_cuda:
             raise RuntimeError(
-                "FusedNoRepeatNGramLogitsProcessor: expected tensors on a ROCm device "
-                "(this library has no CPU path)"
+                "FusedNoRepeatNGramLogitsProcessor: input_ids and scores must both be on the "
+                f"device or both on the host, got {input_ids.device} and {scores.device}"
             )
+        if not input_ids.is_cuda:
+            for i, tokens in enumerate(_banned_tokens_on_host(self.ngram_size, input_ids)):
+                scores[i, tokens] = -float("inf")
+            return scores
         cur_len = input_ids.shape[-1]
         return NGramRepeatBlockFunction.apply(
             input_ids.contiguous(),
@@ -853,10 +878,6 @@ class FusedNoRepeatNGramLogitsProcessor(object):
             self.ngram_size,
         )
 
-
-# ---------------------------------------------------------------------------
-# model.fuse()
-# ---------------------------------------------------------------------------
 
 class FusedKernelMixin(object):
     """oslo/fused_kernels_utils.py:524-566: swaps the class of every fusable

@@ -64,6 +64,32 @@ def test_workspace_bytes(lib):
     assert lib.oslo_colsum_workspace_bytes(16385, 10) == 513 * 10 * 4
 
 
+def test_softmax_row_limit_is_on_rows_not_elements(lib):
+    """A call takes at most 2^31 - 1 rows (batch * heads * S); more is refused
+    with OSLO_E_UNSUPPORTED before any pointer is looked at. The number of
+    elements is not limited: the gate admits [32,16,2048,2048] (2^31 elements)
+    and [2,16,8192,8192] (2^32)."""
+    import torch
+
+    from oslo_amd import FusedScaleMaskSoftmax
+
+    null, one = ctypes.c_void_p(0), ctypes.c_void_p(16)
+    rows_ok, rows_too_many = (2 ** 31 - 8) // 8, 2 ** 31 // 8      # heads of S = 8
+    assert lib.oslo_softmax_causal_fwd(one, one, null, 1.0, 1, rows_too_many, 8, 1, null) == -2
+    assert b"rows" in lib.oslo_last_error()
+    assert lib.oslo_softmax_causal_bwd(one, one, one, 1.0, rows_too_many, 8, 1, null) == -2
+    assert lib.oslo_softmax_causal_window_fwd(one, one, null, 1.0, 4, 1, rows_too_many, 8, 1, null) == -2
+    assert lib.oslo_softmax_masked_fwd(one, one, null, 0, 0, 0, 1.0, 2 ** 16, 2 ** 15, 1, 8, 1, null) == -2
+    assert lib.oslo_softmax_masked_bwd(one, one, one, 1.0, 2 ** 31, 8, 1, null) == -2
+    assert rows_ok * 8 < 2 ** 31
+    for dtype in (torch.half, torch.bfloat16, torch.float32):
+        assert FusedScaleMaskSoftmax.is_available(dtype, 32, 16, 2048, 2048, True)
+        assert FusedScaleMaskSoftmax.is_available(dtype, 2, 16, 8192, 8192, True)
+        assert FusedScaleMaskSoftmax.is_available(dtype, 64, 16, 2048, 1024, False)
+        assert not FusedScaleMaskSoftmax.is_available(dtype, 2 ** 16, 2 ** 12, 8, 8, True)   # 2^31 rows
+        assert FusedScaleMaskSoftmax.is_available(dtype, 2 ** 16 - 1, 2 ** 12, 8, 8, True)
+
+
 def test_argument_screening_without_a_device(lib):
     null = ctypes.c_void_p(0)
     one = ctypes.c_void_p(16)  # never dereferenced: every call below fails or returns first

@@ -45,6 +45,27 @@ def test_oracle_matches_transformers_processor(n):
         assert torch.equal(torch.isinf(want), torch.isinf(got)), (n, length)
 
 
+@pytest.mark.parametrize("n", [1, 2, 3, 4])
+def test_processor_host_branch_matches_transformers_and_oracle(n):
+    """Host tensors take the processor's host branch, as in the reference
+    (oslo/fused_kernels_utils.py:505-517): same bans as the installed
+    transformers' processor and as the oracle, written into `scores` in place,
+    the other scores untouched."""
+    from transformers.generation.logits_process import NoRepeatNGramLogitsProcessor
+
+    from oslo_amd.fused_kernels_utils import FusedNoRepeatNGramLogitsProcessor
+
+    for length in (1, 2, 3, 5, 17, 40):
+        tokens = random_tokens(6, length, 7, seed=length * 10 + n)
+        scores = torch.randn(6, 7, generator=torch.Generator().manual_seed(length))
+        want = NoRepeatNGramLogitsProcessor(n)(tokens, scores.clone())
+        mine = scores.clone()
+        got = FusedNoRepeatNGramLogitsProcessor(n, 3, 2)(tokens, mine)
+        assert got.data_ptr() == mine.data_ptr()
+        assert torch.equal(got, want), (n, length)
+        assert torch.equal(got, oracle_scores(tokens, scores, n)), (n, length)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("n", [1, 2, 3, 5])
 @pytest.mark.parametrize("length", [1, 2, 4, 33, 257, 1500])
@@ -81,7 +102,7 @@ def test_kernel_argument_errors():
     with pytest.raises(RuntimeError):
         kernels.ngram_repeat_block_forward(tok, sc, 1, 4, 3, 2)          # rows != bsz * beam
     with pytest.raises(RuntimeError):
-        FusedNoRepeatNGramLogitsProcessor(2, 1, 2)(tok.cpu(), sc.cpu())  # no CPU path
+        FusedNoRepeatNGramLogitsProcessor(2, 1, 2)(tok.cpu(), sc)        # one on the host, one on the device
     with pytest.raises(ValueError):
         FusedNoRepeatNGramLogitsProcessor(0, 1, 2)
     # token ids outside the vocabulary are ignored, not written
