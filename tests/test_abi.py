@@ -68,7 +68,7 @@ def test_softmax_row_limit_is_on_rows_not_elements(lib):
     """A call takes at most 2^31 - 1 rows (batch * heads * S); more is refused
     with OSLO_E_UNSUPPORTED before any pointer is looked at. The number of
     elements is not limited: the gate admits [32,16,2048,2048] (2^31 elements)
-    and [2,16,8192,8192] (2^32)."""
+    and [4,16,8192,8192] (2^32)."""
     import torch
 
     from oslo_amd import FusedScaleMaskSoftmax
@@ -84,7 +84,7 @@ def test_softmax_row_limit_is_on_rows_not_elements(lib):
     assert rows_ok * 8 < 2 ** 31
     for dtype in (torch.half, torch.bfloat16, torch.float32):
         assert FusedScaleMaskSoftmax.is_available(dtype, 32, 16, 2048, 2048, True)
-        assert FusedScaleMaskSoftmax.is_available(dtype, 2, 16, 8192, 8192, True)
+        assert FusedScaleMaskSoftmax.is_available(dtype, 4, 16, 8192, 8192, True)
         assert FusedScaleMaskSoftmax.is_available(dtype, 64, 16, 2048, 1024, False)
         assert not FusedScaleMaskSoftmax.is_available(dtype, 2 ** 16, 2 ** 12, 8, 8, True)   # 2^31 rows
         assert FusedScaleMaskSoftmax.is_available(dtype, 2 ** 16 - 1, 2 ** 12, 8, 8, True)
