@@ -282,6 +282,22 @@ int oslo_bias_dropout_add_fwd(void *out, const void *x, const void *bias,
                               oslo_stream_t stream);
 
 /*
+ * The same with a second residual:
+ * out = keep * (x + bias) / (1-p) + residual + residual2, the sum formed in
+ * fp32 in that order and rounded once. residual2 may be NULL (then exactly
+ * oslo_bias_dropout_add_fwd); with residual2 given, residual must be too.
+ * For GPT-J's block, whose output is attention output + feed-forward output +
+ * residual stream (oslo/models/gptj/modeling_gptj.py:319-320; the reference
+ * adds the three with two torch additions, each rounding to the storage
+ * type). The backward is oslo_bias_dropout_add_bwd: both residuals receive g.
+ */
+int oslo_bias_dropout_add2_fwd(void *out, const void *x, const void *bias,
+                               const void *residual, const void *residual2,
+                               float p, uint64_t philox_seed,
+                               uint64_t philox_offset, int64_t rows,
+                               int64_t cols, int dtype, oslo_stream_t stream);
+
+/*
  * dx[r,c] = keep[r,c] * g[r,c] / (1-p) with the mask regenerated from the same
  * (seed, offset); if dbias != NULL, dbias[c] = sum_r dx[r,c] (workspace as for
  * oslo_bias_gelu_bwd). The gradient of the residual is g itself. dx may alias

@@ -347,9 +347,10 @@ def dropout_keep_mask(seed, offset, n, p, start=0):
     return dropout_bits(seed, offset, n, start) >= np.uint32(dropout_threshold(p))
 
 
-def bias_dropout_add_fwd(x, bias, residual, p, keep, dtype=np.float32):
-    """F.dropout(x + bias, p) + residual with the keep mask given. keep: bool
-    array of x's shape (ignored when p == 0)."""
+def bias_dropout_add_fwd(x, bias, residual, p, keep, dtype=np.float32, residual2=None):
+    """F.dropout(x + bias, p) + residual (+ residual2, the third term of GPT-J's
+    block sum, oslo/models/gptj/modeling_gptj.py:319-320) with the keep mask
+    given. keep: bool array of x's shape (ignored when p == 0)."""
     t = _acc(dtype)
     out = np.asarray(x, dtype=dtype)
     if bias is not None:
@@ -359,6 +360,8 @@ def bias_dropout_add_fwd(x, bias, residual, p, keep, dtype=np.float32):
         out = np.where(keep, out * scale, t(0))
     if residual is not None:
         out = out + np.asarray(residual, dtype=dtype)
+    if residual2 is not None:
+        out = out + np.asarray(residual2, dtype=dtype)
     return out
 
 

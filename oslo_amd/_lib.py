@@ -46,6 +46,8 @@ PROTOTYPES = {
         _c.c_int, [_P, _P, _P, _P, _P, _I64, _I64, _c.c_int, _P]),
     "oslo_bias_dropout_add_fwd": (
         _c.c_int, [_P, _P, _P, _P, _c.c_float, _U64, _U64, _I64, _I64, _c.c_int, _P]),
+    "oslo_bias_dropout_add2_fwd": (
+        _c.c_int, [_P, _P, _P, _P, _P, _c.c_float, _U64, _U64, _I64, _I64, _c.c_int, _P]),
     "oslo_bias_dropout_add_bwd": (
         _c.c_int, [_P, _P, _P, _P, _c.c_float, _U64, _U64, _I64, _I64, _c.c_int, _P]),
     "oslo_rotary_qkv": (

@@ -48,9 +48,8 @@ constexpr float kLog2e = 1.4426950408889634f;
 // lane's sum of 16 exponentials: none of them exceeds the sum, and a sum above
 // 2^kSlack means a score more than kSlack - 4 = kRaise above the maximum, so
 // that doing such a tile again in plain order (redo_tile) does raise it.
-constexpr float kSlack = 8.0f;
 constexpr float kRaise = 4.0f;
-constexpr float kSumLimit = 256.0f; // 2^kSlack
+constexpr float kSumLimit = 256.0f; // 2^kSlack, kSlack = 8
 // The reference of a query that has not seen a key yet (sliding windows): any
 // finite score lies more than kRaise above it, and 2^(score - floor) is +inf.
 constexpr float kReferenceFloor = -3.0e38f;
@@ -101,7 +100,6 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   constexpr int kSteps = D / 16;   // contraction steps of Q K^T
   constexpr int kBlocksD = D / 32; // 32-row blocks of O^T
   constexpr int kLoadsK = kKeysPerTile * kChunks / kBlockThreads; // per thread and tile
-  constexpr int kRowsPerPass = kBlockThreads / kChunks;
   constexpr int kTile = kKeysPerTile * D;      // elements of a K or V buffer
   constexpr int kRowBytes = D * (int)sizeof(T);
   constexpr int kKeyShift = D == 64 ? 1 : 0;   // rows of 128 bytes: two keys share a set of banks

@@ -742,13 +742,13 @@ def _next_philox(device):
 
 class _BiasDropoutAdd(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, bias, residual, p):
+    def forward(ctx, x, bias, residual, p, residual2=None):
         if p > 0.0:
             seed, offset = _next_philox(x.device)
         else:
             seed, offset = 0, 0
         ctx.p, ctx.seed, ctx.offset = p, seed, offset
-        return get_custom_kernels().bias_dropout_add_forward(x, bias, residual, p, seed, offset)
+        return get_custom_kernels().bias_dropout_add_forward(x, bias, residual, p, seed, offset, residual2)
 
     @staticmethod
     @once_differentiable
@@ -760,24 +760,28 @@ class _BiasDropoutAdd(torch.autograd.Function):
                 grad_output, ctx.p, ctx.seed, ctx.offset, want_dbias
             )
         dres = grad_output if ctx.needs_input_grad[2] else None
-        return dx, dbias, dres, None
+        dres2 = grad_output if ctx.needs_input_grad[4] else None
+        return dx, dbias, dres, None, dres2
 
 
-def _bias_dropout_add(x, bias, residual, training, drop_prop):
+def _bias_dropout_add(x, bias, residual, training, drop_prop, residual2=None):
     p = float(drop_prop) if training else 0.0
     if not x.is_cuda:
         raise RuntimeError(f"expected a tensor on a ROCm device, got {x.device} (this library has no CPU path)")
     if p < 0.0 or p > 1.0:
         raise ValueError(f"dropout probability has to be between 0 and 1, but got {p}")
+    if residual is None and residual2 is not None:
+        residual, residual2 = residual2, None
     if p == 1.0:  # everything dropped: F.dropout returns zeros
         out = torch.zeros_like(x)
-        return out if residual is None else out + residual
+        out = out if residual is None else out + residual
+        return out if residual2 is None else out + residual2
     if p == 0.0 and bias is None and residual is None:
         return x  # nothing to add and nothing to drop
-    if not _needs_grad(x, bias, residual):
+    if not _needs_grad(x, bias, residual, residual2):
         seed, offset = _next_philox(x.device) if p > 0.0 else (0, 0)
-        return get_custom_kernels().bias_dropout_add_forward(x, bias, residual, p, seed, offset)
-    return _BiasDropoutAdd.apply(x, bias, residual, p)
+        return get_custom_kernels().bias_dropout_add_forward(x, bias, residual, p, seed, offset, residual2)
+    return _BiasDropoutAdd.apply(x, bias, residual, p, residual2)
 
 
 class FusedBiasDropout(object):
@@ -800,11 +804,16 @@ class FusedBiasDropoutResidual(object):
 
     Before fusion: MLP FFN2 -> (Bias Addition -> Dropout -> Residual Addition) -> LayerNorm -> ...
     After fusion: MLP FFN2 -> Fused Bias Dropout Residual -> LayerNorm -> ...
+
+    ``residual2`` (not in the reference's signature, optional): a second tensor
+    added in the same pass, for blocks whose output is a sum of three terms
+    (GPT-J: attention output + feed-forward output + residual stream). The sum
+    is formed in fp32 and rounded once.
     """
 
     @staticmethod
-    def apply(x, bias, residual, training, drop_prop):
-        return _bias_dropout_add(x, bias, residual, training, drop_prop)
+    def apply(x, bias, residual, training, drop_prop, residual2=None):
+        return _bias_dropout_add(x, bias, residual, training, drop_prop, residual2)
 
 
 # ---------------------------------------------------------------------------

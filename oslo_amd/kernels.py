@@ -351,21 +351,32 @@ def bias_gelu_backward(grad, y, bias, want_dbias=True):
     return dy, dbias
 
 
-def bias_dropout_add_forward(x, bias, residual, p, seed, offset):
+def bias_dropout_add_forward(x, bias, residual, p, seed, offset, residual2=None):
+    """dropout(x + bias, p) + residual (+ residual2): every term but x may be
+    None; a second residual needs a first. The sum is formed in fp32 and
+    rounded once."""
     rows, cols, code = _as_rows_cols(x, bias, "input")
     x = x.contiguous()
     if bias is not None:
         bias = bias.contiguous()
-    if residual is not None:
-        _device_tensor(residual, "residual", x)
-        _require(residual.shape == x.shape and residual.dtype == x.dtype,
-                 "residual and input differ in shape or dtype")
-        residual = residual.contiguous()
+    _require(residual2 is None or residual is not None, "a second residual without a first")
+    res = []
+    for what, r in (("residual", residual), ("residual2", residual2)):
+        if r is not None:
+            _device_tensor(r, what, x)
+            _require(r.shape == x.shape and r.dtype == x.dtype, f"{what} and input differ in shape or dtype")
+            r = r.contiguous()
+        res.append(r)
     out = torch.empty_like(x, requires_grad=False)
     with _on_device(x):
-        _lib.check(_lib.load().oslo_bias_dropout_add_fwd(
-            _ptr(out), _ptr(x), _ptr(bias), _ptr(residual), float(p), int(seed), int(offset),
-            rows, cols, code, _stream(x)))
+        if res[1] is None:
+            _lib.check(_lib.load().oslo_bias_dropout_add_fwd(
+                _ptr(out), _ptr(x), _ptr(bias), _ptr(res[0]), float(p), int(seed), int(offset),
+                rows, cols, code, _stream(x)))
+        else:
+            _lib.check(_lib.load().oslo_bias_dropout_add2_fwd(
+                _ptr(out), _ptr(x), _ptr(bias), _ptr(res[0]), _ptr(res[1]), float(p), int(seed), int(offset),
+                rows, cols, code, _stream(x)))
     return out
 
 

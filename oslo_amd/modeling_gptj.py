@@ -268,24 +268,27 @@ class GPTJMLP(nn.Module):
 class FusedGPTJMLP(GPTJMLP):
     """oslo/models/gptj/modeling_gptj.py:1041-1065."""
 
-    def forward(self, x, residual=None):
-        """``residual``: added to the output (the residual connection of the block)."""
+    def forward(self, x, residual=None, residual2=None):
+        """``residual``, ``residual2``: added to the output (the residual
+        connection of the block and, for the block's three-term sum, the
+        attention output)."""
         if FusedLinearRows.is_available(x, self.fc_in.weight, self.fc_in.bias) and \
                 FusedLinearRows.is_available(None, self.fc_out.weight, self.fc_out.bias, rows_of=x):
             # a decoding step: each projection is one pass over its weight with
             # the bias (and the activation, and the residual) applied to the fp32 sums
             x = FusedLinearRows.apply(x, self.fc_in.weight, self.fc_in.bias, self.config.activation_function)
-            if not (self.training and self.dropout.p > 0.0):
+            if residual2 is None and not (self.training and self.dropout.p > 0.0):
                 return FusedLinearRows.apply(x, self.fc_out.weight, self.fc_out.bias, residual=residual)
             x = FusedLinearRows.apply(x, self.fc_out.weight)
         else:
             x = x @ self.fc_in.weight.t()
             x = FusedBiasActivation.apply(x, self.fc_in.bias, self.config.activation_function)
             x = x @ self.fc_out.weight.t()
-        if residual is None:
+        if residual is None and residual2 is None:
             return FusedBiasDropout.apply(x, self.fc_out.bias, self.training, self.dropout.p)
-        # bias, dropout and the block's residual addition in one pass
-        return FusedBiasDropoutResidual.apply(x, self.fc_out.bias, residual, self.training, self.dropout.p)
+        # bias, dropout and the block's residual addition(s) in one pass
+        return FusedBiasDropoutResidual.apply(x, self.fc_out.bias, residual, self.training, self.dropout.p,
+                                              residual2)
 
 
 class GPTJBlock(nn.Module):
@@ -306,18 +309,28 @@ class GPTJBlock(nn.Module):
 
 
 class FusedGPTJBlock(GPTJBlock):
-    """The block with its residual additions handed to the fused modules,
-    which take them into their last projection's launch in a decoding step:
-    attention output + residual first, then the feed-forward output on top (the
-    unfused block adds attention, feed-forward and residual in that order,
-    oslo/models/gptj/modeling_gptj.py:306-327). No counterpart in the
-    reference, which fuses attention and MLP only
-    (oslo/models/gptj/configuration_gptj.py:155-167)."""
+    """The block with its residual additions handed to the fused modules. The
+    unfused block adds attention output, feed-forward output and residual
+    stream with two torch additions (oslo/models/gptj/modeling_gptj.py:306-327).
+    Over a prompt (and in training) the feed-forward's epilogue kernel takes
+    all three: bias + dropout of its own term, then the attention output and
+    the residual stream, summed in fp32 and rounded once -- one rounding at the
+    magnitude of the residual stream per layer, as in the unfused block (adding
+    the attention output into the stream first and the feed-forward output in a
+    second pass rounds there twice, and 28 layers of it showed in the logits).
+    In a decoding step the two modules take the additions into the launches of
+    their last projections instead (attention output + residual first, the
+    feed-forward output on top). No counterpart in the reference, which fuses
+    attention and MLP only (oslo/models/gptj/configuration_gptj.py:155-167)."""
 
     def forward(self, hidden_states, layer_past=None, attention_mask=None, head_mask=None, use_cache=False):
         if not (isinstance(self.attn, FusedGPTJAttention) and isinstance(self.mlp, FusedGPTJMLP)):
             return super().forward(hidden_states, layer_past, attention_mask, head_mask, use_cache)
         normed = self.ln_1(hidden_states)
+        if hidden_states.shape[-2] > 1 and hidden_states.is_cuda:
+            a = self.attn(normed, layer_past=layer_past, attention_mask=attention_mask, head_mask=head_mask,
+                          use_cache=use_cache)
+            return self.mlp(normed, residual=hidden_states, residual2=a[0]), a[1]
         a = self.attn(normed, layer_past=layer_past, attention_mask=attention_mask, head_mask=head_mask,
                       use_cache=use_cache, residual=hidden_states)
         return self.mlp(normed, residual=a[0]), a[1]

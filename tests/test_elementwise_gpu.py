@@ -86,6 +86,53 @@ def test_bias_dropout_add_forward_backward(rows, cols, dtype, p):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("rows,cols", [(1, 8), (37, 264), (64, 1000), (129, 4096), (5, 7)])
+def test_bias_dropout_add_two_residuals(rows, cols, dtype):
+    """out = dropout(x + bias) + residual + residual2 in one pass (GPT-J's block
+    sum): against the oracle with the kernel's keep mask; at p = 0 the exact
+    fp32 sum of the four terms rounded once; without a bias; and through the
+    operator under autograd, where both residuals receive the gradient itself."""
+    from oslo_amd import FusedBiasDropoutResidual
+
+    seed, offset, p = 99, 4, 0.25
+    x, res, res2 = (randn((rows, cols), dtype, seed=rows + cols + i) for i in range(3))
+    b = randn((cols,), dtype, seed=cols, std=0.02)
+    keep = orc.dropout_keep_mask(seed, offset, rows * cols, p).reshape(rows, cols)
+    dev = [t.to(DEV) for t in (x, b, res, res2)]
+    out = kernels.bias_dropout_add_forward(dev[0], dev[1], dev[2], p, seed, offset, dev[3])
+    want = orc.bias_dropout_add_fwd(f32(x), f32(b), f32(res), p, keep, residual2=f32(res2))
+    assert_close(out, want, dtype, f"two residuals {rows}x{cols}")
+    out = kernels.bias_dropout_add_forward(dev[0], None, dev[2], p, seed, offset, dev[3])
+    assert_close(out, orc.bias_dropout_add_fwd(f32(x), None, f32(res), p, keep, residual2=f32(res2)), dtype)
+    exact = kernels.bias_dropout_add_forward(dev[0], dev[1], dev[2], 0.0, 0, 0, dev[3])
+    if dtype == torch.float32:
+        want0 = ((x + b) + res) + res2                       # the kernel's order of fp32 additions
+    else:
+        want0 = (x.double() + b.double() + res.double() + res2.double())
+        # (the fp32 sum of four 16-bit values may be off the exact sum by an fp32 ulp before its one rounding)
+        assert (exact.cpu().double() - want0).abs().max() <= (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11) * \
+            want0.abs().max() + 1e-6
+        want0 = None
+    if want0 is not None:
+        assert torch.equal(exact.cpu(), want0)
+    with pytest.raises(RuntimeError):
+        kernels.bias_dropout_add_forward(dev[0], dev[1], None, p, seed, offset, dev[3])   # second without first
+    # the operator: reference signature plus the optional second residual
+    xs = [t.clone().requires_grad_(True) for t in dev]
+    torch.manual_seed(5)
+    y = FusedBiasDropoutResidual.apply(xs[0], xs[1], xs[2], True, p, xs[3])
+    go = randn((rows, cols), dtype, seed=7).to(DEV)
+    y.backward(go)
+    assert torch.equal(xs[2].grad, go) and torch.equal(xs[3].grad, go)
+    dropped = f32(xs[0].grad) == 0
+    assert_close(xs[0].grad, np.where(dropped, 0.0, f32(go) / (1 - p)), dtype, "dx")
+    assert abs(dropped.mean() - p) <= 0.2 or rows * cols < 200
+    # in eval mode the operator is the plain four-term sum
+    y0 = FusedBiasDropoutResidual.apply(dev[0], dev[1], dev[2], False, p, dev[3])
+    assert torch.equal(y0, exact)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
 def test_bias_dropout_add_p0_is_exact(dtype):
     x = randn((37, 264), dtype, seed=1)
     res = randn((37, 264), dtype, seed=2)

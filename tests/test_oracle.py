@@ -302,8 +302,17 @@ def test_bias_dropout_add_closed_forms():
     b = r.standard_normal(10)
     # p = 0: exactly x + b + res
     np.testing.assert_array_equal(orc.bias_dropout_add_fwd(x, b, res, 0.0, None, dtype=np.float64), x + b + res)
+    # a second residual is one more term of the same sum, whatever the dropout: the block sum of GPT-J
+    res2 = r.standard_normal((6, 10))
+    np.testing.assert_array_equal(orc.bias_dropout_add_fwd(x, b, res, 0.0, None, dtype=np.float64, residual2=res2),
+                                  x + b + res + res2)
     keep = r.random((6, 10)) < 0.7
     p = 0.3
+    np.testing.assert_allclose(
+        orc.bias_dropout_add_fwd(x, b, res, p, keep, dtype=np.float64, residual2=res2),
+        (torch.from_numpy(x + b) * torch.from_numpy(keep) / (1 - float(np.float32(p)))
+         + torch.from_numpy(res) + torch.from_numpy(res2)).numpy(),
+        rtol=1e-12)
     out = orc.bias_dropout_add_fwd(x, b, res, p, keep, dtype=np.float64)
     # same as torch: (x + b) * mask / (1 - p) + res
     want = (torch.from_numpy(x + b) * torch.from_numpy(keep) / (1 - float(np.float32(p)))
