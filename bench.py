@@ -35,8 +35,10 @@ HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 # Matrix products per visible (query, key) tile that the attention backward's
 # passes issue, by head size (oslo_amd/csrc/attention_prefill_bwd.hip: the dQ
-# pass 3, the dK pass 3, the dV pass 2); the mathematics has 5.
-BWD_PRODUCTS_ISSUED = {64: 8, 128: 8, 256: 8}
+# pass 3, then dK and dV in one pass 4, or at 256 features, where both
+# accumulators do not fit a lane's registers, 3 + 2 in two passes); the
+# mathematics has 5.
+BWD_PRODUCTS_ISSUED = {64: 7, 128: 7, 256: 8}
 
 # HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` and
 # `--pmc WRITE_SIZE` (KiB per dispatch, scaled by the reading of a 1 GiB copy
@@ -87,7 +89,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gptj", action="store_true", help="skip the GPT-J-6B-shaped forward comparison")
-    ap.add_argument("--only", default="", help="run only the named kernel of the table (for profiling)")
+    ap.add_argument("--only", default="",
+                    help="run only the named kernel of the table, or one model-level pass "
+                         "(gptj_fwd_fused, gptj_fwd_unfused, gptj_train_fused, gptj_train_unfused), for profiling")
     ap.add_argument("--zero-operands", action="store_true",
                     help="with --only attention_prefill: q, k, v of zeros (clock and power readings)")
     return ap.parse_args()
@@ -533,6 +537,9 @@ def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
     """--only causal_fwd | causal_bwd | attention_prefill | copy: launch one kernel `steps` times
     (profiling runs). `copy` is torch's device copy of 1 GiB, the kernel of
     known traffic that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
+    if args.only.startswith("gptj_"):
+        model_pass_only(args, torch, dev)
+        return
     if args.only == "copy":
         a = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
         b = torch.empty_like(a)
@@ -556,6 +563,53 @@ def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
         fwd()
     t = time_launches(fn, args.steps, args.warmup)
     print(json.dumps({"only": args.only, "us": round(t * 1e6, 2), "launches": args.steps}))
+
+
+def model_pass_only(args, torch, dev):
+    """--only gptj_fwd_fused | gptj_fwd_unfused: `steps` forward passes of the
+    GPT-J-6B-shaped model of the `gptj_fwd` section (28 layers, batch 8 x 2048,
+    eval), after fuse() or before it; --only gptj_train_fused |
+    gptj_train_unfused: `steps` forward + backward passes of the 4-layer stack
+    of the `gptj_train_step` section (attention and residual dropout 0.1).
+    Nothing else runs: a kernel trace of the command is the model's kernel mix."""
+    from oslo_amd import GPTJConfig, GPTJForCausalLM
+
+    what, fused = args.only.rsplit("_", 1)
+    if what not in ("gptj_fwd", "gptj_train") or fused not in ("fused", "unfused"):
+        sys.exit("--only takes gptj_fwd_fused, gptj_fwd_unfused, gptj_train_fused or gptj_train_unfused")
+    train = what == "gptj_train"
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(dev):
+            torch.manual_seed(0)
+            cfg = GPTJConfig(n_layer=4, attn_pdrop=0.1, resid_pdrop=0.1) if train else GPTJConfig(n_layer=28)
+            model = GPTJForCausalLM(cfg)
+    finally:
+        torch.set_default_dtype(old)
+    model = model.train() if train else model.eval()
+    if fused == "fused":
+        model.fuse()
+    ids = torch.randint(0, 50400, (8, 2048), device=dev)
+
+    def run():
+        if train:
+            model.zero_grad(set_to_none=True)
+            model(ids, labels=ids)["loss"].backward()
+        else:
+            with torch.no_grad():
+                model(ids)
+
+    for _ in range(args.warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    print(json.dumps({"only": args.only, "ms": round(ms, 2), "tokens_per_s": round(8 * 2048 / ms * 1e3, 1),
+                      "passes": args.steps}))
 
 
 def gptj_forward(torch, dev, layers=28, batch=8, seq=2048, reps=5):

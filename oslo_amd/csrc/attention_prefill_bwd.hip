@@ -27,8 +27,10 @@
 // the own position are per-lane scalars, those indexed by the other position
 // are read per tile from LDS. Each block sums in a fixed order and no two
 // blocks write the same element: the gradients are deterministic. The price is
-// that scores are computed once per gradient: dQ takes three matrix products
-// per visible (query, key) tile, dK three, dV two, 8 instead of 5.
+// that scores are computed once per owner kind: dQ takes three matrix products
+// per visible (query, key) tile and dK and dV together four (7 instead of 5)
+// where one pass can hold both accumulators (heads of 64 and 128 features);
+// at 256 features dK takes three and dV two in passes of their own (8).
 //
 // The kernel is built the way the forward is: tiles of 32 positions of the
 // other kind loaded straight into LDS (four buffers per tensor), stored as they
@@ -48,7 +50,16 @@ namespace {
 constexpr int kOwnPerBlock = 128;
 constexpr float kLog2eB = 1.4426950408889634f;
 
-enum Role { kRoleDQ = 0, kRoleDK = 1, kRoleDV = 2 };
+// kRoleDKV: dK and dV in one pass (both own keys and walk queries: the scores
+// and the probabilities are computed once for the two, 4 products per tile
+// where the two passes have 5; it needs both accumulators in registers).
+enum Role { kRoleDQ = 0, kRoleDK = 1, kRoleDV = 2, kRoleDKV = 3 };
+
+// Blocks per CU the kernel is compiled for (a wave per SIMD each).
+constexpr int bwd_blocks_per_cu(int D, int role) {
+  if (role == kRoleDKV) return D == 256 ? 1 : D == 128 ? 1 : 2;
+  return D == 256 ? 1 : D == 128 ? 2 : 3;
+}
 
 struct Strides3 {
   int64_t b, h, s; // element strides: batch, head, position
@@ -76,13 +87,14 @@ constexpr unsigned sched_lds_bytes() {
 }
 
 template <typename T, int D, int ROLE, bool HAS_PAD, bool HAS_WINDOW, bool DROP>
-__global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) void attention_bwd_kernel(
+__global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void attention_bwd_kernel(
     const BwdArgs a) {
-  static_assert(ROLE == kRoleDQ || ROLE == kRoleDK || ROLE == kRoleDV, "one gradient per pass");
+  static_assert(ROLE >= kRoleDQ && ROLE <= kRoleDKV, "unknown pass");
   using Op = MatrixOp<T>;
   using Frag = typename Op::Frag;
   constexpr bool kKeysOwn = ROLE != kRoleDQ;
   constexpr bool kNeedT2 = ROLE != kRoleDV;
+  constexpr bool kTwoAcc = ROLE == kRoleDKV; // acc = dK^T, acc2 = dV^T
   constexpr int kChunks = D / 8;   // 16-byte chunks of a position
   constexpr int kSteps = D / 16;   // contraction steps over the features
   constexpr int kBlocksD = D / 32; // 32-row blocks of the accumulator
@@ -289,17 +301,26 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     return __builtin_bit_cast(Frag, __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
-  f32x16 acc[kBlocksD];
+  f32x16 acc[kBlocksD], acc2[kTwoAcc ? kBlocksD : 1];
 #pragma unroll
   for (int i = 0; i < kBlocksD; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
-  Frag xf[2]; // what the accumulating product takes of the last tile computed: P or P o (dP - delta)
+  if constexpr (kTwoAcc) {
+#pragma unroll
+    for (int i = 0; i < kBlocksD; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc2[i][r] = 0.f;
+  }
+  // what the accumulating products take of the last tile computed: xf = P (dV
+  // pass) or P o (dP - delta); in the combined pass xp = P as well
+  Frag xf[2], xp[2];
 
   // which tensor the accumulating product reads transposed: K (dQ), Q (dK), dO (dV)
   auto transposed_tile = [&](int d) __attribute__((always_inline)) {
     return (ROLE == kRoleDV ? o2_lds : o1_lds) + buffer_of(d) * kTile;
   };
+  auto transposed_tile2 = [&](int d) __attribute__((always_inline)) { return o2_lds + buffer_of(d) * kTile; }; // dO (combined pass)
   // slice `n` of `slices` of a tile's elementwise work: P = exp2(scale*log2e *
   // T1 + pad*log2e - lse), X = P (dV) or P (T2 - delta) (the scale goes onto
   // the result). With attention dropout the forward multiplied V with
@@ -322,7 +343,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
       if constexpr (kKeysOwn && kNeedT2) row_b[r] = rows[kRowSlots];
     }
   };
-  auto elementwise = [&]<bool MASKED>(f32x16 &t1, const f32x16 &t2, int n, int slices, Frag (&x)[2])
+  auto elementwise = [&]<bool MASKED>(f32x16 &t1, f32x16 &t2, int n, int slices, Frag (&x)[2], Frag (&x2)[2])
                          __attribute__((always_inline)) {
     if constexpr (DROP) {
       if (n == 0) {
@@ -358,21 +379,33 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
         p = visible ? p : 0.f;
       }
       float grad = t2[r];
+      float kept = p; // the probability the values met (the combined pass keeps it beside dS)
       if constexpr (DROP) {
         const bool keep = kKeysOwn ? ((keep_words[r >> 2][r & 3] >> col) & 1u) != 0
                                    : ((keep_bits >> (8 * (r >> 2) + (r & 3))) & 1u) != 0;
         grad = keep ? grad * a.drop.keep_scale : 0.f;
         if constexpr (!kNeedT2) p = keep ? p : 0.f;
+        if constexpr (kTwoAcc) kept = keep ? p : 0.f;
       }
       if constexpr (kNeedT2) p *= grad - delta_r;
       t1[r] = p;
       asm volatile("" : "+v"(t1[r])); // (keeps the computation in its slice)
+      if constexpr (kTwoAcc) {
+        t2[r] = kept;
+        asm volatile("" : "+v"(t2[r]));
+      }
     }
     if (n == slices - 1) {
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int i = 0; i < 8; ++i) x[u][i] = static_cast<T>(t1[8 * u + i]);
+      if constexpr (kTwoAcc) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) x2[u][i] = static_cast<T>(t2[8 * u + i]);
+      }
     }
   };
 
@@ -403,7 +436,7 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
     }
 #pragma unroll
     for (int r = 0; r < kAhead; ++r) read_row_values(r);
-    elementwise.template operator()<true>(t1, t2, 0, 1, xf);
+    elementwise.template operator()<true>(t1, t2, 0, 1, xf, xp);
     ++t;
   }
 
@@ -414,15 +447,22 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   auto scheduled_tile = [&]<bool MASKED>() __attribute__((always_inline)) {
     constexpr int kRing = 4;
     constexpr int kProducts = 2 * kBlocksD;
-    constexpr int kOperands = kSteps + (kNeedT2 ? kSteps : 0) + kProducts;
+    // the combined pass: the products of dV^T (dO^T x P) first, then those of dK^T (Q^T x dS)
+    constexpr int kAccProducts = (kTwoAcc ? 2 : 1) * kProducts;
+    constexpr int kOperands = kSteps + (kNeedT2 ? kSteps : 0) + kAccProducts;
     constexpr int kPerStep = (kItems + kSteps - 1) / kSteps;
     const T *b1 = o1_lds + buffer_of(0) * kTile, *b2 = o2_lds + buffer_of(0) * kTile;
     const T *bt = transposed_tile(-1);
+    const T *bt2 = transposed_tile2(-1);
     Frag ring[kRing];
     auto read_operand = [&](int p) __attribute__((always_inline)) {
       if (p < kSteps) ring[p % kRing] = read_natural(b1, p);
       else if (kNeedT2 && p < 2 * kSteps) ring[p % kRing] = read_natural(b2, p - kSteps);
-      else ring[p % kRing] = read_transposed(bt, p - (kNeedT2 ? 2 : 1) * kSteps);
+      else {
+        const int q = p - (kNeedT2 ? 2 : 1) * kSteps;
+        if (kTwoAcc && q < kProducts) ring[p % kRing] = read_transposed(bt2, q);
+        else ring[p % kRing] = read_transposed(bt, q - (kTwoAcc ? kProducts : 0));
+      }
     };
 #pragma unroll
     for (int p = 0; p < kRing; ++p) read_operand(p);
@@ -447,18 +487,24 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    Frag xn[2];
+    Frag xn[2], xpn[2];
 #pragma unroll
     for (int r = 0; r < kAhead; ++r) read_row_values(r);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int n = 0; n < kProducts; ++n, ++p) {
-      acc[n % kBlocksD] = Op::run(ring[p % kRing], xf[n / kBlocksD], acc[n % kBlocksD]);
+    for (int n = 0; n < kAccProducts; ++n, ++p) {
+      if (kTwoAcc && n < kProducts) {
+        acc2[n % kBlocksD] = Op::run(ring[p % kRing], xp[n / kBlocksD], acc2[n % kBlocksD]);
+      } else {
+        const int m = n - (kTwoAcc ? kProducts : 0);
+        acc[m % kBlocksD] = Op::run(ring[p % kRing], xf[m / kBlocksD], acc[m % kBlocksD]);
+      }
       if (p + kRing < kOperands) read_operand(p + kRing);
-      elementwise.template operator()<MASKED>(t1, t2, n, kProducts, xn);
+      elementwise.template operator()<MASKED>(t1, t2, n, kAccProducts, xn, xpn);
       __builtin_amdgcn_sched_barrier(0);
     }
     xf[0] = xn[0], xf[1] = xn[1];
+    if constexpr (kTwoAcc) xp[0] = xpn[0], xp[1] = xpn[1];
   };
   // each kind of tile in a loop of its own
   auto run_tiles = [&]<bool MASKED>(int end) __attribute__((always_inline)) {
@@ -476,6 +522,12 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
   __syncthreads();
   {
     const T *bt = transposed_tile(-1);
+    if constexpr (kTwoAcc) {
+      const T *bt2 = transposed_tile2(-1);
+#pragma unroll
+      for (int n = 0; n < 2 * kBlocksD; ++n)
+        acc2[n % kBlocksD] = Op::run(read_transposed(bt2, n), xp[n / kBlocksD], acc2[n % kBlocksD]);
+    }
 #pragma unroll
     for (int n = 0; n < 2 * kBlocksD; ++n)
       acc[n % kBlocksD] = Op::run(read_transposed(bt, n), xf[n / kBlocksD], acc[n % kBlocksD]);
@@ -483,19 +535,27 @@ __global__ __launch_bounds__(kBlockThreads, D == 256 ? 1 : D == 128 ? 2 : 3) voi
 
   if (own >= S) return;
   typedef T Out4 __attribute__((ext_vector_type(4)));
-  const Strides3 &st_out = ROLE == kRoleDQ ? a.sdq : ROLE == kRoleDK ? a.sdk : a.sdv;
-  void *out_base = ROLE == kRoleDQ ? a.dq : ROLE == kRoleDK ? a.dk : a.dv;
-  const float factor = kNeedT2 ? a.scale : DROP ? a.drop.keep_scale : 1.0f;
-  T *op = static_cast<T *>(out_base) + b * st_out.b + hd * st_out.h + (int64_t)own * st_out.s;
+  auto store = [&](const f32x16 (&sums)[kBlocksD], void *out_base, const Strides3 &st_out, float factor)
+                   __attribute__((always_inline)) {
+    T *op = static_cast<T *>(out_base) + b * st_out.b + hd * st_out.h + (int64_t)own * st_out.s;
 #pragma unroll
-  for (int i = 0; i < kBlocksD; ++i)
+    for (int i = 0; i < kBlocksD; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      Out4 w;
+      for (int j = 0; j < 4; ++j) {
+        Out4 w;
 #pragma unroll
-      for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(acc[i][4 * j + tt] * factor);
-      *reinterpret_cast<Out4 *>(op + 32 * i + 8 * j + 4 * half) = w;
-    }
+        for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(sums[i][4 * j + tt] * factor);
+        *reinterpret_cast<Out4 *>(op + 32 * i + 8 * j + 4 * half) = w;
+      }
+  };
+  const float p_factor = DROP ? a.drop.keep_scale : 1.0f; // the 1/(1-p) of the kept probabilities
+  if constexpr (ROLE == kRoleDQ) store(acc, a.dq, a.sdq, a.scale);
+  else if constexpr (ROLE == kRoleDK) store(acc, a.dk, a.sdk, a.scale);
+  else if constexpr (ROLE == kRoleDV) store(acc, a.dv, a.sdv, p_factor);
+  else {
+    store(acc, a.dk, a.sdk, a.scale);
+    store(acc2, a.dv, a.sdv, p_factor);
+  }
 }
 
 template <typename T, int D, int ROLE>
@@ -553,12 +613,22 @@ int launch_bwd_dim(const BwdArgs &a, float *delta, const void *out, const Stride
       delta, static_cast<const T *>(out), static_cast<const T *>(a.dout), so, a.sdo, a.S, a.heads, rows);
   int s = check_launch("attention_prefill_bwd(delta)");
   if (s != OSLO_OK) return s;
-  // a pass per gradient
   s = launch_role<T, D, kRoleDQ>(a, stream);
   if (s != OSLO_OK) return s;
-  s = launch_role<T, D, kRoleDK>(a, stream);
-  if (s != OSLO_OK) return s;
-  return launch_role<T, D, kRoleDV>(a, stream);
+  // dK and dV: one combined pass where both accumulators fit a lane's registers
+  // (heads of 64 and 128 features: 2 x 32 and 2 x 64 accumulator registers; timed
+  // at [8,32,2048,64] 692 against 816 us for the whole backward, at [8,16,2048,128]
+  // 635 against 648, with dropout 778 against 873). At 256 features they are 2 x
+  // 128 beside 128 registers of fixed operands: the compiler spills 47 to 178
+  // registers per lane, 39 scratch accesses in every tile, and the backward takes
+  // 2917 us instead of 1382; there each gradient keeps a pass of its own.
+  if constexpr (D <= 128) {
+    return launch_role<T, D, kRoleDKV>(a, stream);
+  } else {
+    s = launch_role<T, D, kRoleDK>(a, stream);
+    if (s != OSLO_OK) return s;
+    return launch_role<T, D, kRoleDV>(a, stream);
+  }
 }
 
 template <typename T>
