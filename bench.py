@@ -534,7 +534,8 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
 
 
 def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
-    """--only causal_fwd | causal_bwd | attention_prefill | copy: launch one kernel `steps` times
+    """--only causal_fwd | causal_bwd | attention_prefill | attention_prefill_bwd | copy: launch one kernel
+    (the backward: its four) `steps` times
     (profiling runs). `copy` is torch's device copy of 1 GiB, the kernel of
     known traffic that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
     if args.only.startswith("gptj_"):
@@ -544,6 +545,21 @@ def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
         a = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
         b = torch.empty_like(a)
         fn = lambda: b.copy_(a)
+    elif args.only == "attention_prefill_bwd":
+        import ctypes
+        B, Hh, S, D = 8, 16, 2048, 256  # the GPT-J shape of the kernel table
+        q, k, v, do = (torch.randn(B, Hh, S, D, device=dev).to(torch.bfloat16) for _ in range(4))
+        o = torch.empty((B, Hh, S, D), dtype=torch.bfloat16, device=dev)
+        lse = torch.empty((B, Hh, S), dtype=torch.float32, device=dev)
+        dense = [Hh * S * D, S * D, D]
+        check(lib.oslo_attention_prefill_fwd_lse(P(o), P(lse), P(q), P(k), P(v), None, D ** -0.5, 0.0, 0, 0,
+                                                 B, Hh, S, D, 0, (ctypes.c_int64 * 12)(*(4 * dense)), 2, st))
+        dq, dk, dv = (torch.empty_like(q) for _ in range(3))
+        ws = torch.empty(lib.oslo_attention_prefill_bwd_workspace_bytes(B, Hh, S) // 4, dtype=torch.float32, device=dev)
+        bstr = (ctypes.c_int64 * 24)(*(8 * dense))
+        fn = lambda: check(lib.oslo_attention_prefill_bwd(
+            P(dq), P(dk), P(dv), P(do), P(q), P(k), P(v), P(o), P(lse), P(ws), None, D ** -0.5, 0.0, 0, 0,
+            B, Hh, S, D, 0, bstr, 2, st))
     elif args.only == "attention_prefill":
         import ctypes
         B, Hh, S, D = 8, 16, 2048, 256  # the GPT-J shape of the kernel table
@@ -558,7 +574,7 @@ def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
     else:
         fn = {"causal_fwd": fwd, "causal_bwd": bwd}.get(args.only)
     if fn is None:
-        sys.exit("--only takes causal_fwd, causal_bwd, attention_prefill or copy")
+        sys.exit("--only takes causal_fwd, causal_bwd, attention_prefill, attention_prefill_bwd, copy or a gptj_* pass")
     if args.only == "causal_bwd":
         fwd()
     t = time_launches(fn, args.steps, args.warmup)

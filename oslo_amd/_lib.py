@@ -7,7 +7,10 @@ build fails, oslo/fused_kernels_utils.py:226-230)."""
 import ctypes
 import os
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "liboslo_amd.so")
+# The library lies beside this file. OSLO_AMD_LIB names another build of it
+# (``python -m oslo_amd.build`` writes there too when the variable is set): a
+# library built with other tuning switches, for measurements.
+LIB_PATH = os.environ.get("OSLO_AMD_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "liboslo_amd.so")
 
 _c = ctypes
 _P = _c.c_void_p

@@ -7,6 +7,13 @@ ahead of time for gfx950 only and loaded with ctypes; nothing is compiled when
 a model runs.
 
     python -m oslo_amd.build
+
+Two environment variables make a second build for measurements without
+touching the one in the tree: ``OSLO_AMD_LIB=/some/where/lib.so`` is where the
+library is written (and where ``oslo_amd._lib`` then loads it from), and
+``OSLO_BWD_COMBINED_MAX_DIM=256`` compiles the attention backward with dK and
+dV in one pass at head_dim 256 as well (it spills there; the default, 128, is
+what measures fastest).
 """
 
 import os
@@ -15,8 +22,9 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "liboslo_amd.so")
-OBJ_DIR = os.path.join(CSRC, "build")
+_VARIANT = os.environ.get("OSLO_AMD_LIB")
+LIB_PATH = _VARIANT or os.path.join(os.path.dirname(os.path.abspath(__file__)), "liboslo_amd.so")
+OBJ_DIR = (_VARIANT + ".objs") if _VARIANT else os.path.join(CSRC, "build")
 
 SOURCES = [
     "runtime.hip",
@@ -61,6 +69,9 @@ EXTRA_FLAGS = {
     "attention_prefill.hip": ["-Wno-inline-asm"],
     "attention_prefill_bwd.hip": ["-Wno-inline-asm"],
 }
+if os.environ.get("OSLO_BWD_COMBINED_MAX_DIM"):
+    EXTRA_FLAGS["attention_prefill_bwd.hip"].append(
+        "-DOSLO_BWD_COMBINED_MAX_DIM=" + str(int(os.environ["OSLO_BWD_COMBINED_MAX_DIM"])))
 
 
 def _compile(src):

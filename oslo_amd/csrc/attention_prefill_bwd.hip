@@ -47,6 +47,12 @@
 namespace oslo {
 namespace {
 
+// Largest head size whose dK and dV share a pass (a build switch for
+// measurements: 256 compiles the combined pass there too, where it spills).
+#ifndef OSLO_BWD_COMBINED_MAX_DIM
+#define OSLO_BWD_COMBINED_MAX_DIM 128
+#endif
+
 constexpr int kOwnPerBlock = 128;
 constexpr float kLog2eB = 1.4426950408889634f;
 
@@ -622,7 +628,7 @@ int launch_bwd_dim(const BwdArgs &a, float *delta, const void *out, const Stride
   // 128 beside 128 registers of fixed operands: the compiler spills 47 to 178
   // registers per lane, 39 scratch accesses in every tile, and the backward takes
   // 2917 us instead of 1382; there each gradient keeps a pass of its own.
-  if constexpr (D <= 128) {
+  if constexpr (D <= OSLO_BWD_COMBINED_MAX_DIM) {
     return launch_role<T, D, kRoleDKV>(a, stream);
   } else {
     s = launch_role<T, D, kRoleDK>(a, stream);
