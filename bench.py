@@ -93,7 +93,7 @@ def parse():
                     help="run only the named kernel of the table, or one model-level pass "
                          "(gptj_fwd_fused, gptj_fwd_unfused, gptj_train_fused, gptj_train_unfused), for profiling")
     ap.add_argument("--zero-operands", action="store_true",
-                    help="with --only attention_prefill: q, k, v of zeros (clock and power readings)")
+                    help="with --only attention_prefill or gemm: operands of zeros (clock and power readings)")
     return ap.parse_args()
 
 
@@ -360,7 +360,8 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         n_el = rows * cols
         n_sets = 1 if 6 * n_el >= (1 << 30) else 4
         sets = [(randn((rows, cols), 10 * i, 1.0, torch.bfloat16), randn((rows, cols), 10 * i + 1, 1.0, torch.bfloat16),
-                 torch.empty((rows, cols), dtype=torch.bfloat16, device=dev)) for i in range(n_sets)]
+                 torch.empty((rows, cols), dtype=torch.bfloat16, device=dev),
+                 randn((rows, cols), 10 * i + 2, 1.0, torch.bfloat16)) for i in range(n_sets)]
         bias = randn((cols,), 3, 0.02, torch.bfloat16)
         db = torch.empty_like(bias)
         ws = torch.empty(lib.oslo_colsum_workspace_bytes(rows, cols) // 4, dtype=torch.float32, device=dev)
@@ -378,6 +379,10 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
             P(b[2]), P(db), P(ws), P(b[1]), 0.1, 1234, 0, rows, cols, BF16, st))), n, 3)
         res.append(roof(f"bias_dropout_add_bwd+dbias p=0.1 {shape}", 4 * n_el, t, n_el, n_sets))
         if n_sets > 1:
+            # GPT-J's three-term block sum in the same pass: dropout(x + bias) + residual + a second residual
+            t = time_launches(rotating(sets, lambda b: check(lib.oslo_bias_dropout_add2_fwd(
+                P(b[2]), P(b[0]), P(bias), P(b[1]), P(b[3]), 0.1, 1234, 0, rows, cols, BF16, st))), n, 3)
+            res.append(roof(f"bias_dropout_add2_fwd (two residuals) p=0.1 {shape}", 8 * n_el, t, n_el, n_sets))
             # without the bias gradient (one launch, no partial rows): what the second launch and the
             # partial rows of the rows above cost at this size
             t = time_launches(rotating(sets, lambda b: check(lib.oslo_bias_gelu_bwd(
@@ -534,7 +539,7 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
 
 
 def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
-    """--only causal_fwd | causal_bwd | attention_prefill | attention_prefill_bwd | copy: launch one kernel
+    """--only causal_fwd | causal_bwd | attention_prefill | attention_prefill_bwd | gemm | copy: launch one kernel
     (the backward: its four) `steps` times
     (profiling runs). `copy` is torch's device copy of 1 GiB, the kernel of
     known traffic that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
@@ -545,6 +550,13 @@ def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
         a = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
         b = torch.empty_like(a)
         fn = lambda: b.copy_(a)
+    elif args.only == "gemm":
+        # the calibration of the matrix-core rows: the library's dense bf16 GEMM, 8192^3
+        ga, gb = (torch.randn(8192, 8192, device=dev).to(torch.bfloat16) for _ in range(2))
+        if args.zero_operands:
+            ga.zero_(), gb.zero_()
+        gc = torch.empty_like(ga)
+        fn = lambda: torch.matmul(ga, gb, out=gc)
     elif args.only == "attention_prefill_bwd":
         import ctypes
         B, Hh, S, D = 8, 16, 2048, 256  # the GPT-J shape of the kernel table
@@ -574,7 +586,7 @@ def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
     else:
         fn = {"causal_fwd": fwd, "causal_bwd": bwd}.get(args.only)
     if fn is None:
-        sys.exit("--only takes causal_fwd, causal_bwd, attention_prefill, attention_prefill_bwd, copy or a gptj_* pass")
+        sys.exit("--only takes causal_fwd, causal_bwd, attention_prefill, attention_prefill_bwd, gemm, copy or a gptj_* pass")
     if args.only == "causal_bwd":
         fwd()
     t = time_launches(fn, args.steps, args.warmup)
