@@ -110,6 +110,11 @@ def test_argument_screening_without_a_device(lib):
     assert lib.oslo_bias_dropout_add_fwd(one, one, null, null, 1.0, 1, 0, 4, 8, 1, null) == -1
     assert lib.oslo_bias_dropout_add_fwd(one, one, null, null, -0.1, 1, 0, 4, 8, 1, null) == -1
     assert lib.oslo_bias_dropout_add_bwd(one, null, null, one, float("nan"), 1, 0, 4, 8, 1, null) == -1
+    # a second residual needs a first; the variant screens like the one-residual entry
+    assert lib.oslo_bias_dropout_add2_fwd(one, one, null, null, one, 0.1, 1, 0, 4, 8, 1, null) == -1
+    assert b"second residual" in lib.oslo_last_error()
+    assert lib.oslo_bias_dropout_add2_fwd(one, one, null, one, one, 1.0, 1, 0, 4, 8, 1, null) == -1
+    assert lib.oslo_bias_dropout_add2_fwd(null, null, null, null, null, 0.1, 1, 0, 0, 8, 1, null) == 0
     # softmax with fused dropout: p, the statistics buffer, sizes
     assert lib.oslo_softmax_causal_dropout_fwd(one, one, one, null, 1.0, 1.0, 1, 0, 1, 1, 8, 1, null) == -1
     assert lib.oslo_softmax_causal_dropout_fwd(one, null, one, null, 1.0, 0.1, 1, 0, 1, 1, 8, 1, null) == -1
