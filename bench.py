@@ -46,39 +46,42 @@ BWD_PRODUCTS_ISSUED = {64: 7, 128: 7, 256: 8}
 # profiles/bench_kernels_hbm_traffic.md and, for the two kernels of the step,
 # profiles/causal_softmax_fp16_8x16x2048x2048_hbm_traffic.md.
 MEASURED_TRAFFIC = {
-    "linear_rows fc_in + bias + gelu bf16 1 x [16384,4096]": 134699021,
-    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135284935,
-    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134601375,
-    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136610080,
-    "linear_rows attention projection bf16 1 x [4096,4096]": 33740800,
-    "linear_rows attention projection bf16 8 x [4096,4096]": 34370560,
-    "attention_decode bf16 1 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 17573904,
-    "attention_decode bf16 8 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 136477708,
-    "causal_fwd fp16 [8,16,2048,2048]": 1627471921,
-    "causal_bwd fp16 [8,16,2048,2048]": 2181120049,
-    "causal_fwd bf16 [8,16,2048,2048]": 1627459649,
-    "causal_bwd bf16 [8,16,2048,2048] (in place)": 2181120131,
-    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635900143,
-    "causal_dropout_bwd p=0.1 bf16 [8,16,2048,2048] (in place)": 2214719508,
+    "causal_fwd fp16 [8,16,2048,2048]": 1627471923,
+    "causal_bwd fp16 [8,16,2048,2048]": 2181120048,
+    "causal_fwd bf16 [8,16,2048,2048]": 1627459656,
+    "causal_bwd bf16 [8,16,2048,2048] (in place)": 2181120137,
+    "causal_dropout_fwd p=0.1 bf16 [8,16,2048,2048]": 1635900230,
+    "causal_dropout_bwd p=0.1 bf16 [8,16,2048,2048] (in place)": 2214719499,
     "causal_fwd fp32 [8,16,2048,2048]": 3238067310,
-    "causal_bwd fp32 [8,16,2048,2048] (in place)": 4328580380,
-    "causal_fwd bf16 [1,16,8192,8192]": 3229695246,
-    "masked_fwd bf16 [16,16,1024,1024] key mask": 1082175281,
+    "causal_bwd fp32 [8,16,2048,2048] (in place)": 4328580363,
+    "causal_fwd bf16 [1,16,8192,8192]": 3229695250,
+    "masked_fwd bf16 [16,16,1024,1024] key mask": 1082271801,
     "masked_bwd bf16 [16,16,1024,1024]": 1610650634,
-    "bias_gelu_fwd bf16 [16384,16384]": 1073876258,
-    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677948211,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610759309,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141068691,
-    "bias_gelu_fwd bf16 [16384,4096]": 268493592,
-    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419584569,
-    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402709938,
-    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285361651,
-    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807983113,
-    "causal_fwd bf16 [8,16,2048,2048] with padding mask": 1628022937,
-    "causal_window_fwd window 256 bf16 [8,16,2048,2048]": 1230656579,
-    "causal_window_bwd window 256 bf16 [8,16,2048,2048] (in place)": 1387504736,
+    "bias_gelu_fwd bf16 [16384,16384]": 1073877195,
+    "bias_gelu_bwd+dbias bf16 [16384,16384]": 1677948106,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,16384]": 1610758935,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,16384]": 1141071052,
+    "bias_gelu_fwd bf16 [16384,4096]": 268493535,
+    "bias_gelu_bwd+dbias bf16 [16384,4096]": 419584379,
+    "bias_dropout_add_fwd p=0.1 bf16 [16384,4096]": 402709849,
+    "bias_dropout_add_bwd+dbias p=0.1 bf16 [16384,4096]": 285361737,
+    "bias_dropout_add2_fwd (two residuals) p=0.1 bf16 [16384,4096]": 536945004,
+    "bias_gelu_bwd without dbias bf16 [16384,4096]": 402744320,
+    "bias_dropout_add_bwd without dbias p=0.1 bf16 [16384,4096]": 268517376,
+    "rotary_qkv bf16 q,k,v [8,2048,16,256] rotary 64": 807985633,
+    "causal_fwd bf16 [8,16,2048,2048] with padding mask": 1628022852,
+    "causal_window_fwd window 256 bf16 [8,16,2048,2048]": 1230656581,
+    "causal_window_bwd window 256 bf16 [8,16,2048,2048] (in place)": 1387504650,
     "causal_fwd bf16 [4,16,4096,4096]": 3238084608,
     "causal_bwd bf16 [4,16,4096,4096] (in place)": 4328603740,
+    "linear_rows fc_in + bias + gelu bf16 1 x [16384,4096]": 134699022,
+    "linear_rows fc_in + bias + gelu bf16 8 x [16384,4096]": 135284935,
+    "linear_rows fc_out + bias bf16 1 x [4096,16384]": 134600960,
+    "linear_rows fc_out + bias bf16 8 x [4096,16384]": 136611520,
+    "linear_rows attention projection bf16 1 x [4096,4096]": 33740800,
+    "linear_rows attention projection bf16 8 x [4096,4096]": 34370560,
+    "attention_decode bf16 1 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 17573905,
+    "attention_decode bf16 8 x 16 heads, 1024 of 1152 keys, head 256 (two launches)": 136477703,
 }
 
 
