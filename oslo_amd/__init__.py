@@ -11,6 +11,7 @@ from .fused_kernels_utils import (  # noqa: F401
     FusedDecodeAttention,
     FusedPrefillAttention,
     FusedKernelMixin,
+    FusedLinearBiasActivation,
     FusedLinearRows,
     FusedMergeHeads,
     FusedNoRepeatNGramLogitsProcessor,

@@ -14,7 +14,7 @@ import torch
 from torch import nn
 
 from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedBiasDropoutResidual,
-                                 FusedDecodeAttention, FusedLinearRows, FusedPrefillAttention,
+                                 FusedDecodeAttention, FusedLinearBiasActivation, FusedLinearRows, FusedPrefillAttention,
                                  FusedMergeHeads,
                                  FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedSplitHeads)
@@ -255,8 +255,13 @@ class FusedGPT2MLP(GPT2MLP):
                                              residual=residual)
             x = FusedLinearRows.apply(x, self.c_proj.weight, conv1d=True)
         else:
-            x = x @ self.c_fc.weight
-            x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
+            act = self.config.activation_function
+            if FusedLinearBiasActivation.is_available(x, self.c_fc.weight, self.c_fc.bias, act):
+                # bias and GeLU on the product's fp32 sums, in its own launch
+                x = FusedLinearBiasActivation.apply(x, self.c_fc.weight, self.c_fc.bias, act, conv1d=True)
+            else:
+                x = x @ self.c_fc.weight
+                x = FusedBiasActivation.apply(x, self.c_fc.bias, act)
             x = x @ self.c_proj.weight
         if residual is None:
             return FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)

@@ -17,7 +17,7 @@ import torch
 from torch import nn
 
 from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedBiasDropoutResidual,
-                                 FusedDecodeAttention, FusedLinearRows, FusedPrefillAttention,
+                                 FusedDecodeAttention, FusedLinearBiasActivation, FusedLinearRows, FusedPrefillAttention,
                                  FusedMergeHeads,
                                  FusedRotaryPositionEmbedding, FusedScaleMaskSoftmax,
                                  FusedScaleMaskSoftmaxDropout, FusedScaleMaskWindowSoftmax)
@@ -260,8 +260,13 @@ class FusedGPTNeoMLP(GPTNeoMLP):
                 return FusedLinearRows.apply(x, self.c_proj.weight, self.c_proj.bias, residual=residual)
             x = FusedLinearRows.apply(x, self.c_proj.weight)
         else:
-            x = x @ self.c_fc.weight.t()
-            x = FusedBiasActivation.apply(x, self.c_fc.bias, self.config.activation_function)
+            act = self.config.activation_function
+            if FusedLinearBiasActivation.is_available(x, self.c_fc.weight, self.c_fc.bias, act):
+                # bias and GeLU on the product's fp32 sums, in its own launch
+                x = FusedLinearBiasActivation.apply(x, self.c_fc.weight, self.c_fc.bias, act)
+            else:
+                x = x @ self.c_fc.weight.t()
+                x = FusedBiasActivation.apply(x, self.c_fc.bias, act)
             x = x @ self.c_proj.weight.t()
         if residual is None:
             return FusedBiasDropout.apply(x, self.c_proj.bias, self.training, self.dropout.p)

@@ -19,7 +19,7 @@ import torch
 from torch import nn
 
 from .fused_kernels_utils import (FusedBiasActivation, FusedBiasDropout, FusedBiasDropoutResidual,
-                                 FusedDecodeAttention, FusedLinearRows, FusedPrefillAttention,
+                                 FusedDecodeAttention, FusedLinearBiasActivation, FusedLinearRows, FusedPrefillAttention,
                                  FusedMergeHeads,
                                  FusedRotaryPositionEmbedding,
                                  FusedScaleMaskSoftmax, FusedScaleMaskSoftmaxDropout)
@@ -281,8 +281,13 @@ class FusedGPTJMLP(GPTJMLP):
                 return FusedLinearRows.apply(x, self.fc_out.weight, self.fc_out.bias, residual=residual)
             x = FusedLinearRows.apply(x, self.fc_out.weight)
         else:
-            x = x @ self.fc_in.weight.t()
-            x = FusedBiasActivation.apply(x, self.fc_in.bias, self.config.activation_function)
+            act = self.config.activation_function
+            if FusedLinearBiasActivation.is_available(x, self.fc_in.weight, self.fc_in.bias, act):
+                # bias and GeLU on the product's fp32 sums, in its own launch
+                x = FusedLinearBiasActivation.apply(x, self.fc_in.weight, self.fc_in.bias, act)
+            else:
+                x = x @ self.fc_in.weight.t()
+                x = FusedBiasActivation.apply(x, self.fc_in.bias, act)
             x = x @ self.fc_out.weight.t()
         if residual is None and residual2 is None:
             return FusedBiasDropout.apply(x, self.fc_out.bias, self.training, self.dropout.p)

@@ -210,3 +210,37 @@ def test_full_size_bias_gelu_and_dropout_properties():
     assert torch.equal(o[dropped], res[dropped])                # dropped elements are the residual, exactly
     dx, db = kernels.bias_dropout_add_backward(x, p, 1234, 0)
     assert torch.count_nonzero(dx[dropped]) == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS.get)
+@pytest.mark.parametrize("conv1d", [False, True], ids=["linear", "conv1d"])
+def test_linear_bias_gelu_in_the_products_launch(dtype, conv1d):
+    """FusedLinearBiasActivation (bias and GeLU applied by the matrix product
+    itself, where autograd records nothing) against the float64 oracle of
+    tanh-GeLU(x . W + b), beside product + bias-GeLU kernel on the same inputs:
+    it is the tanh form (the error form differs from it by up to 2e-4 at
+    these magnitudes) and, rounded once, it is at least as close."""
+    from oslo_amd.fused_kernels_utils import FusedBiasActivation, FusedLinearBiasActivation
+
+    m, k, n = 48, 256, 384
+    x = randn((2, m // 2, k), dtype, seed=3)
+    w = randn((n, k), dtype, seed=4, std=1.0 / 16)
+    b = randn((n,), dtype, seed=5, std=0.5)
+    want = orc.linear_rows(f32(x).reshape(m, k), f32(w), f32(b), gelu=True)
+    weight = (w.t().contiguous() if conv1d else w).to(DEV)
+    xd, bd = x.to(DEV), b.to(DEV)
+    assert FusedLinearBiasActivation.is_available(xd, weight, bd, "gelu_new")
+    out = FusedLinearBiasActivation.apply(xd, weight, bd, "gelu_new", conv1d=conv1d)
+    assert out.shape == (2, m // 2, n) and out.dtype == dtype
+    two = FusedBiasActivation.apply(xd @ (weight if conv1d else weight.t()), bd, "gelu_new")
+    err = np.abs(f32(out).reshape(m, n).astype(np.float64) - want)
+    err_two = np.abs(f32(two).reshape(m, n).astype(np.float64) - want)
+    if dtype == torch.float32:
+        assert err.max() <= 2e-5, err.max()      # fp32 sums of 256 products of magnitude up to 1
+    else:
+        assert_close(out.reshape(m, n), want, dtype, "linear + bias + gelu")
+        assert err.mean() <= err_two.mean() * 1.02, (err.mean(), err_two.mean())
+    # recorded by autograd: not available, the callers keep the kernel with its backward
+    assert not FusedLinearBiasActivation.is_available(xd.requires_grad_(), weight, bd, "gelu_new")
+    assert not FusedLinearBiasActivation.is_available(xd.detach(), weight, bd, "relu")
+    assert not FusedLinearBiasActivation.is_available(xd.detach(), weight, None, "gelu_new")

@@ -426,3 +426,27 @@ def test_decoding_step_falls_back_when_only_the_second_projection_fits_no_kernel
         got = m(ids, use_cache=True)
         got_step = m(ids[:, :1], past_key_values=got["past_key_values"])["logits"].float()
     assert (got_step - want_step).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("family", ["gpt2", "gptj", "gpt_neo"])
+def test_mlp_takes_the_products_epilogue_at_inference_and_the_kernel_in_training(family, monkeypatch):
+    """Without gradients the fused MLP's first projection applies bias and
+    GeLU in the matrix product's launch; with gradients it is product +
+    bias-GeLU kernel (whose backward reads the product)."""
+    torch.manual_seed(0)
+    m = models()[family]().to(DEV, torch.bfloat16).eval().fuse()
+    ids = torch.randint(0, 512, (2, 48), device=DEV)
+    epilogue, kernel = [], []
+    real_e, real_k = fku.FusedLinearBiasActivation.apply, fku.FusedBiasActivation.apply
+    monkeypatch.setattr(fku.FusedLinearBiasActivation, "apply",
+                        staticmethod(lambda *a, **kw: (epilogue.append(1), real_e(*a, **kw))[1]))
+    monkeypatch.setattr(fku.FusedBiasActivation, "apply",
+                        staticmethod(lambda *a, **kw: (kernel.append(1), real_k(*a, **kw))[1]))
+    with torch.no_grad():
+        quiet = m(ids)["logits"]
+    assert len(epilogue) == 2 and not kernel
+    epilogue.clear()
+    recorded = m(ids)["logits"]
+    assert len(kernel) == 2 and not epilogue
+    recorded.float().square().mean().backward()
+    assert (quiet.float() - recorded.float()).abs().max().item() <= 0.05
