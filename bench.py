@@ -560,7 +560,7 @@ def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
             ga.zero_(), gb.zero_()
         gc = torch.empty_like(ga)
         fn = lambda: torch.matmul(ga, gb, out=gc)
-    elif args.only == "attention_prefill_bwd":
+    elif args.only in ("attention_prefill_bwd", "attention_prefill_bwd_recompute"):
         import ctypes
         B, Hh, S, D = 8, 16, 2048, 256  # the GPT-J shape of the kernel table
         q, k, v, do = (torch.randn(B, Hh, S, D, device=dev).to(torch.bfloat16) for _ in range(4))
@@ -572,9 +572,16 @@ def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
         dq, dk, dv = (torch.empty_like(q) for _ in range(3))
         ws = torch.empty(lib.oslo_attention_prefill_bwd_workspace_bytes(B, Hh, S) // 4, dtype=torch.float32, device=dev)
         bstr = (ctypes.c_int64 * 24)(*(8 * dense))
-        fn = lambda: check(lib.oslo_attention_prefill_bwd(
-            P(dq), P(dk), P(dv), P(do), P(q), P(k), P(v), P(o), P(lse), P(ws), None, D ** -0.5, 0.0, 0, 0,
-            B, Hh, S, D, 0, bstr, 2, st))
+        if args.only.endswith("_recompute"):  # every pass computes its scores: nothing of [S, S] in memory
+            fn = lambda: check(lib.oslo_attention_prefill_bwd(
+                P(dq), P(dk), P(dv), P(do), P(q), P(k), P(v), P(o), P(lse), P(ws), None, D ** -0.5, 0.0, 0, 0,
+                B, Hh, S, D, 0, bstr, 2, st))
+        else:  # what the operator runs at this head size: P and dS handed to the dK/dV pass through a tile store
+            store_bytes = lib.oslo_attention_prefill_bwd_store_bytes(B, Hh, S)
+            store = torch.empty(store_bytes, dtype=torch.uint8, device=dev)
+            fn = lambda: check(lib.oslo_attention_prefill_bwd_stored(
+                P(dq), P(dk), P(dv), P(do), P(q), P(k), P(v), P(o), P(lse), P(ws), P(store), store_bytes, None,
+                D ** -0.5, 0.0, 0, 0, B, Hh, S, D, 0, bstr, 2, st))
     elif args.only == "attention_prefill":
         import ctypes
         B, Hh, S, D = 8, 16, 2048, 256  # the GPT-J shape of the kernel table
@@ -589,7 +596,8 @@ def run_only(args, lib, torch, dev, st, P, check, time_launches, fwd, bwd):
     else:
         fn = {"causal_fwd": fwd, "causal_bwd": bwd}.get(args.only)
     if fn is None:
-        sys.exit("--only takes causal_fwd, causal_bwd, attention_prefill, attention_prefill_bwd, gemm, copy or a gptj_* pass")
+        sys.exit("--only takes causal_fwd, causal_bwd, attention_prefill, attention_prefill_bwd, "
+                 "attention_prefill_bwd_recompute, gemm, copy or a gptj_* pass")
     if args.only == "causal_bwd":
         fwd()
     t = time_launches(fn, args.steps, args.warmup)

@@ -539,6 +539,41 @@ int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const void *dout,
                                int64_t window, const int64_t *strides,
                                int dtype, oslo_stream_t stream);
 
+/*
+ * The same gradients with the probabilities handed from pass to pass through
+ * memory: the pass that computes dq also writes, for every tile of 32 queries
+ * x 32 keys on or below the diagonal, P (after dropout) and dS / scale in the
+ * storage type (4 KiB a tile) into `store`, and one more pass accumulates dk
+ * and dv from them: 5 matrix products per tile, where the entry point above
+ * computes the scores once per pass (7 or 8). The results obey the same
+ * formulas and the same rounding (P and dS are rounded to the storage type
+ * before the products either way), sums run in the same order, and they are
+ * as reproducible.
+ * store: store_bytes bytes, 16-byte aligned, contents irrelevant before and
+ * after. oslo_attention_prefill_bwd_store_bytes(batch, heads, S) holds every
+ * head at once; with less the heads are processed in groups of 8 x k, as many
+ * as fit, and oslo_attention_prefill_bwd_store_bytes(1, 8, S) is the least
+ * (less: OSLO_E_BAD_ARG). Everything else as above, workspace included.
+ * Replaces the same reference code as oslo_attention_prefill_bwd; autograd
+ * there keeps P and dS as whole [B, H, S, S] tensors between forward and
+ * backward, here they exist for the heads of one launch during the call.
+ */
+size_t oslo_attention_prefill_bwd_store_bytes(int64_t batch, int64_t heads,
+                                              int64_t S);
+int oslo_attention_prefill_bwd_stored(void *dq, void *dk, void *dv,
+                                      const void *dout, const void *q,
+                                      const void *k, const void *v,
+                                      const void *out, const float *lse,
+                                      float *workspace, void *store,
+                                      size_t store_bytes, const float *pad,
+                                      float scale, float p,
+                                      uint64_t philox_seed,
+                                      uint64_t philox_offset, int64_t batch,
+                                      int64_t heads, int64_t S,
+                                      int64_t head_dim, int64_t window,
+                                      const int64_t *strides, int dtype,
+                                      oslo_stream_t stream);
+
 /* Repeated n-gram blocking (beam search) ------------------------------------ */
 
 /*

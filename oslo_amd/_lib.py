@@ -74,6 +74,10 @@ PROTOTYPES = {
     "oslo_attention_prefill_bwd": (
         _c.c_int, [_P] * 11 + [_c.c_float, _c.c_float, _U64, _U64, _I64, _I64, _I64, _I64, _I64,
                                _c.POINTER(_c.c_int64), _c.c_int, _P]),
+    "oslo_attention_prefill_bwd_store_bytes": (_c.c_size_t, [_I64, _I64, _I64]),
+    "oslo_attention_prefill_bwd_stored": (
+        _c.c_int, [_P] * 11 + [_c.c_size_t, _P, _c.c_float, _c.c_float, _U64, _U64, _I64, _I64, _I64, _I64, _I64,
+                               _c.POINTER(_c.c_int64), _c.c_int, _P]),
     "oslo_ngram_repeat_block": (
         _c.c_int, [_P, _P, _I64, _I64, _I64, _I64, _c.c_int, _P]),
     "oslo_sample_idx_rows": (_I64, [_c.c_int32, _c.c_int32, _I64]),

@@ -42,6 +42,8 @@
 // gradients worked out between them. One permutation of a row's 16-byte chunks
 // serves both reads (f(row) below).
 
+#include <algorithm>
+
 #include "attention.hpp"
 
 namespace oslo {
@@ -81,7 +83,28 @@ struct BwdArgs {
   float scale, scale_log2e;
   int S, heads, batch_heads, head_groups, own_blocks, window;
   DropArgs drop; // attention dropout of the forward (the DROP variants)
+  // The passes that exchange the probabilities through memory (below): the
+  // tile store, the first head of the launch (a launch covers the heads
+  // [bh0, bh0 + 8 * head_groups) below batch_heads; tiles of head bh0 come
+  // first in the store), and the number of tiles a head has there.
+  unsigned char *tiles;
+  int bh0;
+  int64_t head_tiles;
 };
+
+// The tile store. P (after dropout) and dS / scale of the 32 queries x 32 keys of
+// query tile Qb and key tile Kb <= Qb of a head are 2 KiB each, one behind the
+// other at tile index Qb (Qb + 1) / 2 + Kb: [query][slot], slot 16 u + 8 h + i
+// holding key 16 u + 8 (i / 4) + 4 h + i % 4, which is what lane (query, half
+// h) of the pass that computes them holds as the B operands u = 0, 1 of its
+// own accumulating product, 16 bytes each. The pass that consumes them reads a
+// tile through the transposing LDS read, key slot in the lane.
+constexpr int kStoredTileBytes = 2048;                      // one of the two
+constexpr int kStoredPairBytes = 2 * kStoredTileBytes;      // P, then dS
+__host__ __device__ constexpr int64_t stored_head_tiles(int64_t own_blocks) {
+  const int64_t n = own_blocks * (kOwnPerBlock / 32);
+  return n * (n + 1) / 2;
+}
 
 constexpr int kSchedTile = 32;
 constexpr int kSchedBuffers = 4;
@@ -92,15 +115,17 @@ constexpr unsigned sched_lds_bytes() {
          kWavesPerBlock * 32u * sizeof(uint32_t);
 }
 
-template <typename T, int D, int ROLE, bool HAS_PAD, bool HAS_WINDOW, bool DROP>
+template <typename T, int D, int ROLE, bool HAS_PAD, bool HAS_WINDOW, bool DROP, bool STORE = false>
 __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void attention_bwd_kernel(
     const BwdArgs a) {
   static_assert(ROLE >= kRoleDQ && ROLE <= kRoleDKV, "unknown pass");
+  static_assert(!STORE || ROLE == kRoleDQ, "the pass that owns queries writes the tile store");
   using Op = MatrixOp<T>;
   using Frag = typename Op::Frag;
   constexpr bool kKeysOwn = ROLE != kRoleDQ;
   constexpr bool kNeedT2 = ROLE != kRoleDV;
   constexpr bool kTwoAcc = ROLE == kRoleDKV; // acc = dK^T, acc2 = dV^T
+  constexpr bool kKeepP = kTwoAcc || STORE;  // the probabilities are wanted beside dS
   constexpr int kChunks = D / 8;   // 16-byte chunks of a position
   constexpr int kSteps = D / 16;   // contraction steps over the features
   constexpr int kBlocksD = D / 32; // 32-row blocks of the accumulator
@@ -126,7 +151,7 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
 
   const int xcd = blockIdx.x & 7;
   const int slot = blockIdx.x >> 3;
-  const int bh = xcd + 8 * (slot % a.head_groups);
+  const int bh = a.bh0 + xcd + 8 * (slot % a.head_groups);
   const int idx = slot / a.head_groups;
   const int own_block = kKeysOwn ? idx : a.own_blocks - 1 - idx;
   if (bh >= a.batch_heads) return; // the whole block
@@ -173,14 +198,14 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
     }
   }
   const int64_t stat_row = (int64_t)bh * S;
-  float own_lse = 0.f, own_delta = 0.f, own_pad = 0.f; // (the padding value in log2 units)
+  float own_lse = 0.f, own_delta = 0.f, own_pad = 0.f; // (the padding value, floored)
   if constexpr (!kKeysOwn) {
     if (own < S) {
       own_lse = a.lse[stat_row + own];
       own_delta = a.delta[stat_row + own];
     }
   } else if constexpr (HAS_PAD) {
-    if (own < S) own_pad = fmaxf(a.pad[(int64_t)b * S + own], kMaskFloor) * kLog2eB;
+    if (own < S) own_pad = fmaxf(a.pad[(int64_t)b * S + own], kMaskFloor);
   }
 
   // Tiles [first_tile, tiles) of the other kind this block walks. Those before
@@ -370,7 +395,8 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
       if (r + kAhead < 16) read_row_values(r + kAhead);
       float shift, delta_r = own_delta;
       if constexpr (kKeysOwn) {
-        shift = own_pad - row_a[r];
+        // (the same fused multiply-add as in the pass that owns queries: every pass sees the same P, bit for bit)
+        shift = HAS_PAD ? __builtin_fmaf(own_pad, kLog2eB, -row_a[r]) : -row_a[r];
         if constexpr (kNeedT2) delta_r = row_b[r];
       } else if constexpr (HAS_PAD) {
         shift = __builtin_fmaf(fmaxf(row_a[r], kMaskFloor), kLog2eB, -own_lse);
@@ -391,12 +417,12 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
                                    : ((keep_bits >> (8 * (r >> 2) + (r & 3))) & 1u) != 0;
         grad = keep ? grad * a.drop.keep_scale : 0.f;
         if constexpr (!kNeedT2) p = keep ? p : 0.f;
-        if constexpr (kTwoAcc) kept = keep ? p : 0.f;
+        if constexpr (kKeepP) kept = keep ? p : 0.f;
       }
       if constexpr (kNeedT2) p *= grad - delta_r;
       t1[r] = p;
       asm volatile("" : "+v"(t1[r])); // (keeps the computation in its slice)
-      if constexpr (kTwoAcc) {
+      if constexpr (kKeepP) {
         t2[r] = kept;
         asm volatile("" : "+v"(t2[r]));
       }
@@ -406,7 +432,7 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
       for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int i = 0; i < 8; ++i) x[u][i] = static_cast<T>(t1[8 * u + i]);
-      if constexpr (kTwoAcc) {
+      if constexpr (kKeepP) {
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -414,6 +440,26 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
       }
     }
   };
+  // The wave's tiles of the store: query tile own0 / 32 + wave, key tile t. A
+  // tile that lies wholly above the diagonal has no place there (and holds zeros).
+  unsigned char *tile_row = nullptr;
+  const int own_tile = own0 / 32 + wave;
+  if constexpr (STORE)
+    tile_row = a.tiles + ((int64_t)(bh - a.bh0) * a.head_tiles + (int64_t)own_tile * (own_tile + 1) / 2) * kStoredPairBytes +
+               col * 64 + half * 16;
+  auto store_tiles = [&](const Frag (&ds)[2], const Frag (&pk)[2]) __attribute__((always_inline)) {
+    if constexpr (STORE) {
+      if (t <= own_tile) {
+        unsigned char *at = tile_row + (int64_t)t * kStoredPairBytes;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          *reinterpret_cast<Frag *>(at + 32 * u) = pk[u];
+          *reinterpret_cast<Frag *>(at + kStoredTileBytes + 32 * u) = ds[u];
+        }
+      }
+    }
+  };
+  constexpr int kStoresPerTile = STORE ? 4 : 0;
 
   // prologue: the first two tiles on their way
 #pragma unroll
@@ -443,6 +489,7 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
 #pragma unroll
     for (int r = 0; r < kAhead; ++r) read_row_values(r);
     elementwise.template operator()<true>(t1, t2, 0, 1, xf, xp);
+    store_tiles(xf, xp);
     ++t;
   }
 
@@ -510,12 +557,16 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
       __builtin_amdgcn_sched_barrier(0);
     }
     xf[0] = xn[0], xf[1] = xn[1];
-    if constexpr (kTwoAcc) xp[0] = xpn[0], xp[1] = xpn[1];
+    if constexpr (kKeepP) xp[0] = xpn[0], xp[1] = xpn[1];
+    store_tiles(xf, xp);
   };
   // each kind of tile in a loop of its own
   auto run_tiles = [&]<bool MASKED>(int end) __attribute__((always_inline)) {
     for (; t < end; ++t) {
-      wait_vm<kLoadsPerTile>();
+      // (vector-memory operations finish in order: behind the loads of tile t
+      // are those of tile t + 1 and the stores of the tile before this one)
+      if (!STORE || t - 1 <= own_tile) wait_vm<kLoadsPerTile + kStoresPerTile>();
+      else wait_vm<kLoadsPerTile>(); // (a wave past its diagonal stored nothing)
       __syncthreads(); // tile t is in LDS; the buffer written next (tile t - 2's) has been read
       scheduled_tile.template operator()<MASKED>();
     }
@@ -564,13 +615,13 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
   }
 }
 
-template <typename T, int D, int ROLE>
+template <typename T, int D, int ROLE, bool STORE = false>
 int launch_role(const BwdArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)(8 * a.head_groups * a.own_blocks));
   constexpr unsigned kLds = sched_lds_bytes<T, D, ROLE>();
   auto go = [&]<bool HAS_PAD, bool DROP>() -> int {
-    auto *kernel = a.window > 0 ? attention_bwd_kernel<T, D, ROLE, HAS_PAD, true, DROP>
-                                : attention_bwd_kernel<T, D, ROLE, HAS_PAD, false, DROP>;
+    auto *kernel = a.window > 0 ? attention_bwd_kernel<T, D, ROLE, HAS_PAD, true, DROP, STORE>
+                                : attention_bwd_kernel<T, D, ROLE, HAS_PAD, false, DROP, STORE>;
     if (kLds > 64u * 1024u) {
       const int s = raise_lds_limit(reinterpret_cast<const void *>(kernel), kLds, "oslo_attention_prefill_bwd");
       if (s != OSLO_OK) return s;
@@ -584,6 +635,224 @@ int launch_role(const BwdArgs &a, hipStream_t stream) {
   }
   if (a.drop.drop) return go.template operator()<false, true>();
   return go.template operator()<false, false>();
+}
+
+// dK and dV from the tile store: dK^T += Q^T dS and dV^T += dO^T P over the query
+// tiles from the diagonal on, nothing else: no scores, no exponentials, no
+// mask, no dropout (all of it is in the stored tiles). A block owns 128 keys
+// and has eight waves, two per SIMD: waves 0..3 accumulate dK of 32 keys each,
+// waves 4..7 dV of the same keys, so a wave holds one accumulator (D / 2
+// registers) and no fixed operands. The tiles of Q and dO go through LDS as in
+// the other passes (three buffers: tile t is read while t + 1 and t + 2 are on
+// their way), shared by the block; every wave loads its own 2 KiB tile of dS
+// or P beside them and reads it back transposed, key slot in the lane: lane c
+// holds the key at slot c of the store's rows, key c with bits 2 and 3 swapped.
+constexpr int kStoredWaves = 8;
+constexpr int kStoredThreads = kStoredWaves * kWave;
+constexpr int kStoredBuffers = 3;
+
+template <typename T, int D>
+constexpr unsigned stored_lds_bytes() {
+  return 2u * kStoredBuffers * kSchedTile * D * sizeof(T) + kStoredWaves * kStoredBuffers * kStoredTileBytes;
+}
+
+template <typename T, int D, bool HAS_WINDOW>
+__global__ __launch_bounds__(kStoredThreads, D == 64 ? 2 : 1) void attention_bwd_stored_kernel(const BwdArgs a) {
+  using Op = MatrixOp<T>;
+  using Frag = typename Op::Frag;
+  constexpr int kChunks = D / 8;
+  constexpr int kBlocksD = D / 32;
+  constexpr int kTile = kSchedTile * D;
+  constexpr int kRowBytes = D * (int)sizeof(T);
+  constexpr int kSwizzle = kChunks >= 16 ? 15 : 7;
+  constexpr int kLoadsN = kChunks / 8; // loads per thread and tile, Q and dO together (D = 64: a tensor per four waves)
+  constexpr int kItems = kLoadsN + 2;  // and the wave's own tile of the store
+  constexpr int kProducts = 2 * kBlocksD;
+
+  extern __shared__ __align__(1024) unsigned char lds_raw[];
+  T *const q_lds = reinterpret_cast<T *>(lds_raw);  // [3][query][chunk ^ f(query)][8]
+  T *const do_lds = q_lds + kStoredBuffers * kTile; // the same for dO
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int half = lane >> 5;
+  const int col = lane & 31;
+  const bool for_dv = wave >= 4;
+  const int key_wave = wave & 3;
+  unsigned char *const x_lds = reinterpret_cast<unsigned char *>(do_lds + kStoredBuffers * kTile) +
+                               wave * (kStoredBuffers * kStoredTileBytes); // [3][query][slot]
+
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  // The blocks of a head follow one another on one XCD, the longest walk
+  // first: the two or three heads an XCD works on at a time keep their Q and dO
+  // (2 x S x D values each) in its L2 while every block of the head reads them.
+  const int bh = a.bh0 + xcd + 8 * (slot / a.own_blocks);
+  const int own_block = slot % a.own_blocks;
+  if (bh >= a.batch_heads) return; // the whole block
+  const int b = bh / a.heads;
+  const int hd = bh - b * a.heads;
+  const int S = a.S;
+  const int own0 = own_block * kOwnPerBlock;
+  const int key_tile = own0 / 32 + key_wave;
+  const int window = HAS_WINDOW ? a.window : 0;
+
+  const int first_tile = own0 / kSchedTile;
+  int last_query = S - 1;
+  if (HAS_WINDOW && own0 + kOwnPerBlock - 1 + window - 1 < last_query) last_query = own0 + kOwnPerBlock - 1 + window - 1;
+  const int tiles = last_query / kSchedTile + 1;
+
+  const T *q_p = static_cast<const T *>(a.q) + b * a.sq.b + hd * a.sq.h;
+  const T *do_p = static_cast<const T *>(a.dout) + b * a.sdo.b + hd * a.sdo.h;
+  const uint32_t q_row = (uint32_t)a.sq.s * sizeof(T), do_row = (uint32_t)a.sdo.s * sizeof(T);
+  auto f_of = [](int r) __attribute__((always_inline)) { return (((r & 3) << 1) | ((r >> 2) & 1) | (r & 8)) & kSwizzle; };
+  // load j of a thread: entry (8 j + wave) * 64 + lane of [Q tile; dO tile]
+  // (a wave's 64 entries lie in one of the two tiles, so every load of a wave
+  // has one source tensor: a stream of tiles per load)
+  uint32_t src_off[kLoadsN];
+  TileStream src[kLoadsN];
+  uint32_t dst_off[kLoadsN]; // elements from q_lds, buffer 0
+#pragma unroll
+  for (int j = 0; j < kLoadsN; ++j) {
+    const int entry = (8 * j + wave) * kWave;
+    const bool is_do = entry >= kSchedTile * kChunks;
+    const int within = entry % (kSchedTile * kChunks) + lane;
+    const int row = within / kChunks, at = within % kChunks;
+    const uint32_t row_bytes = is_do ? do_row : q_row;
+    src_off[j] = (uint32_t)row * row_bytes + (uint32_t)(at ^ f_of(row)) * 16u;
+    const Strides3 &st = is_do ? a.sdo : a.sq;
+    src[j].start(is_do ? do_p : q_p, (uint32_t)(((int64_t)(S - 1) * st.s + D) * sizeof(T)), row_bytes, kSchedTile,
+                 first_tile, tiles);
+    dst_off[j] = (uint32_t)((is_do ? kStoredBuffers * kTile : 0) + (entry % (kSchedTile * kChunks)) * 8);
+  }
+  // The wave's tile of the store for query tile qt: nothing (zeros, without a
+  // memory access) where the pass that writes the store left none: above the
+  // diagonal, past the last query tile, and before the first key tile that the
+  // block owning qt walks under a window.
+  uint64_t store_at = reinterpret_cast<uint64_t>(a.tiles) +
+                      (uint64_t)(((int64_t)(bh - a.bh0) * a.head_tiles + (int64_t)first_tile * (first_tile + 1) / 2 + key_tile) *
+                                     kStoredPairBytes +
+                                 (for_dv ? 0 : kStoredTileBytes));
+  int store_tile = first_tile; // the query tile store_at belongs to
+  auto store_descriptor = [&]() __attribute__((always_inline)) {
+    bool there = store_tile >= key_tile && store_tile < tiles;
+    if constexpr (HAS_WINDOW) {
+      const int walk0 = (store_tile / 4) * kOwnPerBlock - window + 1;
+      there = there && key_tile >= (walk0 > 0 ? walk0 / kSchedTile : 0);
+    }
+    u32x4 d;
+    d[0] = __builtin_amdgcn_readfirstlane((uint32_t)store_at);
+    d[1] = __builtin_amdgcn_readfirstlane((uint32_t)(store_at >> 32) & 0xffffu);
+    d[2] = __builtin_amdgcn_readfirstlane(there ? (uint32_t)kStoredTileBytes : 0u);
+    d[3] = 0x00020000u;
+    return d;
+  };
+  int t = first_tile;
+  int buf_now = 0, buf_load = 0; // buffers of tile t and of the tile being loaded (t + 2 in the loop)
+  auto next_buffer = [](int b) __attribute__((always_inline)) { return b == kStoredBuffers - 1 ? 0 : b + 1; };
+  // item `it` of the loads of the next tile to load
+  auto stage_item = [&](int it) __attribute__((always_inline)) {
+    if (it < kLoadsN) {
+      lds_load_b128(src[it].descriptor(), q_lds + buf_load * kTile + dst_off[it], src_off[it]);
+      src[it].advance();
+      return;
+    }
+    it -= kLoadsN;
+    lds_load_b128(store_descriptor(), x_lds + buf_load * kStoredTileBytes + it * 1024, (uint32_t)(it * 1024 + lane * 16));
+    if (it == 1) {
+      store_at += (uint64_t)(store_tile + 1) * kStoredPairBytes;
+      ++store_tile;
+      buf_load = next_buffer(buf_load);
+    }
+  };
+
+  // transposed operands of the tiles of Q and dO (the passes above read them the same way)
+  typedef short Short4 __attribute__((ext_vector_type(4)));
+  uint32_t tr_lane[2], x_lane;
+  {
+    const int j = lane & 15, group = lane >> 4;
+    const int kq = j >> 2, fb = j & 3, hh = group >> 1, fg = group & 1;
+    const int flow = ((kq << 1) | hh) & kSwizzle;
+    const int x = (2 * fg + (fb >> 1)) ^ (flow & 3);
+    const int flip = flow >> 2;
+    const uint32_t base = (uint32_t)(4 * hh + kq) * kRowBytes + (uint32_t)x * 16u + (uint32_t)(fb & 1) * 8u;
+    tr_lane[0] = base + 64u * (uint32_t)flip;
+    tr_lane[1] = base + 64u * (uint32_t)(1 ^ flip);
+    // the same read of a stored tile: rows of 64 bytes, no permutation of chunks
+    x_lane = (uint32_t)(4 * hh + kq) * 64u + (uint32_t)fg * 32u + (uint32_t)fb * 8u;
+  }
+  auto read_transposed = [&](const T *base, int n) __attribute__((always_inline)) {
+    const int u = n / kBlocksD, i = n % kBlocksD;
+    Short4 part[2];
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+      const int ii = kSwizzle >= 8 ? i ^ (2 * jj) : i;
+      const char *at = reinterpret_cast<const char *>(base) + tr_lane[ii & 1] + 64 * (ii & ~1) +
+                       (16 * u + 8 * jj) * kRowBytes;
+      part[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) Short4 *)(at));
+    }
+    return __builtin_bit_cast(Frag, __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+  auto read_stored = [&](const unsigned char *base, int u) __attribute__((always_inline)) {
+    Short4 part[2];
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj)
+      part[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) Short4 *)(base + x_lane + (16 * u + 8 * jj) * 64));
+    return __builtin_bit_cast(Frag, __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+
+  f32x16 acc[kBlocksD];
+#pragma unroll
+  for (int i = 0; i < kBlocksD; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+
+  // the first two tiles on their way
+#pragma unroll
+  for (int rep = 0; rep < 2; ++rep)
+#pragma unroll
+    for (int it = 0; it < kItems; ++it) stage_item(it);
+  // A tile as one straight run of code: operands are read from LDS kRing
+  // products ahead, the loads of the tile after next go between the products.
+  constexpr int kRing = 4;
+  for (; t < tiles; ++t) {
+    wait_vm<kItems>();
+    __syncthreads(); // tile t is in LDS; the buffers written next (tile t - 1's) have been read
+    const T *bt = (for_dv ? do_lds : q_lds) + buf_now * kTile;
+    const unsigned char *bx = x_lds + buf_now * kStoredTileBytes;
+    Frag x[2], ring[kRing];
+    x[0] = read_stored(bx, 0), x[1] = read_stored(bx, 1);
+#pragma unroll
+    for (int p = 0; p < kRing; ++p) ring[p] = read_transposed(bt, p);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = 0; n < kProducts; ++n) {
+      acc[n % kBlocksD] = Op::run(ring[n % kRing], x[n / kBlocksD], acc[n % kBlocksD]);
+      if (n + kRing < kProducts) ring[n % kRing] = read_transposed(bt, n + kRing);
+      if (n < kItems) stage_item(n);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    buf_now = next_buffer(buf_now);
+  }
+  wait_vm<0>(); // (nothing may still be on its way into LDS when the block ends)
+
+  const int own = own0 + 32 * key_wave + ((col & 0x13) | ((col & 4) << 1) | ((col & 8) >> 1));
+  if (own >= S) return;
+  typedef T Out4 __attribute__((ext_vector_type(4)));
+  const Strides3 &st_out = for_dv ? a.sdv : a.sdk;
+  const float factor = for_dv ? (a.drop.drop ? a.drop.keep_scale : 1.0f) : a.scale;
+  T *op = static_cast<T *>(for_dv ? a.dv : a.dk) + b * st_out.b + hd * st_out.h + (int64_t)own * st_out.s;
+#pragma unroll
+  for (int i = 0; i < kBlocksD; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      Out4 w;
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(acc[i][4 * j + tt] * factor);
+      *reinterpret_cast<Out4 *>(op + 32 * i + 8 * j + 4 * half) = w;
+    }
 }
 
 // delta[bh, q] = sum_d dO[q, d] * O[q, d], fp32. D / 8 lanes share a row.
@@ -610,15 +879,49 @@ __global__ __launch_bounds__(kBlockThreads) void attention_delta_kernel(
   if (live && part == 0) delta[row] = s;
 }
 
+// dK and dV of the heads [a.bh0, a.bh0 + 8 * a.head_groups) from the tile store
+template <typename T, int D>
+int launch_stored(const BwdArgs &a, hipStream_t stream) {
+  const dim3 grid((unsigned)(8 * a.head_groups * a.own_blocks));
+  constexpr unsigned kLds = stored_lds_bytes<T, D>();
+  auto *kernel = a.window > 0 ? attention_bwd_stored_kernel<T, D, true> : attention_bwd_stored_kernel<T, D, false>;
+  if (kLds > 64u * 1024u) {
+    const int s = raise_lds_limit(reinterpret_cast<const void *>(kernel), kLds, "oslo_attention_prefill_bwd_stored");
+    if (s != OSLO_OK) return s;
+  }
+  kernel<<<grid, dim3(kStoredThreads), kLds, stream>>>(a);
+  return check_launch("attention_prefill_bwd_stored");
+}
+
 template <typename T, int D>
 int launch_bwd_dim(const BwdArgs &a, float *delta, const void *out, const Strides3 &so,
-                   hipStream_t stream) {
+                   hipStream_t stream, size_t store_bytes) {
   const int64_t rows = (int64_t)a.batch_heads * a.S;
   constexpr int kRows = kBlockThreads / (D / 8);
   attention_delta_kernel<T, D><<<dim3((unsigned)((rows + kRows - 1) / kRows)), dim3(kBlockThreads), 0, stream>>>(
       delta, static_cast<const T *>(out), static_cast<const T *>(a.dout), so, a.sdo, a.S, a.heads, rows);
   int s = check_launch("attention_prefill_bwd(delta)");
   if (s != OSLO_OK) return s;
+  if (a.tiles != nullptr) {
+    // The probabilities through memory: the dQ pass writes P and dS of every tile
+    // on or below the diagonal, a second pass accumulates dK and dV from them (5
+    // matrix products per tile, the number the mathematics has). Groups of 8
+    // heads, as many at a time as the store holds, in launches of equal size.
+    const int64_t per_group = 8 * a.head_tiles * kStoredPairBytes;
+    const int fit = (int)std::min<int64_t>((int64_t)(store_bytes / (size_t)per_group), a.head_groups);
+    const int launches = (a.head_groups + fit - 1) / fit;
+    const int each = (a.head_groups + launches - 1) / launches;
+    for (int g = 0; g < a.head_groups; g += each) {
+      BwdArgs part = a;
+      part.bh0 = 8 * g;
+      part.head_groups = std::min(each, a.head_groups - g);
+      s = launch_role<T, D, kRoleDQ, true>(part, stream);
+      if (s != OSLO_OK) return s;
+      s = launch_stored<T, D>(part, stream);
+      if (s != OSLO_OK) return s;
+    }
+    return OSLO_OK;
+  }
   s = launch_role<T, D, kRoleDQ>(a, stream);
   if (s != OSLO_OK) return s;
   // dK and dV: one combined pass where both accumulators fit a lane's registers
@@ -639,13 +942,14 @@ int launch_bwd_dim(const BwdArgs &a, float *delta, const void *out, const Stride
 
 template <typename T>
 int launch_bwd(const BwdArgs &a, float *delta, const void *out, const Strides3 &so, int head_dim,
-               hipStream_t stream) {
+               hipStream_t stream, size_t store_bytes) {
   switch (head_dim) {
-    case 64: return launch_bwd_dim<T, 64>(a, delta, out, so, stream);
-    case 128: return launch_bwd_dim<T, 128>(a, delta, out, so, stream);
-    default: return launch_bwd_dim<T, 256>(a, delta, out, so, stream);
+    case 64: return launch_bwd_dim<T, 64>(a, delta, out, so, stream, store_bytes);
+    case 128: return launch_bwd_dim<T, 128>(a, delta, out, so, stream, store_bytes);
+    default: return launch_bwd_dim<T, 256>(a, delta, out, so, stream, store_bytes);
   }
 }
+
 
 } // namespace
 } // namespace oslo
@@ -655,18 +959,14 @@ extern "C" size_t oslo_attention_prefill_bwd_workspace_bytes(int64_t batch, int6
   return (size_t)batch * (size_t)heads * (size_t)S * sizeof(float);
 }
 
-extern "C" int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const void *dout,
-                                          const void *q, const void *k, const void *v,
-                                          const void *out, const float *lse,
-                                          float *workspace, const float *pad, float scale,
-                                          float p, uint64_t philox_seed,
-                                          uint64_t philox_offset,
-                                          int64_t batch, int64_t heads, int64_t S,
-                                          int64_t head_dim, int64_t window,
-                                          const int64_t *strides, int dtype,
-                                          oslo_stream_t stream) {
-  using namespace oslo;
-  const char *name = "oslo_attention_prefill_bwd";
+namespace oslo {
+
+// Both entry points: `store` null = every pass computes the scores it needs.
+static int prefill_bwd(const char *name, void *dq, void *dk, void *dv, const void *dout, const void *q, const void *k,
+                const void *v, const void *out, const float *lse, float *workspace, void *store,
+                size_t store_bytes, const float *pad, float scale, float p, uint64_t philox_seed,
+                uint64_t philox_offset, int64_t batch, int64_t heads, int64_t S, int64_t head_dim,
+                int64_t window, const int64_t *strides, int dtype, oslo_stream_t stream) {
   if (batch < 0 || heads < 0 || S < 0 || head_dim < 0 || window < 0)
     return fail(OSLO_E_BAD_ARG, "%s: negative size", name);
   if (dtype != OSLO_F16 && dtype != OSLO_BF16) {
@@ -701,8 +1001,8 @@ extern "C" int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const vo
   if (pad != nullptr && (S % 4 != 0 || !aligned16(pad)))
     return fail(OSLO_E_UNSUPPORTED,
                 "%s: with a padding mask S must be a multiple of 4 and the mask 16-byte aligned", name);
-  if (!aligned16(lse) || !aligned16(workspace))
-    return fail(OSLO_E_UNSUPPORTED, "%s: lse and workspace must be 16-byte aligned", name);
+  if (!aligned16(lse) || !aligned16(workspace) || !aligned16(store))
+    return fail(OSLO_E_UNSUPPORTED, "%s: lse and the workspaces must be 16-byte aligned", name);
   auto st = [&](int i) { return Strides3{strides[3 * i], strides[3 * i + 1], strides[3 * i + 2]}; };
   BwdArgs a;
   a.q = q, a.k = k, a.v = v, a.dout = dout, a.dq = dq, a.dk = dk, a.dv = dv;
@@ -716,9 +1016,58 @@ extern "C" int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const vo
   a.head_groups = (a.batch_heads + 7) / 8;
   a.own_blocks = (int)((S + kOwnPerBlock - 1) / kOwnPerBlock);
   a.window = window >= S ? 0 : (int)window;
+  a.tiles = static_cast<unsigned char *>(store);
+  a.bh0 = 0;
+  a.head_tiles = stored_head_tiles(a.own_blocks);
+  if (store != nullptr && store_bytes < (size_t)(8 * a.head_tiles * kStoredPairBytes))
+    return fail(OSLO_E_BAD_ARG, "%s: a store of %zu bytes; 8 heads of %lld positions need %lld", name, store_bytes,
+                (long long)S, (long long)(8 * a.head_tiles * kStoredPairBytes));
   if ((int64_t)8 * a.head_groups * a.own_blocks > (int64_t)0x7fffffff)
     return fail(OSLO_E_UNSUPPORTED, "%s: too many blocks for one launch", name);
   hipStream_t stm = static_cast<hipStream_t>(stream);
-  if (dtype == OSLO_F16) return launch_bwd<f16>(a, workspace, out, st(3), (int)head_dim, stm);
-  return launch_bwd<bf16>(a, workspace, out, st(3), (int)head_dim, stm);
+  if (dtype == OSLO_F16) return launch_bwd<f16>(a, workspace, out, st(3), (int)head_dim, stm, store_bytes);
+  return launch_bwd<bf16>(a, workspace, out, st(3), (int)head_dim, stm, store_bytes);
 }
+
+} // namespace oslo
+
+extern "C" size_t oslo_attention_prefill_bwd_store_bytes(int64_t batch, int64_t heads, int64_t S) {
+  if (batch <= 0 || heads <= 0 || S <= 0) return 0;
+  const int64_t groups = (batch * heads + 7) / 8;
+  const int64_t own_blocks = (S + oslo::kOwnPerBlock - 1) / oslo::kOwnPerBlock;
+  return (size_t)(8 * groups) * (size_t)oslo::stored_head_tiles(own_blocks) * (size_t)oslo::kStoredPairBytes;
+}
+
+extern "C" int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const void *dout,
+                                          const void *q, const void *k, const void *v,
+                                          const void *out, const float *lse,
+                                          float *workspace, const float *pad, float scale,
+                                          float p, uint64_t philox_seed,
+                                          uint64_t philox_offset,
+                                          int64_t batch, int64_t heads, int64_t S,
+                                          int64_t head_dim, int64_t window,
+                                          const int64_t *strides, int dtype,
+                                          oslo_stream_t stream) {
+  return oslo::prefill_bwd("oslo_attention_prefill_bwd", dq, dk, dv, dout, q, k, v, out, lse, workspace, nullptr, 0,
+                           pad, scale, p, philox_seed, philox_offset, batch, heads, S, head_dim, window, strides,
+                           dtype, stream);
+}
+
+extern "C" int oslo_attention_prefill_bwd_stored(void *dq, void *dk, void *dv, const void *dout,
+                                                 const void *q, const void *k, const void *v,
+                                                 const void *out, const float *lse,
+                                                 float *workspace, void *store, size_t store_bytes,
+                                                 const float *pad, float scale,
+                                                 float p, uint64_t philox_seed,
+                                                 uint64_t philox_offset,
+                                                 int64_t batch, int64_t heads, int64_t S,
+                                                 int64_t head_dim, int64_t window,
+                                                 const int64_t *strides, int dtype,
+                                                 oslo_stream_t stream) {
+  if (store == nullptr)
+    return oslo::fail(OSLO_E_BAD_ARG, "oslo_attention_prefill_bwd_stored: null store");
+  return oslo::prefill_bwd("oslo_attention_prefill_bwd_stored", dq, dk, dv, dout, q, k, v, out, lse, workspace, store,
+                           store_bytes, pad, scale, p, philox_seed, philox_offset, batch, heads, S, head_dim, window,
+                           strides, dtype, stream);
+}
+

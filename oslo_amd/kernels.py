@@ -659,14 +659,28 @@ def attention_prefill_forward(query, key, value, scale, pad=None, window=0, want
     return (out, lse) if want_lse else out
 
 
+# Bytes of tile store a call of the attention's backward may allocate: the
+# store of a call is freed when it returns (the next layer's call reuses the
+# block), so this bounds what the backward adds to a training step's peak.
+PREFILL_BWD_STORE_LIMIT = 2 << 30
+
+
 def attention_prefill_backward(grad_out, query, key, value, out, lse, scale, pad=None, window=0, p=0.0, seed=0,
-                               offset=0):
+                               offset=0, store=None):
     """Gradients of ``attention_prefill_forward`` with respect to query, key and
     value (each [B, H, S, D], dense), from the gradient of its output, its
     inputs, its output and the log-sum-exp it returned with ``want_lse`` (and
     its ``p``, ``seed``, ``offset`` if it dropped attention probabilities). The
-    [S, S] probabilities and their keep mask are recomputed tile by tile;
-    nothing of that size is stored."""
+    [S, S] probabilities and their keep mask are recomputed tile by tile.
+    ``store``: True = the pass that computes dQ hands the probabilities and their
+    gradients to the pass for dK and dV through a workspace (16-bit, the tiles
+    on and below the diagonal, for as many heads at a time as
+    ``PREFILL_BWD_STORE_LIMIT`` bytes hold; freed on return); False = every pass
+    computes the scores it needs and nothing of that size is in memory. Both
+    give the same bits. None = whichever is faster: the store for heads of 256
+    features and, with attention dropout, of 128 (the traffic of the store does
+    not depend on the head size, the matrix products it saves do), if 8 heads
+    fit the limit."""
     code, pad = _prefill_args(query, key, value, pad)
     _device_tensor(grad_out, "grad_out", query)
     _device_tensor(out, "out", query)
@@ -684,11 +698,23 @@ def attention_prefill_backward(grad_out, query, key, value, out, lse, scale, pad
     ws = torch.empty(max(lib.oslo_attention_prefill_bwd_workspace_bytes(b, h, s) // 4, 1), dtype=torch.float32,
                      device=query.device)
     strides = _stride_table((q, k, v, o, g, dq, dk, dv))
+    least = lib.oslo_attention_prefill_bwd_store_bytes(1, 8, s)
+    if store is None:
+        store = (d == 256 or (d == 128 and p > 0.0)) and least <= PREFILL_BWD_STORE_LIMIT
     with _on_device(q):
-        _lib.check(lib.oslo_attention_prefill_bwd(
-            _ptr(dq), _ptr(dk), _ptr(dv), _ptr(g), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(ws),
-            _ptr(pad), float(scale), float(p), int(seed), int(offset), b, h, s, d, int(window), strides, code,
-            _stream(q)))
+        if store:
+            want = lib.oslo_attention_prefill_bwd_store_bytes(b, h, s)
+            size = max(least, min(want, PREFILL_BWD_STORE_LIMIT // least * least))
+            tiles = torch.empty(size, dtype=torch.uint8, device=query.device)
+            _lib.check(lib.oslo_attention_prefill_bwd_stored(
+                _ptr(dq), _ptr(dk), _ptr(dv), _ptr(g), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(ws),
+                _ptr(tiles), size, _ptr(pad), float(scale), float(p), int(seed), int(offset), b, h, s, d,
+                int(window), strides, code, _stream(q)))
+        else:
+            _lib.check(lib.oslo_attention_prefill_bwd(
+                _ptr(dq), _ptr(dk), _ptr(dv), _ptr(g), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(ws),
+                _ptr(pad), float(scale), float(p), int(seed), int(offset), b, h, s, d, int(window), strides, code,
+                _stream(q)))
     return dq, dk, dv
 
 

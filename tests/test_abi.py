@@ -164,6 +164,19 @@ def test_argument_screening_without_a_device(lib):
     assert lib.oslo_attention_decode_fwd(one, two, three, three, one, one, 2, 100, one, null, 3, 0, 1.0, 4, 64, 64, 1, null) == -1  # stride below heads*head_dim
     assert lib.oslo_attention_decode_workspace_bytes(16, 1152, 256, 2) == 16 * 18 * 258 * 4
     assert lib.oslo_attention_decode_workspace_bytes(16, 1152, 48, 2) == 0
+    # the attention's backward with a tile store: its size, a store too small for 8 heads, none at all
+    assert lib.oslo_attention_prefill_bwd_store_bytes(0, 16, 2048) == 0
+    assert lib.oslo_attention_prefill_bwd_store_bytes(8, 16, 2048) == 128 * (64 * 65 // 2) * 4096
+    assert lib.oslo_attention_prefill_bwd_store_bytes(1, 3, 100) == 8 * (4 * 5 // 2) * 4096    # 8 heads, one block of 128
+    strides = (ctypes.c_int64 * 24)(*(8 * [2 * 100 * 64, 100 * 64, 64]))
+    args = (one, one, one, one, one, one, one, one, one, one)
+    tail = (null, 0.125, 0.0, 0, 0, 1, 2, 100, 64, 0, strides, 2, null)
+    assert lib.oslo_attention_prefill_bwd_stored(*args, null, 1 << 20, *tail) == -1
+    assert b"null store" in lib.oslo_last_error()
+    assert lib.oslo_attention_prefill_bwd_stored(*args, one, 8 * 10 * 4096 - 1, *tail) == -1
+    assert b"8 heads" in lib.oslo_last_error()
+    assert lib.oslo_attention_prefill_bwd_stored(*args, ctypes.c_void_p(24), 1 << 30, *tail) == -2   # misaligned
+    assert lib.oslo_attention_prefill_bwd_stored(*args, one, 1 << 30, *(tail[:6] + (0,) + tail[7:])) == 0  # no positions
     # n-gram blocking
     assert lib.oslo_ngram_repeat_block(one, one, 2, 4, 3, 8, 0, null) == -1
     assert lib.oslo_ngram_repeat_block(null, one, 2, 4, 3, 8, 2, null) == -1

@@ -59,9 +59,21 @@ def reference(q, k, v, do, scale, pad=None, window=0, keep=None, p_drop=0.0):
     return o, {"dq": dq, "dk": dk, "dv": dv}, bounds
 
 
+def backward_both_ways(do, q, k, v, out, lse, scale, pad=None, window=0, p=0.0, seed=0, offset=0):
+    """The backward with every pass computing its scores and with the
+    probabilities handed from the dQ pass to the dK/dV pass through the tile
+    store: the same bits (the same products, rounded and summed in the same
+    order), whatever the head size."""
+    plain = kernels.attention_prefill_backward(do, q, k, v, out, lse, scale, pad, window, p, seed, offset, store=False)
+    stored = kernels.attention_prefill_backward(do, q, k, v, out, lse, scale, pad, window, p, seed, offset, store=True)
+    for name, a, b in zip(("dq", "dk", "dv"), plain, stored):
+        assert torch.equal(a, b), (name, tuple(q.shape), window, p, (a.float() - b.float()).abs().max().item())
+    return stored
+
+
 def run(q, k, v, do, scale, pad=None, window=0):
     out, lse = kernels.attention_prefill_forward(q, k, v, scale, pad, window, want_lse=True)
-    dq, dk, dv = kernels.attention_prefill_backward(do, q, k, v, out, lse, scale, pad, window)
+    dq, dk, dv = backward_both_ways(do, q, k, v, out, lse, scale, pad, window)
     return out, lse, {"dq": dq, "dk": dk, "dv": dv}
 
 
@@ -220,7 +232,7 @@ def test_attention_dropout_forward_and_backward(s, d, dtype):
         vmax = 4.0 / (1 - p)
         excess = ((out.double() - o_ref).abs() - REL[dtype] * (o_ref.abs() + vmax)).max().item()
         assert excess <= 1e-4, (excess, s, d, "forward")
-        dq, dk, dv = kernels.attention_prefill_backward(dev[3], *dev[:3], out, lse, scale, padd, window, p, seed, offset)
+        dq, dk, dv = backward_both_ways(dev[3], *dev[:3], out, lse, scale, padd, window, p, seed, offset)
         check({"dq": dq, "dk": dk, "dv": dv}, want, bounds, dtype, (s, d, pad is not None, window))
         if pad is None and window == 0 and s <= 64:
             flat = [f32(t).reshape(b * h, s, d) for t in (q, k, v, do)]
@@ -260,7 +272,7 @@ def test_random_combinations_forward_and_backward():
         what = (case, dt, b, h, s, d, scale, window, pad is not None, p)
         out, lse = kernels.attention_prefill_forward(q, k, v, scale, pad, window, want_lse=True, p=p, seed=seed,
                                                      offset=offset)
-        dq, dk, dv = kernels.attention_prefill_backward(do, q, k, v, out, lse, scale, pad, window, p, seed, offset)
+        dq, dk, dv = backward_both_ways(do, q, k, v, out, lse, scale, pad, window, p, seed, offset)
         o_ref, want, bounds = reference(q, k, v, do, scale, pad, window, keep, p)
         excess = ((out.double() - o_ref).abs() - REL[dt] * (o_ref.abs() + 5.0 / (1 - p))).max().item()
         assert torch.isfinite(out).all() and excess <= 1e-4, (excess, what)
@@ -292,6 +304,34 @@ def test_attention_dropout_long_prompt_and_operator():
                                              seed=seed, offset=off0)[0][..., 0].double()
     want_frac = (keep.double().tril().sum(-1) / (1 - p)) / torch.arange(1, s + 1, device=DEV)
     assert (frac - want_frac).abs().max().item() <= 2.0 ** -7 * 2
+
+
+@pytest.mark.parametrize("d", [64, 256])
+def test_tile_store_smaller_than_the_heads(d, monkeypatch):
+    """A store that holds 8 heads (16 with the second limit) where the call has
+    20: the heads go through it in launches of 8, 8 and 4 (16 and 4), with a
+    window, a padding mask and dropout; the same bits as without a store,
+    whatever the default picks for the head size."""
+    dtype, b, h, s, p, seed, offset = torch.bfloat16, 4, 5, 264, 0.2, 5, 12
+    q, k, v, do = (randn((b, h, s, d), dtype, seed=70 + i).to(DEV) for i in range(4))
+    pad = padding(b, s, 9).to(DEV)
+    lib = kernels._lib.load()
+    least = lib.oslo_attention_prefill_bwd_store_bytes(1, 8, s)
+    assert lib.oslo_attention_prefill_bwd_store_bytes(b, h, s) == 3 * least     # 20 heads: three groups of 8
+    assert least == 8 * (12 * 13 // 2) * 4096                                    # 264 positions: 12 tiles of 32 (3 blocks of 128)
+    for window in (0, 70):
+        out, lse = kernels.attention_prefill_forward(q, k, v, 0.1, pad, window, want_lse=True, p=p, seed=seed, offset=offset)
+        want = kernels.attention_prefill_backward(do, q, k, v, out, lse, 0.1, pad, window, p, seed, offset, store=False)
+        for limit in (least, 2 * least + 100, 1 << 40):
+            monkeypatch.setattr(kernels, "PREFILL_BWD_STORE_LIMIT", limit)
+            got = kernels.attention_prefill_backward(do, q, k, v, out, lse, 0.1, pad, window, p, seed, offset, store=True)
+            assert all(torch.equal(x, y) for x, y in zip(got, want)), (window, limit)
+        auto = kernels.attention_prefill_backward(do, q, k, v, out, lse, 0.1, pad, window, p, seed, offset)
+        assert all(torch.equal(x, y) for x, y in zip(auto, want))
+    # a limit below 8 heads: the default does without a store
+    monkeypatch.setattr(kernels, "PREFILL_BWD_STORE_LIMIT", least - 1)
+    auto = kernels.attention_prefill_backward(do, q, k, v, out, lse, 0.1, pad, 70, p, seed, offset)
+    assert all(torch.equal(x, y) for x, y in zip(auto, want))
 
 
 def test_backward_rejects_what_it_cannot_take():
