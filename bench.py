@@ -34,10 +34,12 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 # Matrix products per visible (query, key) tile that the attention backward's
-# passes issue, by head size (oslo_amd/csrc/attention_prefill_bwd.hip: the dQ
-# pass 3, then dK and dV in one pass 4, or at 256 features, where both
-# accumulators do not fit a lane's registers, 3 + 2 in two passes); the
-# mathematics has 5.
+# passes issue when every pass computes the scores it needs, by head size
+# (oslo_amd/csrc/attention_prefill_bwd.hip: the dQ pass 3, then dK and dV in
+# one pass 4, or at 256 features, where both accumulators do not fit a lane's
+# registers, 3 + 2 in two passes); the mathematics has 5, and so has the
+# backward that hands P and dS from the dQ pass to the dK/dV pass through a
+# tile store (what runs at 256 features).
 BWD_PRODUCTS_ISSUED = {64: 7, 128: 7, 256: 8}
 
 # HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` and
@@ -493,8 +495,8 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
             continue
         # its backward (the forward that stores the log-sum-exp first). Algorithmic work: the five
         # matrix products of the mathematics (S, dP, dV, dQ, dK) where the forward has two, 10 flops per
-        # visible score and feature; `frac` is that over the time. The kernels issue more, because each
-        # owner kind recomputes the scores (`issued_flops`: BWD_PRODUCTS_ISSUED products per visible tile).
+        # visible score and feature; `frac` is that over the time. Where each owner kind recomputes the
+        # scores the kernels issue more (`issued_flops`: BWD_PRODUCTS_ISSUED products per visible tile).
         lse = torch.empty((B, Hh, S), dtype=torch.float32, device=dev)
         check(lib.oslo_attention_prefill_fwd_lse(P(o), P(lse), P(q), P(k), P(v), None, D ** -0.5, 0.0, 0, 0,
                                                  B, Hh, S, D, 0, strides, BF16, st))
@@ -503,17 +505,38 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
         wsb = torch.empty(lib.oslo_attention_prefill_bwd_workspace_bytes(B, Hh, S) // 4, dtype=torch.float32, device=dev)
         dense, merged = [Hh * S * D, S * D, D], [S * Hh * D, D, Hh * D]
         bstr = (ctypes.c_int64 * 24)(*(3 * dense + 2 * merged + 3 * dense))
-        t = time_launches(lambda: check(lib.oslo_attention_prefill_bwd(
+        recompute = lambda: check(lib.oslo_attention_prefill_bwd(
             P(dq), P(dk), P(dv), P(do), P(q), P(k), P(v), P(o), P(lse), P(wsb), None, D ** -0.5, 0.0, 0, 0,
-            B, Hh, S, D, 0, bstr, BF16, st)), max(5, n // 4), 3)
+            B, Hh, S, D, 0, bstr, BF16, st))
+        backward = recompute
         bflops = 5 * flops // 2
-        issued = BWD_PRODUCTS_ISSUED[D] * flops // 2
-        res.append({"kernel": f"attention_prefill_bwd bf16 [{B},{Hh},{S},{D}] causal (dq, dk, dv)",
-                    "bound": "mfma",
-                    "achieved": round(bflops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(bflops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "us": round(t * 1e6, 1),
-                    "algorithmic_flops": bflops, "issued_flops": issued,
-                    "issued_TFLOPs": round(issued / t / 1e12, 1), "traffic": None})
+        if D == 256:
+            # what the operator runs at this head size: the dQ pass hands P and dS to the dK/dV pass
+            # through a tile store (16-bit, the tiles on and below the diagonal), 5 products per tile
+            store_bytes = lib.oslo_attention_prefill_bwd_store_bytes(B, Hh, S)
+            store = torch.empty(store_bytes, dtype=torch.uint8, device=dev)
+            backward = lambda: check(lib.oslo_attention_prefill_bwd_stored(
+                P(dq), P(dk), P(dv), P(do), P(q), P(k), P(v), P(o), P(lse), P(wsb), P(store), store_bytes, None,
+                D ** -0.5, 0.0, 0, 0, B, Hh, S, D, 0, bstr, BF16, st))
+            t = time_launches(recompute, max(5, n // 4), 3)
+            issued = BWD_PRODUCTS_ISSUED[D] * flops // 2
+            res.append({"kernel": f"attention_prefill_bwd bf16 [{B},{Hh},{S},{D}] causal, every pass computing its "
+                                  "scores (no tile store)", "bound": "mfma",
+                        "achieved": round(bflops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                        "frac": round(bflops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "us": round(t * 1e6, 1),
+                        "algorithmic_flops": bflops, "issued_flops": issued,
+                        "issued_TFLOPs": round(issued / t / 1e12, 1), "traffic": None})
+        t = time_launches(backward, max(5, n // 4), 3)
+        issued = (5 if D == 256 else BWD_PRODUCTS_ISSUED[D]) * flops // 2
+        row = {"kernel": f"attention_prefill_bwd bf16 [{B},{Hh},{S},{D}] causal (dq, dk, dv)",
+               "bound": "mfma",
+               "achieved": round(bflops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+               "frac": round(bflops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "us": round(t * 1e6, 1),
+               "algorithmic_flops": bflops, "issued_flops": issued,
+               "issued_TFLOPs": round(issued / t / 1e12, 1), "traffic": None}
+        if D == 256:
+            row["tile_store_bytes"] = store_bytes
+        res.append(row)
         if D == 256:
             # The same launches on zero operands: the same instructions in the same order (no branch of
             # these kernels looks at the data), without the switching activity of the matrix cores'
@@ -529,15 +552,15 @@ def other_kernels(lib, torch, dev, st, P, check, time_launches, roof, n):
                         "us": round(t * 1e6, 1), "algorithmic_flops": flops, "traffic": None})
             check(lib.oslo_attention_prefill_fwd_lse(P(o), P(lse), P(q), P(k), P(v), None, D ** -0.5, 0.0, 0, 0,
                                                      B, Hh, S, D, 0, strides, BF16, st))
-            t = time_launches(lambda: check(lib.oslo_attention_prefill_bwd(
-                P(dq), P(dk), P(dv), P(do), P(q), P(k), P(v), P(o), P(lse), P(wsb), None, D ** -0.5, 0.0, 0, 0,
-                B, Hh, S, D, 0, bstr, BF16, st)), max(5, n // 4), 3)
+            t = time_launches(backward, max(5, n // 4), 3)
             res.append({"kernel": f"attention_prefill_bwd bf16 [{B},{Hh},{S},{D}] causal, zero operands (same instruction stream)",
                         "bound": "mfma", "achieved": round(bflops / t / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                         "unit": "TFLOP/s", "frac": round(bflops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                         "us": round(t * 1e6, 1), "algorithmic_flops": bflops, "issued_flops": issued,
                         "issued_TFLOPs": round(issued / t / 1e12, 1), "traffic": None})
         del q, k, v, o, do, dq, dk, dv, lse, wsb
+        if D == 256:
+            del store
     return res
 
 

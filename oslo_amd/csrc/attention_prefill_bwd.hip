@@ -242,7 +242,15 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
   // get 16 values of f, the 16 lanes of a transposing read (rows 4c .. 4c + 3,
   // two chunks, both halves of each) four values that differ above bit 0: f
   // puts the row's two low bits at bits 1 and 2, bit 2 at bit 0, bit 3 stays.
-  auto f_of = [](int r) __attribute__((always_inline)) { return (((r & 3) << 1) | ((r >> 2) & 1) | (r & 8)) & kSwizzle; };
+  // (At 256 features, where the registers for eight lane offsets are there, f is
+  // 4 (r % 4) + r / 4 % 4 instead: the four rows of a transposing read then use four
+  // different quarters of the banks for both 16-feature halves at once; with the
+  // f above two of the four share theirs, two more cycles for every such read.)
+  constexpr bool kQuads = D == 256;
+  auto f_of = [](int r) __attribute__((always_inline)) {
+    if (kQuads) return ((r & 3) << 2) | ((r >> 2) & 3);
+    return (((r & 3) << 1) | ((r >> 2) & 1) | (r & 8)) & kSwizzle;
+  };
   uint32_t o1_off[kLoadsN], o2_off[kLoadsN];
 #pragma unroll
   for (int j = 0; j < kLoadsN; ++j) {
@@ -306,27 +314,42 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
   // are positions 16u + 4h + 0..3, slots 4..7 positions 16u + 8 + 4h + 0..3 (h
   // the lane's half of the wave): the rows the accumulator layout gives a lane.
   typedef short Short4 __attribute__((ext_vector_type(4)));
-  uint32_t tr_lane[2]; // for even and odd blocks of 32 features
+  uint32_t tr_lane[kQuads ? 8 : 2]; // for even and odd blocks of 32 features (kQuads: per block % 4 and read of the two)
   {
     const int j = lane & 15, group = lane >> 4;
     const int kq = j >> 2, fb = j & 3, hh = group >> 1, fg = group & 1;
-    // f of the lane's rows 16u + 8jj + 4hh + kq is 2 kq | hh | 8 jj; the part below bit 3:
-    const int flow = ((kq << 1) | hh) & kSwizzle;
-    const int x = (2 * fg + (fb >> 1)) ^ (flow & 3);
-    const int flip = flow >> 2; // its bit 2 swaps neighbouring blocks of four chunks
-    const uint32_t base = (uint32_t)(4 * hh + kq) * kRowBytes + (uint32_t)x * 16u + (uint32_t)(fb & 1) * 8u;
-    tr_lane[0] = base + 64u * (uint32_t)flip;
-    tr_lane[1] = base + 64u * (uint32_t)(1 ^ flip);
+    if constexpr (kQuads) {
+      // row 16 u + 8 jj + 4 hh + kq, chunk 4 i + w of it, w = 2 fg + fb / 2: f is 4 kq + 2 jj + hh, so the chunk lies
+      // at 16 (i / 4) + 4 (i % 4 ^ kq) + (w ^ hh ^ 2 jj): the lane's part, with the read's i % 4 and jj folded in
+      const uint32_t own_part = (uint32_t)(4 * hh + kq) * kRowBytes + 64u * (uint32_t)kq +
+                                16u * (uint32_t)((2 * fg + (fb >> 1)) ^ hh) + 8u * (uint32_t)(fb & 1);
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) tr_lane[2 * v + jj] = own_part ^ (uint32_t)(64 * v + 32 * jj);
+    } else {
+      // f of the lane's rows 16u + 8jj + 4hh + kq is 2 kq | hh | 8 jj; the part below bit 3:
+      const int flow = ((kq << 1) | hh) & kSwizzle;
+      const int x = (2 * fg + (fb >> 1)) ^ (flow & 3);
+      const int flip = flow >> 2; // its bit 2 swaps neighbouring blocks of four chunks
+      const uint32_t base = (uint32_t)(4 * hh + kq) * kRowBytes + (uint32_t)x * 16u + (uint32_t)(fb & 1) * 8u;
+      tr_lane[0] = base + 64u * (uint32_t)flip;
+      tr_lane[1] = base + 64u * (uint32_t)(1 ^ flip);
+    }
   }
   auto read_transposed = [&](const T *base, int n) __attribute__((always_inline)) {
     const int u = n / kBlocksD, i = n % kBlocksD;
     Short4 part[2];
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj) {
-      // rows with bit 3 set (jj = 1) have bit 3 of f set: blocks two apart swap (head sizes of 16 chunks and more)
-      const int ii = kSwizzle >= 8 ? i ^ (2 * jj) : i;
-      const char *at = reinterpret_cast<const char *>(base) + tr_lane[ii & 1] + 64 * (ii & ~1) +
-                       (16 * u + 8 * jj) * kRowBytes;
+      const char *at;
+      if constexpr (kQuads) {
+        at = reinterpret_cast<const char *>(base) + tr_lane[2 * (i & 3) + jj] + 256 * (i >> 2) + (16 * u + 8 * jj) * kRowBytes;
+      } else {
+        // rows with bit 3 set (jj = 1) have bit 3 of f set: blocks two apart swap (head sizes of 16 chunks and more)
+        const int ii = kSwizzle >= 8 ? i ^ (2 * jj) : i;
+        at = reinterpret_cast<const char *>(base) + tr_lane[ii & 1] + 64 * (ii & ~1) + (16 * u + 8 * jj) * kRowBytes;
+      }
       part[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) Short4 *)(at));
     }
     return __builtin_bit_cast(Frag, __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7));
@@ -640,24 +663,31 @@ int launch_role(const BwdArgs &a, hipStream_t stream) {
 // dK and dV from the tile store: dK^T += Q^T dS and dV^T += dO^T P over the query
 // tiles from the diagonal on, nothing else: no scores, no exponentials, no
 // mask, no dropout (all of it is in the stored tiles). A block owns 128 keys
-// and has eight waves, two per SIMD: waves 0..3 accumulate dK of 32 keys each,
-// waves 4..7 dV of the same keys, so a wave holds one accumulator (D / 2
-// registers) and no fixed operands. The tiles of Q and dO go through LDS as in
-// the other passes (three buffers: tile t is read while t + 1 and t + 2 are on
-// their way), shared by the block; every wave loads its own 2 KiB tile of dS
-// or P beside them and reads it back transposed, key slot in the lane: lane c
-// holds the key at slot c of the store's rows, key c with bits 2 and 3 swapped.
-constexpr int kStoredWaves = 8;
+// and one of the two gradients (even blocks dK, odd blocks dV); of its four
+// waves a pair has 64 keys and each wave of the pair half of the features, so
+// a wave holds one accumulator of 64 keys x D / 2 features (D / 2 registers),
+// no fixed operands, and uses every transposed operand of Q (or dO) it reads
+// from LDS for two products. The tiles of Q (or dO) go through LDS as in the
+// other passes (three buffers: tile t is read while t + 1 and t + 2 are on
+// their way), shared by the block; every wave loads one 2 KiB tile of dS (or
+// P) beside them, which it and its partner read back transposed, key slot in
+// the lane: lane c holds the key at slot c of the store's rows, key c with
+// bits 2 and 3 swapped. A tile is only 16 products per wave between two
+// barriers, and the waves of a block wait for their first operands of a tile
+// together: two or more blocks share a CU (72 KiB of LDS each at 256
+// features) so that one block's products run while another waits.
+constexpr int kStoredWaves = 4;
 constexpr int kStoredThreads = kStoredWaves * kWave;
 constexpr int kStoredBuffers = 3;
 
 template <typename T, int D>
 constexpr unsigned stored_lds_bytes() {
-  return 2u * kStoredBuffers * kSchedTile * D * sizeof(T) + kStoredWaves * kStoredBuffers * kStoredTileBytes;
+  return (unsigned)kStoredBuffers * (kSchedTile * D * sizeof(T) + kStoredWaves * kStoredTileBytes);
 }
 
 template <typename T, int D, bool HAS_WINDOW>
-__global__ __launch_bounds__(kStoredThreads, D == 64 ? 2 : 1) void attention_bwd_stored_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(kStoredThreads, D == 256 ? 2 : D == 128 ? 3 : 4) void attention_bwd_stored_kernel(
+    const BwdArgs a) {
   using Op = MatrixOp<T>;
   using Frag = typename Op::Frag;
   constexpr int kChunks = D / 8;
@@ -665,26 +695,30 @@ __global__ __launch_bounds__(kStoredThreads, D == 64 ? 2 : 1) void attention_bwd
   constexpr int kTile = kSchedTile * D;
   constexpr int kRowBytes = D * (int)sizeof(T);
   constexpr int kSwizzle = kChunks >= 16 ? 15 : 7;
-  constexpr int kLoadsN = kChunks / 8; // loads per thread and tile, Q and dO together (D = 64: a tensor per four waves)
+  constexpr int kLoadsN = kChunks / 8; // loads per thread and tile of Q (or dO)
   constexpr int kItems = kLoadsN + 2;  // and the wave's own tile of the store
-  constexpr int kProducts = 2 * kBlocksD;
+  constexpr int kHalfBlocks = kBlocksD / 2; // 32-feature blocks of a wave's half of the features
+  constexpr int kOperands = 2 * kHalfBlocks; // transposed operands of Q or dO per tile, each used for both key tiles
 
   extern __shared__ __align__(1024) unsigned char lds_raw[];
-  T *const q_lds = reinterpret_cast<T *>(lds_raw);  // [3][query][chunk ^ f(query)][8]
-  T *const do_lds = q_lds + kStoredBuffers * kTile; // the same for dO
+  T *const t_lds = reinterpret_cast<T *>(lds_raw); // [3][query][chunk ^ f(query)][8]
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int half = lane >> 5;
   const int col = lane & 31;
-  const bool for_dv = wave >= 4;
-  const int key_wave = wave & 3;
-  unsigned char *const x_lds = reinterpret_cast<unsigned char *>(do_lds + kStoredBuffers * kTile) +
+  // two pairs of waves, 64 keys each; of a pair, a wave per half of the features
+  const int feature_half = wave & 1;
+  unsigned char *const x_lds = reinterpret_cast<unsigned char *>(t_lds + kStoredBuffers * kTile) +
                                wave * (kStoredBuffers * kStoredTileBytes); // [3][query][slot]
+  // the two stored tiles the wave multiplies with: its own and its partner's
+  const unsigned char *const x_pair = reinterpret_cast<unsigned char *>(t_lds + kStoredBuffers * kTile) +
+                                      (wave & ~1) * (kStoredBuffers * kStoredTileBytes);
 
   const int xcd = blockIdx.x & 7;
-  const int slot = blockIdx.x >> 3;
+  const int slot = blockIdx.x >> 4;
+  const bool for_dv = ((blockIdx.x >> 3) & 1) != 0;
   // The blocks of a head follow one another on one XCD, the longest walk
   // first: the two or three heads an XCD works on at a time keep their Q and dO
   // (2 x S x D values each) in its L2 while every block of the head reads them.
@@ -695,7 +729,7 @@ __global__ __launch_bounds__(kStoredThreads, D == 64 ? 2 : 1) void attention_bwd
   const int hd = bh - b * a.heads;
   const int S = a.S;
   const int own0 = own_block * kOwnPerBlock;
-  const int key_tile = own0 / 32 + key_wave;
+  const int key_tile = own0 / 32 + wave; // the key tile whose stored tiles this wave loads
   const int window = HAS_WINDOW ? a.window : 0;
 
   const int first_tile = own0 / kSchedTile;
@@ -703,29 +737,30 @@ __global__ __launch_bounds__(kStoredThreads, D == 64 ? 2 : 1) void attention_bwd
   if (HAS_WINDOW && own0 + kOwnPerBlock - 1 + window - 1 < last_query) last_query = own0 + kOwnPerBlock - 1 + window - 1;
   const int tiles = last_query / kSchedTile + 1;
 
-  const T *q_p = static_cast<const T *>(a.q) + b * a.sq.b + hd * a.sq.h;
-  const T *do_p = static_cast<const T *>(a.dout) + b * a.sdo.b + hd * a.sdo.h;
-  const uint32_t q_row = (uint32_t)a.sq.s * sizeof(T), do_row = (uint32_t)a.sdo.s * sizeof(T);
-  auto f_of = [](int r) __attribute__((always_inline)) { return (((r & 3) << 1) | ((r >> 2) & 1) | (r & 8)) & kSwizzle; };
-  // load j of a thread: entry (8 j + wave) * 64 + lane of [Q tile; dO tile]
-  // (a wave's 64 entries lie in one of the two tiles, so every load of a wave
-  // has one source tensor: a stream of tiles per load)
+  const Strides3 &st_in = for_dv ? a.sdo : a.sq;
+  const T *in_p = static_cast<const T *>(for_dv ? a.dout : a.q) + b * st_in.b + hd * st_in.h;
+  const uint32_t in_row = (uint32_t)st_in.s * sizeof(T);
+  // The permutation of a row's 16-byte chunks in LDS: chunk c of row r lies at
+  // c ^ f(r). A transposing read takes, per half of the wave, 4 chunks (64 bytes)
+  // of 4 consecutive rows, and rows lie a multiple of 256 bytes apart: with the
+  // rows' low two bits in bits 2 and 3 of f the four rows use four different
+  // quarters of the banks. (The permutation of the other passes, which leaves two
+  // rows on the same banks, costs every such read two cycles.)
+  constexpr bool kQuads = kChunks >= 16;
+  auto f_of = [](int r) __attribute__((always_inline)) {
+    if (kQuads) return ((r & 3) << 2) | ((r >> 2) & 3);
+    return (((r & 3) << 1) | ((r >> 2) & 1) | (r & 8)) & kSwizzle;
+  };
+  // load j of a thread: entry (4 j + wave) * 64 + lane of the tile
   uint32_t src_off[kLoadsN];
-  TileStream src[kLoadsN];
-  uint32_t dst_off[kLoadsN]; // elements from q_lds, buffer 0
 #pragma unroll
   for (int j = 0; j < kLoadsN; ++j) {
-    const int entry = (8 * j + wave) * kWave;
-    const bool is_do = entry >= kSchedTile * kChunks;
-    const int within = entry % (kSchedTile * kChunks) + lane;
-    const int row = within / kChunks, at = within % kChunks;
-    const uint32_t row_bytes = is_do ? do_row : q_row;
-    src_off[j] = (uint32_t)row * row_bytes + (uint32_t)(at ^ f_of(row)) * 16u;
-    const Strides3 &st = is_do ? a.sdo : a.sq;
-    src[j].start(is_do ? do_p : q_p, (uint32_t)(((int64_t)(S - 1) * st.s + D) * sizeof(T)), row_bytes, kSchedTile,
-                 first_tile, tiles);
-    dst_off[j] = (uint32_t)((is_do ? kStoredBuffers * kTile : 0) + (entry % (kSchedTile * kChunks)) * 8);
+    const int entry = (4 * j + wave) * kWave + lane;
+    const int row = entry / kChunks, at = entry % kChunks;
+    src_off[j] = (uint32_t)row * in_row + (uint32_t)(at ^ f_of(row)) * 16u;
   }
+  TileStream src; // the next tile to load
+  src.start(in_p, (uint32_t)(((int64_t)(S - 1) * st_in.s + D) * sizeof(T)), in_row, kSchedTile, first_tile, tiles);
   // The wave's tile of the store for query tile qt: nothing (zeros, without a
   // memory access) where the pass that writes the store left none: above the
   // diagonal, past the last query tile, and before the first key tile that the
@@ -754,8 +789,8 @@ __global__ __launch_bounds__(kStoredThreads, D == 64 ? 2 : 1) void attention_bwd
   // item `it` of the loads of the next tile to load
   auto stage_item = [&](int it) __attribute__((always_inline)) {
     if (it < kLoadsN) {
-      lds_load_b128(src[it].descriptor(), q_lds + buf_load * kTile + dst_off[it], src_off[it]);
-      src[it].advance();
+      lds_load_b128(src.descriptor(), t_lds + buf_load * kTile + (4 * it + wave) * (kWave * 8), src_off[it]);
+      if (it == kLoadsN - 1) src.advance();
       return;
     }
     it -= kLoadsN;
@@ -769,27 +804,40 @@ __global__ __launch_bounds__(kStoredThreads, D == 64 ? 2 : 1) void attention_bwd
 
   // transposed operands of the tiles of Q and dO (the passes above read them the same way)
   typedef short Short4 __attribute__((ext_vector_type(4)));
-  uint32_t tr_lane[2], x_lane;
+  // Transposed operand (u, ib): 16 queries u of block feature_half * kHalfBlocks + ib of 32 features; two reads
+  // (jj) each. tr_lane[ib][jj]: the lane's byte offset in the tile, the row of the read apart.
+  uint32_t tr_lane[kHalfBlocks][2], x_lane;
   {
     const int j = lane & 15, group = lane >> 4;
     const int kq = j >> 2, fb = j & 3, hh = group >> 1, fg = group & 1;
-    const int flow = ((kq << 1) | hh) & kSwizzle;
-    const int x = (2 * fg + (fb >> 1)) ^ (flow & 3);
-    const int flip = flow >> 2;
-    const uint32_t base = (uint32_t)(4 * hh + kq) * kRowBytes + (uint32_t)x * 16u + (uint32_t)(fb & 1) * 8u;
-    tr_lane[0] = base + 64u * (uint32_t)flip;
-    tr_lane[1] = base + 64u * (uint32_t)(1 ^ flip);
+#pragma unroll
+    for (int ib = 0; ib < kHalfBlocks; ++ib) {
+      const int i = feature_half * kHalfBlocks + ib;
+      if constexpr (kQuads) {
+        // row 16 u + 8 jj + 4 hh + kq, chunk 4 i + w of it, w = 2 fg + fb / 2: f is 4 kq + 2 jj + hh, so the chunk
+        // lies at 16 (i / 4) + 4 (i % 4 ^ kq) + (w ^ hh ^ 2 jj)
+        const uint32_t own = (uint32_t)(4 * hh + kq) * kRowBytes + 64u * (uint32_t)kq +
+                             16u * (uint32_t)((2 * fg + (fb >> 1)) ^ hh) + 8u * (uint32_t)(fb & 1);
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj)
+          tr_lane[ib][jj] = (own ^ (uint32_t)(64 * (i & 3) + 32 * jj)) + 256u * (uint32_t)(i >> 2);
+      } else {
+        const int flow = ((kq << 1) | hh) & kSwizzle;
+        const int x = (2 * fg + (fb >> 1)) ^ (flow & 3);
+        const int flip = flow >> 2;
+        const uint32_t base = (uint32_t)(4 * hh + kq) * kRowBytes + (uint32_t)x * 16u + (uint32_t)(fb & 1) * 8u;
+        tr_lane[ib][0] = tr_lane[ib][1] = base + 64u * (uint32_t)(flip ^ (i & 1)) + 64u * (uint32_t)(i & ~1);
+      }
+    }
     // the same read of a stored tile: rows of 64 bytes, no permutation of chunks
     x_lane = (uint32_t)(4 * hh + kq) * 64u + (uint32_t)fg * 32u + (uint32_t)fb * 8u;
   }
   auto read_transposed = [&](const T *base, int n) __attribute__((always_inline)) {
-    const int u = n / kBlocksD, i = n % kBlocksD;
+    const int u = n / kHalfBlocks, ib = n % kHalfBlocks;
     Short4 part[2];
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj) {
-      const int ii = kSwizzle >= 8 ? i ^ (2 * jj) : i;
-      const char *at = reinterpret_cast<const char *>(base) + tr_lane[ii & 1] + 64 * (ii & ~1) +
-                       (16 * u + 8 * jj) * kRowBytes;
+      const char *at = reinterpret_cast<const char *>(base) + tr_lane[ib][jj] + (16 * u + 8 * jj) * kRowBytes;
       part[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) Short4 *)(at));
     }
     return __builtin_bit_cast(Frag, __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7));
@@ -803,11 +851,13 @@ __global__ __launch_bounds__(kStoredThreads, D == 64 ? 2 : 1) void attention_bwd
     return __builtin_bit_cast(Frag, __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
-  f32x16 acc[kBlocksD];
+  f32x16 acc[2][kHalfBlocks]; // [key tile of the pair][block of features]
 #pragma unroll
-  for (int i = 0; i < kBlocksD; ++i)
+  for (int g = 0; g < 2; ++g)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+    for (int i = 0; i < kHalfBlocks; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[g][i][r] = 0.f;
 
   // the first two tiles on their way
 #pragma unroll
@@ -815,44 +865,56 @@ __global__ __launch_bounds__(kStoredThreads, D == 64 ? 2 : 1) void attention_bwd
 #pragma unroll
     for (int it = 0; it < kItems; ++it) stage_item(it);
   // A tile as one straight run of code: operands are read from LDS kRing
-  // products ahead, the loads of the tile after next go between the products.
-  constexpr int kRing = 4;
+  // operands ahead, the loads of the tile after next go between the products.
+  constexpr int kRing = kOperands < 4 ? kOperands : 4;
+  constexpr int kPerOperand = (kItems + kOperands - 1) / kOperands;
   for (; t < tiles; ++t) {
     wait_vm<kItems>();
     __syncthreads(); // tile t is in LDS; the buffers written next (tile t - 1's) have been read
-    const T *bt = (for_dv ? do_lds : q_lds) + buf_now * kTile;
-    const unsigned char *bx = x_lds + buf_now * kStoredTileBytes;
-    Frag x[2], ring[kRing];
-    x[0] = read_stored(bx, 0), x[1] = read_stored(bx, 1);
+    const T *bt = t_lds + buf_now * kTile;
+    const unsigned char *bx = x_pair + buf_now * kStoredTileBytes;
+    Frag x[2][2], ring[kRing];
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) x[g][u] = read_stored(bx + g * (kStoredBuffers * kStoredTileBytes), u);
 #pragma unroll
     for (int p = 0; p < kRing; ++p) ring[p] = read_transposed(bt, p);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int n = 0; n < kProducts; ++n) {
-      acc[n % kBlocksD] = Op::run(ring[n % kRing], x[n / kBlocksD], acc[n % kBlocksD]);
-      if (n + kRing < kProducts) ring[n % kRing] = read_transposed(bt, n + kRing);
-      if (n < kItems) stage_item(n);
+    for (int n = 0; n < kOperands; ++n) {
+      const int u = n / kHalfBlocks, ib = n % kHalfBlocks;
+      acc[0][ib] = Op::run(ring[n % kRing], x[0][u], acc[0][ib]);
+      acc[1][ib] = Op::run(ring[n % kRing], x[1][u], acc[1][ib]);
+      if (n + kRing < kOperands) ring[n % kRing] = read_transposed(bt, n + kRing);
+#pragma unroll
+      for (int it = n * kPerOperand; it < (n + 1) * kPerOperand && it < kItems; ++it) stage_item(it);
       __builtin_amdgcn_sched_barrier(0);
     }
     buf_now = next_buffer(buf_now);
   }
   wait_vm<0>(); // (nothing may still be on its way into LDS when the block ends)
 
-  const int own = own0 + 32 * key_wave + ((col & 0x13) | ((col & 4) << 1) | ((col & 8) >> 1));
-  if (own >= S) return;
   typedef T Out4 __attribute__((ext_vector_type(4)));
   const Strides3 &st_out = for_dv ? a.sdv : a.sdk;
   const float factor = for_dv ? (a.drop.drop ? a.drop.keep_scale : 1.0f) : a.scale;
-  T *op = static_cast<T *>(for_dv ? a.dv : a.dk) + b * st_out.b + hd * st_out.h + (int64_t)own * st_out.s;
 #pragma unroll
-  for (int i = 0; i < kBlocksD; ++i)
+  for (int g = 0; g < 2; ++g) {
+    // lane c holds the key at slot c of the store's rows: c with bits 2 and 3 swapped
+    const int own = own0 + 32 * ((wave & ~1) + g) + ((col & 0x13) | ((col & 4) << 1) | ((col & 8) >> 1));
+    if (own >= S) continue;
+    T *op = static_cast<T *>(for_dv ? a.dv : a.dk) + b * st_out.b + hd * st_out.h + (int64_t)own * st_out.s +
+            32 * kHalfBlocks * feature_half;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      Out4 w;
+    for (int i = 0; i < kHalfBlocks; ++i)
 #pragma unroll
-      for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(acc[i][4 * j + tt] * factor);
-      *reinterpret_cast<Out4 *>(op + 32 * i + 8 * j + 4 * half) = w;
-    }
+      for (int j = 0; j < 4; ++j) {
+        Out4 w;
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) w[tt] = static_cast<T>(acc[g][i][4 * j + tt] * factor);
+        *reinterpret_cast<Out4 *>(op + 32 * i + 8 * j + 4 * half) = w;
+      }
+  }
 }
 
 // delta[bh, q] = sum_d dO[q, d] * O[q, d], fp32. D / 8 lanes share a row.
@@ -882,7 +944,7 @@ __global__ __launch_bounds__(kBlockThreads) void attention_delta_kernel(
 // dK and dV of the heads [a.bh0, a.bh0 + 8 * a.head_groups) from the tile store
 template <typename T, int D>
 int launch_stored(const BwdArgs &a, hipStream_t stream) {
-  const dim3 grid((unsigned)(8 * a.head_groups * a.own_blocks));
+  const dim3 grid((unsigned)(2 * 8 * a.head_groups * a.own_blocks)); // a block per gradient
   constexpr unsigned kLds = stored_lds_bytes<T, D>();
   auto *kernel = a.window > 0 ? attention_bwd_stored_kernel<T, D, true> : attention_bwd_stored_kernel<T, D, false>;
   if (kLds > 64u * 1024u) {
@@ -1019,10 +1081,11 @@ static int prefill_bwd(const char *name, void *dq, void *dk, void *dv, const voi
   a.tiles = static_cast<unsigned char *>(store);
   a.bh0 = 0;
   a.head_tiles = stored_head_tiles(a.own_blocks);
+
   if (store != nullptr && store_bytes < (size_t)(8 * a.head_tiles * kStoredPairBytes))
     return fail(OSLO_E_BAD_ARG, "%s: a store of %zu bytes; 8 heads of %lld positions need %lld", name, store_bytes,
                 (long long)S, (long long)(8 * a.head_tiles * kStoredPairBytes));
-  if ((int64_t)8 * a.head_groups * a.own_blocks > (int64_t)0x7fffffff)
+  if ((int64_t)16 * a.head_groups * a.own_blocks > (int64_t)0x7fffffff)
     return fail(OSLO_E_UNSUPPORTED, "%s: too many blocks for one launch", name);
   hipStream_t stm = static_cast<hipStream_t>(stream);
   if (dtype == OSLO_F16) return launch_bwd<f16>(a, workspace, out, st(3), (int)head_dim, stm, store_bytes);
