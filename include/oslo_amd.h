@@ -545,7 +545,8 @@ int oslo_attention_prefill_bwd(void *dq, void *dk, void *dv, const void *dout,
  * x 32 keys on or below the diagonal, P (after dropout) and dS / scale in the
  * storage type (4 KiB a tile) into `store`, and one more pass accumulates dk
  * and dv from them: 5 matrix products per tile, where the entry point above
- * computes the scores once per pass (7 or 8). The results obey the same
+ * computes the scores once per pass (7 or 8); worth its memory traffic at
+ * head_dim 256, not at 64 or 128. The results obey the same
  * formulas and the same rounding (P and dS are rounded to the storage type
  * before the products either way), sums run in the same order, and they are
  * as reproducible.

@@ -119,6 +119,11 @@ __device__ __forceinline__ void lds_load_b128(const u32x4 &desc, const void *dst
   const uint32_t at = __builtin_amdgcn_readfirstlane((uint32_t)reinterpret_cast<uintptr_t>(dst));
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");
 }
+// The same load with the non-temporal hint: data that is read once.
+__device__ __forceinline__ void lds_load_b128_once(const u32x4 &desc, const void *dst, uint32_t offset) {
+  const uint32_t at = __builtin_amdgcn_readfirstlane((uint32_t)reinterpret_cast<uintptr_t>(dst));
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen nt lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");
+}
 __device__ __forceinline__ void lds_load_b32(const u32x4 &desc, const void *dst, uint32_t offset) {
   const uint32_t at = __builtin_amdgcn_readfirstlane((uint32_t)reinterpret_cast<uintptr_t>(dst));
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(at), "v"(offset), "s"(desc) : "m0");

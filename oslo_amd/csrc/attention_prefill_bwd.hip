@@ -54,6 +54,11 @@ namespace {
 #ifndef OSLO_BWD_COMBINED_MAX_DIM
 #define OSLO_BWD_COMBINED_MAX_DIM 128
 #endif
+// Waves of a block of the pass that reads the tile store (32 keys each), heads
+// of 128 and 256 features (a build switch for measurements: 4 or 8).
+#ifndef OSLO_STORED_WAVES
+#define OSLO_STORED_WAVES 8
+#endif
 
 constexpr int kOwnPerBlock = 128;
 constexpr float kLog2eB = 1.4426950408889634f;
@@ -476,8 +481,9 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
         unsigned char *at = tile_row + (int64_t)t * kStoredPairBytes;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-          *reinterpret_cast<Frag *>(at + 32 * u) = pk[u];
-          *reinterpret_cast<Frag *>(at + kStoredTileBytes + 32 * u) = ds[u];
+          // (written once and read once by the next pass: non-temporal, so that K and V stay in the caches)
+          __builtin_nontemporal_store(pk[u], reinterpret_cast<Frag *>(at + 32 * u));
+          __builtin_nontemporal_store(ds[u], reinterpret_cast<Frag *>(at + kStoredTileBytes + 32 * u));
         }
       }
     }
@@ -662,32 +668,41 @@ int launch_role(const BwdArgs &a, hipStream_t stream) {
 
 // dK and dV from the tile store: dK^T += Q^T dS and dV^T += dO^T P over the query
 // tiles from the diagonal on, nothing else: no scores, no exponentials, no
-// mask, no dropout (all of it is in the stored tiles). A block owns 128 keys
-// and one of the two gradients (even blocks dK, odd blocks dV); of its four
-// waves a pair has 64 keys and each wave of the pair half of the features, so
-// a wave holds one accumulator of 64 keys x D / 2 features (D / 2 registers),
-// no fixed operands, and uses every transposed operand of Q (or dO) it reads
-// from LDS for two products. The tiles of Q (or dO) go through LDS as in the
-// other passes (three buffers: tile t is read while t + 1 and t + 2 are on
-// their way), shared by the block; every wave loads one 2 KiB tile of dS (or
-// P) beside them, which it and its partner read back transposed, key slot in
-// the lane: lane c holds the key at slot c of the store's rows, key c with
-// bits 2 and 3 swapped. A tile is only 16 products per wave between two
-// barriers, and the waves of a block wait for their first operands of a tile
-// together: two or more blocks share a CU (72 KiB of LDS each at 256
-// features) so that one block's products run while another waits.
-constexpr int kStoredWaves = 4;
-constexpr int kStoredThreads = kStoredWaves * kWave;
+// mask, no dropout (all of it is in the stored tiles). A block owns 32 keys per
+// wave (256 with eight waves) and one of the two gradients (even blocks dK, odd
+// blocks dV); a pair of waves has 64 keys and each wave of the pair half of the
+// features, so a wave holds one accumulator of 64 keys x D / 2 features (D / 2
+// registers), no fixed operands, and uses every transposed operand of Q (or
+// dO) it reads from LDS for two products. The tiles of Q (or dO) go through LDS
+// as in the other passes (three buffers: tile t is read while t + 1 and t + 2
+// are on their way), shared by the block; every wave loads one 2 KiB tile of dS
+// (or P) beside them, which it and its partner read back transposed, key slot
+// in the lane: lane c holds the key at slot c of the store's rows, key c with
+// bits 2 and 3 swapped. What this pass waits for is its loads (with none of
+// them issued it takes 0.22 ms instead of 0.40 at [8,16,2048,256], without its
+// products still 0.39): the more keys share a tile of Q, the fewer bytes per
+// product, hence eight waves.
 constexpr int kStoredBuffers = 3;
+// waves of a block (32 keys each), by head size
+constexpr int stored_waves(int D) { return D == 64 ? 4 : OSLO_STORED_WAVES; }
 
 template <typename T, int D>
 constexpr unsigned stored_lds_bytes() {
-  return (unsigned)kStoredBuffers * (kSchedTile * D * sizeof(T) + kStoredWaves * kStoredTileBytes);
+  return (unsigned)kStoredBuffers * (kSchedTile * D * sizeof(T) + stored_waves(D) * kStoredTileBytes);
+}
+
+// blocks that share a CU: what the 160 KiB of LDS hold, four at most
+template <typename T, int D>
+constexpr int stored_blocks_per_cu() {
+  const unsigned fit = 160u * 1024u / stored_lds_bytes<T, D>();
+  return fit > 4u ? 4 : (int)fit;
 }
 
 template <typename T, int D, bool HAS_WINDOW>
-__global__ __launch_bounds__(kStoredThreads, D == 256 ? 2 : D == 128 ? 3 : 4) void attention_bwd_stored_kernel(
+__global__ __launch_bounds__(stored_waves(D) * kWave, (stored_blocks_per_cu<T, D>())) void attention_bwd_stored_kernel(
     const BwdArgs a) {
+  constexpr int kStoredWaves = stored_waves(D);
+  constexpr int kStoredKeys = 32 * kStoredWaves; // keys of a block
   using Op = MatrixOp<T>;
   using Frag = typename Op::Frag;
   constexpr int kChunks = D / 8;
@@ -695,7 +710,8 @@ __global__ __launch_bounds__(kStoredThreads, D == 256 ? 2 : D == 128 ? 3 : 4) vo
   constexpr int kTile = kSchedTile * D;
   constexpr int kRowBytes = D * (int)sizeof(T);
   constexpr int kSwizzle = kChunks >= 16 ? 15 : 7;
-  constexpr int kLoadsN = kChunks / 8; // loads per thread and tile of Q (or dO)
+  constexpr int kLoadsN = kSchedTile * kChunks / (kStoredWaves * kWave); // loads per thread and tile of Q (or dO)
+  static_assert(kLoadsN >= 1, "a tile of fewer entries than the block has threads");
   constexpr int kItems = kLoadsN + 2;  // and the wave's own tile of the store
   constexpr int kHalfBlocks = kBlocksD / 2; // 32-feature blocks of a wave's half of the features
   constexpr int kOperands = 2 * kHalfBlocks; // transposed operands of Q or dO per tile, each used for both key tiles
@@ -722,19 +738,20 @@ __global__ __launch_bounds__(kStoredThreads, D == 256 ? 2 : D == 128 ? 3 : 4) vo
   // The blocks of a head follow one another on one XCD, the longest walk
   // first: the two or three heads an XCD works on at a time keep their Q and dO
   // (2 x S x D values each) in its L2 while every block of the head reads them.
-  const int bh = a.bh0 + xcd + 8 * (slot / a.own_blocks);
-  const int own_block = slot % a.own_blocks;
+  const int S = a.S;
+  const int key_blocks = (S + kStoredKeys - 1) / kStoredKeys;
+  const int bh = a.bh0 + xcd + 8 * (slot / key_blocks);
+  const int own_block = slot % key_blocks;
   if (bh >= a.batch_heads) return; // the whole block
   const int b = bh / a.heads;
   const int hd = bh - b * a.heads;
-  const int S = a.S;
-  const int own0 = own_block * kOwnPerBlock;
+  const int own0 = own_block * kStoredKeys;
   const int key_tile = own0 / 32 + wave; // the key tile whose stored tiles this wave loads
   const int window = HAS_WINDOW ? a.window : 0;
 
   const int first_tile = own0 / kSchedTile;
   int last_query = S - 1;
-  if (HAS_WINDOW && own0 + kOwnPerBlock - 1 + window - 1 < last_query) last_query = own0 + kOwnPerBlock - 1 + window - 1;
+  if (HAS_WINDOW && own0 + kStoredKeys - 1 + window - 1 < last_query) last_query = own0 + kStoredKeys - 1 + window - 1;
   const int tiles = last_query / kSchedTile + 1;
 
   const Strides3 &st_in = for_dv ? a.sdo : a.sq;
@@ -751,11 +768,11 @@ __global__ __launch_bounds__(kStoredThreads, D == 256 ? 2 : D == 128 ? 3 : 4) vo
     if (kQuads) return ((r & 3) << 2) | ((r >> 2) & 3);
     return (((r & 3) << 1) | ((r >> 2) & 1) | (r & 8)) & kSwizzle;
   };
-  // load j of a thread: entry (4 j + wave) * 64 + lane of the tile
+  // load j of a thread: entry (kStoredWaves j + wave) * 64 + lane of the tile
   uint32_t src_off[kLoadsN];
 #pragma unroll
   for (int j = 0; j < kLoadsN; ++j) {
-    const int entry = (4 * j + wave) * kWave + lane;
+    const int entry = (kStoredWaves * j + wave) * kWave + lane;
     const int row = entry / kChunks, at = entry % kChunks;
     src_off[j] = (uint32_t)row * in_row + (uint32_t)(at ^ f_of(row)) * 16u;
   }
@@ -789,12 +806,13 @@ __global__ __launch_bounds__(kStoredThreads, D == 256 ? 2 : D == 128 ? 3 : 4) vo
   // item `it` of the loads of the next tile to load
   auto stage_item = [&](int it) __attribute__((always_inline)) {
     if (it < kLoadsN) {
-      lds_load_b128(src.descriptor(), t_lds + buf_load * kTile + (4 * it + wave) * (kWave * 8), src_off[it]);
+      lds_load_b128(src.descriptor(), t_lds + buf_load * kTile + (kStoredWaves * it + wave) * (kWave * 8), src_off[it]);
       if (it == kLoadsN - 1) src.advance();
       return;
     }
     it -= kLoadsN;
-    lds_load_b128(store_descriptor(), x_lds + buf_load * kStoredTileBytes + it * 1024, (uint32_t)(it * 1024 + lane * 16));
+    // (read once: past the caches' usual replacement, so that the tiles of Q and dO stay)
+    lds_load_b128_once(store_descriptor(), x_lds + buf_load * kStoredTileBytes + it * 1024, (uint32_t)(it * 1024 + lane * 16));
     if (it == 1) {
       store_at += (uint64_t)(store_tile + 1) * kStoredPairBytes;
       ++store_tile;
@@ -944,14 +962,15 @@ __global__ __launch_bounds__(kBlockThreads) void attention_delta_kernel(
 // dK and dV of the heads [a.bh0, a.bh0 + 8 * a.head_groups) from the tile store
 template <typename T, int D>
 int launch_stored(const BwdArgs &a, hipStream_t stream) {
-  const dim3 grid((unsigned)(2 * 8 * a.head_groups * a.own_blocks)); // a block per gradient
+  const int key_blocks = (a.S + 32 * stored_waves(D) - 1) / (32 * stored_waves(D));
+  const dim3 grid((unsigned)(2 * 8 * a.head_groups * key_blocks)); // a block per gradient
   constexpr unsigned kLds = stored_lds_bytes<T, D>();
   auto *kernel = a.window > 0 ? attention_bwd_stored_kernel<T, D, true> : attention_bwd_stored_kernel<T, D, false>;
   if (kLds > 64u * 1024u) {
     const int s = raise_lds_limit(reinterpret_cast<const void *>(kernel), kLds, "oslo_attention_prefill_bwd_stored");
     if (s != OSLO_OK) return s;
   }
-  kernel<<<grid, dim3(kStoredThreads), kLds, stream>>>(a);
+  kernel<<<grid, dim3(stored_waves(D) * kWave), kLds, stream>>>(a);
   return check_launch("attention_prefill_bwd_stored");
 }
 

@@ -678,9 +678,9 @@ def attention_prefill_backward(grad_out, query, key, value, out, lse, scale, pad
     ``PREFILL_BWD_STORE_LIMIT`` bytes hold; freed on return); False = every pass
     computes the scores it needs and nothing of that size is in memory. Both
     give the same bits. None = whichever is faster: the store for heads of 256
-    features and, with attention dropout, of 128 (the traffic of the store does
-    not depend on the head size, the matrix products it saves do), if 8 heads
-    fit the limit."""
+    features (its traffic does not depend on the head size, the matrix products
+    it saves do: at 128 features the two are even at best, at 64 the store
+    loses by a factor of two), if 8 heads fit the limit."""
     code, pad = _prefill_args(query, key, value, pad)
     _device_tensor(grad_out, "grad_out", query)
     _device_tensor(out, "out", query)
@@ -700,7 +700,7 @@ def attention_prefill_backward(grad_out, query, key, value, out, lse, scale, pad
     strides = _stride_table((q, k, v, o, g, dq, dk, dv))
     least = lib.oslo_attention_prefill_bwd_store_bytes(1, 8, s)
     if store is None:
-        store = (d == 256 or (d == 128 and p > 0.0)) and least <= PREFILL_BWD_STORE_LIMIT
+        store = d == 256 and least <= PREFILL_BWD_STORE_LIMIT
     with _on_device(q):
         if store:
             want = lib.oslo_attention_prefill_bwd_store_bytes(b, h, s)
