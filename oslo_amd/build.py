@@ -69,6 +69,8 @@ EXTRA_FLAGS = {
     "attention_prefill.hip": ["-Wno-inline-asm"],
     "attention_prefill_bwd.hip": ["-Wno-inline-asm"],
 }
+if os.environ.get("OSLO_STORED_BUFFERS"):
+    EXTRA_FLAGS["attention_prefill_bwd.hip"].append("-DOSLO_STORED_BUFFERS=" + str(int(os.environ["OSLO_STORED_BUFFERS"])))
 if os.environ.get("OSLO_STORED_WAVES"):
     EXTRA_FLAGS["attention_prefill_bwd.hip"].append("-DOSLO_STORED_WAVES=" + str(int(os.environ["OSLO_STORED_WAVES"])))
 if os.environ.get("OSLO_BWD_COMBINED_MAX_DIM"):

@@ -682,13 +682,21 @@ int launch_role(const BwdArgs &a, hipStream_t stream) {
 // them issued it takes 0.22 ms instead of 0.40 at [8,16,2048,256], without its
 // products still 0.39): the more keys share a tile of Q, the fewer bytes per
 // product, hence eight waves.
-constexpr int kStoredBuffers = 3;
+// Tiles of a tensor in LDS: the one that is read and those on their way. (The
+// pass is bound by its loads, but not by their latency: with four or five
+// buffers at 256 features, 128 and 160 KiB, it takes the same time as with three.
+// Nor does it help to issue the loads of half of the waves one operand later
+// than those of the others: 430 against 390 us.)
+#ifndef OSLO_STORED_BUFFERS
+#define OSLO_STORED_BUFFERS 3
+#endif
+constexpr int stored_buffers(int D) { return D == 256 ? OSLO_STORED_BUFFERS : 3; }
 // waves of a block (32 keys each), by head size
 constexpr int stored_waves(int D) { return D == 64 ? 4 : OSLO_STORED_WAVES; }
 
 template <typename T, int D>
 constexpr unsigned stored_lds_bytes() {
-  return (unsigned)kStoredBuffers * (kSchedTile * D * sizeof(T) + stored_waves(D) * kStoredTileBytes);
+  return (unsigned)stored_buffers(D) * (kSchedTile * D * sizeof(T) + stored_waves(D) * kStoredTileBytes);
 }
 
 // blocks that share a CU: what the 160 KiB of LDS hold, four at most
@@ -703,6 +711,7 @@ __global__ __launch_bounds__(stored_waves(D) * kWave, (stored_blocks_per_cu<T, D
     const BwdArgs a) {
   constexpr int kStoredWaves = stored_waves(D);
   constexpr int kStoredKeys = 32 * kStoredWaves; // keys of a block
+  constexpr int kStoredBuffers = stored_buffers(D);
   using Op = MatrixOp<T>;
   using Frag = typename Op::Frag;
   constexpr int kChunks = D / 8;
@@ -801,7 +810,7 @@ __global__ __launch_bounds__(stored_waves(D) * kWave, (stored_blocks_per_cu<T, D
     return d;
   };
   int t = first_tile;
-  int buf_now = 0, buf_load = 0; // buffers of tile t and of the tile being loaded (t + 2 in the loop)
+  int buf_now = 0, buf_load = 0; // buffers of tile t and of the tile being loaded (t + kStoredBuffers - 1 in the loop)
   auto next_buffer = [](int b) __attribute__((always_inline)) { return b == kStoredBuffers - 1 ? 0 : b + 1; };
   // item `it` of the loads of the next tile to load
   auto stage_item = [&](int it) __attribute__((always_inline)) {
@@ -877,9 +886,9 @@ __global__ __launch_bounds__(stored_waves(D) * kWave, (stored_blocks_per_cu<T, D
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[g][i][r] = 0.f;
 
-  // the first two tiles on their way
+  // the first tiles on their way
 #pragma unroll
-  for (int rep = 0; rep < 2; ++rep)
+  for (int rep = 0; rep < kStoredBuffers - 1; ++rep)
 #pragma unroll
     for (int it = 0; it < kItems; ++it) stage_item(it);
   // A tile as one straight run of code: operands are read from LDS kRing
@@ -887,7 +896,7 @@ __global__ __launch_bounds__(stored_waves(D) * kWave, (stored_blocks_per_cu<T, D
   constexpr int kRing = kOperands < 4 ? kOperands : 4;
   constexpr int kPerOperand = (kItems + kOperands - 1) / kOperands;
   for (; t < tiles; ++t) {
-    wait_vm<kItems>();
+    wait_vm<(kStoredBuffers - 2) * kItems>(); // (the tiles after t may still be on their way)
     __syncthreads(); // tile t is in LDS; the buffers written next (tile t - 1's) have been read
     const T *bt = t_lds + buf_now * kTile;
     const unsigned char *bx = x_pair + buf_now * kStoredTileBytes;
