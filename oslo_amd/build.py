@@ -8,12 +8,14 @@ a model runs.
 
     python -m oslo_amd.build
 
-Two environment variables make a second build for measurements without
-touching the one in the tree: ``OSLO_AMD_LIB=/some/where/lib.so`` is where the
-library is written (and where ``oslo_amd._lib`` then loads it from), and
+Environment variables make a second build for measurements without touching
+the one in the tree: ``OSLO_AMD_LIB=/some/where/lib.so`` is where the library
+is written (and where ``oslo_amd._lib`` then loads it from);
 ``OSLO_BWD_COMBINED_MAX_DIM=256`` compiles the attention backward with dK and
 dV in one pass at head_dim 256 as well (it spills there; the default, 128, is
-what measures fastest).
+what measures fastest); ``OSLO_STORED_WAVES=4`` and ``OSLO_STORED_BUFFERS=5``
+give the pass of that backward that reads the tile store blocks of 128 keys
+instead of 256, and five tiles per tensor in LDS instead of three.
 """
 
 import os
