@@ -1,6 +1,8 @@
 // Backward of the one-kernel causal prompt attention (attention_prefill.hip):
 // dQ, dK and dV from Q, K, V, dO, the forward's output O and the log-sum-exp
-// of every row, without the [S, S] matrices in memory. With
+// of every row, without the [S, S] matrices in memory (or, for the entry
+// point with a tile store, with their tiles below the diagonal in a workspace
+// between two passes of one call). With
 //   P  = exp2(scale*log2e * Q K^T + pad*log2e - lse)      (the probabilities)
 //   dP = dO V^T,   delta[q] = sum_d dO[q,d] * O[q,d]
 //   dS = scale * P o (dP - delta)

@@ -642,7 +642,10 @@ class FusedPrefillAttention(object):
     heads of 64, 128 or 256 features; no probabilities to return. With
     gradients recorded the forward also keeps the log-sum-exp of every row and
     the backward recomputes the probabilities from it, so a training step
-    stores no [B, H, S, S] tensor either. ``dropout_p`` > 0 (training) drops
+    keeps no [B, H, S, S] tensor between forward and backward either (heads of
+    256 features: the backward's passes hand the 16-bit probabilities of the
+    tiles below the diagonal to one another through a workspace of the call,
+    ``kernels.PREFILL_BWD_STORE_LIMIT`` bytes at most). ``dropout_p`` > 0 (training) drops
     attention probabilities inside the kernel, with the keep mask the softmax
     kernel with fused dropout would draw from the device generator (S must be
     a multiple of 8 then).
