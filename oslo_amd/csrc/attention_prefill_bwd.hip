@@ -101,11 +101,13 @@ struct BwdArgs {
 
 // The tile store. P (after dropout) and dS / scale of the 32 queries x 32 keys of
 // query tile Qb and key tile Kb <= Qb of a head are 2 KiB each, one behind the
-// other at tile index Qb (Qb + 1) / 2 + Kb: [query][slot], slot 16 u + 8 h + i
-// holding key 16 u + 8 (i / 4) + 4 h + i % 4, which is what lane (query, half
-// h) of the pass that computes them holds as the B operands u = 0, 1 of its
-// own accumulating product, 16 bytes each. The pass that consumes them reads a
-// tile through the transposing LDS read, key slot in the lane.
+// other at tile index Qb (Qb + 1) / 2 + Kb, each as the pass that computes
+// them holds it: [operand u][lane][8 values], the B operand u = 0, 1 of that
+// pass's own accumulating product of lane (query, half h), whose value i is
+// key 16 u + 8 (i / 4) + 4 h + i % 4: a store instruction of a wave writes 1 KiB
+// in a row. The pass that consumes them gathers a tile into LDS as rows of
+// [query][slot], slot 16 u + 8 h + i, and reads it through the transposing LDS
+// read, key slot in the lane.
 constexpr int kStoredTileBytes = 2048;                      // one of the two
 constexpr int kStoredPairBytes = 2 * kStoredTileBytes;      // P, then dS
 __host__ __device__ constexpr int64_t stored_head_tiles(int64_t own_blocks) {
@@ -476,7 +478,7 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
   const int own_tile = own0 / 32 + wave;
   if constexpr (STORE)
     tile_row = a.tiles + ((int64_t)(bh - a.bh0) * a.head_tiles + (int64_t)own_tile * (own_tile + 1) / 2) * kStoredPairBytes +
-               col * 64 + half * 16;
+               lane * 16;
   auto store_tiles = [&](const Frag (&ds)[2], const Frag (&pk)[2]) __attribute__((always_inline)) {
     if constexpr (STORE) {
       if (t <= own_tile) {
@@ -484,8 +486,8 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
           // (written once and read once by the next pass: non-temporal, so that K and V stay in the caches)
-          __builtin_nontemporal_store(pk[u], reinterpret_cast<Frag *>(at + 32 * u));
-          __builtin_nontemporal_store(ds[u], reinterpret_cast<Frag *>(at + kStoredTileBytes + 32 * u));
+          __builtin_nontemporal_store(pk[u], reinterpret_cast<Frag *>(at + 1024 * u));
+          __builtin_nontemporal_store(ds[u], reinterpret_cast<Frag *>(at + kStoredTileBytes + 1024 * u));
         }
       }
     }
@@ -594,10 +596,15 @@ __global__ __launch_bounds__(kBlockThreads, bwd_blocks_per_cu(D, ROLE)) void att
   // each kind of tile in a loop of its own
   auto run_tiles = [&]<bool MASKED>(int end) __attribute__((always_inline)) {
     for (; t < end; ++t) {
-      // (vector-memory operations finish in order: behind the loads of tile t
-      // are those of tile t + 1 and the stores of the tile before this one)
-      if (!STORE || t - 1 <= own_tile) wait_vm<kLoadsPerTile + kStoresPerTile>();
-      else wait_vm<kLoadsPerTile>(); // (a wave past its diagonal stored nothing)
+      // (Vector-memory operations are counted in order. Behind the loads of tile t
+      // come the stores of tile t - 2, the loads of tile t + 1 and the stores of
+      // tile t - 1: none of them is waited for here. A store into the tile store
+      // takes long to be acknowledged; waited for a tile after it was issued, the
+      // stores cost this pass 100 us of 600.)
+      if (!STORE) wait_vm<kLoadsPerTile>();
+      else if (t - 1 > own_tile) wait_vm<kLoadsPerTile>(); // (a wave past its diagonal stored nothing)
+      else if (t - 2 < first_tile) wait_vm<kLoadsPerTile + kStoresPerTile>(); // (the block's second tile)
+      else wait_vm<kLoadsPerTile + 2 * kStoresPerTile>();
       __syncthreads(); // tile t is in LDS; the buffer written next (tile t - 2's) has been read
       scheduled_tile.template operator()<MASKED>();
     }
@@ -823,7 +830,11 @@ __global__ __launch_bounds__(stored_waves(D) * kWave, (stored_blocks_per_cu<T, D
     }
     it -= kLoadsN;
     // (read once: past the caches' usual replacement, so that the tiles of Q and dO stay)
-    lds_load_b128_once(store_descriptor(), x_lds + buf_load * kStoredTileBytes + it * 1024, (uint32_t)(it * 1024 + lane * 16));
+    // LDS gets rows of [query][slot] (lane L of load `it`: query 16 it + L / 4, 16-byte chunk L % 4 of its row);
+    // in memory that chunk, operand u = (L % 4) / 2 of half h = L % 2 of the wave that wrote it, lies at
+    // 1024 u + 16 (query + 32 h)
+    lds_load_b128_once(store_descriptor(), x_lds + buf_load * kStoredTileBytes + it * 1024,
+                       (uint32_t)(1024 * ((lane >> 1) & 1) + 16 * (16 * it + (lane >> 2) + 32 * (lane & 1))));
     if (it == 1) {
       store_at += (uint64_t)(store_tile + 1) * kStoredPairBytes;
       ++store_tile;
